@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the contraction hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only NAME]
+
+A step is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM.  The headline workload is the bf16 4096^3 GEMM; the
+int8 MLP layer, the bf16 MLP chain, fused attention and the f32 plumbing case
+are measured in the same run and reported under "others".  One JSON line goes
+to stdout; progress goes to stderr.
+
+Kernel durations come from HIP events recorded on the stream the kernels are
+launched on (torch's current stream), one pair per launch.  Inputs rotate over
+several buffer sets so that no launch finds its operands in the 256 MiB
+Infinity Cache from the previous one.
+"""
+import argparse
+import importlib.util
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"bf16": 2500.0, "int8": 5000.0, "f32": 157.3}  # dense MFMA, TFLOP/s | TOP/s
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def load_package():
+    pkg_dir = os.path.join(ROOT, "graph-compiler_amd")
+    spec = importlib.util.spec_from_file_location("graph_compiler_amd", os.path.join(pkg_dir, "__init__.py"),
+                                                  submodule_search_locations=[pkg_dir])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["graph_compiler_amd"] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def time_launches(torch, fn, nsets, steps, warmup):
+    """fn(i) launches one step on buffer set i.  Returns (ms_per_step over the
+    whole timed region, mean and min per-launch ms from per-launch events)."""
+    for i in range(warmup):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn(i % nsets)
+        stops[i].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per = sorted(s.elapsed_time(e) for s, e in zip(starts, stops))
+    region_ms = starts[0].elapsed_time(stops[-1])
+    return {"ms_per_step": region_ms / steps, "wall_ms_per_step": wall_ms / steps,
+            "kernel_ms_mean": sum(per) / len(per), "kernel_ms_min": per[0], "kernel_ms_median": per[len(per) // 2]}
+
+
+def roofline(ops, ms, peak_tops, traffic=None):
+    ach = ops / (ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": round(ach, 2), "peak": peak_tops, "unit": "TFLOP/s", "frac": round(ach / peak_tops, 4),
+            "traffic": traffic}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32")
+    ap.add_argument("--cpu-rows", type=int, default=512, help="rows of the 4096^3 GEMM the CPU baseline computes")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on ONE GPU (no sharding, no collectives); --gpus %d is not supported. "
+            "Every workload shards without communication over rows / (batch, head) -- run one process per GPU." % args.gpus)
+        sys.exit(2)
+
+    import torch
+    gc = load_package()
+    import importlib
+    wl = importlib.import_module("graph_compiler_amd.workloads")
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible; there is no CPU fallback for the product path")
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    gc.check(gc.lib().gcmi_init(0), "gcmi_init")
+    only = set(x for x in args.only.split(",") if x)
+    want = lambda n: not only or n in only  # noqa: E731
+    K, W = args.steps, args.warmup
+    others = {}
+
+    # ---------------- headline: bf16 GEMM 4096^3 (BASELINE configs[1])
+    M = N = Kd = 4096
+    flops = 2.0 * M * N * Kd
+    res = None
+    if want("gemm"):
+        nsets = 4  # 4 x 100 MB of operands+result > 256 MiB Infinity Cache
+        sets = []
+        for s in range(nsets):
+            A, B = wl.bf16_gemm(seed=10 * s)
+            sets.append((A.to(dev), B.to(dev), torch.empty(M, N, device=dev, dtype=torch.bfloat16)))
+        t = time_launches(torch, lambda i: gc.gemm_bf16(sets[i][0], sets[i][1], out=sets[i][2]), nsets, K, W)
+        res = t
+        log("bf16 gemm 4096^3: %.4f ms/launch  %.1f TFLOP/s" % (t["kernel_ms_mean"], flops / t["kernel_ms_mean"] / 1e9))
+        del sets
+        torch.cuda.empty_cache()
+
+    # ---------------- int8 MLP layer (configs[2])
+    if want("int8"):
+        Mi, Ki, Ni = 4096, 4096, 11008
+        ops = 2.0 * Mi * Ki * Ni
+        nsets = 3
+        sets = []
+        for s in range(nsets):
+            A, Wt, sc, bs = wl.int8_mlp_layer(seed=10 * s)
+            Wd = Wt.to(dev)
+            sets.append((A.to(dev), Wd, gc.colsum_s8(Wd), sc.to(dev), bs.to(dev),
+                         torch.empty(Mi, Ni, device=dev, dtype=torch.bfloat16)))
+        t = time_launches(torch, lambda i: gc.gemm_int8(sets[i][0], sets[i][1], sets[i][2], 128, sets[i][3], sets[i][4],
+                                                        "gelu_erf", gc.BF16, sets[i][5]), nsets, K, W)
+        tc = time_launches(torch, lambda i: gc.colsum_s8(sets[i][1]), nsets, 10, 2)
+        others["int8_mlp_layer"] = {"workload": "u8[4096x4096] x s8[4096x11008] -> s32 -> dequant+bias+GELU -> bf16",
+                                    "value": round(ops / t["ms_per_step"] / 1e9, 2), "unit": "TOP/s", "dtype": "int8",
+                                    "ms_per_step": round(t["ms_per_step"], 5),
+                                    "roofline": roofline(ops, t["kernel_ms_mean"], PEAK["int8"]),
+                                    "weight_colsum_precompute_ms": round(tc["kernel_ms_mean"], 5)}
+        others["int8_mlp_layer"]["roofline"]["unit"] = "TOP/s"
+        log("int8 mlp layer: %.4f ms  %.1f TOP/s" % (t["kernel_ms_mean"], ops / t["kernel_ms_mean"] / 1e9))
+        del sets
+        torch.cuda.empty_cache()
+
+    # ---------------- bf16 MLP chain (configs[3]): two launches per step
+    if want("chain"):
+        Mc, Kc, Hc = 4096, 4096, 11008
+        ops = 2 * 2.0 * Mc * Kc * Hc
+        nsets = 2
+        sets = []
+        for s in range(nsets):
+            x, W1, W2, b2 = wl.bf16_mlp_chain(seed=10 * s)
+            sets.append((x.to(dev), W1.to(dev), W2.to(dev), b2.to(dev),
+                         torch.empty(Mc, Hc, device=dev, dtype=torch.bfloat16),
+                         torch.empty(Mc, Kc, device=dev, dtype=torch.bfloat16)))
+
+        def chain(i):
+            x, W1, W2, b2, h, y = sets[i]
+            gc.gemm_bf16(x, W1, None, "relu", out=h)
+            gc.gemm_bf16(h, W2, b2, None, out=y)
+
+        t = time_launches(torch, chain, nsets, K, W)
+        others["bf16_mlp_chain"] = {"workload": "x[4096x4096] -> W1[4096x11008]+ReLU -> W2[11008x4096]+bias, bf16",
+                                    "value": round(ops / t["ms_per_step"] / 1e9, 2), "unit": "TFLOP/s", "dtype": "bf16",
+                                    "ms_per_step": round(t["ms_per_step"], 5),
+                                    "roofline": roofline(ops, t["kernel_ms_mean"], PEAK["bf16"])}
+        log("bf16 mlp chain: %.4f ms  %.1f TFLOP/s" % (t["kernel_ms_mean"], ops / t["kernel_ms_mean"] / 1e9))
+        del sets
+        torch.cuda.empty_cache()
+
+    # ---------------- fused attention (configs[4])
+    if want("mha"):
+        Bm, Hm, Sm, Dm = 4, 32, 2048, 128
+        ops = 4.0 * Bm * Hm * Sm * Sm * Dm  # dense count: the mask is data
+        nsets = 2
+        sets = []
+        for s in range(nsets):
+            Q, Kk, V, mask, scale = wl.bf16_mha(seed=10 * s)
+            sets.append((Q.to(dev), Kk.to(dev), V.to(dev), mask.to(dev), torch.empty(Bm, Hm, Sm, Dm, device=dev, dtype=torch.bfloat16)))
+        t = time_launches(torch, lambda i: gc.mha_fwd_bf16(sets[i][0], sets[i][1], sets[i][2], sets[i][3], scale, sets[i][4]),
+                          nsets, K, W)
+        others["bf16_mha"] = {"workload": "B4 H32 S2048 D128, additive causal mask f32[2048,2048] read as data",
+                              "value": round(ops / t["ms_per_step"] / 1e9, 2), "unit": "TFLOP/s (dense 4*B*H*S*S*D)",
+                              "dtype": "bf16", "ms_per_step": round(t["ms_per_step"], 5),
+                              "roofline": roofline(ops, t["kernel_ms_mean"], PEAK["bf16"])}
+        log("bf16 mha: %.4f ms  %.1f TFLOP/s (dense count)" % (t["kernel_ms_mean"], ops / t["kernel_ms_mean"] / 1e9))
+        del sets
+        torch.cuda.empty_cache()
+
+    # ---------------- f32 plumbing case (configs[0])
+    if want("f32"):
+        A, B, bias = wl.f32_matmul_bias_relu()
+        Ad, Bd, bd = A.to(dev), B.to(dev), bias.to(dev)
+        out = torch.empty(128, 256, device=dev)
+        t = time_launches(torch, lambda i: gc.gemm_f32(Ad, Bd, bd, "relu", out=out), 1, K, W)
+        others["f32_matmul_bias_relu"] = {"workload": "A[128x512].B[512x256]+bias+ReLU f32 (launch bound)",
+                                          "ms_per_step": round(t["ms_per_step"], 5),
+                                          "value": round(2.0 * 128 * 512 * 256 / t["kernel_ms_mean"] / 1e9, 4), "unit": "TFLOP/s"}
+
+    # ---------------- CPU baseline: the oracle's deep-tile nest on a bounded sample
+    cpu = None
+    if not args.no_cpu and want("gemm"):
+        from oracle import gc_oracle as orc
+        rows = args.cpu_rows
+        A, B = wl.bf16_gemm(M=rows, seed=0)
+        a16, b16 = wl.bf16_bits(A), wl.bf16_bits(B)
+        nt = orc.num_threads()
+        t0 = time.perf_counter()
+        orc.matmul_bf16(a16, b16)
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(2.0 * rows * N * Kd / dt / 1e12, 5), "unit": "TFLOP/s", "cores": nt, "kind": "port",
+               "sample": "first %d of 4096 rows of the same bf16 4096^3 GEMM (deep-tile nest, 32^3 brgemm restatement, "
+                         "gcc -O3 -march=native, OpenMP), %.2f s" % (rows, dt)}
+        log("cpu baseline: %.4f TFLOP/s on %d threads (%.2f s)" % (cpu["value"], nt, dt))
+
+    line = {
+        "metric": "TFLOPS/TOPS + % of MI355X MFMA peak: bf16 4096^3 GEMM, int8 MLP, bf16 MHA",
+        "value": round(flops / res["ms_per_step"] / 1e9, 2) if res else None,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(res["ms_per_step"], 5) if res else None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "bf16 GEMM M=N=K=4096, row-major A and B, N(0,1)*0.1, f32 accumulate, bf16 out, no post-op",
+                   "buffer_sets": 4},
+        "roofline": roofline(flops, res["kernel_ms_mean"], PEAK["bf16"]) if res else None,
+        "cpu_baseline": cpu,
+        "kernel_ms": {k: round(v, 5) for k, v in res.items()} if res else None,
+        "others": others,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

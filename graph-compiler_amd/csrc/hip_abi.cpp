@@ -1,0 +1,236 @@
+// The thin C-ABI layer between host code and the HIP kernels: argument
+// validation, parameter-block assembly, launches.  This and the kernels' own
+// launch stubs are the only translation units that touch the HIP runtime for
+// compute; nothing here allocates device memory.
+#include <hip/hip_runtime_api.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <shared_mutex>
+#include <vector>
+
+#include "gc_brgemm.h"
+#include "gc_hip_kernels.h"
+#include "kernels/gemm_params.h"
+
+using namespace gcmi;
+
+extern "C" {
+int gcmi_launch_gemm_tile256(const GemmParams *p, int es, hipStream_t stream);
+int gcmi_launch_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, void *out, hipStream_t stream);
+int gcmi_launch_gemm_f32(const F32GemmParams *p, hipStream_t stream);
+int gcmi_launch_brgemm(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t LDA,
+                       int64_t LDB, int64_t LDC, int64_t stride_a, int64_t stride_b, int num, int beta_zero, int dtA,
+                       int dtB, hipStream_t stream);
+int gcmi_launch_mha_fwd(const MhaParams *p, hipStream_t stream);
+}
+
+namespace {
+thread_local char g_err[256] = "";
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+enum { ST_OK = 0, ST_INVALID = 2, ST_UNIMPL = 3, ST_RUNTIME = 5 };
+int launched(int rc, const char *what) {
+  if (rc == 0)
+    return ST_OK;
+  return fail(rc, "%s: launch failed (%s)", what, hipGetErrorString(hipPeekAtLastError()));
+}
+} // namespace
+
+extern "C" const char *gcmi_last_error(void) { return g_err; }
+
+extern "C" int gcmi_init(int device) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n <= 0)
+    return fail(ST_RUNTIME, "no HIP device visible");
+  if (device < 0 || device >= n)
+    return fail(ST_INVALID, "device %d out of range (%d visible)", device, n);
+  if (hipSetDevice(device) != hipSuccess)
+    return fail(ST_RUNTIME, "hipSetDevice(%d) failed", device);
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, device) != hipSuccess)
+    return fail(ST_RUNTIME, "hipGetDeviceProperties failed");
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(ST_UNIMPL, "device is %s; these kernels are built for gfx950 only", prop.gcnArchName);
+  return ST_OK;
+}
+
+extern "C" int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                              int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype,
+                              void *stream) {
+  if (M < 0 || N < 0 || K < 0)
+    return fail(ST_INVALID, "gemm_bf16: negative size");
+  if (M == 0 || N == 0)
+    return ST_OK;
+  if (!A || !B || !C)
+    return fail(ST_INVALID, "gemm_bf16: null operand");
+  if (lda < K || ldb < N || ldc < N)
+    return fail(ST_INVALID, "gemm_bf16: leading dimension smaller than the row (lda %lld ldb %lld ldc %lld)",
+                (long long)lda, (long long)ldb, (long long)ldc);
+  if (out_dtype != GCMI_BF16 && out_dtype != GCMI_F32)
+    return fail(ST_UNIMPL, "gemm_bf16: out_dtype %d", out_dtype);
+  if (bias && bias_dtype != GCMI_BF16 && bias_dtype != GCMI_F32)
+    return fail(ST_UNIMPL, "gemm_bf16: bias_dtype %d", bias_dtype);
+  if (act < GCMI_ACT_NONE || act > GCMI_ACT_SIGMOID)
+    return fail(ST_INVALID, "gemm_bf16: act %d", act);
+  GemmParams p{};
+  p.A = A, p.B = B, p.C = C, p.M = M, p.N = N, p.K = K, p.lda = lda, p.ldb = ldb, p.ldc = ldc;
+  p.bias = bias, p.bias_dt = bias_dtype, p.act = act, p.out_dt = out_dtype;
+  return launched(gcmi_launch_gemm_tile256(&p, 2, (hipStream_t)stream), "gemm_bf16");
+}
+
+extern "C" int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K,
+                              int64_t lda, int64_t ldb, int64_t ldc, const int32_t *colsum, int32_t zp_a,
+                              const float *scale, const float *bias, int act, int out_dtype, void *stream) {
+  if (M < 0 || N < 0 || K < 0)
+    return fail(ST_INVALID, "gemm_int8: negative size");
+  if (M == 0 || N == 0)
+    return ST_OK;
+  if (!A || !W || !C)
+    return fail(ST_INVALID, "gemm_int8: null operand");
+  if (a_dtype != GCMI_U8 && a_dtype != GCMI_S8)
+    return fail(ST_UNIMPL, "gemm_int8: a_dtype %d", a_dtype);
+  if (lda < K || ldb < N || ldc < N)
+    return fail(ST_INVALID, "gemm_int8: leading dimension smaller than the row");
+  if (out_dtype != GCMI_S32 && out_dtype != GCMI_F32 && out_dtype != GCMI_BF16)
+    return fail(ST_UNIMPL, "gemm_int8: out_dtype %d", out_dtype);
+  if (act < GCMI_ACT_NONE || act > GCMI_ACT_SIGMOID)
+    return fail(ST_INVALID, "gemm_int8: act %d", act);
+  // The matrix cores multiply signed bytes.  u8 activations enter as
+  // (a ^ 0x80) = a - 128, so acc_true = acc_mfma + 128*colsum, and the
+  // zero-point compensation subtracts zp_a*colsum: both fold into one integer
+  // factor of colsum.
+  const int32_t shift = a_dtype == GCMI_U8 ? 128 : 0;
+  const int32_t comp = out_dtype == GCMI_S32 ? shift : shift - zp_a;
+  if (comp != 0 && !colsum)
+    return fail(ST_INVALID, "gemm_int8: colsum is required for u8 activations or a non-zero zero point");
+  GemmParams p{};
+  p.A = A, p.B = W, p.C = C, p.M = M, p.N = N, p.K = K, p.lda = lda, p.ldb = ldb, p.ldc = ldc;
+  p.bias = bias, p.bias_dt = GCMI_F32, p.scale = scale, p.colsum = comp ? colsum : nullptr, p.comp = comp;
+  p.a_xor = a_dtype == GCMI_U8 ? 0x80808080u : 0u;
+  p.act = out_dtype == GCMI_S32 ? GCMI_ACT_NONE : act, p.out_dt = out_dtype;
+  return launched(gcmi_launch_gemm_tile256(&p, 1, (hipStream_t)stream), "gemm_int8");
+}
+
+extern "C" int gcmi_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, int32_t *colsum, void *stream) {
+  if (K < 0 || N < 0 || ldw < N)
+    return fail(ST_INVALID, "colsum_s8: bad shape");
+  if (N == 0)
+    return ST_OK;
+  if (!W || !colsum)
+    return fail(ST_INVALID, "colsum_s8: null operand");
+  return launched(gcmi_launch_colsum_s8(W, K, N, ldw, colsum, (hipStream_t)stream), "colsum_s8");
+}
+
+extern "C" int gcmi_gemm_f32(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                             int64_t ldb, int64_t ldc, int trans_a, int trans_b, const float *bias, int act,
+                             void *stream) {
+  if (M < 0 || N < 0 || K < 0)
+    return fail(ST_INVALID, "gemm_f32: negative size");
+  if (M == 0 || N == 0)
+    return ST_OK;
+  if (!A || !B || !C)
+    return fail(ST_INVALID, "gemm_f32: null operand");
+  if (lda < (trans_a ? M : K) || ldb < (trans_b ? K : N) || ldc < N)
+    return fail(ST_INVALID, "gemm_f32: leading dimension smaller than the row");
+  if (act < GCMI_ACT_NONE || act > GCMI_ACT_SIGMOID)
+    return fail(ST_INVALID, "gemm_f32: act %d", act);
+  F32GemmParams p{};
+  p.A = A, p.B = B, p.C = C, p.M = M, p.N = N, p.K = K;
+  p.a_rs = trans_a ? 1 : lda, p.a_cs = trans_a ? lda : 1;
+  p.b_rs = trans_b ? 1 : ldb, p.b_cs = trans_b ? ldb : 1;
+  p.ldc = ldc, p.bias = bias, p.act = act, p.beta = 0.0f;
+  return launched(gcmi_launch_gemm_f32(&p, (hipStream_t)stream), "gemm_f32");
+}
+
+extern "C" int gcmi_mha_fwd_bf16(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld,
+                                 void *O, int64_t BH, int64_t Sq, int64_t Sk, int64_t D, float scale, void *stream) {
+  if (BH < 0 || Sq < 0 || Sk < 0)
+    return fail(ST_INVALID, "mha_fwd: negative size");
+  if (D != 128)
+    return fail(ST_UNIMPL, "mha_fwd: head_dim %lld (only 128 is built)", (long long)D);
+  if (BH == 0 || Sq == 0)
+    return ST_OK;
+  if (Sk == 0)
+    return fail(ST_INVALID, "mha_fwd: no keys");
+  if (!Q || !K || !V || !O)
+    return fail(ST_INVALID, "mha_fwd: null operand");
+  if (mask && mask_ld < Sk)
+    return fail(ST_INVALID, "mha_fwd: mask_ld < Sk");
+  if (BH > 0x7fffffff || Sq > 0x7fffffff || Sk > 0x7fffffff)
+    return fail(ST_INVALID, "mha_fwd: size too large");
+  MhaParams p{};
+  p.Q = Q, p.K = K, p.V = V, p.O = O, p.mask = mask, p.mask_ld = mask_ld;
+  p.BH = (int)BH, p.Sq = (int)Sq, p.Sk = (int)Sk, p.D = (int)D, p.scale = scale;
+  int rc = gcmi_launch_mha_fwd(&p, (hipStream_t)stream);
+  if (rc == 2)
+    return fail(ST_INVALID, "mha_fwd: Q/K/V/O must be 16-byte aligned");
+  return launched(rc, "mha_fwd");
+}
+
+// ---------------------------------------------------------------------------
+// Microkernel ABI: dispatch-once / execute-many, as the reference's runtime
+// (lib/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmOnednn.cpp:74-168).
+namespace {
+struct BrgemmDesc {
+  int64_t M, N, K, LDA, LDB, LDC, stride_a, stride_b;
+  float beta;
+  int64_t dtA, dtB;
+};
+std::shared_mutex g_brgemm_lock;
+std::vector<BrgemmDesc> &brgemm_table() {
+  static std::vector<BrgemmDesc> *t = new std::vector<BrgemmDesc>(); // never freed: handles stay valid at exit
+  return *t;
+}
+bool brgemm_pair_ok(int64_t a, int64_t b) {
+  auto i8 = [](int64_t d) { return d == GCMI_S8 || d == GCMI_U8; };
+  return (a == GCMI_F32 && b == GCMI_F32) || (a == GCMI_BF16 && b == GCMI_BF16) || (i8(a) && i8(b));
+}
+} // namespace
+
+extern "C" int64_t dnnl_brgemm_dispatch(int64_t M, int64_t N, int64_t K, int64_t LDA, int64_t LDB, int64_t LDC,
+                                        int64_t stride_a, int64_t stride_b, float beta, int64_t dtypeA,
+                                        int64_t dtypeB) {
+  if (M < 0 || N < 0 || K < 0 || !brgemm_pair_ok(dtypeA, dtypeB)) {
+    fail(ST_INVALID, "brgemm_dispatch: unsupported shape or dtype pair (%lld,%lld)", (long long)dtypeA,
+         (long long)dtypeB);
+    return -1;
+  }
+  std::unique_lock<std::shared_mutex> g(g_brgemm_lock);
+  auto &t = brgemm_table();
+  t.push_back(BrgemmDesc{M, N, K, LDA, LDB, LDC, stride_a, stride_b, beta, dtypeA, dtypeB});
+  return (int64_t)t.size() - 1;
+}
+
+extern "C" void dnnl_brgemm_tileconfig(int64_t) {}
+extern "C" void dnnl_brgemm_tilerelease(void) {}
+
+extern "C" void dnnl_brgemm_execute(int64_t kernel, void *A, uint64_t A_offset, void *B, uint64_t B_offset, void *C,
+                                    uint64_t C_offset, int num) {
+  BrgemmDesc d;
+  {
+    std::shared_lock<std::shared_mutex> g(g_brgemm_lock);
+    auto &t = brgemm_table();
+    if (kernel < 0 || kernel >= (int64_t)t.size()) {
+      fail(ST_INVALID, "brgemm_execute: invalid kernel handle %lld", (long long)kernel);
+      return;
+    }
+    d = t[(size_t)kernel];
+  }
+  const int es = d.dtA == GCMI_F32 ? 4 : (d.dtA == GCMI_BF16 ? 2 : 1);
+  const int ces = 4;
+  const char *a = (const char *)A + A_offset * es;
+  const char *b = (const char *)B + B_offset * es;
+  char *c = (char *)C + C_offset * ces;
+  int rc = gcmi_launch_brgemm(a, b, c, d.M, d.N, d.K, d.LDA, d.LDB, d.LDC, d.stride_a, d.stride_b, num,
+                              d.beta == 0.0f ? 1 : 0, (int)d.dtA, (int)d.dtB, nullptr);
+  if (rc)
+    fail(rc, "brgemm_execute: launch failed");
+}

@@ -1,0 +1,61 @@
+// Shared device-side vocabulary for the gfx950 kernels: vector types, bf16
+// rounding, post-op (epilogue) math.  Wave size is 64 throughout.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gcmi {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x16_t __attribute__((ext_vector_type(16)));
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x4_t __attribute__((ext_vector_type(4)));
+
+#define GCMI_LDS __attribute__((address_space(3)))
+
+// post-op kinds fused into a GEMM epilogue
+enum Act : int { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU_ERF = 2, ACT_GELU_TANH = 3, ACT_SIGMOID = 4 };
+
+// dnnl_data_type_t values used across the C ABI
+enum DType : int { DT_F16 = 1, DT_BF16 = 2, DT_F32 = 3, DT_S32 = 4, DT_S8 = 5, DT_U8 = 6 };
+
+// f32 -> bf16, round to nearest even, NaN -> 0x7FC0: the reference's bf16_t
+// constructor (include/gc/ExecutionEngine/CPURuntime/Microkernel/
+// BrgemmInterface.h:83-92).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) {
+  uint32_t bits = __float_as_uint(v);
+  uint32_t r = (bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16;
+  return (v != v) ? (uint16_t)0x7FC0u : (uint16_t)r;
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+__device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+// Activation in f32.  Operation order follows the reference graphs:
+// ReLU   = max(x, 0), NaN propagates (lib/gc/Transforms/OneDNNGraphToLinalg.cpp:355-358)
+// GELU   = ((erf(x*c)+1)*x)*0.5, c = 0x3f3504f3 (legacy/core/src/ops/gelu.cpp:110-131)
+// tanh   = (x*(tanh((((x*x)*0.044715+1)*x)*0.79788458)+1))*0.5 (gelu.cpp:78-108)
+// sigmoid= 1/(1+exp(-x)) (lib/gc/Dialect/Linalgx/LinalgxOps.cpp:42-61)
+__device__ __forceinline__ float apply_act(float x, int act) {
+  switch (act) {
+  case ACT_RELU:
+    return (x != x) ? x : fmaxf(x, 0.0f);
+  case ACT_GELU_ERF: {
+    const float c = __uint_as_float(0x3f3504f3u);
+    return ((erff(x * c) + 1.0f) * x) * 0.5f;
+  }
+  case ACT_GELU_TANH: {
+    float t = (((x * x) * 0.044715f + 1.0f) * x) * 0.79788458f;
+    return (x * (tanhf(t) + 1.0f)) * 0.5f;
+  }
+  case ACT_SIGMOID:
+    return 1.0f / (1.0f + expf(-x));
+  default:
+    return x;
+  }
+}
+
+} // namespace gcmi

@@ -1,0 +1,288 @@
+// Fused multi-head attention forward for gfx950 (bf16, head_dim 128):
+//   O = softmax(Q K^T * scale + mask) V
+// i.e. the composition batch_matmul_transpose_b -> scale -> +mask -> softmax ->
+// batch_matmul that the reference would run as separate ops
+// (lib/gc/Transforms/DecomposeAggregatedOps.cpp:24-38 for the softmax;
+// test/benchgc/src/benchgc/linalg/matmul.py:29-32,65-68 for the two batch
+// matmuls), computed in one pass with an online softmax so the [Sq,Sk] score
+// matrix never leaves registers.
+//
+// Work split: one workgroup = 128 query rows of one (batch, head); 4 waves x 32
+// rows.  Keys/values stream through LDS in blocks of 64 (K 16 KiB + V 16 KiB,
+// double buffered = 64 KiB, two workgroups per CU).
+//
+// Everything is kept TRANSPOSED in the accumulators:
+//   S^T[key, q] = K . Q^T      MFMA 32x32x16: first operand = K rows (d is
+//                              contiguous in memory -> ds_read_b128), second =
+//                              Q rows held in registers for the whole kernel
+//   O^T[d, q]  += V^T . P^T    first operand = V^T, read from the row-major V
+//                              tile with ds_read_b64_tr_b16; second = P^T taken
+//                              straight from the S^T accumulator registers
+// In the 32x32 accumulator layout a lane owns ONE query column and 16 of the 32
+// keys of a tile, so row max / row sum are in-lane reductions plus a single
+// exchange with lane^32, and the softmax weights feed the second MFMA without
+// any cross-lane movement: the contraction index of that MFMA is simply
+// enumerated in the order the accumulator registers hold the keys
+// (lane half h, register e -> key 16*j + 8*(e/4) + 4*h + e%4), and the V^T
+// fragment is fetched in the same order.
+//
+// Workgroup order: query block is the fast index, (batch, head) the slow one.
+// Consecutive workgroup ids go to different XCDs, so XCD x only ever touches
+// the mask rows of query blocks congruent to x mod 8: a few MiB that stay
+// resident in its L2 while K/V of successive heads stream through.
+#include "common.hpp"
+#include "gemm_params.h"
+
+namespace gcmi {
+
+static constexpr int FA_BQ = 128, FA_BK = 64, FA_D = 128, FA_THREADS = 256;
+static constexpr int FA_TILE_BYTES = FA_BK * FA_D * 2; // 16 KiB
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+template <bool HAS_MASK, bool EDGE> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fwd_kernel(MhaParams p) {
+  __shared__ __align__(16) char smem[2][2][FA_TILE_BYTES]; // [stage][0=K,1=V]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, lh = lane >> 5;
+  const int nqb = (p.Sq + FA_BQ - 1) / FA_BQ;
+  const int qb = blockIdx.x % nqb, bh = blockIdx.x / nqb;
+  const int q_lane = qb * FA_BQ + wave * 32 + l32; // the query row this lane owns
+  const bool q_ok = !EDGE || q_lane < p.Sq;
+
+  const char *Qb = reinterpret_cast<const char *>(p.Q) + (int64_t)bh * p.Sq * FA_D * 2;
+  const char *Kb = reinterpret_cast<const char *>(p.K) + (int64_t)bh * p.Sk * FA_D * 2;
+  const char *Vb = reinterpret_cast<const char *>(p.V) + (int64_t)bh * p.Sk * FA_D * 2;
+
+  // Q^T fragments (second MFMA operand): lane = query, 8 consecutive d per 16-step
+  uint4 qf[8];
+#pragma unroll
+  for (int ds = 0; ds < 8; ds++)
+    qf[ds] = q_ok ? *reinterpret_cast<const uint4 *>(Qb + (int64_t)q_lane * FA_D * 2 + ds * 32 + lh * 16)
+                  : make_uint4(0, 0, 0, 0);
+
+  // global -> LDS staging: 4 chunks of K and 4 of V per thread per block
+  const int st_key0 = tid >> 4, st_c = tid & 15; // keys st_key0 + 16*i
+  uint32_t k_st[4], v_st[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    int key = st_key0 + 16 * i;
+    k_st[i] = key * 256 + ((st_c ^ (key & 15)) << 4);
+    v_st[i] = key * 256 + ((st_c ^ ((key & 3) << 2)) << 4);
+  }
+  // LDS fragment offsets
+  uint32_t k_ld[8]; // + kt*8192
+#pragma unroll
+  for (int ds = 0; ds < 8; ds++)
+    k_ld[ds] = l32 * 256 + (((ds * 2 + lh) ^ (l32 & 15)) << 4);
+  uint32_t v_ld[4]; // + (kt*32 + 16*h2 + 8*rd)*256
+  {
+    const int g = lane >> 4, i16 = lane & 15, kk = i16 >> 2, cc = i16 & 3;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+      v_ld[dt] = (4 * lh + kk) * 256 + (((dt * 4 + 2 * (g & 1) + (cc >> 1)) ^ (kk << 2)) << 4) + (cc & 1) * 8;
+  }
+
+  f32x16_t o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+      o[dt][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  const float LOG2E = 1.4426950408889634f;
+  const float sl2 = p.scale * LOG2E;
+  const int nkb = (p.Sk + FA_BK - 1) / FA_BK;
+  uint4 rk[4], rv[4];
+
+  auto gload = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      int key = kb * FA_BK + st_key0 + 16 * i;
+      if (!EDGE || key < p.Sk) {
+        rk[i] = *reinterpret_cast<const uint4 *>(Kb + (int64_t)key * FA_D * 2 + st_c * 16);
+        rv[i] = *reinterpret_cast<const uint4 *>(Vb + (int64_t)key * FA_D * 2 + st_c * 16);
+      } else {
+        rk[i] = make_uint4(0, 0, 0, 0);
+        rv[i] = make_uint4(0, 0, 0, 0);
+      }
+    }
+  };
+  auto lstore = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      *reinterpret_cast<uint4 *>(&smem[stage][0][k_st[i]]) = rk[i];
+      *reinterpret_cast<uint4 *>(&smem[stage][1][v_st[i]]) = rv[i];
+    }
+  };
+
+  gload(0);
+  lstore(0);
+  __syncthreads();
+
+  for (int kb = 0; kb < nkb; kb++) {
+    const int cur = kb & 1;
+    if (kb + 1 < nkb)
+      gload(kb + 1);
+    const char *sK = &smem[cur][0][0];
+    const char *sV = &smem[cur][1][0];
+
+    // ---- S^T = K . Q^T for 64 keys x 32 queries
+    f32x16_t s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        s[kt][r] = 0.0f;
+#pragma unroll
+      for (int ds = 0; ds < 8; ds++) {
+        uint4 kf = *reinterpret_cast<const uint4 *>(sK + k_ld[ds] + kt * 8192);
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf),
+                                                        __builtin_bit_cast(bf16x8_t, qf[ds]), s[kt], 0, 0, 0);
+      }
+    }
+
+    // ---- scale, additive mask, to log2 domain; block max
+    float m_blk = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const int key = kb * FA_BK + kt * 32 + 8 * q4 + 4 * lh;
+        float mk[4] = {0.f, 0.f, 0.f, 0.f};
+        if (HAS_MASK) {
+          if (!EDGE) {
+            f32x4_t mv = *reinterpret_cast<const f32x4_t *>(p.mask + (int64_t)q_lane * p.mask_ld + key);
+            mk[0] = mv[0];
+            mk[1] = mv[1];
+            mk[2] = mv[2];
+            mk[3] = mv[3];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              mk[e] = (q_ok && key + e < p.Sk) ? p.mask[(int64_t)q_lane * p.mask_ld + key + e] : 0.0f;
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          float v = s[kt][4 * q4 + e] * sl2;
+          if (HAS_MASK)
+            v = v + mk[e] * LOG2E;
+          if (EDGE && key + e >= p.Sk)
+            v = -INFINITY;
+          s[kt][4 * q4 + e] = v;
+          m_blk = fmaxf(m_blk, v);
+        }
+      }
+    }
+    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32));
+
+    // ---- online softmax update
+    const float m_new = fmaxf(m_run, m_blk);
+    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new; // fully masked so far: keep exp2 finite
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    m_run = m_new;
+    float l_blk = 0.0f;
+    uint32_t pk[2][8]; // bf16 pairs: pk[kt][e2] = (p[2*e2], p[2*e2+1])
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        float p0 = __builtin_amdgcn_exp2f(s[kt][r] - m_use);
+        float p1 = __builtin_amdgcn_exp2f(s[kt][r + 1] - m_use);
+        l_blk += p0 + p1;
+        pk[kt][r >> 1] = pack_bf16x2(p0, p1);
+      }
+    }
+    l_run = l_run * alpha + l_blk;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          o[dt][r] *= alpha;
+    }
+
+    // ---- O^T += V^T . P^T
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+      for (int h2 = 0; h2 < 2; h2++) {
+        uint4 pf = make_uint4(pk[kt][4 * h2 + 0], pk[kt][4 * h2 + 1], pk[kt][4 * h2 + 2], pk[kt][4 * h2 + 3]);
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+          const char *vp = sV + v_ld[dt] + (kt * 32 + 16 * h2) * 256;
+          bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((GCMI_LDS bf16x4_t *)vp);
+          bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((GCMI_LDS bf16x4_t *)(vp + 8 * 256));
+          uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+          uint4 vf = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf),
+                                                          __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
+        }
+      }
+    }
+
+    if (kb + 1 < nkb)
+      lstore(cur ^ 1);
+    __syncthreads();
+  }
+
+  // ---- normalise and store: lane owns query q_lane, d = dt*32 + 8*q4 + 4*lh + e
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = 1.0f / l_tot; // l_tot == 0 (row fully masked): 0 * inf = NaN, as softmax of all -inf
+  if (q_ok) {
+    char *Ob = reinterpret_cast<char *>(p.O) + ((int64_t)bh * p.Sq + q_lane) * FA_D * 2;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        uint16_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          h[e] = f32_to_bf16_bits(o[dt][4 * q4 + e] * inv);
+        *reinterpret_cast<uint2 *>(Ob + (dt * 32 + 8 * q4 + 4 * lh) * 2) =
+            make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+      }
+  }
+}
+
+} // namespace gcmi
+
+using namespace gcmi;
+
+extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
+  MhaParams p = *pp;
+  if (p.D != FA_D)
+    return 3;
+  if (p.BH <= 0 || p.Sq <= 0 || p.Sk <= 0)
+    return 0;
+  const int nqb = (p.Sq + FA_BQ - 1) / FA_BQ;
+  const int64_t nblk = (int64_t)nqb * p.BH;
+  if (nblk > 0x7fffffff)
+    return 2;
+  auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  bool fast = p.Sq % FA_BQ == 0 && p.Sk % FA_BK == 0 && al16(p.Q) && al16(p.K) && al16(p.V) && al16(p.O) &&
+              (!p.mask || (al16(p.mask) && p.mask_ld % 4 == 0));
+  if (!(al16(p.Q) && al16(p.K) && al16(p.V) && al16(p.O)))
+    return 2; // rows are 256 bytes: a 16-byte aligned base is required
+  dim3 grid((unsigned)nblk), block(FA_THREADS);
+  if (p.mask) {
+    if (fast)
+      hipLaunchKernelGGL((mha_fwd_kernel<true, false>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((mha_fwd_kernel<true, true>), grid, block, 0, stream, p);
+  } else {
+    if (fast)
+      hipLaunchKernelGGL((mha_fwd_kernel<false, false>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((mha_fwd_kernel<false, true>), grid, block, 0, stream, p);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : 5;
+}

@@ -1,0 +1,396 @@
+// Whole-problem MFMA GEMM for gfx950 with a register-fused epilogue.
+//
+// Replaces the reference's "outer loops + brgemm microkernel call" structure
+// (lib/gc/Transforms/DeepTileContractionOp.cpp:506-540 calling
+// dnnl_brgemm_execute, lib/gc/ExecutionEngine/CPURuntime/Microkernel/
+// BrgemmOnednn.cpp:145-168) by one kernel per matmul:
+//   C[M,N] = epilogue( A[M,K] . B[K,N] ),  A and B plain row-major.
+// ES = 2: bf16 x bf16 -> f32 accumulate (v_mfma_f32_32x32x16_bf16)
+// ES = 1: (u8|s8) x s8 -> s32 accumulate (v_mfma_i32_32x32x32_i8)
+//
+// Workgroup tile 256 x 256, 128 bytes of K per stage (64 bf16 / 128 int8),
+// 8 waves as 2 (M) x 4 (N), wave tile 128 x 64 = 4 x 2 MFMA tiles of 32 x 32.
+// LDS: two stages of {A 256 rows x 128 B, B (128/ES) rows x 256*ES B} = 128 KiB.
+//
+// Operand roles are swapped on purpose: the MFMA's first operand is the B
+// fragment (rows = n), the second the A fragment (columns = m).  The 32x32
+// accumulator then gives every lane 4 consecutive n for one m, so the epilogue
+// stores 8 (bf16) or 16 (f32/s32) contiguous bytes per lane and reads bias /
+// scale / colsum as 4-vectors.
+//
+// B is row-major [K,N] (n contiguous) while the MFMA wants k-contiguous
+// fragments: the transposition happens in the LDS read with
+// ds_read_b64_tr_b16 / ds_read_b64_tr_b8, so the tile is stored exactly as it
+// lies in memory.  This is the GPU analogue of the VNNI re-layout the
+// reference's brgemm requires of B (lib/gc/Dialect/Microkernel/
+// MicrokernelOps.cpp:380-389) without a separate packing pass.
+//
+// LDS swizzles (16-byte chunk index XOR):
+//   A: chunk ^= (row >> 1) & 7        -> ds_read_b128 of 32 rows x 16 B is
+//                                        conflict free over 64 banks
+//   B: chunk ^= (krow % RG) * CW      -> RG = rows per transpose group (4 for
+//                                        16-bit, 8 for 8-bit), CW = 16-byte
+//                                        chunks one read touches per row
+#include "common.hpp"
+#include "gemm_params.h"
+
+namespace gcmi {
+
+static constexpr int G_BM = 256, G_BN = 256, G_KBYTES = 128;
+static constexpr int G_THREADS = 512;
+static constexpr int G_STAGE_BYTES = 65536; // A 32 KiB + B 32 KiB
+
+template <int ES> struct MfmaOp;
+template <> struct MfmaOp<2> {
+  typedef f32x16_t acc_t;
+  typedef float acc_elem_t;
+  static __device__ __forceinline__ acc_t run(const uint4 &a, const uint4 &b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
+                                                   0, 0, 0);
+  }
+  // 8 bytes: k..k+3 of one n
+  static __device__ __forceinline__ uint2 tr_read(const char *p) {
+    bf16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((GCMI_LDS bf16x4_t *)p);
+    return __builtin_bit_cast(uint2, v);
+  }
+};
+template <> struct MfmaOp<1> {
+  typedef i32x16_t acc_t;
+  typedef int acc_elem_t;
+  static __device__ __forceinline__ acc_t run(const uint4 &a, const uint4 &b, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, a), __builtin_bit_cast(i32x4_t, b), c, 0,
+                                                 0, 0);
+  }
+  // 8 bytes: k..k+7 of one n
+  static __device__ __forceinline__ uint2 tr_read(const char *p) {
+    i32x2_t v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((GCMI_LDS i32x2_t *)p);
+    return __builtin_bit_cast(uint2, v);
+  }
+};
+
+// 16-byte chunk from global memory, zero filled outside [0,rows) x [0,row_bytes)
+template <bool EDGE>
+__device__ __forceinline__ uint4 load_chunk(const char *base, int64_t row, int64_t rows, int64_t col_byte,
+                                            int64_t row_bytes, int64_t ld_bytes) {
+  if (!EDGE) {
+    return *reinterpret_cast<const uint4 *>(base + row * ld_bytes + col_byte);
+  } else {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (row >= rows || col_byte >= row_bytes)
+      return v;
+    const char *p = base + row * ld_bytes + col_byte;
+    int64_t nvalid = row_bytes - col_byte;
+    if (nvalid >= 16 && ((reinterpret_cast<uintptr_t>(p) & 15) == 0))
+      return *reinterpret_cast<const uint4 *>(p);
+    unsigned char tmp[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      tmp[i] = i < nvalid ? (unsigned char)p[i] : (unsigned char)0;
+    v.x = tmp[0] | (tmp[1] << 8) | (tmp[2] << 16) | ((uint32_t)tmp[3] << 24);
+    v.y = tmp[4] | (tmp[5] << 8) | (tmp[6] << 16) | ((uint32_t)tmp[7] << 24);
+    v.z = tmp[8] | (tmp[9] << 8) | (tmp[10] << 16) | ((uint32_t)tmp[11] << 24);
+    v.w = tmp[12] | (tmp[13] << 8) | (tmp[14] << 16) | ((uint32_t)tmp[15] << 24);
+    return v;
+  }
+}
+
+// Map a linear workgroup id to a tile so that the workgroups one XCD receives
+// (hardware deals consecutive ids round-robin over 8 XCDs) cover a compact
+// rectangle of tiles and share A/B panels in that XCD's L2.
+__device__ __forceinline__ void tile_of_block(int bid, int nblk, int tiles_m, int tiles_n, int group_m, int &tm,
+                                              int &tn) {
+  int id = bid;
+  if ((nblk & 7) == 0)
+    id = (bid & 7) * (nblk >> 3) + (bid >> 3);
+  int per_group = group_m * tiles_n;
+  int g = id / per_group;
+  int first_m = g * group_m;
+  int gm = min(group_m, tiles_m - first_m);
+  int in_g = id - g * per_group;
+  tm = first_m + in_g % gm;
+  tn = in_g / gm;
+}
+
+template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_kernel(GemmParams p) {
+  typedef MfmaOp<ES> Op;
+  typedef typename Op::acc_t acc_t;
+  constexpr int BK = G_KBYTES / ES;        // K elements per stage
+  constexpr int B_ROW_BYTES = G_BN * ES;   // bytes per k-row of the B tile
+  constexpr int B_CPR = B_ROW_BYTES / 16;  // 16-byte chunks per B row
+  constexpr int RG = ES == 2 ? 4 : 8;      // k-rows per transpose-read group
+  constexpr int CW = ES == 2 ? 4 : 2;      // chunks per row one transpose read spans
+  constexpr int KSTEP = 32 / ES;           // K elements one MFMA consumes
+
+  __shared__ __align__(16) char smem[2 * G_STAGE_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  const int tiles_m = (int)((p.M + G_BM - 1) / G_BM), tiles_n = (int)((p.N + G_BN - 1) / G_BN);
+  int tm, tn;
+  tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
+  const int64_t m0 = (int64_t)tm * G_BM, n0 = (int64_t)tn * G_BN;
+
+  const int64_t lda_b = p.lda * ES, ldb_b = p.ldb * ES;
+  const char *Ab = reinterpret_cast<const char *>(p.A);
+  const char *Bb = reinterpret_cast<const char *>(p.B);
+
+  // ---- global -> register staging assignment: 4 A chunks + 4 B chunks per thread
+  const int a_row0 = tid >> 3, a_c = tid & 7;             // rows a_row0 + 64*i
+  const int b_row0 = tid / B_CPR, b_c = tid % B_CPR;      // rows b_row0 + (512/B_CPR)*i
+  constexpr int B_ROW_STEP = G_THREADS / B_CPR;
+  uint32_t a_st[4], b_st[4]; // LDS store offsets inside a stage
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    int row = a_row0 + 64 * i;
+    a_st[i] = row * 128 + ((a_c ^ ((row >> 1) & 7)) << 4);
+    int krow = b_row0 + B_ROW_STEP * i;
+    b_st[i] = 32768 + krow * B_ROW_BYTES + ((b_c ^ ((krow % RG) * CW)) << 4);
+  }
+
+  // ---- LDS read offsets of this lane's MFMA fragments
+  const int sw = (l32 >> 1) & 7;
+  uint32_t a_ld[4]; // per k-step chunk offset; + lane row base + i*4096
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++)
+    a_ld[ks] = (wm * 128 + l32) * 128 + (((2 * ks + lh) ^ sw) << 4);
+  const int g = lane >> 4, i16 = lane & 15;
+  uint32_t b_ld[2]; // + ks*8192 + jj*2048
+  {
+    const int kk = ES == 2 ? (i16 >> 2) : (i16 >> 1);
+    const int cc = ES == 2 ? (i16 & 3) : (i16 & 1);
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      int chunk = ES == 2 ? (wn * 8 + j * 4 + 2 * (g & 1) + (cc >> 1)) : (wn * 4 + j * 2 + (g & 1));
+      int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
+      int krow_lane = (ES == 2 ? 8 : 16) * (g >> 1) + kk;
+      b_ld[j] = 32768 + krow_lane * B_ROW_BYTES + ((chunk ^ (kk * CW)) << 4) + sub;
+    }
+  }
+
+  acc_t acc[2][4];
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        acc[j][i][r] = 0;
+
+  const int64_t k_bytes = p.K * ES;
+  const int KT = (int)((p.K + BK - 1) / BK);
+  uint4 ra[4], rb[4];
+
+  auto gload = [&](int kt) {
+    const int64_t kb = (int64_t)kt * G_KBYTES; // byte offset along K of A
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      ra[i] = load_chunk<EDGE>(Ab, m0 + a_row0 + 64 * i, p.M, kb + a_c * 16, k_bytes, lda_b);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      rb[i] = load_chunk<EDGE>(Bb, (int64_t)kt * BK + b_row0 + B_ROW_STEP * i, p.K, n0 * ES + b_c * 16,
+                               p.N * ES, ldb_b);
+  };
+  auto lstore = [&](int stage) {
+    char *s = smem + stage * G_STAGE_BYTES;
+    const uint32_t x = p.a_xor;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint4 v = ra[i];
+      if (ES == 1) { // u8 activations: a - 128 as s8 == a ^ 0x80
+        v.x ^= x;
+        v.y ^= x;
+        v.z ^= x;
+        v.w ^= x;
+      }
+      *reinterpret_cast<uint4 *>(s + a_st[i]) = v;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      *reinterpret_cast<uint4 *>(s + b_st[i]) = rb[i];
+  };
+
+  gload(0);
+  lstore(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < KT; kt++) {
+    const int cur = kt & 1;
+    if (kt + 1 < KT)
+      gload(kt + 1);
+    const char *s = smem + cur * G_STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      uint4 af[4], bf[2];
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        af[i] = *reinterpret_cast<const uint4 *>(s + a_ld[ks] + i * 4096);
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        uint2 lo = Op::tr_read(s + b_ld[j] + ks * 8192);
+        uint2 hi = Op::tr_read(s + b_ld[j] + ks * 8192 + 2048);
+        bf[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          acc[j][i] = Op::run(bf[j], af[i], acc[j][i]);
+    }
+    if (kt + 1 < KT)
+      lstore(cur ^ 1);
+    __syncthreads();
+  }
+  (void)KSTEP;
+
+  // ---- epilogue: lane owns m = mrow(i), n = ncol(j,q) .. +3
+  const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
+  char *Cb = reinterpret_cast<char *>(p.C);
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int64_t n = n0 + wn * 64 + j * 32 + 8 * q + 4 * lh;
+      float bias4[4] = {0.f, 0.f, 0.f, 0.f}, scale4[4] = {1.f, 1.f, 1.f, 1.f};
+      int cs4[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if (!EDGE || n + e < p.N) {
+          if (p.bias)
+            bias4[e] = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n + e])
+                                            : reinterpret_cast<const float *>(p.bias)[n + e];
+          if (ES == 1) {
+            if (p.scale)
+              scale4[e] = p.scale[n + e];
+            if (p.colsum)
+              cs4[e] = p.colsum[n + e];
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int64_t m = m0 + wm * 128 + i * 32 + l32;
+        if (EDGE && m >= p.M)
+          continue;
+        uint32_t o32[4];
+        uint16_t o16[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          if (ES == 1) {
+            // s32 accumulator of (a ^ 0x80) * w; comp restores / applies the
+            // zero-point term in exact integer arithmetic.
+            int c = acc[j][i][4 * q + e] + p.comp * cs4[e];
+            if (p.out_dt == DT_S32) {
+              o32[e] = (uint32_t)c;
+            } else {
+              float x = (float)c * scale4[e];
+              if (p.bias)
+                x = x + bias4[e];
+              x = apply_act(x, p.act);
+              o32[e] = __float_as_uint(x);
+              o16[e] = f32_to_bf16_bits(x);
+            }
+          } else {
+            float x = (float)acc[j][i][4 * q + e];
+            if (p.out_dt == DT_BF16) {
+              // bf16 graph: round after the matmul and after every bf16 op
+              // (lib/gc/Transforms/Pipeline.cpp:79-95)
+              x = round_bf16(x);
+              if (p.bias)
+                x = round_bf16(x + bias4[e]);
+              if (p.act != ACT_NONE)
+                x = round_bf16(apply_act(x, p.act));
+              o16[e] = f32_to_bf16_bits(x);
+            } else {
+              if (p.bias)
+                x = x + bias4[e];
+              x = apply_act(x, p.act);
+              o32[e] = __float_as_uint(x);
+            }
+          }
+        }
+        char *dst = Cb + (m * p.ldc + n) * out_es;
+        if (!EDGE) {
+          if (out_es == 2)
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
+          else
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(o32[0], o32[1], o32[2], o32[3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            if (n + e < p.N) {
+              if (out_es == 2)
+                reinterpret_cast<uint16_t *>(dst)[e] = o16[e];
+              else
+                reinterpret_cast<uint32_t *>(dst)[e] = o32[e];
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// column sums of an s8 [K,N] weight in s32 (weight-only constant of the
+// asymmetric-activation compensation, legacy/core/src/ops/matmul_core.cpp:
+// 546-557).  One thread per column, coalesced along n; K split over blockDim.y
+// with an LDS reduction.
+__global__ void colsum_s8_kernel(const int8_t *W, int64_t K, int64_t N, int64_t ldw, int32_t *out) {
+  __shared__ int part[8][64];
+  const int64_t n = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  int s = 0;
+  if (n < N)
+    for (int64_t k = threadIdx.y; k < K; k += 8)
+      s += (int)W[k * ldw + n];
+  part[threadIdx.y][threadIdx.x] = s;
+  __syncthreads();
+  if (threadIdx.y == 0 && n < N) {
+    int t = 0;
+#pragma unroll
+    for (int y = 0; y < 8; y++)
+      t += part[y][threadIdx.x];
+    out[n] = t;
+  }
+}
+
+} // namespace gcmi
+
+using namespace gcmi;
+
+extern "C" int gcmi_launch_gemm_tile256(const GemmParams *pp, int es, hipStream_t stream) {
+  GemmParams p = *pp;
+  const int tiles_m = (int)((p.M + G_BM - 1) / G_BM), tiles_n = (int)((p.N + G_BN - 1) / G_BN);
+  const int64_t nblk = (int64_t)tiles_m * tiles_n;
+  if (nblk <= 0 || nblk > 0x7fffffff)
+    return 2;
+  const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
+  auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const int BK = G_KBYTES / es;
+  bool fast = p.M % G_BM == 0 && p.N % G_BN == 0 && p.K % BK == 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
+              (p.lda * es) % 16 == 0 && (p.ldb * es) % 16 == 0 && (p.ldc * out_es) % 16 == 0;
+  if (p.group_m <= 0)
+    p.group_m = 4;
+  dim3 grid((unsigned)nblk), block(G_THREADS);
+  if (es == 2) {
+    if (fast)
+      hipLaunchKernelGGL((gemm_tile256_kernel<2, false>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((gemm_tile256_kernel<2, true>), grid, block, 0, stream, p);
+  } else {
+    if (fast)
+      hipLaunchKernelGGL((gemm_tile256_kernel<1, false>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((gemm_tile256_kernel<1, true>), grid, block, 0, stream, p);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : 5;
+}
+
+extern "C" int gcmi_launch_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, void *out, hipStream_t stream) {
+  if (N <= 0)
+    return 0;
+  dim3 grid((unsigned)((N + 63) / 64)), block(64, 8);
+  hipLaunchKernelGGL(colsum_s8_kernel, grid, block, 0, stream, (const int8_t *)W, K, N, ldw, (int32_t *)out);
+  return hipGetLastError() == hipSuccess ? 0 : 5;
+}

@@ -1,0 +1,45 @@
+// Plain-data argument blocks passed by value to the GEMM / attention kernels.
+#pragma once
+#include <stdint.h>
+
+namespace gcmi {
+
+struct GemmParams {
+  const void *A;   // [M,K] row-major, lda elements between rows
+  const void *B;   // [K,N] row-major, ldb elements between rows
+  void *C;         // [M,N] row-major, ldc elements between rows
+  int64_t M, N, K;
+  int64_t lda, ldb, ldc;
+  const void *bias;      // [N] or null; dtype bias_dt (bf16 or f32)
+  const float *scale;    // int8 only: per-output-channel dequant scale [N] or null
+  const int32_t *colsum; // int8 only: sum_k W[k,n] in s32, [N] or null
+  int32_t comp;          // int8 only: integer factor of colsum added to the accumulator
+  uint32_t a_xor;        // int8 only: 0x80808080 when A is u8, else 0
+  int32_t act;           // gcmi::Act
+  int32_t out_dt;        // gcmi::DType of C
+  int32_t bias_dt;       // gcmi::DType of bias
+  int32_t group_m;       // tile-order group height (XCD/L2 locality), 0 = default
+};
+
+struct F32GemmParams {
+  const float *A, *B;
+  float *C;
+  int64_t M, N, K;
+  int64_t a_rs, a_cs; // element strides of A along m and k (transposes fold in here)
+  int64_t b_rs, b_cs; // element strides of B along k and n
+  int64_t ldc;
+  const float *bias;
+  int32_t act;
+  float beta; // 0: overwrite, 1: accumulate into C before the epilogue
+};
+
+struct MhaParams {
+  const void *Q, *K, *V; // bf16 [B*H, S, D] contiguous
+  void *O;               // bf16 [B*H, Sq, D]
+  const float *mask;     // f32 [Sq, Sk] additive, shared by every (batch, head); or null
+  int64_t mask_ld;
+  int32_t BH, Sq, Sk, D;
+  float scale;
+};
+
+} // namespace gcmi

@@ -1,0 +1,103 @@
+/*
+ * gc_hip_kernels.h -- C ABI of the MI355X (gfx950) kernels behind the graph
+ * compiler's contraction hot path.  Every pointer is a DEVICE pointer unless
+ * stated otherwise; sizes and leading dimensions are in elements; `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream).  Calls are
+ * asynchronous on `stream`.  No function allocates device memory.
+ *
+ * Return value: a dnnl_status_t-compatible int (0 success, 2 invalid
+ * arguments, 3 unimplemented, 5 runtime error); gcmi_last_error() gives text.
+ *
+ * Each entry point names the reference interface whose work it takes over
+ * (paths relative to the intel/graph-compiler tree).
+ */
+#ifndef GC_HIP_KERNELS_H
+#define GC_HIP_KERNELS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#pragma GCC visibility push(default)
+
+/* dnnl_data_type_t values, as the reference passes them across its microkernel
+ * ABI (test/mlir/unittests/ExecutionEngine/BrgemmRuntime.cpp:61-62,117-118). */
+enum { GCMI_F16 = 1, GCMI_BF16 = 2, GCMI_F32 = 3, GCMI_S32 = 4, GCMI_S8 = 5, GCMI_U8 = 6 };
+
+/* fused post-op of a GEMM epilogue */
+enum { GCMI_ACT_NONE = 0, GCMI_ACT_RELU = 1, GCMI_ACT_GELU_ERF = 2, GCMI_ACT_GELU_TANH = 3, GCMI_ACT_SIGMOID = 4 };
+
+/* Library / device set-up.  Selects `device`, checks it is a gfx950 part and
+ * returns 0.  Optional: every entry point works on the current device. */
+int gcmi_init(int device);
+const char *gcmi_last_error(void);
+
+/*
+ * bf16 matmul with fused epilogue:  C = act( (A.B) [+ bias] ).
+ * Takes over: linalg.matmul lowered by DeepTileMatmul to a loop nest of
+ * dnnl_brgemm_execute calls plus the fused consumers
+ * (lib/gc/Transforms/DeepTileContractionOp.cpp:958-1014,
+ *  lib/gc/Transforms/IterativeTilingAndFusion.cpp:585-611,
+ *  include/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmInterface.h:31-63).
+ * A [M,K] and B [K,N] row-major bf16 (B is NOT VNNI packed).  f32 accumulate
+ * over all of K.  out_dtype GCMI_BF16: bf16 graph semantics, the value is
+ * rounded to bf16 after the matmul, after the bias add and after the
+ * activation (lib/gc/Transforms/Pipeline.cpp:79-95).  out_dtype GCMI_F32: no
+ * intermediate rounding.  bias: [N] of bias_dtype (GCMI_BF16 or GCMI_F32) or
+ * NULL.
+ */
+int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                   int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
+
+/*
+ * 8-bit matmul with s32 accumulation and fused dequantise epilogue.
+ * Takes over: the u8/s8 brgemm (lib/gc/ExecutionEngine/CPURuntime/Microkernel/
+ * BrgemmNaive.cpp:102-140) under the deep-tile nest, the asymmetric-activation
+ * compensation (legacy/core/src/ops/matmul_core.cpp:529-571), Dequantize
+ * (legacy/core/src/compiler/ir/graph/quantization/quantize_op.cpp:230-277) and
+ * GELU (legacy/core/src/ops/gelu.cpp:72-133).
+ * A [M,K] of a_dtype (GCMI_U8 or GCMI_S8), W [K,N] s8, both row-major.
+ *   acc[m,n]  = sum_k A[m,k]*W[k,n]                       (s32, exact)
+ *   out_dtype GCMI_S32 : C = acc                          (raw accumulators)
+ *   otherwise          : x = f32(acc - zp_a*colsum[n]) * scale[n] (+ bias[n]);
+ *                        C = act(x) as GCMI_F32 or GCMI_BF16 (one RNE rounding)
+ * colsum [N] s32 = sum_k W[k,n] (gcmi_colsum_s8); required when a_dtype is
+ * GCMI_U8 or zp_a != 0.  scale, bias: f32 [N] or NULL (scale 1, no bias).
+ */
+int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                   int64_t ldb, int64_t ldc, const int32_t *colsum, int32_t zp_a, const float *scale,
+                   const float *bias, int act, int out_dtype, void *stream);
+
+/* Column sums of an s8 weight [K,N] into s32 [N]: the weight-only constant of
+ * the compensation term (legacy/core/src/ops/matmul_core.cpp:546-557). */
+int gcmi_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, int32_t *colsum, void *stream);
+
+/*
+ * f32 matmul (+bias, +activation), transposes folded into strides.
+ * Takes over: onednn_graph.matmul{transpose_a,transpose_b} + bias + ReLU on
+ * f32 (lib/gc/Transforms/OneDNNGraphToLinalg.cpp:421-499, :355-358).
+ * Logical A is [M,K], logical B is [K,N]; when trans_a the stored A is [K,M]
+ * with leading dimension lda, likewise trans_b.  Plain f32 FMA arithmetic.
+ */
+int gcmi_gemm_f32(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                  int64_t ldc, int trans_a, int trans_b, const float *bias, int act, void *stream);
+
+/*
+ * Fused multi-head attention forward, bf16, head_dim 128:
+ *   O = softmax(Q K^T * scale + mask) V,  softmax over keys in f32.
+ * Takes over the composition batch_matmul_transpose_b -> mul -> add -> softmax
+ * -> batch_matmul (lib/gc/Transforms/DecomposeAggregatedOps.cpp:24-38;
+ * test/benchgc/src/benchgc/linalg/matmul.py:29-32,65-68).
+ * Q [BH,Sq,D], K and V [BH,Sk,D], O [BH,Sq,D], contiguous bf16; mask f32
+ * [Sq,Sk] with row stride mask_ld, added to every (batch, head), or NULL.
+ * A query row whose keys are all masked with -inf yields NaN.
+ */
+int gcmi_mha_fwd_bf16(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld, void *O,
+                      int64_t BH, int64_t Sq, int64_t Sk, int64_t D, float scale, void *stream);
+
+#pragma GCC visibility pop
+#ifdef __cplusplus
+}
+#endif
+#endif /* GC_HIP_KERNELS_H */

@@ -1,0 +1,171 @@
+"""GPU parity: MFMA GEMMs through the C ABI against the CPU oracle.
+bf16/f32 outputs: max relative error (see conftest.close_report) <= 1e-2 / 1e-4;
+s32 accumulators: bit exact."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import assert_close
+
+pytestmark = pytest.mark.gpu
+
+BF16_SHAPES = [(256, 256, 64), (512, 512, 256), (256, 512, 1024), (300, 200, 100), (257, 511, 129), (1, 7, 5),
+               (33, 1, 64), (128, 256, 8)]
+
+
+@pytest.mark.parametrize("M,N,K", BF16_SHAPES)
+@pytest.mark.parametrize("epi", ["none", "bias", "bias_relu", "gelu"])
+def test_bf16_gemm_matches_oracle(gc, orc, wl, dev, M, N, K, epi):
+    torch.manual_seed(0)
+    A = (torch.randn(M, K) * 0.5).to(torch.bfloat16)
+    torch.manual_seed(1)
+    B = (torch.randn(K, N) * 0.5).to(torch.bfloat16)
+    torch.manual_seed(2)
+    bias = torch.randn(N).to(torch.bfloat16) if "bias" in epi else None
+    act = {"none": None, "bias": None, "bias_relu": "relu", "gelu": "gelu_erf"}[epi]
+    ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B),
+                                          None if bias is None else wl.bf16_bits(bias), act))
+    mm = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B))) if bias is not None else None
+    out = gc.gemm_bf16(A.to(dev), B.to(dev), None if bias is None else bias.to(dev), act)
+    torch.cuda.synchronize()
+    # 1e-2 per bf16 rounding point of the reference graph: the matmul result is
+    # rounded once; a bias add or activation after it rounds a second time, and
+    # the two one-ulp (2^-7) differences of a different f32 summation order add.
+    rtol = 1e-2 if epi == "none" else 2e-2
+    assert_close(ref, out.float().cpu().numpy(), rtol, "bf16 %dx%dx%d %s" % (M, N, K, epi), mag=mm)
+
+
+def test_bf16_gemm_f32_out_and_strided_operands(gc, orc, wl, dev):
+    M, N, K = 260, 264, 200
+    torch.manual_seed(0)
+    Abig = torch.randn(M, K + 24).to(torch.bfloat16).to(dev)
+    Bbig = torch.randn(K, N + 8).to(torch.bfloat16).to(dev)
+    A, B = Abig[:, :K], Bbig[:, :N]
+    Cbig = torch.full((M, N + 4), 7.0, device=dev)
+    out = gc.gemm_bf16(A, B, None, None, gc.F32, out=Cbig[:, :N])
+    torch.cuda.synchronize()
+    ref = orc.deep_tile_matmul(wl.bf16_bits(A.cpu().contiguous()), wl.bf16_bits(B.cpu().contiguous()), orc.BF16, orc.BF16)
+    assert_close(ref, out.cpu().numpy(), 1e-4, "bf16->f32 strided")
+    assert (Cbig[:, N:] == 7.0).all()  # nothing written past the row
+
+
+def test_bf16_identity_is_exact_at_full_size(gc, dev):
+    """A . I == A bit for bit: every product is exact and every sum has one term."""
+    n = 4096
+    torch.manual_seed(3)
+    A = torch.randn(n, n, device=dev).to(torch.bfloat16)
+    eye = torch.eye(n, device=dev, dtype=torch.bfloat16)
+    out = gc.gemm_bf16(A, eye)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), A.view(torch.int16))
+
+
+def test_bf16_full_size_rows_against_oracle(gc, orc, wl, dev):
+    """BASELINE config 2 (4096^3): 48 rows spread over every row tile."""
+    A, B = wl.bf16_gemm()
+    out = gc.gemm_bf16(A.to(dev), B.to(dev))
+    torch.cuda.synchronize()
+    rows = sorted(set(list(range(0, 4096, 256)) + list(range(255, 4096, 256)) + [1, 130, 2049, 3000] +
+                      list(range(97, 4096, 331))))[:48]
+    ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A[rows]), wl.bf16_bits(B)))
+    assert_close(ref, out[rows].float().cpu().numpy(), 1e-2, "bf16 4096^3 sampled rows")
+    # column checksum over all rows in f64 (every output element takes part)
+    want = (A.double().sum(0, keepdim=True) @ B.double()).squeeze(0)
+    got = out.double().sum(0).cpu()
+    scale = (A.double().abs().sum(0, keepdim=True) @ B.double().abs()).squeeze(0)
+    assert ((got - want).abs() <= 2 ** -8 * scale).all()
+
+
+INT8_SHAPES = [(256, 256, 128), (512, 768, 384), (100, 130, 77), (1, 5, 3), (260, 40, 500)]
+
+
+@pytest.mark.parametrize("M,N,K", INT8_SHAPES)
+@pytest.mark.parametrize("a_signed", [False, True])
+def test_int8_accumulators_bit_exact(gc, orc, dev, M, N, K, a_signed):
+    torch.manual_seed(0)
+    A = torch.randint(-128, 128, (M, K), dtype=torch.int32).to(torch.int8) if a_signed else \
+        torch.randint(0, 256, (M, K), dtype=torch.int32).to(torch.uint8)
+    torch.manual_seed(1)
+    W = torch.randint(-128, 128, (K, N), dtype=torch.int32).to(torch.int8)
+    ref = orc.deep_tile_matmul(A.numpy(), W.numpy(), orc.S8 if a_signed else orc.U8, orc.S8)
+    Wd = W.to(dev)
+    cs = gc.colsum_s8(Wd)
+    torch.cuda.synchronize()
+    assert (cs.cpu().numpy() == orc.colsum_s8(W.numpy())).all()
+    raw = gc.gemm_int8(A.to(dev), Wd, cs, 0, None, None, None, gc.S32)
+    torch.cuda.synchronize()
+    assert (raw.cpu().numpy() == ref).all()
+
+
+@pytest.mark.parametrize("M,N,K", INT8_SHAPES[:4])
+@pytest.mark.parametrize("act,zp", [("gelu_erf", 128), ("relu", 3), (None, 0), ("gelu_tanh", 128)])
+def test_int8_layer_matches_oracle(gc, orc, dev, M, N, K, act, zp):
+    torch.manual_seed(0)
+    A = torch.randint(0, 256, (M, K), dtype=torch.int32).to(torch.uint8)
+    torch.manual_seed(1)
+    W = torch.randint(-127, 128, (K, N), dtype=torch.int32).to(torch.int8)
+    torch.manual_seed(2)
+    sc = torch.rand(N) * 0.009 + 0.001
+    torch.manual_seed(3)
+    bs = torch.randn(N)
+    _, y = orc.int8_layer(A.numpy(), W.numpy(), sc.numpy(), bs.numpy(), zp, act)
+    Wd = W.to(dev)
+    out = gc.gemm_int8(A.to(dev), Wd, gc.colsum_s8(Wd), zp, sc.to(dev), bs.to(dev), act, gc.BF16)
+    torch.cuda.synchronize()
+    assert_close(orc.bf16_to_f32(y), out.float().cpu().numpy(), 1e-2, "int8 layer")
+    _, yf = orc.int8_layer(A.numpy(), W.numpy(), sc.numpy(), bs.numpy(), zp, act, out_bf16=False)
+    outf = gc.gemm_int8(A.to(dev), Wd, gc.colsum_s8(Wd), zp, sc.to(dev), bs.to(dev), act, gc.F32)
+    torch.cuda.synchronize()
+    assert_close(yf, outf.cpu().numpy(), 1e-4, "int8 layer f32 out")
+
+
+def test_int8_full_size_exact_checksums_and_rows(gc, orc, wl, dev):
+    """BASELINE config 3 (4096 x 4096 x 11008).  Exactness of all 45M
+    accumulators through integer checksums (row sums and column sums of the
+    s32 result against int64 products of the operand sums), exact rows against
+    the oracle, and the fused epilogue against the oracle on those rows."""
+    A, W, scale, bias = wl.int8_mlp_layer()
+    Ad, Wd = A.to(dev), W.to(dev)
+    cs = gc.colsum_s8(Wd)
+    raw = gc.gemm_int8(Ad, Wd, cs, 0, None, None, None, gc.S32)
+    torch.cuda.synchronize()
+    assert (cs.cpu() == W.to(torch.int64).sum(0)).all()
+    raw64 = raw.to(torch.int64)
+    col_want = (A.to(torch.int64).sum(0, keepdim=True) @ W.to(torch.int64)).squeeze(0)   # 1^T A W
+    row_want = (A.to(torch.int64) @ W.to(torch.int64).sum(1, keepdim=True)).squeeze(1)   # A W 1
+    assert (raw64.sum(0).cpu() == col_want).all()
+    assert (raw64.sum(1).cpu() == row_want).all()
+    rows = [0, 255, 256, 1027, 2048, 3333, 4095] + list(range(61, 4096, 449))
+    acc, y = orc.int8_layer(A[rows].numpy(), W.numpy(), scale.numpy(), bias.numpy(), 128, "gelu_erf")
+    assert (raw[rows].cpu().numpy() == acc).all()
+    out = gc.gemm_int8(Ad, Wd, cs, 128, scale.to(dev), bias.to(dev), "gelu_erf", gc.BF16)
+    torch.cuda.synchronize()
+    assert_close(orc.bf16_to_f32(y), out[rows].float().cpu().numpy(), 1e-2, "int8 mlp rows")
+
+
+@pytest.mark.parametrize("M,N,K,ta,tb", [(128, 256, 512, False, False), (512, 64, 128, True, False),
+                                         (70, 33, 45, False, True), (65, 67, 19, True, True), (1, 1, 1, False, False)])
+def test_f32_gemm_bias_relu(gc, orc, dev, M, N, K, ta, tb):
+    torch.manual_seed(0)
+    A = torch.rand((K, M) if ta else (M, K)) * 2 - 1
+    torch.manual_seed(1)
+    B = torch.rand((N, K) if tb else (K, N)) * 2 - 1
+    torch.manual_seed(2)
+    bias = torch.rand(N) * 2 - 1
+    ref = orc.matmul_f32(A.numpy(), B.numpy(), bias.numpy(), "relu", ta, tb)
+    out = gc.gemm_f32(A.to(dev), B.to(dev), bias.to(dev), "relu", ta, tb)
+    torch.cuda.synchronize()
+    assert_close(ref, out.cpu().numpy(), 1e-4, "f32 gemm")
+
+
+def test_mlp_chain_bf16_reduced(gc, orc, wl, dev):
+    """BASELINE config 4 at 1/8 size: x W1 -> ReLU -> W2 + bias, bf16 rounding
+    points after the matmul, the add and the ReLU."""
+    x, W1, W2, b2 = wl.bf16_mlp_chain(M=512, K=512, H=1376)
+    h = gc.gemm_bf16(x.to(dev), W1.to(dev), None, "relu")
+    y = gc.gemm_bf16(h, W2.to(dev), b2.to(dev), None)
+    torch.cuda.synchronize()
+    href, yref = orc.mlp_chain_bf16(wl.bf16_bits(x), wl.bf16_bits(W1), wl.bf16_bits(W2), wl.bf16_bits(b2))
+    assert_close(orc.bf16_to_f32(href), h.float().cpu().numpy(), 1e-2, "mlp hidden")
+    mm = orc.bf16_to_f32(orc.matmul_bf16(href, wl.bf16_bits(W2)))
+    assert_close(orc.bf16_to_f32(yref), y.float().cpu().numpy(), 2e-2, "mlp out (two rounding points)", mag=mm)

@@ -1,0 +1,88 @@
+"""GPU parity: fused attention through the C ABI against the oracle's
+batch_matmul -> scale -> +mask -> softmax -> batch_matmul composition."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import assert_close
+
+pytestmark = pytest.mark.gpu
+
+def _pv_mag(Q, K, V, mask, scale):
+    """sum_j softmax(S)_ij |V_jd| in f64: the magnitude of the terms whose
+    weights are rounded to bf16 before the second matmul (in the reference
+    graph P is a bf16 tensor).  One half-ulp of each term, 2^-9 p|v|, is the
+    error unit of an output element, however much the signed sum cancels."""
+    S = Q.double() @ K.double().transpose(-1, -2) * scale
+    if mask is not None:
+        S = S + mask.double()
+    return (torch.softmax(S, -1) @ V.double().abs()).numpy()
+
+
+CASES = [(1, 2, 128, 128, "causal"), (1, 1, 256, 192, "none"), (2, 2, 100, 77, "causal"), (1, 2, 384, 384, "neg1e9"),
+         (1, 1, 1, 1, "none"), (1, 3, 130, 64, "random"), (1, 1, 64, 300, "neg30000")]
+
+
+def _mask(kind, Sq, Sk):
+    if kind == "none":
+        return None
+    if kind == "causal":
+        return torch.triu(torch.full((Sq, Sk), float("-inf")), diagonal=1)
+    if kind == "neg1e9":
+        return torch.triu(torch.full((Sq, Sk), -1e9), diagonal=1)
+    if kind == "neg30000":
+        return torch.triu(torch.full((Sq, Sk), -30000.0), diagonal=1)
+    torch.manual_seed(9)
+    return torch.randn(Sq, Sk) * 2
+
+
+@pytest.mark.parametrize("B,H,Sq,Sk,kind", CASES)
+def test_mha_matches_oracle(gc, orc, wl, dev, B, H, Sq, Sk, kind):
+    D = 128
+    torch.manual_seed(0)
+    Q = torch.randn(B, H, Sq, D).to(torch.bfloat16)
+    torch.manual_seed(1)
+    K = torch.randn(B, H, Sk, D).to(torch.bfloat16)
+    torch.manual_seed(2)
+    V = torch.randn(B, H, Sk, D).to(torch.bfloat16)
+    mask = _mask(kind, Sq, Sk)
+    scale = 1 / np.sqrt(D)
+    ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q), wl.bf16_bits(K), wl.bf16_bits(V),
+                                       None if mask is None else mask.numpy(), scale))
+    out = gc.mha_fwd_bf16(Q.to(dev), K.to(dev), V.to(dev), None if mask is None else mask.to(dev), scale)
+    torch.cuda.synchronize()
+    assert_close(ref, out.float().cpu().numpy(), 1e-2, "mha %s" % kind, mag=_pv_mag(Q, K, V, mask, scale))
+
+
+def test_fully_masked_rows_are_nan_like_the_reference_softmax(gc, orc, wl, dev):
+    torch.manual_seed(0)
+    Q = torch.randn(1, 1, 128, 128).to(torch.bfloat16)
+    K = torch.randn(1, 1, 128, 128).to(torch.bfloat16)
+    V = torch.randn(1, 1, 128, 128).to(torch.bfloat16)
+    mask = torch.zeros(128, 128)
+    mask[5, :] = float("-inf")
+    mask[70, :64] = float("-inf")  # first key block fully masked, second one live
+    ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q), wl.bf16_bits(K), wl.bf16_bits(V), mask.numpy(), 0.1))
+    out = gc.mha_fwd_bf16(Q.to(dev), K.to(dev), V.to(dev), mask.to(dev), 0.1).float().cpu().numpy()
+    assert np.isnan(out[0, 0, 5]).all() and np.isnan(ref[0, 0, 5]).all()
+    assert not np.isnan(np.delete(out[0, 0], 5, axis=0)).any()
+    assert_close(ref, out, 1e-2, "mha masked rows", mag=_pv_mag(Q, K, V, mask, 0.1))
+
+
+def test_mha_full_size_heads_and_invariants(gc, orc, wl, dev):
+    """BASELINE config 5 (B4 H32 S2048 D128, additive causal mask): three
+    (batch, head) slices against the oracle; first row equals V[0] exactly;
+    V == 1 gives 1 (weights sum to one)."""
+    Q, K, V, mask, scale = wl.bf16_mha()
+    Qd, Kd, Vd, md = Q.to(dev), K.to(dev), V.to(dev), mask.to(dev)
+    out = gc.mha_fwd_bf16(Qd, Kd, Vd, md, scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out[:, :, 0].view(torch.int16), Vd[:, :, 0].view(torch.int16))
+    for (b, h) in [(0, 0), (2, 17), (3, 31)]:
+        ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q[b:b + 1, h:h + 1]), wl.bf16_bits(K[b:b + 1, h:h + 1]),
+                                           wl.bf16_bits(V[b:b + 1, h:h + 1]), mask.numpy(), scale))
+        mag = _pv_mag(Q[b:b + 1, h:h + 1], K[b:b + 1, h:h + 1], V[b:b + 1, h:h + 1], mask, scale)
+        assert_close(ref, out[b:b + 1, h:h + 1].float().cpu().numpy(), 1e-2, "mha full size (%d,%d)" % (b, h), mag=mag)
+    ones = gc.mha_fwd_bf16(Qd, Kd, torch.ones_like(Vd), md, scale)
+    torch.cuda.synchronize()
+    assert (ones.float() - 1).abs().max().item() <= 2 ** -7
