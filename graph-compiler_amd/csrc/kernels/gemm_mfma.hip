@@ -31,6 +31,8 @@
 //   B: chunk ^= (krow % RG) * CW      -> RG = rows per transpose group (4 for
 //                                        16-bit, 8 for 8-bit), CW = 16-byte
 //                                        chunks one read touches per row
+#include <type_traits>
+
 #include "common.hpp"
 #include "gemm_params.h"
 
@@ -109,6 +111,136 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblk, int tiles_m, in
   int in_g = id - g * per_group;
   tm = first_m + in_g % gm;
   tn = in_g / gm;
+}
+
+// compile-time loop: the body receives std::integral_constant<int, I>, so every
+// accumulator index is a constant and the accumulators stay in registers
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+template <int ACT> __device__ __forceinline__ float act_const(float x) { return apply_act(x, ACT); }
+
+// Epilogue shared by both kernels.  acc[j][i][r] holds
+//   m = m0 + wm*128 + i*32 + (lane & 31),  n = n0 + wn*64 + j*32 + 8*(r/4) + 4*(lane >> 5) + r%4.
+// Instantiated once per activation so that each copy unrolls completely.
+template <int ES, bool EDGE, int ACT>
+__device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[2][4],
+                                                  int64_t m0, int64_t n0, int wm, int wn, int l32, int lh) {
+  const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
+  char *Cb = reinterpret_cast<char *>(p.C);
+  static_for<0, 2>([&](auto jc) {
+    constexpr int j = decltype(jc)::value;
+    static_for<0, 4>([&](auto qc) {
+      constexpr int q = decltype(qc)::value;
+      const int64_t n = n0 + wn * 64 + j * 32 + 8 * q + 4 * lh;
+      float bias4[4] = {0.f, 0.f, 0.f, 0.f}, scale4[4] = {1.f, 1.f, 1.f, 1.f};
+      int cs4[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if (!EDGE || n + e < p.N) {
+          if (p.bias)
+            bias4[e] = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n + e])
+                                            : reinterpret_cast<const float *>(p.bias)[n + e];
+          if (ES == 1) {
+            if (p.scale)
+              scale4[e] = p.scale[n + e];
+            if (p.colsum)
+              cs4[e] = p.colsum[n + e];
+          }
+        }
+      }
+      static_for<0, 4>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        const int64_t m = m0 + wm * 128 + i * 32 + l32;
+        if (EDGE && m >= p.M)
+          return;
+        uint32_t o32[4];
+        uint16_t o16[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          if (ES == 1) {
+            // s32 accumulator of (a ^ 0x80) * w; comp restores / applies the
+            // zero-point term in exact integer arithmetic.
+            int c = (int)acc[j][i][4 * q + e] + p.comp * cs4[e];
+            if (p.out_dt == DT_S32) {
+              o32[e] = (uint32_t)c;
+              o16[e] = 0;
+            } else {
+              float x = (float)c * scale4[e];
+              if (p.bias)
+                x = x + bias4[e];
+              x = act_const<ACT>(x);
+              o32[e] = __float_as_uint(x);
+              o16[e] = f32_to_bf16_bits(x);
+            }
+          } else {
+            float x = (float)acc[j][i][4 * q + e];
+            if (p.out_dt == DT_BF16) {
+              // bf16 graph: round after the matmul and after every bf16 op
+              // (lib/gc/Transforms/Pipeline.cpp:79-95)
+              x = round_bf16(x);
+              if (p.bias)
+                x = round_bf16(x + bias4[e]);
+              if (ACT != ACT_NONE)
+                x = round_bf16(act_const<ACT>(x));
+              o16[e] = f32_to_bf16_bits(x);
+              o32[e] = 0;
+            } else {
+              if (p.bias)
+                x = x + bias4[e];
+              x = act_const<ACT>(x);
+              o32[e] = __float_as_uint(x);
+              o16[e] = 0;
+            }
+          }
+        }
+        char *dst = Cb + (m * p.ldc + n) * out_es;
+        if (!EDGE) {
+          if (out_es == 2)
+            *reinterpret_cast<uint2 *>(dst) =
+                make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
+          else
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(o32[0], o32[1], o32[2], o32[3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            if (n + e < p.N) {
+              if (out_es == 2)
+                reinterpret_cast<uint16_t *>(dst)[e] = o16[e];
+              else
+                reinterpret_cast<uint32_t *>(dst)[e] = o32[e];
+            }
+          }
+        }
+      });
+    });
+  });
+}
+
+template <int ES, bool EDGE>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[2][4], int64_t m0,
+                                              int64_t n0, int wm, int wn, int l32, int lh) {
+  switch (p.act) {
+  case ACT_RELU:
+    gemm_epilogue_act<ES, EDGE, ACT_RELU>(p, acc, m0, n0, wm, wn, l32, lh);
+    break;
+  case ACT_GELU_ERF:
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_ERF>(p, acc, m0, n0, wm, wn, l32, lh);
+    break;
+  case ACT_GELU_TANH:
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_TANH>(p, acc, m0, n0, wm, wn, l32, lh);
+    break;
+  case ACT_SIGMOID:
+    gemm_epilogue_act<ES, EDGE, ACT_SIGMOID>(p, acc, m0, n0, wm, wn, l32, lh);
+    break;
+  default:
+    gemm_epilogue_act<ES, EDGE, ACT_NONE>(p, acc, m0, n0, wm, wn, l32, lh);
+    break;
+  }
 }
 
 template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_kernel(GemmParams p) {
@@ -245,92 +377,193 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
   }
   (void)KSTEP;
 
-  // ---- epilogue: lane owns m = mrow(i), n = ncol(j,q) .. +3
-  const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
-  char *Cb = reinterpret_cast<char *>(p.C);
+  gemm_epilogue<ES, EDGE>(p, acc, m0, n0, wm, wn, l32, lh);
+}
+
+// ---------------------------------------------------------------------------
+// Fast path: every dimension a multiple of the tile, 16-byte aligned operands.
+//  * global -> LDS goes through global_load_lds_dwordx4: each wave instruction
+//    drops 1 KiB straight into LDS (lane l at base + 16*l), no staging
+//    registers and no ds_write.  The swizzle is applied on the GLOBAL side: the
+//    lane that fills physical chunk P fetches logical chunk P ^ f(row).
+//  * MFMA fragments are double buffered in registers: the LDS reads of k-step
+//    s+1 are issued in the shadow of the MFMAs of k-step s, interleaved 1:1 by
+//    the scheduler hints; the reads of the next stage's first k-step are issued
+//    right after the stage barrier, under the last 8 MFMAs of the stage.
+//  * The two LDS stages are separate arrays and the K loop is unrolled by two,
+//    so every LDS address is static and the compiler never has to order a
+//    fragment read after the in-flight DMA into the other stage.
+#define GCMI_GLB __attribute__((address_space(1)))
+
+template <int ES> struct FastGemm {
+  typedef MfmaOp<ES> Op;
+  typedef typename Op::acc_t acc_t;
+  static constexpr int BK = G_KBYTES / ES;
+  static constexpr int B_ROW_BYTES = G_BN * ES;
+  static constexpr int RG = ES == 2 ? 4 : 8;
+  static constexpr int CW = ES == 2 ? 4 : 2;
+  static constexpr int B_ROWS_PER_DMA = 1024 / B_ROW_BYTES; // 2 (bf16) or 4 (int8)
+  static constexpr int B_CPR = B_ROW_BYTES / 16;
+
+  uint32_t a_src[4], b_src[4]; // per-lane byte offsets of this wave's 4+4 DMA instructions
+  uint32_t a_ld[4], b_ld[2];   // fragment read offsets
+  uint32_t a_xor;
+  int wave_u;                  // wave id, wave-uniform
+
+  __device__ __forceinline__ void issue_loads(char *__restrict__ stage, const char *a_base, const char *b_base) const {
 #pragma unroll
-  for (int j = 0; j < 2; j++) {
+    for (int i = 0; i < 4; i++) {
+      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(a_base + a_src[i]),
+                                       (GCMI_LDS void *)(stage + (wave_u * 4 + i) * 1024), 16, 0, 0);
+    }
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      const int64_t n = n0 + wn * 64 + j * 32 + 8 * q + 4 * lh;
-      float bias4[4] = {0.f, 0.f, 0.f, 0.f}, scale4[4] = {1.f, 1.f, 1.f, 1.f};
-      int cs4[4] = {0, 0, 0, 0};
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        if (!EDGE || n + e < p.N) {
-          if (p.bias)
-            bias4[e] = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n + e])
-                                            : reinterpret_cast<const float *>(p.bias)[n + e];
-          if (ES == 1) {
-            if (p.scale)
-              scale4[e] = p.scale[n + e];
-            if (p.colsum)
-              cs4[e] = p.colsum[n + e];
-          }
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int64_t m = m0 + wm * 128 + i * 32 + l32;
-        if (EDGE && m >= p.M)
-          continue;
-        uint32_t o32[4];
-        uint16_t o16[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          if (ES == 1) {
-            // s32 accumulator of (a ^ 0x80) * w; comp restores / applies the
-            // zero-point term in exact integer arithmetic.
-            int c = acc[j][i][4 * q + e] + p.comp * cs4[e];
-            if (p.out_dt == DT_S32) {
-              o32[e] = (uint32_t)c;
-            } else {
-              float x = (float)c * scale4[e];
-              if (p.bias)
-                x = x + bias4[e];
-              x = apply_act(x, p.act);
-              o32[e] = __float_as_uint(x);
-              o16[e] = f32_to_bf16_bits(x);
-            }
-          } else {
-            float x = (float)acc[j][i][4 * q + e];
-            if (p.out_dt == DT_BF16) {
-              // bf16 graph: round after the matmul and after every bf16 op
-              // (lib/gc/Transforms/Pipeline.cpp:79-95)
-              x = round_bf16(x);
-              if (p.bias)
-                x = round_bf16(x + bias4[e]);
-              if (p.act != ACT_NONE)
-                x = round_bf16(apply_act(x, p.act));
-              o16[e] = f32_to_bf16_bits(x);
-            } else {
-              if (p.bias)
-                x = x + bias4[e];
-              x = apply_act(x, p.act);
-              o32[e] = __float_as_uint(x);
-            }
-          }
-        }
-        char *dst = Cb + (m * p.ldc + n) * out_es;
-        if (!EDGE) {
-          if (out_es == 2)
-            *reinterpret_cast<uint2 *>(dst) = make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
-          else
-            *reinterpret_cast<uint4 *>(dst) = make_uint4(o32[0], o32[1], o32[2], o32[3]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            if (n + e < p.N) {
-              if (out_es == 2)
-                reinterpret_cast<uint16_t *>(dst)[e] = o16[e];
-              else
-                reinterpret_cast<uint32_t *>(dst)[e] = o32[e];
-            }
-          }
-        }
-      }
+    for (int i = 0; i < 4; i++) {
+      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(b_base + b_src[i]),
+                                       (GCMI_LDS void *)(stage + 32768 + (wave_u * 4 + i) * 1024), 16, 0, 0);
     }
   }
+
+  __device__ __forceinline__ void load_frags(const char *__restrict__ s, int ks, uint4 (&af)[4], uint4 (&bf)[2]) const {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint4 v = *reinterpret_cast<const uint4 *>(s + a_ld[ks] + i * 4096);
+      if (ES == 1) // u8 activations: a - 128 as s8 == a ^ 0x80
+        v = make_uint4(v.x ^ a_xor, v.y ^ a_xor, v.z ^ a_xor, v.w ^ a_xor);
+      af[i] = v;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      uint2 lo = Op::tr_read(s + b_ld[j] + ks * 8192);
+      uint2 hi = Op::tr_read(s + b_ld[j] + ks * 8192 + 2048);
+      bf[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+    }
+  }
+
+  static __device__ __forceinline__ void mfma_all(acc_t (&acc)[2][4], const uint4 (&af)[4], const uint4 (&bf)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        acc[j][i] = Op::run(bf[j], af[i], acc[j][i]);
+  }
+
+  // ask the scheduler for MFMA, DS read, MFMA, DS read, ... over the region
+  static __device__ __forceinline__ void interleave_hint() {
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // 1 DS read
+    }
+  }
+
+  // One stage: `cur` holds k-block kt (already landed and barriered, fragments
+  // of k-step 0 already in f0); loads of k-block kt+1 go into `nxt`.
+  __device__ __forceinline__ void stage(char *__restrict__ cur, char *__restrict__ nxt, bool has_next, const char *a_next, const char *b_next,
+                                        acc_t (&acc)[2][4], uint4 (&a0)[4], uint4 (&b0)[2], uint4 (&a1)[4],
+                                        uint4 (&b1)[2]) const {
+    if (has_next)
+      issue_loads(nxt, a_next, b_next);
+    load_frags(cur, 1, a1, b1);
+    mfma_all(acc, a0, b0);
+    interleave_hint();
+    load_frags(cur, 2, a0, b0);
+    mfma_all(acc, a1, b1);
+    interleave_hint();
+    load_frags(cur, 3, a1, b1);
+    mfma_all(acc, a0, b0);
+    interleave_hint();
+    // every wave has its last fragments of `cur` in registers and its DMA into
+    // `nxt` landed before anyone moves on
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    if (has_next)
+      load_frags(nxt, 0, a0, b0);
+    mfma_all(acc, a1, b1);
+    interleave_hint();
+  }
+};
+
+template <int ES> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast_kernel(GemmParams p) {
+  typedef FastGemm<ES> FG;
+  typedef typename FG::acc_t acc_t;
+  __shared__ __align__(1024) char smem0[G_STAGE_BYTES];
+  __shared__ __align__(1024) char smem1[G_STAGE_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  const int tiles_m = (int)(p.M / G_BM), tiles_n = (int)(p.N / G_BN);
+  int tm, tn;
+  tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
+  const int64_t m0 = (int64_t)tm * G_BM, n0 = (int64_t)tn * G_BN;
+  const int64_t lda_b = p.lda * ES, ldb_b = p.ldb * ES;
+
+  FG g;
+  g.wave_u = wave;
+  g.a_xor = p.a_xor;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    // A: this instruction fills LDS rows (wave*4+i)*8 .. +7, lane -> (row, physical chunk)
+    int row = (wave * 4 + i) * 8 + (lane >> 3);
+    int c = (lane & 7) ^ ((row >> 1) & 7);
+    g.a_src[i] = (uint32_t)(row * lda_b + c * 16);
+    // B: rows (wave*4+i)*B_ROWS_PER_DMA .. , lane -> (krow, physical chunk)
+    int krow = (wave * 4 + i) * FG::B_ROWS_PER_DMA + lane / FG::B_CPR;
+    int cb = (lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW);
+    g.b_src[i] = (uint32_t)(krow * ldb_b + cb * 16);
+  }
+  const int sw = (l32 >> 1) & 7;
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++)
+    g.a_ld[ks] = (wm * 128 + l32) * 128 + (((2 * ks + lh) ^ sw) << 4);
+  {
+    const int gq = lane >> 4, i16 = lane & 15;
+    const int kk = ES == 2 ? (i16 >> 2) : (i16 >> 1);
+    const int cc = ES == 2 ? (i16 & 3) : (i16 & 1);
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      int chunk = ES == 2 ? (wn * 8 + j * 4 + 2 * (gq & 1) + (cc >> 1)) : (wn * 4 + j * 2 + (gq & 1));
+      int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
+      int krow_lane = (ES == 2 ? 8 : 16) * (gq >> 1) + kk;
+      g.b_ld[j] = 32768 + krow_lane * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + sub;
+    }
+  }
+
+  acc_t acc[2][4];
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        acc[j][i][r] = 0;
+
+  const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b; // advances 128 B per k-block
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * ES;    // advances BK rows per k-block
+  const int64_t b_step = (int64_t)FG::BK * ldb_b;
+  const int KT = (int)(p.K / FG::BK);
+
+  uint4 a0[4], b0[2], a1[4], b1[2];
+  g.issue_loads(smem0, a_ptr, b_ptr);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  g.load_frags(smem0, 0, a0, b0);
+
+  for (int kt = 0; kt < KT; kt += 2) {
+    a_ptr += G_KBYTES;
+    b_ptr += b_step;
+    g.stage(smem0, smem1, kt + 1 < KT, a_ptr, b_ptr, acc, a0, b0, a1, b1);
+    if (kt + 1 < KT) {
+      a_ptr += G_KBYTES;
+      b_ptr += b_step;
+      g.stage(smem1, smem0, kt + 2 < KT, a_ptr, b_ptr, acc, a0, b0, a1, b1);
+    }
+  }
+
+  gemm_epilogue<ES, false>(p, acc, m0, n0, wm, wn, l32, lh);
 }
 
 // column sums of an s8 [K,N] weight in s32 (weight-only constant of the
@@ -368,19 +601,21 @@ extern "C" int gcmi_launch_gemm_tile256(const GemmParams *pp, int es, hipStream_
   const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const int BK = G_KBYTES / es;
-  bool fast = p.M % G_BM == 0 && p.N % G_BN == 0 && p.K % BK == 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
-              (p.lda * es) % 16 == 0 && (p.ldb * es) % 16 == 0 && (p.ldc * out_es) % 16 == 0;
+  // fast path: whole tiles, 16-byte aligned rows, and a tile's rows reachable with 32-bit byte offsets
+  bool fast = p.M % G_BM == 0 && p.N % G_BN == 0 && p.K % BK == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
+              (p.lda * es) % 16 == 0 && (p.ldb * es) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
+              p.lda * es * G_BM < (int64_t)1 << 31 && p.ldb * es * BK < (int64_t)1 << 31;
   if (p.group_m <= 0)
     p.group_m = 4;
   dim3 grid((unsigned)nblk), block(G_THREADS);
   if (es == 2) {
     if (fast)
-      hipLaunchKernelGGL((gemm_tile256_kernel<2, false>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((gemm_tile256_fast_kernel<2>), grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL((gemm_tile256_kernel<2, true>), grid, block, 0, stream, p);
   } else {
     if (fast)
-      hipLaunchKernelGGL((gemm_tile256_kernel<1, false>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((gemm_tile256_fast_kernel<1>), grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL((gemm_tile256_kernel<1, true>), grid, block, 0, stream, p);
   }
