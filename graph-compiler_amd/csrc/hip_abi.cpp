@@ -18,7 +18,8 @@
 using namespace gcmi;
 
 extern "C" {
-int gcmi_launch_gemm_tile256(const GemmParams *p, int es, hipStream_t stream);
+int gcmi_launch_gemm_bf16(const GemmParams *p, hipStream_t stream);
+int gcmi_launch_gemm_int8(const GemmParams *p, hipStream_t stream);
 int gcmi_launch_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, void *out, hipStream_t stream);
 int gcmi_launch_gemm_f32(const F32GemmParams *p, hipStream_t stream);
 int gcmi_launch_brgemm(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t LDA,
@@ -83,7 +84,7 @@ extern "C" int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, 
   GemmParams p{};
   p.A = A, p.B = B, p.C = C, p.M = M, p.N = N, p.K = K, p.lda = lda, p.ldb = ldb, p.ldc = ldc;
   p.bias = bias, p.bias_dt = bias_dtype, p.act = act, p.out_dt = out_dtype;
-  return launched(gcmi_launch_gemm_tile256(&p, 2, (hipStream_t)stream), "gemm_bf16");
+  return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
 }
 
 extern "C" int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K,
@@ -116,7 +117,7 @@ extern "C" int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C
   p.bias = bias, p.bias_dt = GCMI_F32, p.scale = scale, p.colsum = comp ? colsum : nullptr, p.comp = comp;
   p.a_xor = a_dtype == GCMI_U8 ? 0x80808080u : 0u;
   p.act = out_dtype == GCMI_S32 ? GCMI_ACT_NONE : act, p.out_dt = out_dtype;
-  return launched(gcmi_launch_gemm_tile256(&p, 1, (hipStream_t)stream), "gemm_int8");
+  return launched(gcmi_launch_gemm_int8(&p, (hipStream_t)stream), "gemm_int8");
 }
 
 extern "C" int gcmi_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, int32_t *colsum, void *stream) {

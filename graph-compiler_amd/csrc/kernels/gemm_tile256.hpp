@@ -31,6 +31,7 @@
 //   B: chunk ^= (krow % RG) * CW      -> RG = rows per transpose group (4 for
 //                                        16-bit, 8 for 8-bit), CW = 16-byte
 //                                        chunks one read touches per row
+#pragma once
 #include <type_traits>
 
 #include "common.hpp"
@@ -127,9 +128,17 @@ template <int ACT> __device__ __forceinline__ float act_const(float x) { return 
 // Epilogue shared by both kernels.  acc[j][i][r] holds
 //   m = m0 + wm*128 + i*32 + (lane & 31),  n = n0 + wn*64 + j*32 + 8*(r/4) + 4*(lane >> 5) + r%4.
 // Instantiated once per activation so that each copy unrolls completely.
-template <int ES, bool EDGE, int ACT>
+// STAGED (whole tiles, bf16 output): the wave first lays its 128 x 64 result out
+// in a private LDS region (rows of 128 B at a 144 B pitch), then reads it back
+// row-wise so that every global store instruction writes eight complete
+// 128-byte lines (16 B per lane) instead of 32 scattered 16-byte pieces.
+static constexpr int G_STG_PITCH = 144;
+static constexpr int G_STG_WAVE_BYTES = 128 * G_STG_PITCH; // 18 KiB per wave
+
+template <int ES, bool EDGE, int ACT, bool STAGED>
 __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[2][4],
-                                                  int64_t m0, int64_t n0, int wm, int wn, int l32, int lh) {
+                                                  int64_t m0, int64_t n0, int wm, int wn, int l32, int lh,
+                                                  char *stg) {
   const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
   char *Cb = reinterpret_cast<char *>(p.C);
   static_for<0, 2>([&](auto jc) {
@@ -198,6 +207,11 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
             }
           }
         }
+        if (STAGED) {
+          *reinterpret_cast<uint2 *>(stg + (i * 32 + l32) * G_STG_PITCH + j * 64 + q * 16 + lh * 8) =
+              make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
+          return;
+        }
         char *dst = Cb + (m * p.ldc + n) * out_es;
         if (!EDGE) {
           if (out_es == 2)
@@ -219,26 +233,38 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
       });
     });
   });
+  if (STAGED) {
+    // wave-private region: only this wave's own LDS writes have to land
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const int lane = lh * 32 + l32;
+    const int r8 = lane >> 3, c8 = lane & 7;
+#pragma unroll
+    for (int it = 0; it < 16; it++) {
+      const int row = it * 8 + r8;
+      uint4 v = *reinterpret_cast<const uint4 *>(stg + row * G_STG_PITCH + c8 * 16);
+      *reinterpret_cast<uint4 *>(Cb + ((m0 + wm * 128 + row) * p.ldc + n0 + wn * 64 + c8 * 8) * 2) = v;
+    }
+  }
 }
 
-template <int ES, bool EDGE>
+template <int ES, bool EDGE, bool STAGED>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[2][4], int64_t m0,
-                                              int64_t n0, int wm, int wn, int l32, int lh) {
+                                              int64_t n0, int wm, int wn, int l32, int lh, char *stg) {
   switch (p.act) {
   case ACT_RELU:
-    gemm_epilogue_act<ES, EDGE, ACT_RELU>(p, acc, m0, n0, wm, wn, l32, lh);
+    gemm_epilogue_act<ES, EDGE, ACT_RELU, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   case ACT_GELU_ERF:
-    gemm_epilogue_act<ES, EDGE, ACT_GELU_ERF>(p, acc, m0, n0, wm, wn, l32, lh);
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_ERF, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   case ACT_GELU_TANH:
-    gemm_epilogue_act<ES, EDGE, ACT_GELU_TANH>(p, acc, m0, n0, wm, wn, l32, lh);
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_TANH, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   case ACT_SIGMOID:
-    gemm_epilogue_act<ES, EDGE, ACT_SIGMOID>(p, acc, m0, n0, wm, wn, l32, lh);
+    gemm_epilogue_act<ES, EDGE, ACT_SIGMOID, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   default:
-    gemm_epilogue_act<ES, EDGE, ACT_NONE>(p, acc, m0, n0, wm, wn, l32, lh);
+    gemm_epilogue_act<ES, EDGE, ACT_NONE, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   }
 }
@@ -377,7 +403,7 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
   }
   (void)KSTEP;
 
-  gemm_epilogue<ES, EDGE>(p, acc, m0, n0, wm, wn, l32, lh);
+  gemm_epilogue<ES, EDGE, false>(p, acc, m0, n0, wm, wn, l32, lh, nullptr);
 }
 
 // ---------------------------------------------------------------------------
@@ -406,6 +432,8 @@ template <int ES> struct FastGemm {
   static constexpr int B_CPR = B_ROW_BYTES / 16;
 
   uint32_t a_src[4], b_src[4]; // per-lane byte offsets of this wave's 4+4 DMA instructions
+  uint32_t pf_src;             // per-lane byte offset of the cache line this lane touches when prefetching
+  bool pf_is_a;                // waves 0-3 prefetch the A tile (256 lines), waves 4-7 the B tile
   uint32_t a_ld[4], b_ld[2];   // fragment read offsets
   uint32_t a_xor;
   int wave_u;                  // wave id, wave-uniform
@@ -421,6 +449,14 @@ template <int ES> struct FastGemm {
       __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(b_base + b_src[i]),
                                        (GCMI_LDS void *)(stage + 32768 + (wave_u * 4 + i) * 1024), 16, 0, 0);
     }
+  }
+
+  // Touch one 128-byte line per lane of a k-block that will be DMA-ed two
+  // stages from now, so that its lines are in this XCD's L2 by then: a 4-byte
+  // LDS-DMA into a dump area nobody reads (no VGPR is written).
+  __device__ __forceinline__ void issue_prefetch(char *__restrict__ dump, const char *a_base, const char *b_base) const {
+    const char *src = (pf_is_a ? a_base : b_base) + pf_src;
+    __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)src, (GCMI_LDS void *)(dump + wave_u * 256), 4, 0, 0);
   }
 
   __device__ __forceinline__ void load_frags(const char *__restrict__ s, int ks, uint4 (&af)[4], uint4 (&bf)[2]) const {
@@ -458,11 +494,14 @@ template <int ES> struct FastGemm {
 
   // One stage: `cur` holds k-block kt (already landed and barriered, fragments
   // of k-step 0 already in f0); loads of k-block kt+1 go into `nxt`.
-  __device__ __forceinline__ void stage(char *__restrict__ cur, char *__restrict__ nxt, bool has_next, const char *a_next, const char *b_next,
-                                        acc_t (&acc)[2][4], uint4 (&a0)[4], uint4 (&b0)[2], uint4 (&a1)[4],
-                                        uint4 (&b1)[2]) const {
+  __device__ __forceinline__ void stage(char *__restrict__ cur, char *__restrict__ nxt, char *__restrict__ dump,
+                                        bool has_next, const char *a_next, const char *b_next, bool has_pf,
+                                        const char *a_pf, const char *b_pf, acc_t (&acc)[2][4], uint4 (&a0)[4],
+                                        uint4 (&b0)[2], uint4 (&a1)[4], uint4 (&b1)[2]) const {
     if (has_next)
       issue_loads(nxt, a_next, b_next);
+    if (has_pf)
+      issue_prefetch(dump, a_pf, b_pf);
     load_frags(cur, 1, a1, b1);
     mfma_all(acc, a0, b0);
     interleave_hint();
@@ -474,7 +513,11 @@ template <int ES> struct FastGemm {
     interleave_hint();
     // every wave has its last fragments of `cur` in registers and its DMA into
     // `nxt` landed before anyone moves on
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    // (the prefetch, issued after the DMA, may stay in flight: loads retire in order)
+    if (has_pf)
+      asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     if (has_next)
       load_frags(nxt, 0, a0, b0);
@@ -486,8 +529,10 @@ template <int ES> struct FastGemm {
 template <int ES> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast_kernel(GemmParams p) {
   typedef FastGemm<ES> FG;
   typedef typename FG::acc_t acc_t;
-  __shared__ __align__(1024) char smem0[G_STAGE_BYTES];
-  __shared__ __align__(1024) char smem1[G_STAGE_BYTES];
+  // two 64 KiB stages; the epilogue reuses the whole array as 8 x 18 KiB staging regions
+  __shared__ __align__(1024) char smem[8 * G_STG_WAVE_BYTES];
+  __shared__ __align__(256) char dump[8 * 256]; // landing area of the prefetch touches, never read
+  char *smem0 = smem, *smem1 = smem + G_STAGE_BYTES;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -546,8 +591,22 @@ template <int ES> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast
   const int64_t b_step = (int64_t)FG::BK * ldb_b;
   const int KT = (int)(p.K / FG::BK);
 
+  // L2 prefetch assignment: one 128-byte line of the A tile (waves 0-3, one row
+  // each) or of the B tile (waves 4-7) per lane
+  constexpr int PF_DIST = 2; // k-blocks between the prefetch and the DMA of the same data
+  g.pf_is_a = wave < 4;
+  {
+    const int t = tid & 255;
+    constexpr int B_LPR = FG::B_ROW_BYTES / 128; // lines per B row: 4 (bf16) or 2 (int8)
+    g.pf_src = wave < 4 ? (uint32_t)(t * lda_b) : (uint32_t)((t / B_LPR) * ldb_b + (t % B_LPR) * 128);
+  }
+
   uint4 a0[4], b0[2], a1[4], b1[2];
   g.issue_loads(smem0, a_ptr, b_ptr);
+#pragma unroll
+  for (int d = 1; d <= PF_DIST; d++)
+    if (d < KT)
+      g.issue_prefetch(dump, a_ptr + d * G_KBYTES, b_ptr + d * b_step);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
   g.load_frags(smem0, 0, a0, b0);
@@ -555,44 +614,27 @@ template <int ES> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast
   for (int kt = 0; kt < KT; kt += 2) {
     a_ptr += G_KBYTES;
     b_ptr += b_step;
-    g.stage(smem0, smem1, kt + 1 < KT, a_ptr, b_ptr, acc, a0, b0, a1, b1);
+    g.stage(smem0, smem1, dump, kt + 1 < KT, a_ptr, b_ptr, kt + 1 + PF_DIST < KT, a_ptr + PF_DIST * G_KBYTES,
+            b_ptr + PF_DIST * b_step, acc, a0, b0, a1, b1);
     if (kt + 1 < KT) {
       a_ptr += G_KBYTES;
       b_ptr += b_step;
-      g.stage(smem1, smem0, kt + 2 < KT, a_ptr, b_ptr, acc, a0, b0, a1, b1);
+      g.stage(smem1, smem0, dump, kt + 2 < KT, a_ptr, b_ptr, kt + 2 + PF_DIST < KT, a_ptr + PF_DIST * G_KBYTES,
+              b_ptr + PF_DIST * b_step, acc, a0, b0, a1, b1);
     }
   }
 
-  gemm_epilogue<ES, false>(p, acc, m0, n0, wm, wn, l32, lh);
+  // no wave reads fragments any more (the last stage's barrier came after its
+  // final fragment reads), so the stage buffers can be overwritten
+  if (p.out_dt == DT_BF16)
+    gemm_epilogue<ES, false, true>(p, acc, m0, n0, wm, wn, l32, lh, smem + wave * G_STG_WAVE_BYTES);
+  else
+    gemm_epilogue<ES, false, false>(p, acc, m0, n0, wm, wn, l32, lh, nullptr);
 }
 
-// column sums of an s8 [K,N] weight in s32 (weight-only constant of the
-// asymmetric-activation compensation, legacy/core/src/ops/matmul_core.cpp:
-// 546-557).  One thread per column, coalesced along n; K split over blockDim.y
-// with an LDS reduction.
-__global__ void colsum_s8_kernel(const int8_t *W, int64_t K, int64_t N, int64_t ldw, int32_t *out) {
-  __shared__ int part[8][64];
-  const int64_t n = (int64_t)blockIdx.x * 64 + threadIdx.x;
-  int s = 0;
-  if (n < N)
-    for (int64_t k = threadIdx.y; k < K; k += 8)
-      s += (int)W[k * ldw + n];
-  part[threadIdx.y][threadIdx.x] = s;
-  __syncthreads();
-  if (threadIdx.y == 0 && n < N) {
-    int t = 0;
-#pragma unroll
-    for (int y = 0; y < 8; y++)
-      t += part[y][threadIdx.x];
-    out[n] = t;
-  }
-}
 
-} // namespace gcmi
-
-using namespace gcmi;
-
-extern "C" int gcmi_launch_gemm_tile256(const GemmParams *pp, int es, hipStream_t stream) {
+// Host-side launch of the 256x256 tile kernels for one element size.
+template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t stream) {
   GemmParams p = *pp;
   const int tiles_m = (int)((p.M + G_BM - 1) / G_BM), tiles_n = (int)((p.N + G_BN - 1) / G_BN);
   const int64_t nblk = (int64_t)tiles_m * tiles_n;
@@ -600,32 +642,19 @@ extern "C" int gcmi_launch_gemm_tile256(const GemmParams *pp, int es, hipStream_
     return 2;
   const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
-  const int BK = G_KBYTES / es;
+  const int BK = G_KBYTES / ES;
   // fast path: whole tiles, 16-byte aligned rows, and a tile's rows reachable with 32-bit byte offsets
   bool fast = p.M % G_BM == 0 && p.N % G_BN == 0 && p.K % BK == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
-              (p.lda * es) % 16 == 0 && (p.ldb * es) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
-              p.lda * es * G_BM < (int64_t)1 << 31 && p.ldb * es * BK < (int64_t)1 << 31;
+              (p.lda * ES) % 16 == 0 && (p.ldb * ES) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
+              p.lda * ES * G_BM < (int64_t)1 << 31 && p.ldb * ES * BK < (int64_t)1 << 31;
   if (p.group_m <= 0)
     p.group_m = 4;
   dim3 grid((unsigned)nblk), block(G_THREADS);
-  if (es == 2) {
-    if (fast)
-      hipLaunchKernelGGL((gemm_tile256_fast_kernel<2>), grid, block, 0, stream, p);
-    else
-      hipLaunchKernelGGL((gemm_tile256_kernel<2, true>), grid, block, 0, stream, p);
-  } else {
-    if (fast)
-      hipLaunchKernelGGL((gemm_tile256_fast_kernel<1>), grid, block, 0, stream, p);
-    else
-      hipLaunchKernelGGL((gemm_tile256_kernel<1, true>), grid, block, 0, stream, p);
-  }
+  if (fast)
+    hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((gemm_tile256_kernel<ES, true>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 
-extern "C" int gcmi_launch_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, void *out, hipStream_t stream) {
-  if (N <= 0)
-    return 0;
-  dim3 grid((unsigned)((N + 63) / 64)), block(64, 8);
-  hipLaunchKernelGGL(colsum_s8_kernel, grid, block, 0, stream, (const int8_t *)W, K, N, ldw, (int32_t *)out);
-  return hipGetLastError() == hipSuccess ? 0 : 5;
-}
+} // namespace gcmi
