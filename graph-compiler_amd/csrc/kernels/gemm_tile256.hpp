@@ -42,6 +42,9 @@ namespace gcmi {
 static constexpr int G_BM = 256, G_BN = 256, G_KBYTES = 128;
 static constexpr int G_THREADS = 512;
 static constexpr int G_STAGE_BYTES = 65536; // A 32 KiB + B 32 KiB
+#ifndef G_FAST_KS
+#define G_FAST_KS 2 // MFMA k-steps per LDS stage of the fast path: 2 (4-stage ring) or 4 (2-stage ring)
+#endif
 
 template <int ES> struct MfmaOp;
 template <> struct MfmaOp<2> {
@@ -408,6 +411,11 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
 
 // ---------------------------------------------------------------------------
 // Fast path: every dimension a multiple of the tile, 16-byte aligned operands.
+//  * K is consumed in stages of KS MFMA k-steps (KS*32 bytes of K per row); the
+//    LDS holds a ring of NST = 8/KS such stages (KS=2: 4 x 32 KiB, KS=4:
+//    2 x 64 KiB).  Stage kt+NST-1 is requested while stage kt is computed, so
+//    two to three stages of global->LDS traffic are always in flight: a CU's
+//    L2->LDS path only delivers ~100 GB/s and has to stream without gaps.
 //  * global -> LDS goes through global_load_lds_dwordx4: each wave instruction
 //    drops 1 KiB straight into LDS (lane l at base + 16*l), no staging
 //    registers and no ds_write.  The swizzle is applied on the GLOBAL side: the
@@ -416,53 +424,48 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
 //    s+1 are issued in the shadow of the MFMAs of k-step s, interleaved 1:1 by
 //    the scheduler hints; the reads of the next stage's first k-step are issued
 //    right after the stage barrier, under the last 8 MFMAs of the stage.
-//  * The two LDS stages are separate arrays and the K loop is unrolled by two,
-//    so every LDS address is static and the compiler never has to order a
-//    fragment read after the in-flight DMA into the other stage.
+//  * The stage loop is unrolled over the ring, so every LDS address is static.
 #define GCMI_GLB __attribute__((address_space(1)))
 
-template <int ES> struct FastGemm {
+template <int ES, int KS> struct FastGemm {
   typedef MfmaOp<ES> Op;
   typedef typename Op::acc_t acc_t;
-  static constexpr int BK = G_KBYTES / ES;
+  static constexpr int NST = 8 / KS;                  // stages in the LDS ring
+  static constexpr int KB = KS * 32;                  // bytes of K per A row per stage
+  static constexpr int BK = KB / ES;                  // K elements per stage
+  static constexpr int A_BYTES = G_BM * KB;           // 16 or 32 KiB
+  static constexpr int STAGE_BYTES = 2 * A_BYTES;     // B tile has the same size
+  static constexpr int A_CPR = KB / 16;               // 16-byte chunks per A row: 4 or 8
+  static constexpr int A_ROWS_PER_DMA = 1024 / KB;    // 16 or 8
   static constexpr int B_ROW_BYTES = G_BN * ES;
   static constexpr int RG = ES == 2 ? 4 : 8;
   static constexpr int CW = ES == 2 ? 4 : 2;
   static constexpr int B_ROWS_PER_DMA = 1024 / B_ROW_BYTES; // 2 (bf16) or 4 (int8)
   static constexpr int B_CPR = B_ROW_BYTES / 16;
+  static constexpr int NDMA = KS;                     // DMA instructions per operand per wave per stage
 
-  uint32_t a_src[4], b_src[4]; // per-lane byte offsets of this wave's 4+4 DMA instructions
-  uint32_t pf_src;             // per-lane byte offset of the cache line this lane touches when prefetching
-  bool pf_is_a;                // waves 0-3 prefetch the A tile (256 lines), waves 4-7 the B tile
-  uint32_t a_ld[4], b_ld[2];   // fragment read offsets
+  static __device__ __forceinline__ int a_swz(int row) { return KS == 4 ? ((row >> 1) & 7) : ((row >> 2) & 3); }
+
+  uint32_t a_src[NDMA], b_src[NDMA]; // per-lane byte offsets of this wave's DMA instructions
+  uint32_t a_ld[KS], b_ld[2];        // fragment read offsets
   uint32_t a_xor;
-  int wave_u;                  // wave id, wave-uniform
+  int wave_u; // wave id, wave-uniform
 
   __device__ __forceinline__ void issue_loads(char *__restrict__ stage, const char *a_base, const char *b_base) const {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < NDMA; i++)
       __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(a_base + a_src[i]),
-                                       (GCMI_LDS void *)(stage + (wave_u * 4 + i) * 1024), 16, 0, 0);
-    }
+                                       (GCMI_LDS void *)(stage + (wave_u * NDMA + i) * 1024), 16, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < NDMA; i++)
       __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(b_base + b_src[i]),
-                                       (GCMI_LDS void *)(stage + 32768 + (wave_u * 4 + i) * 1024), 16, 0, 0);
-    }
-  }
-
-  // Touch one 128-byte line per lane of a k-block that will be DMA-ed two
-  // stages from now, so that its lines are in this XCD's L2 by then: a 4-byte
-  // LDS-DMA into a dump area nobody reads (no VGPR is written).
-  __device__ __forceinline__ void issue_prefetch(char *__restrict__ dump, const char *a_base, const char *b_base) const {
-    const char *src = (pf_is_a ? a_base : b_base) + pf_src;
-    __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)src, (GCMI_LDS void *)(dump + wave_u * 256), 4, 0, 0);
+                                       (GCMI_LDS void *)(stage + A_BYTES + (wave_u * NDMA + i) * 1024), 16, 0, 0);
   }
 
   __device__ __forceinline__ void load_frags(const char *__restrict__ s, int ks, uint4 (&af)[4], uint4 (&bf)[2]) const {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      uint4 v = *reinterpret_cast<const uint4 *>(s + a_ld[ks] + i * 4096);
+      uint4 v = *reinterpret_cast<const uint4 *>(s + a_ld[ks] + i * 32 * KB);
       if (ES == 1) // u8 activations: a - 128 as s8 == a ^ 0x80
         v = make_uint4(v.x ^ a_xor, v.y ^ a_xor, v.z ^ a_xor, v.w ^ a_xor);
       af[i] = v;
@@ -492,47 +495,52 @@ template <int ES> struct FastGemm {
     }
   }
 
-  // One stage: `cur` holds k-block kt (already landed and barriered, fragments
-  // of k-step 0 already in f0); loads of k-block kt+1 go into `nxt`.
-  __device__ __forceinline__ void stage(char *__restrict__ cur, char *__restrict__ nxt, char *__restrict__ dump,
-                                        bool has_next, const char *a_next, const char *b_next, bool has_pf,
-                                        const char *a_pf, const char *b_pf, acc_t (&acc)[2][4], uint4 (&a0)[4],
+  // wait until at most BEHIND later stages of this wave's DMA are still in flight
+  // (and all of its LDS reads have returned)
+  template <int BEHIND> static __device__ __forceinline__ void wait_dma() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(BEHIND * 2 * NDMA) : "memory");
+  }
+
+  // One stage, branch free.  `cur` holds k-block kt (landed and barriered;
+  // fragments of its k-step 0 are in a0/b0); the DMA of k-block kt+NST-1 goes
+  // into `fill`, the buffer that was computed from one stage ago; `nxt` holds
+  // k-block kt+1, behind which BEHIND more blocks are in flight.
+  template <bool HAS_FILL, bool HAS_NEXT, int BEHIND>
+  __device__ __forceinline__ void stage(char *__restrict__ cur, char *__restrict__ nxt, char *__restrict__ fill,
+                                        const char *a_fill, const char *b_fill, acc_t (&acc)[2][4], uint4 (&a0)[4],
                                         uint4 (&b0)[2], uint4 (&a1)[4], uint4 (&b1)[2]) const {
-    if (has_next)
-      issue_loads(nxt, a_next, b_next);
-    if (has_pf)
-      issue_prefetch(dump, a_pf, b_pf);
-    load_frags(cur, 1, a1, b1);
-    mfma_all(acc, a0, b0);
-    interleave_hint();
-    load_frags(cur, 2, a0, b0);
-    mfma_all(acc, a1, b1);
-    interleave_hint();
-    load_frags(cur, 3, a1, b1);
-    mfma_all(acc, a0, b0);
-    interleave_hint();
-    // every wave has its last fragments of `cur` in registers and its DMA into
-    // `nxt` landed before anyone moves on
-    // (the prefetch, issued after the DMA, may stay in flight: loads retire in order)
-    if (has_pf)
-      asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    if (HAS_FILL)
+      issue_loads(fill, a_fill, b_fill);
+#pragma unroll
+    for (int ks = 0; ks + 1 < KS; ks++) {
+      if (ks & 1) {
+        load_frags(cur, ks + 1, a0, b0);
+        mfma_all(acc, a1, b1);
+      } else {
+        load_frags(cur, ks + 1, a1, b1);
+        mfma_all(acc, a0, b0);
+      }
+      interleave_hint();
+    }
+    // every wave has its last fragments of `cur` in registers and its share of
+    // k-block kt+1 landed in `nxt` before anyone moves on
+    wait_dma<BEHIND>();
     __builtin_amdgcn_s_barrier();
-    if (has_next)
-      load_frags(nxt, 0, a0, b0);
+    // with a 2-stage ring the next block lives in the buffer just filled: read it
+    // through the same pointer the DMA was issued with
+    if (HAS_NEXT)
+      load_frags(NST == 2 ? fill : nxt, 0, a0, b0);
     mfma_all(acc, a1, b1);
     interleave_hint();
   }
 };
 
-template <int ES> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast_kernel(GemmParams p) {
-  typedef FastGemm<ES> FG;
+template <int ES, int KS> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast_kernel(GemmParams p) {
+  typedef FastGemm<ES, KS> FG;
   typedef typename FG::acc_t acc_t;
-  // two 64 KiB stages; the epilogue reuses the whole array as 8 x 18 KiB staging regions
+  constexpr int NST = FG::NST;
+  // ring of NST stages (128 KiB); the epilogue reuses the whole array as 8 x 18 KiB staging regions
   __shared__ __align__(1024) char smem[8 * G_STG_WAVE_BYTES];
-  __shared__ __align__(256) char dump[8 * 256]; // landing area of the prefetch touches, never read
-  char *smem0 = smem, *smem1 = smem + G_STAGE_BYTES;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -550,20 +558,21 @@ template <int ES> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast
   g.wave_u = wave;
   g.a_xor = p.a_xor;
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    // A: this instruction fills LDS rows (wave*4+i)*8 .. +7, lane -> (row, physical chunk)
-    int row = (wave * 4 + i) * 8 + (lane >> 3);
-    int c = (lane & 7) ^ ((row >> 1) & 7);
+  for (int i = 0; i < FG::NDMA; i++) {
+    // A: this instruction fills 1 KiB = A_ROWS_PER_DMA rows; lane -> (row, physical chunk)
+    int row = (wave * FG::NDMA + i) * FG::A_ROWS_PER_DMA + lane / FG::A_CPR;
+    int c = (lane % FG::A_CPR) ^ FG::a_swz(row);
     g.a_src[i] = (uint32_t)(row * lda_b + c * 16);
-    // B: rows (wave*4+i)*B_ROWS_PER_DMA .. , lane -> (krow, physical chunk)
-    int krow = (wave * 4 + i) * FG::B_ROWS_PER_DMA + lane / FG::B_CPR;
+    // B: B_ROWS_PER_DMA k-rows; lane -> (krow, physical chunk)
+    int krow = (wave * FG::NDMA + i) * FG::B_ROWS_PER_DMA + lane / FG::B_CPR;
     int cb = (lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW);
     g.b_src[i] = (uint32_t)(krow * ldb_b + cb * 16);
   }
-  const int sw = (l32 >> 1) & 7;
 #pragma unroll
-  for (int ks = 0; ks < 4; ks++)
-    g.a_ld[ks] = (wm * 128 + l32) * 128 + (((2 * ks + lh) ^ sw) << 4);
+  for (int ks = 0; ks < KS; ks++) {
+    int row = wm * 128 + l32; // + i*32: a multiple of 32 leaves the swizzle unchanged
+    g.a_ld[ks] = row * FG::KB + (((2 * ks + lh) ^ FG::a_swz(row)) << 4);
+  }
   {
     const int gq = lane >> 4, i16 = lane & 15;
     const int kk = ES == 2 ? (i16 >> 2) : (i16 >> 1);
@@ -573,7 +582,7 @@ template <int ES> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast
       int chunk = ES == 2 ? (wn * 8 + j * 4 + 2 * (gq & 1) + (cc >> 1)) : (wn * 4 + j * 2 + (gq & 1));
       int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
       int krow_lane = (ES == 2 ? 8 : 16) * (gq >> 1) + kk;
-      g.b_ld[j] = 32768 + krow_lane * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + sub;
+      g.b_ld[j] = FG::A_BYTES + krow_lane * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + sub;
     }
   }
 
@@ -586,43 +595,42 @@ template <int ES> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast
       for (int r = 0; r < 16; r++)
         acc[j][i][r] = 0;
 
-  const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b; // advances 128 B per k-block
-  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * ES;    // advances BK rows per k-block
+  const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b; // k-block 0; KB bytes per k-block
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * ES;    // k-block 0; BK rows per k-block
   const int64_t b_step = (int64_t)FG::BK * ldb_b;
   const int KT = (int)(p.K / FG::BK);
 
-  // L2 prefetch assignment: one 128-byte line of the A tile (waves 0-3, one row
-  // each) or of the B tile (waves 4-7) per lane
-  constexpr int PF_DIST = 2; // k-blocks between the prefetch and the DMA of the same data
-  g.pf_is_a = wave < 4;
-  {
-    const int t = tid & 255;
-    constexpr int B_LPR = FG::B_ROW_BYTES / 128; // lines per B row: 4 (bf16) or 2 (int8)
-    g.pf_src = wave < 4 ? (uint32_t)(t * lda_b) : (uint32_t)((t / B_LPR) * ldb_b + (t % B_LPR) * 128);
-  }
-
   uint4 a0[4], b0[2], a1[4], b1[2];
-  g.issue_loads(smem0, a_ptr, b_ptr);
+  // prologue: request k-blocks 0 .. NST-2 (KT is a positive multiple of NST), wait for block 0
 #pragma unroll
-  for (int d = 1; d <= PF_DIST; d++)
-    if (d < KT)
-      g.issue_prefetch(dump, a_ptr + d * G_KBYTES, b_ptr + d * b_step);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  for (int d = 0; d < NST - 1; d++)
+    g.issue_loads(smem + d * FG::STAGE_BYTES, a_ptr + d * FG::KB, b_ptr + d * b_step);
+  FG::template wait_dma<NST - 2>();
   __builtin_amdgcn_s_barrier();
-  g.load_frags(smem0, 0, a0, b0);
+  g.load_frags(smem, 0, a0, b0);
 
-  for (int kt = 0; kt < KT; kt += 2) {
-    a_ptr += G_KBYTES;
-    b_ptr += b_step;
-    g.stage(smem0, smem1, dump, kt + 1 < KT, a_ptr, b_ptr, kt + 1 + PF_DIST < KT, a_ptr + PF_DIST * G_KBYTES,
-            b_ptr + PF_DIST * b_step, acc, a0, b0, a1, b1);
-    if (kt + 1 < KT) {
-      a_ptr += G_KBYTES;
-      b_ptr += b_step;
-      g.stage(smem1, smem0, dump, kt + 2 < KT, a_ptr, b_ptr, kt + 2 + PF_DIST < KT, a_ptr + PF_DIST * G_KBYTES,
-              b_ptr + PF_DIST * b_step, acc, a0, b0, a1, b1);
-    }
+  // steady state: groups of NST stages in which every stage still has a block to request
+  int kt0 = 0;
+  for (; kt0 + 2 * NST <= KT; kt0 += NST) {
+    static_for<0, NST>([&](auto sc) {
+      constexpr int st = decltype(sc)::value;
+      constexpr int cur = st, nxt = (st + 1) % NST, fill = (st + NST - 1) % NST;
+      const int kf = kt0 + st + NST - 1;
+      g.template stage<true, true, NST - 2>(smem + cur * FG::STAGE_BYTES, smem + nxt * FG::STAGE_BYTES,
+                                            smem + fill * FG::STAGE_BYTES, a_ptr + (int64_t)kf * FG::KB,
+                                            b_ptr + kf * b_step, acc, a0, b0, a1, b1);
+    });
   }
+  // last group: only its first stage requests a block (the last one); the ring drains
+  static_for<0, NST>([&](auto sc) {
+    constexpr int st = decltype(sc)::value;
+    constexpr int cur = st, nxt = (st + 1) % NST, fill = (st + NST - 1) % NST;
+    constexpr int behind = NST - 2 - st > 0 ? NST - 2 - st : 0;
+    const int kf = kt0 + st + NST - 1;
+    g.template stage<st == 0, (st < NST - 1), behind>(smem + cur * FG::STAGE_BYTES, smem + nxt * FG::STAGE_BYTES,
+                                                      smem + fill * FG::STAGE_BYTES, a_ptr + (int64_t)kf * FG::KB,
+                                                      b_ptr + kf * b_step, acc, a0, b0, a1, b1);
+  });
 
   // no wave reads fragments any more (the last stage's barrier came after its
   // final fragment reads), so the stage buffers can be overwritten
@@ -631,7 +639,6 @@ template <int ES> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast
   else
     gemm_epilogue<ES, false, false>(p, acc, m0, n0, wm, wn, l32, lh, nullptr);
 }
-
 
 // Host-side launch of the 256x256 tile kernels for one element size.
 template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t stream) {
@@ -644,14 +651,15 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const int BK = G_KBYTES / ES;
   // fast path: whole tiles, 16-byte aligned rows, and a tile's rows reachable with 32-bit byte offsets
-  bool fast = p.M % G_BM == 0 && p.N % G_BN == 0 && p.K % BK == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
+  const int KGROUP = 256 / ES; // K elements of one trip round the LDS ring
+  bool fast = p.M % G_BM == 0 && p.N % G_BN == 0 && p.K % KGROUP == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
               (p.lda * ES) % 16 == 0 && (p.ldb * ES) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
               p.lda * ES * G_BM < (int64_t)1 << 31 && p.ldb * ES * BK < (int64_t)1 << 31;
   if (p.group_m <= 0)
     p.group_m = 4;
   dim3 grid((unsigned)nblk), block(G_THREADS);
   if (fast)
-    hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS>), grid, block, 0, stream, p);
   else
     hipLaunchKernelGGL((gemm_tile256_kernel<ES, true>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 5;
