@@ -1,0 +1,781 @@
+#include "executable.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <set>
+#include <sstream>
+#include <stdexcept>
+
+#include "gc_hip_kernels.h"
+#include "kernels/eltwise_params.h"
+
+extern "C" {
+int gcmi_launch_eltwise(const gcmi::EltParams *p, hipStream_t stream);
+int gcmi_launch_reduce(const gcmi::ReduceParams *p, hipStream_t stream);
+int gcmi_launch_softmax(const gcmi::SoftmaxParams *p, hipStream_t stream);
+}
+
+namespace gcapi {
+
+namespace {
+
+void hip_check(hipError_t e, const char *what) {
+  if (e != hipSuccess) {
+    if (e == hipErrorOutOfMemory)
+      throw std::bad_alloc();
+    throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+  }
+}
+void gc_check(int rc, const char *what) {
+  if (rc != 0)
+    throw std::runtime_error(std::string(what) + ": " + gcmi_last_error());
+}
+
+std::vector<int64_t> dense_strides(const std::vector<int64_t> &shape) {
+  std::vector<int64_t> s(shape.size(), 1);
+  for (int i = (int)shape.size() - 2; i >= 0; i--)
+    s[i] = s[i + 1] * shape[i + 1];
+  return s;
+}
+bool is_dense(const LTensor &t) { return !t.strided || t.stride == dense_strides(t.shape); }
+int64_t prod(const std::vector<int64_t> &v, size_t lo, size_t hi) {
+  int64_t p = 1;
+  for (size_t i = lo; i < hi; i++)
+    p *= v[i];
+  return p;
+}
+bool is_device_pointer(const void *p) {
+  hipPointerAttribute_t attr;
+  hipError_t e = hipPointerGetAttributes(&attr, p);
+  if (e != hipSuccess) {
+    (void)hipGetLastError(); // plain host memory is reported as an error: clear it
+    return false;
+  }
+  return attr.type == hipMemoryTypeDevice;
+}
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+int act_of(const Op &op) {
+  if (op.kind == "ReLU")
+    return GCMI_ACT_RELU;
+  if (op.kind == "Sigmoid")
+    return GCMI_ACT_SIGMOID;
+  if (op.kind == "GELU") {
+    std::string m = op.attr_str("mode", "gelu_erf");
+    if (m == "gelu_tanh" || m == "tanh")
+      return GCMI_ACT_GELU_TANH;
+    if (m == "gelu_erf" || m == "erf")
+      return GCMI_ACT_GELU_ERF;
+    throw std::logic_error("Unsupported GELU mode: " + m);
+  }
+  return -1;
+}
+
+// [N] or [1,..,1,N]
+bool is_row_vector(const LTensor &t, int64_t N) {
+  if (t.shape.empty() || t.shape.back() != N)
+    return false;
+  for (size_t i = 0; i + 1 < t.shape.size(); i++)
+    if (t.shape[i] != 1)
+      return false;
+  return true;
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------
+int Executable::new_slot(size_t bytes, long tensor_id) {
+  Slot s;
+  s.bytes = bytes ? bytes : 4;
+  s.tensor_id = tensor_id;
+  slots_.push_back(std::move(s));
+  return (int)slots_.size() - 1;
+}
+
+int Executable::slot_for(size_t tid) {
+  auto it = slot_of_tensor_.find(tid);
+  if (it != slot_of_tensor_.end())
+    return it->second;
+  const LTensor &t = g_.tensors.at(tid);
+  int es = dt_size(t.dt);
+  if (es == 0)
+    throw std::logic_error(std::string("Unsupported tensor dtype on this path: ") + dt_name(t.dt));
+  int s = new_slot((size_t)t.numel() * es, (long)tid);
+  slot_of_tensor_[tid] = s;
+  return s;
+}
+
+int Executable::const_slot(const void *data, size_t bytes) {
+  int s = new_slot(bytes);
+  slots_[s].init.assign((const char *)data, (const char *)data + bytes);
+  return s;
+}
+
+void Executable::add_copy(int src, DT sdt, const std::vector<int64_t> &dims, const std::vector<int64_t> &strides,
+                          int dst, DT ddt) {
+  if (dims.size() > (size_t)gcmi::ELT_MAX_RANK)
+    throw std::logic_error("tensor rank above 6 is not supported");
+  Step s;
+  s.kind = Step::Elt;
+  s.note = "copy";
+  s.op = gcmi::ELT_COPY;
+  s.a = src, s.out = dst;
+  s.a_dt = dt_dnnl(sdt), s.out_dt = dt_dnnl(ddt);
+  s.dims = dims, s.sa = strides;
+  steps_.push_back(std::move(s));
+}
+
+// ---------------------------------------------------------------------------
+Executable::Executable(const char *json, bool dry) : g_(parse_graph(json)) {
+  verify_graph(g_);
+  plan();
+  if (dry)
+    return;
+  // arena layout
+  size_t off = 0;
+  for (auto &s : slots_) {
+    s.offset = off;
+    off += align256(s.bytes);
+  }
+  arena_bytes_ = off ? off : 256;
+  hip_check(hipMalloc((void **)&arena_, arena_bytes_), "hipMalloc(arena)");
+  hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
+  for (auto &s : slots_)
+    if (!s.init.empty())
+      hip_check(hipMemcpy(arena_ + s.offset, s.init.data(), s.init.size(), hipMemcpyHostToDevice), "upload constants");
+  ptr_.resize(slots_.size());
+}
+
+Executable::~Executable() {
+  if (stream_)
+    (void)hipStreamDestroy(stream_);
+  if (arena_)
+    (void)hipFree(arena_);
+}
+
+// ---------------------------------------------------------------------------
+void Executable::plan() {
+  const size_t n = g_.ops.size();
+  std::map<size_t, std::vector<size_t>> consumers;
+  for (size_t i = 0; i < n; i++)
+    for (auto id : g_.ops[i].in)
+      consumers[id].push_back(i);
+  std::set<size_t> outs(g_.output_ids.begin(), g_.output_ids.end());
+  std::map<size_t, size_t> producer;
+  for (size_t i = 0; i < n; i++)
+    for (auto id : g_.ops[i].out)
+      producer[id] = i;
+
+  // strided (non-dense) inputs are gathered into dense buffers first
+  for (auto id : g_.input_ids) {
+    const LTensor &t = g_.tensors.at(id);
+    if (!is_dense(t)) {
+      int64_t span = 1;
+      for (size_t d = 0; d < t.shape.size(); d++) {
+        if (t.stride[d] < 0)
+          throw std::logic_error("negative strides are not supported");
+        span += (t.shape[d] - 1) * t.stride[d];
+      }
+      int raw = new_slot((size_t)span * dt_size(t.dt));
+      slots_[raw].is_input = true;
+      slots_[raw].tensor_id = (long)id;
+      int dense = new_slot((size_t)t.numel() * dt_size(t.dt));
+      slot_of_tensor_[id] = dense;
+      add_copy(raw, t.dt, t.shape, t.stride, dense, t.dt);
+    } else {
+      slots_[slot_for(id)].is_input = true;
+    }
+  }
+  for (auto id : g_.output_ids) {
+    const LTensor &t = g_.tensors.at(id);
+    if (!is_dense(t))
+      throw std::logic_error("strided output tensors are not supported");
+    slots_[slot_for(id)].is_output = true;
+  }
+
+  // ---- matching pass: fused groups are emitted where their LAST op stands
+  std::vector<bool> skip(n, false), claimed(n, false);
+  std::map<size_t, std::vector<Step>> emit_at;
+  auto single_use = [&](size_t tid) { return !outs.count(tid) && consumers[tid].size() == 1; };
+
+  for (size_t i = 0; i < n; i++) {
+    const Op &mm = g_.ops[i];
+    if (mm.kind != "MatMul" || claimed[i])
+      continue;
+    auto T = [&](size_t id) -> const LTensor & { return g_.tensors.at(id); };
+    const bool ta = mm.attr_bool("transpose_a", false), tb = mm.attr_bool("transpose_b", false);
+
+    // ---------------- attention: MatMul(Q,K^T) -> [scale] -> [+mask] -> SoftMax -> MatMul(P,V)
+    {
+      const LTensor &q = T(mm.in[0]), &k = T(mm.in[1]);
+      size_t r = q.shape.size();
+      bool ok = mm.in.size() == 2 && !ta && tb && q.dt == DT::bf16 && k.dt == DT::bf16 && r >= 3 &&
+                k.shape.size() == r && q.shape[r - 1] == 128 &&
+                std::equal(q.shape.begin(), q.shape.end() - 2, k.shape.begin());
+      size_t cur = mm.out[0];
+      std::vector<size_t> chain{i};
+      long scale_t = -1, mask_t = -1;
+      bool scale_div = false;
+      size_t last = i;
+      if (ok) {
+        int64_t Sq = q.shape[r - 2], Sk = k.shape[r - 2];
+        bool seen_softmax = false;
+        while (ok) {
+          if (!single_use(cur)) {
+            ok = false;
+            break;
+          }
+          size_t ci = consumers[cur][0];
+          const Op &c = g_.ops[ci];
+          if ((c.kind == "Multiply" || c.kind == "Divide") && scale_t < 0 && mask_t < 0) {
+            size_t other = c.in[0] == cur ? c.in[1] : c.in[0];
+            if (c.kind == "Divide" && c.in[0] != cur) {
+              ok = false;
+              break;
+            }
+            const LTensor &st = T(other);
+            bool is_in = std::find(g_.input_ids.begin(), g_.input_ids.end(), other) != g_.input_ids.end();
+            if (st.numel() != 1 || !is_in || !(st.dt == DT::f32 || st.dt == DT::bf16)) {
+              ok = false;
+              break;
+            }
+            scale_t = (long)other, scale_div = c.kind == "Divide";
+          } else if (c.kind == "Add" && mask_t < 0) {
+            size_t other = c.in[0] == cur ? c.in[1] : c.in[0];
+            const LTensor &mt = T(other);
+            size_t mr = mt.shape.size();
+            bool shape_ok = mr >= 2 && mt.shape[mr - 1] == Sk && mt.shape[mr - 2] == Sq && prod(mt.shape, 0, mr - 2) == 1;
+            if (!shape_ok || !(mt.dt == DT::f32 || mt.dt == DT::bf16) ) {
+              ok = false;
+              break;
+            }
+            mask_t = (long)other;
+          } else if (c.kind == "SoftMax") {
+            int64_t ax = c.attr_s64("axis", 1);
+            if (ax < 0)
+              ax += (int64_t)r;
+            if (ax != (int64_t)r - 1) {
+              ok = false;
+              break;
+            }
+            seen_softmax = true;
+          } else if (c.kind == "MatMul" && seen_softmax) {
+            const LTensor &v = T(c.in[1]);
+            bool fin = c.in.size() == 2 && c.in[0] == cur && !c.attr_bool("transpose_a", false) &&
+                       !c.attr_bool("transpose_b", false) && v.dt == DT::bf16 && v.shape.size() == r &&
+                       v.shape[r - 1] == 128 && v.shape[r - 2] == Sk &&
+                       std::equal(q.shape.begin(), q.shape.end() - 2, v.shape.begin()) && T(c.out[0]).dt == DT::bf16;
+            if (!fin) {
+              ok = false;
+              break;
+            }
+            chain.push_back(ci);
+            last = ci;
+            break;
+          } else {
+            ok = false;
+            break;
+          }
+          if (seen_softmax && c.kind != "SoftMax") {
+            ok = false;
+            break;
+          }
+          chain.push_back(ci);
+          cur = c.out[0];
+        }
+        if (ok && last != i) {
+          const Op &pv = g_.ops[last];
+          std::vector<Step> v;
+          int mask_slot = -1;
+          int64_t mask_ld = 0;
+          if (mask_t >= 0) {
+            const LTensor &mt = T((size_t)mask_t);
+            mask_slot = slot_for((size_t)mask_t);
+            mask_ld = Sk;
+            if (mt.dt != DT::f32) { // the kernel adds an f32 mask
+              int f = new_slot((size_t)mt.numel() * 4);
+              Step cp;
+              cp.kind = Step::Elt, cp.note = "mask -> f32", cp.op = gcmi::ELT_COPY, cp.a = mask_slot, cp.out = f;
+              cp.a_dt = dt_dnnl(mt.dt), cp.out_dt = GCMI_F32;
+              cp.dims = {mt.numel()}, cp.sa = {1};
+              v.push_back(cp);
+              mask_slot = f;
+            }
+          }
+          Step s;
+          s.kind = Step::Mha;
+          s.note = "attention: MatMul+scale+mask+SoftMax+MatMul fused (" + std::to_string(chain.size()) + " ops)";
+          s.a = slot_for(mm.in[0]), s.b = slot_for(mm.in[1]), s.c = slot_for(pv.in[1]), s.out = slot_for(pv.out[0]);
+          s.mask = mask_slot, s.mask_ld = mask_ld;
+          s.BH = prod(q.shape, 0, r - 2), s.Sq = Sq, s.Sk = Sk, s.D = 128;
+          s.scale = 1.0f;
+          if (scale_t >= 0) {
+            s.scale_slot = slot_for((size_t)scale_t);
+            s.scale_div = scale_div;
+            s.a_dt = dt_dnnl(T((size_t)scale_t).dt);
+          }
+          v.push_back(s);
+          for (auto ci : chain)
+            skip[ci] = claimed[ci] = true;
+          skip[last] = false;
+          emit_at[last] = v;
+          continue;
+        }
+      }
+    }
+
+    // ---------------- quantised: Dequantize(A) , Dequantize(W) -> MatMul -> [bias] -> [act] -> [cast]
+    bool int8 = false;
+    size_t dq_a = 0, dq_w = 0;
+    if (!ta && !tb && producer.count(mm.in[0]) && producer.count(mm.in[1]) && T(mm.out[0]).dt == DT::f32) {
+      dq_a = producer[mm.in[0]], dq_w = producer[mm.in[1]];
+      const Op &da = g_.ops[dq_a], &dw = g_.ops[dq_w];
+      if (da.kind == "Dequantize" && dw.kind == "Dequantize" && single_use(mm.in[0]) && single_use(mm.in[1])) {
+        const LTensor &qa = T(da.in[0]), &qw = T(dw.in[0]);
+        const auto &sa = da.attrs.at("scales").fa, &sw = dw.attrs.at("scales").fa;
+        std::vector<int64_t> zw;
+        if (dw.attrs.count("zps"))
+          zw = dw.attrs.at("zps").ia;
+        bool zw0 = std::all_of(zw.begin(), zw.end(), [](int64_t z) { return z == 0; });
+        int64_t axw = dw.attr_s64("axis", 1);
+        if (axw < 0)
+          axw += (int64_t)qw.shape.size();
+        int8 = sa.size() == 1 && qw.dt == DT::s8 && qw.shape.size() == 2 && qa.shape.size() >= 2 && zw0 &&
+               (sw.size() == 1 || axw == 1) && is_dense(qa) && is_dense(qw);
+      }
+    }
+
+    // ---------------- epilogue chain shared by the plain and the quantised GEMM
+    const LTensor &A = T(mm.in[0]), &B = T(mm.in[1]);
+    const size_t ra = A.shape.size(), rb = B.shape.size();
+    // fusable only when the contraction is one flat GEMM: [.., M, K] x [K, N]
+    bool flat = ra >= 2 && rb == 2 && (!ta || ra == 2);
+    int64_t Nn = flat ? (tb ? B.shape[0] : B.shape[1]) : 0;
+    long bias_t = mm.in.size() == 3 ? (long)mm.in[2] : -1;
+    bool bias_in_matmul = bias_t >= 0;
+    if (bias_t >= 0 && !(flat && is_row_vector(T((size_t)bias_t), Nn)))
+      bias_t = -1; // handled as a separate Add below
+    int act = 0;
+    size_t cur = mm.out[0], last = i;
+    std::vector<size_t> chain;
+    DT gemm_dt = int8 ? DT::f32 : A.dt;
+    if (flat && (gemm_dt == DT::f32 || gemm_dt == DT::bf16) && (bias_in_matmul ? bias_t >= 0 : true)) {
+      while (single_use(cur)) {
+        size_t ci = consumers[cur][0];
+        const Op &c = g_.ops[ci];
+        if (claimed[ci])
+          break;
+        if (c.kind == "Add" && bias_t < 0 && act == 0) {
+          size_t other = c.in[0] == cur ? c.in[1] : c.in[0];
+          const LTensor &bt = T(other);
+          bool dt_ok = bt.dt == T(cur).dt;
+          if (!is_row_vector(bt, Nn) || !dt_ok || T(c.out[0]).shape != T(cur).shape)
+            break;
+          bias_t = (long)other;
+        } else if (act_of(c) > 0 && act == 0) {
+          act = act_of(c);
+        } else if (int8 && (c.kind == "Typecast" || c.kind == "TypeCast") && T(c.out[0]).dt == DT::bf16) {
+          chain.push_back(ci);
+          last = ci;
+          cur = c.out[0];
+          break;
+        } else {
+          break;
+        }
+        chain.push_back(ci);
+        last = ci;
+        cur = c.out[0];
+      }
+    }
+
+    std::vector<Step> v;
+    std::string fused;
+    if (bias_t >= 0)
+      fused += "+bias";
+    if (act)
+      fused += "+act";
+    if (int8 && flat) {
+      const Op &da = g_.ops[dq_a], &dw = g_.ops[dq_w];
+      const LTensor &qa = T(da.in[0]), &qw = T(dw.in[0]);
+      const float sA = da.attrs.at("scales").fa[0];
+      const auto &sw = dw.attrs.at("scales").fa;
+      int32_t zpA = 0;
+      if (da.attrs.count("zps") && !da.attrs.at("zps").ia.empty())
+        zpA = (int32_t)da.attrs.at("zps").ia[0];
+      int64_t K = qw.shape[0], N = qw.shape[1], M = qa.numel() / K;
+      // output_scales = data_scales (x) weight_scales
+      // (legacy/core/src/compiler/ir/graph/transform/quantization/graph_reschedule.cpp:220-235)
+      std::vector<float> sc((size_t)N);
+      for (int64_t nI = 0; nI < N; nI++)
+        sc[(size_t)nI] = sA * (sw.size() == 1 ? sw[0] : sw[(size_t)nI]);
+      int sc_slot = const_slot(sc.data(), sc.size() * 4);
+      int cs_slot = new_slot((size_t)N * 4);
+      Step cs;
+      cs.kind = Step::ColSum, cs.note = qw.constant ? "colsum(W), once: W is constant" : "colsum(W)";
+      cs.a = slot_for(dw.in[0]), cs.out = cs_slot, cs.K = K, cs.N = N, cs.lda = N;
+      cs.op = qw.constant ? 1 : 0;
+      v.push_back(cs);
+      Step s;
+      s.kind = Step::GemmInt8;
+      s.note = "Dequantize x2 + MatMul" + fused + (T(cur).dt == DT::bf16 ? "+cast" : "") + " fused";
+      s.a = slot_for(da.in[0]), s.b = slot_for(dw.in[0]), s.out = slot_for(cur);
+      s.M = M, s.N = N, s.K = K, s.lda = K, s.ldb = N, s.ldc = N;
+      s.a_dt = dt_dnnl(qa.dt), s.zp = zpA, s.aux = cs_slot, s.scales_slot = sc_slot;
+      s.bias = bias_t >= 0 ? slot_for((size_t)bias_t) : -1;
+      s.act = act, s.out_dt = dt_dnnl(T(cur).dt);
+      v.push_back(s);
+      skip[dq_a] = skip[dq_w] = claimed[dq_a] = claimed[dq_w] = true;
+    } else {
+      // plain GEMM, possibly batched
+      if (A.dt == DT::f16)
+        throw std::logic_error("f16 MatMul is not supported (bf16 and f32 are)");
+      // stored 2-D views: 1-D operands become [1,K] / [K,1]
+      std::vector<int64_t> as = A.shape, bs = B.shape;
+      bool a1 = ra == 1, b1 = rb == 1;
+      if (a1)
+        as = {1, A.shape[0]};
+      if (b1)
+        bs = {B.shape[0], 1};
+      bool tA = a1 ? false : ta, tB = b1 ? false : tb;
+      size_t Ra = as.size(), Rb = bs.size();
+      int64_t M = tA ? as[Ra - 1] : as[Ra - 2], K = tA ? as[Ra - 2] : as[Ra - 1];
+      int64_t N = tB ? bs[Rb - 2] : bs[Rb - 1];
+      int sa_slot = slot_for(mm.in[0]), sb_slot = slot_for(mm.in[1]);
+      DT out_dt = T(mm.out[0]).dt;
+      if (A.dt == DT::bf16 && (tA || tB)) {
+        // the bf16 kernel reads row-major [M,K] and [K,N]: materialise the transposes
+        auto transposed = [&](int slot, std::vector<int64_t> &shp) {
+          std::vector<int64_t> st = dense_strides(shp), d = shp;
+          std::swap(d[d.size() - 1], d[d.size() - 2]);
+          std::swap(st[st.size() - 1], st[st.size() - 2]);
+          int t = new_slot((size_t)prod(shp, 0, shp.size()) * 2);
+          if (d.size() > (size_t)gcmi::ELT_MAX_RANK)
+            throw std::logic_error("tensor rank above 6 is not supported");
+          Step cp;
+          cp.kind = Step::Elt, cp.note = "transpose copy", cp.op = gcmi::ELT_COPY, cp.a = slot, cp.out = t;
+          cp.a_dt = cp.out_dt = GCMI_BF16, cp.dims = d, cp.sa = st;
+          v.push_back(cp);
+          shp = d;
+          return t;
+        };
+        if (tA)
+          sa_slot = transposed(sa_slot, as), tA = false;
+        if (tB)
+          sb_slot = transposed(sb_slot, bs), tB = false;
+      }
+      std::vector<int64_t> ba(as.begin(), as.end() - 2), bb(bs.begin(), bs.end() - 2), bo;
+      broadcast_shape(ba, bb, bo);
+      int64_t nb = prod(bo, 0, bo.size());
+      bool flatten = bb.empty() && !tA; // [..,M,K] x [K,N]: one GEMM over all rows
+      int64_t a_mat = as[Ra - 1] * as[Ra - 2], b_mat = bs[Rb - 1] * bs[Rb - 2];
+      auto batch_off = [&](const std::vector<int64_t> &bd, int64_t idx) {
+        // index into a (possibly broadcast) batch shape aligned to the right of bo
+        int64_t off = 0, mul = 1;
+        for (int d = (int)bo.size() - 1; d >= 0; d--) {
+          int64_t c = idx % bo[d];
+          idx /= bo[d];
+          int dd = d - ((int)bo.size() - (int)bd.size());
+          if (dd >= 0) {
+            if (bd[dd] != 1)
+              off += c * mul;
+            mul *= bd[dd];
+          }
+        }
+        return off;
+      };
+      int out_slot = slot_for(chain.empty() ? mm.out[0] : cur);
+      int64_t reps = flatten ? 1 : nb;
+      for (int64_t bi = 0; bi < reps; bi++) {
+        Step s;
+        s.kind = A.dt == DT::f32 ? Step::GemmF32 : Step::GemmBf16;
+        s.note = std::string("MatMul") + fused + (reps > 1 ? " (batched)" : "");
+        s.a = sa_slot, s.b = sb_slot, s.out = out_slot;
+        s.M = flatten ? M * nb : M, s.N = N, s.K = K;
+        s.lda = as[Ra - 1], s.ldb = bs[Rb - 1], s.ldc = N;
+        s.ta = tA, s.tb = tB;
+        if (!flatten) {
+          s.a_off = batch_off(ba, bi) * a_mat, s.b_off = batch_off(bb, bi) * b_mat, s.out_off = bi * M * N;
+        }
+        s.bias = bias_t >= 0 ? slot_for((size_t)bias_t) : -1;
+        s.bias_dt = bias_t >= 0 ? dt_dnnl(T((size_t)bias_t).dt) : 0;
+        s.act = act;
+        s.out_dt = dt_dnnl(chain.empty() ? out_dt : T(cur).dt);
+        v.push_back(s);
+      }
+      // a MatMul bias that is not a row vector: separate broadcast add, in place
+      if (bias_in_matmul && bias_t < 0) {
+        const LTensor &bt = T(mm.in[2]), &ot = T(mm.out[0]);
+        Step s;
+        s.kind = Step::Elt, s.note = "bias add", s.op = gcmi::ELT_ADD;
+        s.a = out_slot, s.b = slot_for(mm.in[2]), s.out = out_slot;
+        s.a_dt = s.out_dt = dt_dnnl(ot.dt), s.b_dt = dt_dnnl(bt.dt);
+        s.dims = ot.shape, s.sa = dense_strides(ot.shape);
+        std::vector<int64_t> bst = dense_strides(bt.shape), full(ot.shape.size(), 0);
+        for (size_t d = 0; d < bt.shape.size(); d++) {
+          size_t od = ot.shape.size() - bt.shape.size() + d;
+          full[od] = bt.shape[d] == 1 ? 0 : bst[d];
+        }
+        s.sb = full;
+        if (s.dims.size() > (size_t)gcmi::ELT_MAX_RANK)
+          throw std::logic_error("tensor rank above 6 is not supported");
+        v.push_back(s);
+      }
+    }
+    for (auto ci : chain)
+      skip[ci] = claimed[ci] = true;
+    skip[i] = claimed[i] = true;
+    skip[last] = false;
+    emit_at[last] = v;
+  }
+
+  // ---- emission pass, in op order
+  for (size_t i = 0; i < n; i++) {
+    if (skip[i])
+      continue;
+    auto it = emit_at.find(i);
+    if (it != emit_at.end()) {
+      for (auto &s : it->second)
+        steps_.push_back(s);
+      continue;
+    }
+    plan_generic(g_.ops[i]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+void Executable::plan_generic(const Op &op) {
+  auto T = [&](size_t id) -> const LTensor & { return g_.tensors.at(id); };
+  const std::string &k = op.kind;
+  const LTensor &out = T(op.out[0]);
+  if (out.shape.size() > (size_t)gcmi::ELT_MAX_RANK)
+    throw std::logic_error("tensor rank above 6 is not supported");
+  auto bstrides = [&](const LTensor &t) {
+    std::vector<int64_t> st = dense_strides(t.shape), full(out.shape.size(), 0);
+    for (size_t d = 0; d < t.shape.size(); d++) {
+      size_t od = out.shape.size() - t.shape.size() + d;
+      full[od] = t.shape[d] == 1 ? 0 : st[d];
+    }
+    return full;
+  };
+  Step s;
+  s.kind = Step::Elt;
+  s.note = k;
+  if (k == "Add" || k == "Subtract" || k == "Multiply" || k == "Divide") {
+    s.op = k == "Add" ? gcmi::ELT_ADD : k == "Subtract" ? gcmi::ELT_SUB : k == "Multiply" ? gcmi::ELT_MUL : gcmi::ELT_DIV;
+    s.a = slot_for(op.in[0]), s.b = slot_for(op.in[1]), s.out = slot_for(op.out[0]);
+    s.a_dt = dt_dnnl(T(op.in[0]).dt), s.b_dt = dt_dnnl(T(op.in[1]).dt), s.out_dt = dt_dnnl(out.dt);
+    s.dims = out.shape, s.sa = bstrides(T(op.in[0])), s.sb = bstrides(T(op.in[1]));
+  } else if (k == "ReLU" || k == "Sigmoid" || k == "GELU" || k == "Pow" || k == "Typecast" || k == "TypeCast") {
+    s.op = k == "ReLU" ? gcmi::ELT_RELU
+           : k == "Sigmoid" ? gcmi::ELT_SIGMOID
+           : k == "GELU" ? (act_of(op) == GCMI_ACT_GELU_TANH ? gcmi::ELT_GELU_TANH : gcmi::ELT_GELU_ERF)
+           : k == "Pow" ? gcmi::ELT_POW
+                        : gcmi::ELT_COPY;
+    s.alpha = k == "Pow" ? op.attr_f32("beta", 1.0f) : 0.0f;
+    s.a = slot_for(op.in[0]), s.out = slot_for(op.out[0]);
+    s.a_dt = dt_dnnl(T(op.in[0]).dt), s.out_dt = dt_dnnl(out.dt);
+    s.dims = {out.numel()}, s.sa = {1};
+  } else if (k == "Dequantize" || k == "Quantize") {
+    const LTensor &in = T(op.in[0]);
+    s.op = k == "Dequantize" ? gcmi::ELT_DEQUANT : gcmi::ELT_QUANT;
+    s.a = slot_for(op.in[0]), s.out = slot_for(op.out[0]);
+    s.a_dt = dt_dnnl(in.dt), s.out_dt = dt_dnnl(out.dt);
+    s.dims = out.shape, s.sa = dense_strides(out.shape);
+    const auto &sc = op.attrs.at("scales").fa;
+    s.n_scales = (int)sc.size();
+    s.scales_slot = const_slot(sc.data(), sc.size() * 4);
+    std::vector<int32_t> zp(sc.size(), 0);
+    if (op.attrs.count("zps")) {
+      const auto &z = op.attrs.at("zps").ia;
+      for (size_t i = 0; i < zp.size() && !z.empty(); i++)
+        zp[i] = (int32_t)(z.size() == 1 ? z[0] : z[i]);
+    }
+    s.zps_slot = const_slot(zp.data(), zp.size() * 4);
+    int64_t ax = op.attr_s64("axis", 1);
+    if (ax < 0)
+      ax += (int64_t)out.shape.size();
+    s.ch_axis = (int)ax;
+  } else if (k == "ReduceSum" || k == "ReduceMean") {
+    const LTensor &in = T(op.in[0]);
+    std::vector<int64_t> axes;
+    if (op.attrs.count("axes"))
+      axes = op.attrs.at("axes").ia;
+    auto ca = canonical_axes(axes, (int64_t)in.shape.size());
+    auto st = dense_strides(in.shape);
+    s.kind = Step::Reduce;
+    s.a = slot_for(op.in[0]), s.out = slot_for(op.out[0]);
+    s.a_dt = dt_dnnl(in.dt);
+    s.mean = k == "ReduceMean";
+    for (size_t d = 0; d < in.shape.size(); d++) {
+      bool red = std::find(ca.begin(), ca.end(), (int64_t)d) != ca.end();
+      (red ? s.rdims : s.kdims).push_back(in.shape[d]);
+      (red ? s.rstr : s.kstr).push_back(st[d]);
+    }
+  } else if (k == "SoftMax") {
+    const LTensor &in = T(op.in[0]);
+    int64_t r = (int64_t)in.shape.size(), ax = op.attr_s64("axis", 1);
+    if (ax < 0)
+      ax += r;
+    s.kind = Step::Softmax;
+    s.a = slot_for(op.in[0]), s.out = slot_for(op.out[0]);
+    s.a_dt = dt_dnnl(in.dt), s.out_dt = dt_dnnl(out.dt);
+    s.outer = prod(in.shape, 0, (size_t)ax), s.len = in.shape[(size_t)ax], s.inner = prod(in.shape, (size_t)ax + 1, (size_t)r);
+  } else {
+    throw std::logic_error("Unsupported operation: " + k);
+  }
+  steps_.push_back(std::move(s));
+}
+
+// ---------------------------------------------------------------------------
+void Executable::launch(const Step &s) {
+  auto P = [&](int slot) -> char * { return slot < 0 ? nullptr : (char *)ptr_[(size_t)slot]; };
+  switch (s.kind) {
+  case Step::GemmF32:
+    gc_check(gcmi_gemm_f32((const float *)P(s.a) + s.a_off, (const float *)P(s.b) + s.b_off, (float *)P(s.out) + s.out_off,
+                           s.M, s.N, s.K, s.lda, s.ldb, s.ldc, s.ta, s.tb, (const float *)P(s.bias), s.act, stream_),
+             "MatMul f32");
+    break;
+  case Step::GemmBf16:
+    gc_check(gcmi_gemm_bf16(P(s.a) + s.a_off * 2, P(s.b) + s.b_off * 2, P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4),
+                            s.M, s.N, s.K, s.lda, s.ldb, s.ldc, P(s.bias), s.bias_dt ? s.bias_dt : GCMI_BF16, s.act,
+                            s.out_dt, stream_),
+             "MatMul bf16");
+    break;
+  case Step::ColSum:
+    if (s.op == 1 && colsum_valid_[s.out])
+      break; // constant weight: already summed
+    gc_check(gcmi_colsum_s8(P(s.a), s.K, s.N, s.lda, (int32_t *)P(s.out), stream_), "colsum");
+    colsum_valid_[s.out] = true;
+    break;
+  case Step::GemmInt8:
+    gc_check(gcmi_gemm_int8(P(s.a), s.a_dt, P(s.b), P(s.out), s.M, s.N, s.K, s.lda, s.ldb, s.ldc, (const int32_t *)P(s.aux),
+                            s.zp, (const float *)P(s.scales_slot), (const float *)P(s.bias), s.act, s.out_dt, stream_),
+             "MatMul int8");
+    break;
+  case Step::Mha: {
+    float scale = s.scale;
+    if (s.scale_slot >= 0) {
+      // a one-element input tensor: read it back (blocks until staging is done)
+      uint32_t raw = 0;
+      hip_check(hipMemcpyAsync(&raw, P(s.scale_slot), s.a_dt == GCMI_BF16 ? 2 : 4, hipMemcpyDeviceToHost, stream_), "read scale");
+      hip_check(hipStreamSynchronize(stream_), "read scale");
+      float v;
+      if (s.a_dt == GCMI_BF16)
+        raw <<= 16;
+      memcpy(&v, &raw, 4);
+      scale = s.scale_div ? 1.0f / v : v;
+    }
+    gc_check(gcmi_mha_fwd_bf16(P(s.a), P(s.b), P(s.c), (const float *)P(s.mask), s.mask_ld, P(s.out), s.BH, s.Sq, s.Sk, s.D,
+                               scale, stream_),
+             "attention");
+    break;
+  }
+  case Step::Elt: {
+    gcmi::EltParams p{};
+    p.a = P(s.a), p.b = P(s.b), p.out = P(s.out);
+    p.op = s.op, p.a_dt = s.a_dt, p.b_dt = s.b_dt, p.out_dt = s.out_dt, p.alpha = s.alpha;
+    size_t r = s.dims.size(), pad = gcmi::ELT_MAX_RANK - r;
+    p.n = 1;
+    for (int d = 0; d < gcmi::ELT_MAX_RANK; d++)
+      p.dims[d] = 1, p.sa[d] = 0, p.sb[d] = 0;
+    for (size_t d = 0; d < r; d++) {
+      p.dims[pad + d] = s.dims[d];
+      p.sa[pad + d] = s.sa.empty() ? 0 : s.sa[d];
+      p.sb[pad + d] = s.sb.empty() ? 0 : s.sb[d];
+      p.n *= s.dims[d];
+    }
+    p.scales = (const float *)P(s.scales_slot), p.zps = (const int32_t *)P(s.zps_slot);
+    p.n_scales = s.n_scales, p.ch_axis = s.ch_axis >= 0 ? (int)pad + s.ch_axis : -1;
+    gc_check(gcmi_launch_eltwise(&p, stream_) ? 5 : 0, s.note.c_str());
+    break;
+  }
+  case Step::Reduce: {
+    gcmi::ReduceParams p{};
+    p.in = P(s.a), p.out = P(s.out), p.dt = s.a_dt, p.mean = s.mean;
+    p.n_out = 1, p.n_red = 1;
+    for (int d = 0; d < gcmi::ELT_MAX_RANK; d++)
+      p.kdims[d] = p.rdims[d] = 1, p.kstr[d] = p.rstr[d] = 0;
+    size_t pk = gcmi::ELT_MAX_RANK - s.kdims.size(), pr = gcmi::ELT_MAX_RANK - s.rdims.size();
+    for (size_t d = 0; d < s.kdims.size(); d++)
+      p.kdims[pk + d] = s.kdims[d], p.kstr[pk + d] = s.kstr[d], p.n_out *= s.kdims[d];
+    for (size_t d = 0; d < s.rdims.size(); d++)
+      p.rdims[pr + d] = s.rdims[d], p.rstr[pr + d] = s.rstr[d], p.n_red *= s.rdims[d];
+    gc_check(gcmi_launch_reduce(&p, stream_) ? 5 : 0, s.note.c_str());
+    break;
+  }
+  case Step::Softmax: {
+    gcmi::SoftmaxParams p{};
+    p.in = P(s.a), p.out = P(s.out), p.outer = s.outer, p.len = s.len, p.inner = s.inner, p.in_dt = s.a_dt, p.out_dt = s.out_dt;
+    gc_check(gcmi_launch_softmax(&p, stream_) ? 5 : 0, "SoftMax");
+    break;
+  }
+  }
+}
+
+// src/dnnl/dnnl_graph_compiler.cpp:64-103
+void Executable::execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs) {
+  auto find = [](dnnl_graph_compiler_tensor *ts, size_t n, size_t i, size_t id) -> dnnl_graph_compiler_tensor * {
+    if (!ts)
+      throw std::invalid_argument("Tensor not found");
+    if (ts[i].id == id)
+      return &ts[i];
+    for (size_t j = 0; j < n; j++) // the order may differ from the argument order
+      if (ts[j].id == id)
+        return &ts[j];
+    throw std::invalid_argument("Tensor not found");
+  };
+  for (size_t s = 0; s < slots_.size(); s++)
+    ptr_[s] = arena_ + slots_[s].offset;
+
+  // inputs: device pointers are used in place, host buffers are staged
+  for (size_t i = 0; i < g_.input_ids.size(); i++) {
+    size_t id = g_.input_ids[i];
+    auto *t = find(inputs, g_.input_ids.size(), i, id);
+    if (t->ndims > DNNL_MAX_NDIMS)
+      throw std::invalid_argument("Number of dimensions > DNNL_MAX_NDIMS");
+    int slot = -1;
+    for (size_t s = 0; s < slots_.size(); s++)
+      if (slots_[s].is_input && slots_[s].tensor_id == (long)id)
+        slot = (int)s;
+    if (slot < 0 || !t->data)
+      continue;
+    if (is_device_pointer(t->data))
+      ptr_[(size_t)slot] = t->data;
+    else
+      hip_check(hipMemcpyAsync(ptr_[(size_t)slot], t->data, slots_[(size_t)slot].bytes, hipMemcpyHostToDevice, stream_), "stage input");
+  }
+  std::vector<std::pair<void *, int>> copy_back;
+  for (size_t i = 0; i < g_.output_ids.size(); i++) {
+    size_t id = g_.output_ids[i];
+    auto *t = find(outputs, g_.output_ids.size(), i, id);
+    if (t->ndims > DNNL_MAX_NDIMS)
+      throw std::invalid_argument("Number of dimensions > DNNL_MAX_NDIMS");
+    int slot = slot_of_tensor_.at(id);
+    if (!t->data)
+      throw std::invalid_argument("Output tensor has no buffer");
+    bool also_input = slots_[(size_t)slot].is_input;
+    if (is_device_pointer(t->data) && !also_input)
+      ptr_[(size_t)slot] = t->data;
+    else
+      copy_back.emplace_back(t->data, slot);
+  }
+  for (auto &s : steps_)
+    launch(s);
+  for (auto &cb : copy_back) {
+    hipMemcpyKind kind = is_device_pointer(cb.first) ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost;
+    hip_check(hipMemcpyAsync(cb.first, ptr_[(size_t)cb.second], slots_[(size_t)cb.second].bytes, kind, stream_), "copy result");
+  }
+  hip_check(hipStreamSynchronize(stream_), "execute");
+}
+
+std::string Executable::describe() const {
+  static const char *names[] = {"gemm_f32", "gemm_bf16", "gemm_int8", "colsum", "attention", "eltwise", "reduce", "softmax"};
+  std::ostringstream os;
+  for (auto &s : steps_)
+    os << names[(int)s.kind] << ": " << s.note << "\n";
+  return os.str();
+}
+
+} // namespace gcapi

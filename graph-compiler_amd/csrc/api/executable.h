@@ -1,0 +1,102 @@
+// A compiled partition: a list of kernel launches over device buffers.
+//
+// compile  = parse (graph.h) -> verify -> fuse -> plan.  Fusion replaces the
+//            reference's tiling + consumer fusion passes
+//            (lib/gc/Transforms/DeepTileContractionOp.cpp,
+//             lib/gc/Transforms/IterativeTilingAndFusion.cpp:585-611): a MatMul
+//            absorbs the bias add / activation / cast that follow it into the
+//            GEMM epilogue; Dequantize -> MatMul becomes the int8 GEMM with a
+//            dequantising epilogue; MatMul -> scale -> +mask -> SoftMax ->
+//            MatMul becomes one attention kernel.  Everything else runs as a
+//            generic kernel per op.
+// execute  = match tensors by id (src/dnnl/dnnl_graph_compiler.cpp:64-103),
+//            stage host buffers to the device arena (device pointers are used
+//            in place), launch, copy results back, wait.
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "dnnl_graph_compiler.h"
+#include "graph.h"
+
+namespace gcapi {
+
+struct Step {
+  enum Kind { GemmF32, GemmBf16, GemmInt8, ColSum, Mha, Elt, Reduce, Softmax } kind;
+  std::string note; // what was fused, for introspection
+  // operands are arena slot indices (-1 = none)
+  int a = -1, b = -1, c = -1, out = -1, bias = -1, mask = -1, aux = -1;
+  int64_t M = 0, N = 0, K = 0, lda = 0, ldb = 0, ldc = 0;
+  int64_t a_off = 0, b_off = 0, out_off = 0; // element offsets (batched fallbacks)
+  bool ta = false, tb = false;
+  int act = 0, out_dt = 0, bias_dt = 0, a_dt = 0;
+  int32_t zp = 0;
+  // attention
+  int64_t BH = 0, Sq = 0, Sk = 0, D = 0, mask_ld = 0;
+  float scale = 1.0f;
+  int scale_slot = -1;   // 1-element tensor holding the scale (or its reciprocal)
+  bool scale_div = false;
+  // generic kernels: parameter blocks are filled at plan time with slot ids
+  // resolved to pointers at execute time
+  std::vector<int64_t> dims, sa, sb;
+  int op = 0, b_dt = 0;
+  float alpha = 0;
+  int n_scales = 0, ch_axis = -1, scales_slot = -1, zps_slot = -1;
+  // reduce
+  std::vector<int64_t> kdims, kstr, rdims, rstr;
+  bool mean = false;
+  // softmax
+  int64_t outer = 0, len = 0, inner = 0;
+};
+
+struct Slot {
+  size_t bytes = 0;
+  size_t offset = 0;   // into the arena
+  long tensor_id = -1; // graph tensor it holds, -1 for temporaries / constants
+  bool is_input = false, is_output = false;
+  std::vector<char> init; // constant contents uploaded at compile time
+};
+
+class Executable {
+public:
+  // dry = plan only: no device memory, no stream (host-side tests and explain)
+  explicit Executable(const char *json, bool dry = false);
+  ~Executable();
+  Executable(const Executable &) = delete;
+  Executable &operator=(const Executable &) = delete;
+
+  void execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs);
+
+  const Graph &graph() const { return g_; }
+  const std::vector<Step> &steps() const { return steps_; }
+  std::string describe() const; // one line per step
+
+private:
+  Graph g_;
+  std::vector<Step> steps_;
+  std::vector<Slot> slots_;
+  std::unordered_map<size_t, int> slot_of_tensor_;
+  std::vector<void *> ptr_; // per-slot device pointer during execute
+  char *arena_ = nullptr;
+  size_t arena_bytes_ = 0;
+  hipStream_t stream_ = nullptr;
+  std::unordered_map<int, bool> colsum_valid_; // ColSum results of constant weights are computed once
+
+  int new_slot(size_t bytes, long tensor_id = -1);
+  int slot_for(size_t tensor_id);
+  int const_slot(const void *data, size_t bytes);
+  void plan();
+  void plan_generic(const Op &op);
+  void plan_matmul(size_t op_index, std::vector<bool> &done);
+  bool try_int8(size_t op_index, std::vector<bool> &done);
+  bool try_mha(size_t op_index, std::vector<bool> &done);
+  void add_copy(int src_slot, DT src_dt, const std::vector<int64_t> &dims, const std::vector<int64_t> &strides,
+                int dst_slot, DT dst_dt);
+  void launch(const Step &s);
+};
+
+} // namespace gcapi

@@ -1,0 +1,120 @@
+/*
+ * dnnl_graph_compiler.h -- the oneDNN-Graph compiler-backend C API of
+ * intel/graph-compiler, served by MI355X (gfx950) kernels.
+ *
+ * The reference implements these six entry points in
+ * src/dnnl/dnnl_graph_compiler.cpp:157-226 against a header that lives in a
+ * oneDNN fork (graph/backend/elyzor/include/dnnl_graph_compiler.h) and is not
+ * part of the reference tree.  This header re-declares the same functions and
+ * structures as recovered from every use site:
+ *   context  {num_threads}                      test/dnnl/TestApiBasic.cpp:28
+ *   tensor   {id, ndims, dims, data}            test/dnnl/TestApiOps.cpp:46-48,
+ *                                               src/dnnl/dnnl_graph_compiler.cpp:76-77,121-133
+ *   version  {api_version, gc_version} x {major, minor, patch, hash}
+ *                                               src/dnnl/dnnl_graph_compiler.cpp:159-166
+ * The integer widths of the fork's header are not pinned by the reference
+ * tree; the widths below are the ones its call sites are consistent with.
+ *
+ * Behaviour kept from the reference: JSON partition in, tensors matched by id
+ * (any order), caller-owned buffers, no exception crosses the ABI, statuses
+ * are dnnl_status_t values, an executable must not outlive its compiler.
+ * `data` may be a host pointer (the reference's only mode: inputs are copied
+ * to the GPU and outputs copied back) or a device pointer (used in place).
+ * execute() returns after the work has completed.
+ */
+#ifndef DNNL_GRAPH_COMPILER_H
+#define DNNL_GRAPH_COMPILER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#pragma GCC visibility push(default)
+
+#define DNNL_GC_API_V_MAJOR 0
+#define DNNL_GC_API_V_MINOR 1
+#define DNNL_GC_API_V_PATCH 0
+#define DNNL_GC_API_V_HASH "N/A"
+
+#ifndef DNNL_MAX_NDIMS
+#define DNNL_MAX_NDIMS 12
+#endif
+
+/* dnnl_status_t values of oneDNN (oneapi/dnnl/dnnl_common_types.h) */
+#ifndef DNNL_COMMON_TYPES_H
+typedef enum {
+  dnnl_success = 0,
+  dnnl_out_of_memory = 1,
+  dnnl_invalid_arguments = 2,
+  dnnl_unimplemented = 3,
+  dnnl_last_impl_reached = 4,
+  dnnl_runtime_error = 5,
+  dnnl_not_required = 6,
+  dnnl_invalid_graph = 7,
+  dnnl_invalid_graph_op = 8,
+  dnnl_invalid_shape = 9,
+  dnnl_invalid_data_type = 10
+} dnnl_status_t;
+#endif
+
+struct dnnl_graph_compiler;
+struct dnnl_graph_compiler_executable;
+
+struct dnnl_graph_compiler_version {
+  struct version {
+    uint8_t major;
+    uint8_t minor;
+    uint8_t patch;
+    const char *hash;
+  } api_version, gc_version;
+};
+
+struct dnnl_graph_compiler_context {
+  uint32_t num_threads; /* kept for source compatibility; the GPU path ignores it */
+};
+
+struct dnnl_graph_compiler_tensor {
+  size_t id;
+  uint8_t ndims;
+  int64_t *dims;
+  void *data;
+};
+
+/* src/dnnl/dnnl_graph_compiler.cpp:157-167 */
+const struct dnnl_graph_compiler_version *dnnl_graph_compiler_get_version(void);
+/* :169-183 -- ctx may be NULL */
+dnnl_status_t dnnl_graph_compiler_create(const struct dnnl_graph_compiler_context *ctx,
+                                         const struct dnnl_graph_compiler **gc);
+/* :185-188 */
+void dnnl_graph_compiler_destroy(const struct dnnl_graph_compiler *gc);
+/* :190-207 -- malformed graph: dnnl_invalid_graph; unsupported op, dtype,
+ * engine or attribute type: dnnl_unimplemented; failed verification or device
+ * error: dnnl_runtime_error */
+dnnl_status_t dnnl_graph_compiler_compile(const struct dnnl_graph_compiler *gc, const char *graph_json,
+                                          const struct dnnl_graph_compiler_executable **exe);
+/* :209-212 */
+void dnnl_graph_compiler_destroy_executable(const struct dnnl_graph_compiler_executable *exe);
+/* :214-226 -- inputs/outputs hold as many entries as the graph has inputs and
+ * outputs; a missing id or ndims > DNNL_MAX_NDIMS: dnnl_runtime_error */
+dnnl_status_t dnnl_graph_compiler_execute(const struct dnnl_graph_compiler_executable *exe,
+                                          struct dnnl_graph_compiler_tensor *inputs,
+                                          struct dnnl_graph_compiler_tensor *outputs);
+
+/* Host-side stages only (parse, verify, fuse, plan): writes the kernel launch
+ * plan of the partition, one line per launch, into buf (NUL terminated,
+ * truncated to len) and returns the status compile would return for these
+ * stages.  Needs no GPU.  No counterpart in the reference, whose equivalent is
+ * printing the IR after the pass pipeline (gc-opt --gc-cpu-pipeline). */
+dnnl_status_t dnnl_graph_compiler_explain(const char *graph_json, char *buf, size_t len);
+
+/* Text of the last error raised on the calling thread by the functions above
+ * (no counterpart in the reference, which prints to stderr in debug builds). */
+const char *dnnl_graph_compiler_last_error(void);
+
+#pragma GCC visibility pop
+#ifdef __cplusplus
+}
+#endif
+#endif /* DNNL_GRAPH_COMPILER_H */

@@ -1,0 +1,146 @@
+"""CPU: host side of the oneDNN-Graph backend API -- JSON schema, error classes,
+op verification and the fusion plan -- through the C ABI
+(dnnl_graph_compiler_explain runs parse -> verify -> fuse -> plan without a GPU).
+Cases follow test/dnnl/TestJsonParser.cpp and the error mapping of
+src/dnnl/dnnl_graph_compiler.cpp:190-207 / src/dnnl/JsonParser.cpp."""
+import ctypes as C
+import importlib
+import json
+import os
+
+import pytest
+
+from conftest import ROOT
+
+OK, UNIMPL, RUNTIME, INVALID_GRAPH = 0, 3, 5, 7
+
+
+@pytest.fixture(scope="module")
+def ga(gc):
+    return importlib.import_module("graph_compiler_amd.graph_api")
+
+
+def _res(name):
+    return open(os.path.join(ROOT, "tests", "golden", name)).read()
+
+
+def test_version_struct(ga):
+    v = ga.api().dnnl_graph_compiler_get_version().contents
+    assert (v.api_version.major, v.api_version.minor, v.api_version.patch) == (0, 1, 0)
+    assert v.gc_version.hash == b"gfx950"
+    assert ga.api().dnnl_graph_compiler_get_version().contents.gc_version.major == v.gc_version.major  # static storage
+
+
+def test_create_destroy_without_gpu(ga):
+    for threads in (None, 4):
+        c = ga.Compiler(threads)
+        assert c.h
+        c.close()
+
+
+@pytest.mark.parametrize("name", ["add", "add_relu", "div", "matmul", "mpl", "mul", "pow", "reduce_mean", "reduce_sum",
+                                  "relu", "sigmoid", "sub", "typecast"])
+def test_every_reference_fixture_parses_and_plans(ga, name):
+    st, plan = ga.explain(_res(name + ".json"))
+    assert st == OK, plan
+    assert plan.strip()
+
+
+def test_fusion_plan_of_reference_mlp(ga):
+    """mpl.json (test/dnnl/resources): MatMul+bias -> ReLU -> MatMul -> Add -> ReLU
+    becomes two GEMM launches with everything else in the epilogues."""
+    st, plan = ga.explain(_res("mpl.json"))
+    assert st == OK
+    assert plan.splitlines() == ["gemm_bf16: MatMul+bias+act", "gemm_bf16: MatMul+bias+act"]
+
+
+def test_fusion_plans_of_benchmark_partitions(ga):
+    assert ga.explain(ga.matmul_bias_relu_json(128, 512, 256))[1].splitlines() == ["gemm_f32: MatMul+bias+act"]
+    assert ga.explain(_res("matmul.json"))[1].splitlines() == ["gemm_f32: MatMul+bias"]  # transpose_a folds into strides
+    j, _ = ga.int8_mlp_json(256, 256, 512, 0.02, 128, [0.01] * 512)
+    lines = ga.explain(j)[1].splitlines()
+    assert lines[0].startswith("colsum") and lines[1].startswith("gemm_int8: Dequantize x2 + MatMul+bias+act+cast") and len(lines) == 2
+    assert ga.explain(ga.mlp_chain_json(256, 256, 512))[1].splitlines() == ["gemm_bf16: MatMul+act", "gemm_bf16: MatMul+bias"]
+    assert ga.explain(ga.mha_json(2, 2, 128, 128, 128))[1].startswith("attention:")
+    assert ga.explain(ga.mha_json(2, 2, 128, 128, 128, with_mask=False, scale_op="Divide"))[1].startswith("attention:")
+    # head_dim 64 has no fused kernel: falls back to per-op kernels, still a valid plan
+    unfused = ga.explain(ga.mha_json(1, 2, 64, 64, 64))[1]
+    assert "softmax: SoftMax" in unfused and "attention" not in unfused
+
+
+def test_intermediate_that_is_an_output_is_not_fused_away(ga):
+    g = json.loads(ga.matmul_bias_relu_json(64, 64, 64))
+    g["output_ports"] = [3, 4]  # the pre-activation tensor is wanted too
+    st, plan = ga.explain(json.dumps(g))
+    assert st == OK and plan.splitlines() == ["gemm_f32: MatMul+bias", "eltwise: ReLU"]
+
+
+def _mutate(fn):
+    g = json.loads(_res("add_relu.json"))
+    fn(g)
+    return json.dumps(g)
+
+
+def test_error_classes(ga):
+    ex = ga.explain
+    # malformed / unknown key / missing pieces -> invalid_graph (std::invalid_argument)
+    assert ex("{")[0] == INVALID_GRAPH
+    assert ex(_mutate(lambda g: g.update(foo=1)))[0] == INVALID_GRAPH
+    assert ex(_mutate(lambda g: g["graph"][0].update(bar=1)))[0] == INVALID_GRAPH
+    assert ex(_mutate(lambda g: g["graph"][0]["inputs"][0].update(baz=1)))[0] == INVALID_GRAPH
+    assert ex(_mutate(lambda g: g["graph"][0].pop("kind")))[0] == INVALID_GRAPH
+    assert ex(_mutate(lambda g: g["graph"][0]["inputs"][0].pop("dtype")))[0] == INVALID_GRAPH
+    assert ex(_mutate(lambda g: g.update(output_ports=[99])))[0] == INVALID_GRAPH           # Output value not found
+    assert ex(_mutate(lambda g: g.update(input_ports=[0])))[0] == INVALID_GRAPH              # length mismatch
+    assert ex(_mutate(lambda g: g.update(input_ports=[0, 77])))[0] == INVALID_GRAPH          # input not in input_ports
+    assert ex(_mutate(lambda g: g["graph"][1]["inputs"][0].update(dtype="f32")))[0] == INVALID_GRAPH  # type mismatch
+    assert ex(_mutate(lambda g: g["graph"][1]["outputs"][0].update(id=2)))[0] == INVALID_GRAPH  # duplicate output id
+    # unsupported feature -> unimplemented (std::logic_error)
+    assert ex(_mutate(lambda g: g.update(engine_kind="fpga")))[0] == UNIMPL
+    assert ex(_mutate(lambda g: g.update(fpmath_mode="bf16")))[0] == UNIMPL
+    assert ex(_mutate(lambda g: g["graph"][0].update(kind="Convolution")))[0] == UNIMPL
+    assert ex(_mutate(lambda g: g["graph"][0]["inputs"][0].update(dtype="f128")))[0] == UNIMPL
+    assert ex(_mutate(lambda g: g["graph"][0]["inputs"][0].update(layout_type="blocked")))[0] == UNIMPL
+    assert ex(_mutate(lambda g: g["graph"][0].update(attrs={"x": {"type": "u64", "value": 1}})))[0] == UNIMPL
+    assert ex(_mutate(lambda g: g["graph"][0].update(attrs={"auto_broadcast": {"type": "string", "value": "maybe"}})))[0] == INVALID_GRAPH
+    # a graph that parses but does not verify -> runtime_error, like a failed JitModule::create
+    assert ex(_mutate(lambda g: g["graph"][1]["outputs"][0].update(shape=[3, 3])))[0] == RUNTIME
+    assert "gpu" and ex(_mutate(lambda g: g.update(engine_kind="gpu")))[0] == OK
+    st, msg = ex(_mutate(lambda g: g["graph"][0].update(kind="Convolution")))
+    assert "Unsupported operation" in msg
+
+
+def test_parser_ids_strides_and_op_order(ga):
+    """test/dnnl/TestJsonParser.cpp:71-225: add_relu.json declares a strided input;
+    inputs are numbered in order of first use; outputs default to the last op's."""
+    g = json.loads(_res("add_relu.json"))
+    strided = [t for op in g["graph"] for t in op["inputs"] if t.get("layout_type") == "strided"]
+    assert strided, "fixture lost its strided tensor"
+    st, plan = ga.explain(_res("add_relu.json"))
+    assert st == OK and plan.splitlines()[0] == "eltwise: copy"  # the strided input is gathered first
+    g.pop("output_ports")
+    assert ga.explain(json.dumps(g))[0] == OK  # output_ports absent -> last op's outputs
+
+
+def test_matmul_shape_rules(ga):
+    """lib/gc/Dialect/OneDNNGraph/OneDNNGraphOps.cpp:204-310"""
+    def mm(a, b, o, **attrs):
+        at = {k: {"type": "bool", "value": int(v)} for k, v in attrs.items()}
+        return json.dumps({"graph": [{"kind": "MatMul", "attrs": at,
+                                      "inputs": [{"id": 0, "dtype": "f32", "shape": a}, {"id": 1, "dtype": "f32", "shape": b}],
+                                      "outputs": [{"id": 2, "dtype": "f32", "shape": o}]}]})
+    ok = [([4, 8], [8, 3], [4, 3], {}), ([8, 4], [8, 3], [4, 3], {"transpose_a": 1}), ([4, 8], [3, 8], [4, 3], {"transpose_b": 1}),
+          ([2, 5, 4, 8], [8, 3], [2, 5, 4, 3], {}), ([2, 1, 4, 8], [5, 8, 3], [2, 5, 4, 3], {}), ([8], [8], [1], {}),
+          ([8], [2, 8, 3], [2, 3], {}), ([2, 4, 8], [8], [2, 4], {})]
+    for a, b, o, at in ok:
+        assert ga.explain(mm(a, b, o, **at))[0] == OK, (a, b, o)
+    bad = [([4, 8], [7, 3], [4, 3], {}), ([4, 8], [8, 3], [4, 4], {}), ([2, 4, 8], [3, 8, 3], [2, 4, 3], {})]
+    for a, b, o, at in bad:
+        assert ga.explain(mm(a, b, o, **at))[0] == RUNTIME, (a, b, o)
+
+
+def test_tensor_struct_layout_matches_the_reference_initialisers(ga):
+    """{.id, .ndims, .dims, .data} (test/dnnl/TestApiOps.cpp:46-48) on LP64."""
+    T = ga.Tensor
+    assert (T.id.offset, T.ndims.offset, T.dims.offset, T.data.offset, C.sizeof(T)) == (0, 8, 16, 24, 32)
+    assert C.sizeof(ga.Context) == 4

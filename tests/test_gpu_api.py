@@ -1,0 +1,199 @@
+"""GPU: the oneDNN-Graph backend API end to end (create / compile / execute /
+destroy) with host buffers, as the reference's own API tests drive it
+(test/dnnl/TestApiBasic.cpp:25-58, test/dnnl/TestApiOps.cpp:27-320), plus the
+benchmark partitions against the oracle, with host and with device tensors."""
+import importlib
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ga(gc, dev):
+    return importlib.import_module("graph_compiler_amd.graph_api")
+
+
+def _res(name):
+    return open(os.path.join(ROOT, "tests", "golden", name)).read()
+
+
+def _run(ga, js, ins, outs):
+    cst, est = ga.run(js, ins, outs)
+    assert cst == 0, "compile -> %d: %s" % (cst, ga.api().dnnl_graph_compiler_last_error().decode())
+    assert est == 0, "execute -> %d: %s" % (est, ga.api().dnnl_graph_compiler_last_error().decode())
+
+
+def test_basic_workflow_add(ga):
+    """TestApiBasic.basicWorkflow: add.json on 128 floats, 4 threads requested."""
+    a = np.arange(128, dtype=np.float32)
+    b = np.arange(128, dtype=np.float32) * 2
+    out = np.zeros(128, np.float32)
+    gcomp = ga.Compiler(4)
+    st, exe = gcomp.compile(_res("add.json"))
+    assert st == 0
+    assert exe.execute([(0, a), (1, b)], [(2, out)]) == 0
+    assert (out == a + b).all()
+    # tensors may come in any order: they are matched by id
+    out[:] = 0
+    assert exe.execute([(1, b), (0, a)], [(2, out)]) == 0
+    assert (out == a + b).all()
+    # an id the graph does not know is a runtime error
+    assert exe.execute([(0, a), (7, b)], [(2, out)]) == ga.RUNTIME_ERROR
+    exe.close()
+    gcomp.close()
+
+
+def test_ops_div_mul_sub_pow_relu_sigmoid(ga):
+    i = np.arange(64 * 32 * 32, dtype=np.float32).reshape(64, 32, 32)
+    o = np.zeros_like(i)
+    _run(ga, _res("div.json"), [(0, i), (1, i + 1)], [(2, o)])
+    assert np.allclose(o, i / (i + 1), rtol=1e-6, atol=0)
+    x = np.arange(128, dtype=np.float32)
+    o = np.zeros(128, np.float32)
+    _run(ga, _res("mul.json"), [(0, x), (1, x)], [(2, o)])
+    assert (o == x * x).all()
+    _run(ga, _res("sub.json"), [(0, x), (1, x * x)], [(2, o)])
+    assert (o == x - x * x).all()
+    x64, o64 = np.arange(64, dtype=np.float32), np.zeros(64, np.float32)
+    _run(ga, _res("pow.json"), [(0, x64)], [(1, o64)])
+    assert (o64 == x64 * x64).all()
+    xs = (np.arange(128) - 64).astype(np.float32)
+    _run(ga, _res("relu.json"), [(0, xs)], [(1, o)])
+    assert (o == np.maximum(xs, 0)).all()
+    _run(ga, _res("sigmoid.json"), [(0, xs)], [(1, o)])
+    assert np.allclose(o, 1 / (1 + np.exp(-xs)), rtol=2e-6, atol=1e-30)
+
+
+def test_ops_matmul_transpose_a_bias_closed_form(ga):
+    """TestApiOps.matMul: A[i][j]=i+j (128x512, transpose_a), B[i][j]=i-j, bias=j; exact integers."""
+    i, j = np.meshgrid(np.arange(128), np.arange(512), indexing="ij")
+    A = (i + j).astype(np.float32)
+    i, j = np.meshgrid(np.arange(128), np.arange(64), indexing="ij")
+    B = (i - j).astype(np.float32)
+    bias = np.arange(64, dtype=np.float32)
+    out = np.zeros((512, 64), np.float32)
+    _run(ga, _res("matmul.json"), [(0, A), (1, B), (2, bias)], [(3, out)])
+    want = A.astype(np.int64).T @ B.astype(np.int64) + np.arange(64)
+    assert (out.astype(np.int64) == want).all()
+
+
+def test_ops_reduce_and_typecast(ga):
+    x = np.arange(16 * 64 * 32, dtype=np.float32).reshape(16, 64, 32)
+    o = np.zeros((16, 1, 32), np.float32)
+    _run(ga, _res("reduce_sum.json"), [(0, x)], [(1, o)])
+    want = np.zeros((16, 1, 32), np.float32)
+    for y in range(64):  # the reference test sums in this order, in f32
+        want[:, 0, :] += x[:, y, :]
+    assert np.allclose(o, want, rtol=1e-6)
+    _run(ga, _res("reduce_mean.json"), [(0, x)], [(1, o)])
+    assert np.allclose(o, want / 64, rtol=1e-6)
+    # typecast f32 -> f16 must be round-to-nearest-even bit for bit (TestApiOps.typecast)
+    v = np.array([(k - 64) / np.exp(-(k - 64)) for k in range(128)], np.float32)
+    h = np.zeros(128, np.uint16)
+    _run(ga, _res("typecast.json"), [(0, v)], [(1, h)])
+    assert (h == v.astype(np.float16).view(np.uint16)).all()
+
+
+def test_add_relu_strided_input(ga):
+    """add_relu.json declares input 1 with explicit strides [1,2,3,4]."""
+    g = json.loads(_res("add_relu.json"))
+    shape = g["graph"][0]["inputs"][0]["shape"]
+    stride = g["graph"][0]["inputs"][1]["stride"]
+    span = 1 + sum((d - 1) * s for d, s in zip(shape, stride))
+    torch.manual_seed(0)
+    a = torch.randn(shape).to(torch.bfloat16)
+    braw = torch.randn(span).to(torch.bfloat16)
+    b = torch.as_strided(braw, shape, stride)
+    out = torch.zeros(shape, dtype=torch.bfloat16)
+    _run(ga, _res("add_relu.json"), [(0, a), (1, braw)], [(3, out)])
+    assert torch.equal(out, torch.relu(a + b))
+
+
+def test_reference_mlp_fixture_bf16(ga, orc, wl):
+    """mpl.json: MatMul+bias -> ReLU -> MatMul -> Add -> ReLU, all bf16."""
+    torch.manual_seed(0)
+    x = torch.randn(128, 512).to(torch.bfloat16)
+    w1 = (torch.randn(512, 64) * 0.05).to(torch.bfloat16)
+    b1 = torch.randn(64).to(torch.bfloat16)
+    w2 = (torch.randn(64, 256) * 0.1).to(torch.bfloat16)
+    b2 = torch.randn(256).to(torch.bfloat16)
+    out = torch.zeros(128, 256, dtype=torch.bfloat16)
+    _run(ga, _res("mpl.json"), [(0, x), (1, w1), (2, b1), (5, w2), (7, b2)], [(9, out)])
+    h = orc.matmul_bf16(wl.bf16_bits(x), wl.bf16_bits(w1), wl.bf16_bits(b1), "relu")
+    y = orc.matmul_bf16(h, wl.bf16_bits(w2), wl.bf16_bits(b2), "relu")
+    mm = orc.bf16_to_f32(orc.matmul_bf16(h, wl.bf16_bits(w2)))
+    assert_close(orc.bf16_to_f32(y), out.float().numpy(), 2e-2, "mpl.json", mag=mm)
+
+
+def test_config1_f32_matmul_bias_relu_through_the_api(ga, orc, wl):
+    """BASELINE config 1, host buffers in and out (max relative error <= 1e-4)."""
+    A, B, bias = wl.f32_matmul_bias_relu()
+    out = np.zeros((128, 256), np.float32)
+    _run(ga, ga.matmul_bias_relu_json(128, 512, 256), [(0, A.numpy()), (1, B.numpy()), (2, bias.numpy())], [(4, out)])
+    ref = orc.matmul_f32(A.numpy(), B.numpy(), bias.numpy(), "relu")
+    assert_close(ref, out, 1e-4, "config 1 via API")
+
+
+def test_int8_partition_through_the_api_with_device_tensors(ga, gc, orc, wl, dev):
+    M, K, N = 512, 256, 768
+    A, W, scale, bias = wl.int8_mlp_layer(M, K, N)
+    sA = 0.02
+    js, out_id = ga.int8_mlp_json(M, K, N, sA, 128, scale.tolist())
+    out = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    _run(ga, js, [(0, A.to(dev)), (1, W.to(dev)), (2, bias.to(dev))], [(out_id, out)])
+    torch.cuda.synchronize()
+    eff = (np.float32(sA) * scale.numpy().astype(np.float32)).astype(np.float32)  # data scale x weight scales, in f32
+    _, y = orc.int8_layer(A.numpy(), W.numpy(), eff, bias.numpy(), 128, "gelu_erf")
+    assert_close(orc.bf16_to_f32(y), out.float().cpu().numpy(), 1e-2, "int8 partition")
+    # the same with host buffers and an f32 result, executed twice (constant-weight colsum is cached)
+    js2, oid2 = ga.int8_mlp_json(M, K, N, sA, 128, scale.tolist(), out_dtype="f32")
+    o2 = np.zeros((M, N), np.float32)
+    c = ga.Compiler()
+    st, exe = c.compile(js2)
+    assert st == 0
+    for _ in range(2):
+        o2[:] = 0
+        assert exe.execute([(0, A.numpy()), (1, W.numpy()), (2, bias.numpy())], [(oid2, o2)]) == 0
+        _, yf = orc.int8_layer(A.numpy(), W.numpy(), eff, bias.numpy(), 128, "gelu_erf", out_bf16=False)
+        assert_close(yf, o2, 1e-4, "int8 partition f32")
+    exe.close()
+    c.close()
+
+
+def test_mlp_chain_partition(ga, orc, wl, dev):
+    M, K, H = 512, 512, 1280
+    x, W1, W2, b2 = wl.bf16_mlp_chain(M, K, H)
+    out = torch.zeros(M, K, dtype=torch.bfloat16)
+    _run(ga, ga.mlp_chain_json(M, K, H), [(0, x), (1, W1), (4, W2), (5, b2)], [(6, out)])
+    h, y = orc.mlp_chain_bf16(wl.bf16_bits(x), wl.bf16_bits(W1), wl.bf16_bits(W2), wl.bf16_bits(b2))
+    mm = orc.bf16_to_f32(orc.matmul_bf16(h, wl.bf16_bits(W2)))
+    assert_close(orc.bf16_to_f32(y), out.float().numpy(), 2e-2, "mlp chain partition", mag=mm)
+
+
+@pytest.mark.parametrize("D,with_mask,scale_op", [(128, True, "Multiply"), (128, False, "Divide"), (64, True, "Multiply")])
+def test_attention_partition(ga, orc, wl, dev, D, with_mask, scale_op):
+    """head_dim 128 runs the fused kernel; 64 falls back to per-op kernels with
+    the same results (softmax weights are a bf16 tensor in both)."""
+    B, H, S = 1, 2, 128
+    Q, K, V, mask, scale = wl.bf16_mha(B, H, S, D)
+    sval = np.array([scale if scale_op == "Multiply" else 1.0 / scale], np.float32)
+    out = torch.zeros(B, H, S, D, dtype=torch.bfloat16)
+    ins = [(0, Q), (1, K), (2, sval)] + ([(3, mask)] if with_mask else []) + [(4, V)]
+    _run(ga, ga.mha_json(B, H, S, S, D, with_mask, scale_op), ins, [(9, out)])
+    if D == 128:
+        ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q), wl.bf16_bits(K), wl.bf16_bits(V),
+                                           mask.numpy() if with_mask else None, scale))
+    else:
+        Sm = Q.float() @ K.float().transpose(-1, -2) * scale + (mask if with_mask else 0)
+        P = torch.softmax(Sm, -1).to(torch.bfloat16).float()
+        ref = (P @ V.float()).to(torch.bfloat16).float().numpy()
+    Sd = Q.double() @ K.double().transpose(-1, -2) * scale + (mask.double() if with_mask else 0)
+    mag = (torch.softmax(Sd, -1) @ V.double().abs()).numpy()
+    assert_close(ref, out.float().numpy(), 1e-2, "attention partition", mag=mag)
