@@ -253,6 +253,228 @@ template <bool HAS_MASK, bool EDGE> __global__ __launch_bounds__(FA_THREADS, 2) 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Fast path (Sq % 128 == 0, Sk % 64 == 0, aligned): same tiling and register
+// layout as above, restructured so that a wave never waits on memory inside an
+// iteration:
+//  * K/V blocks go global -> LDS with global_load_lds_dwordx4 (1 KiB per wave
+//    instruction, swizzle applied on the global side), block kb+1 in flight
+//    while block kb is computed; no staging registers, no ds_write.
+//  * the additive mask tile of block kb+1 is loaded into registers while block
+//    kb is computed (the loop is unrolled by two so the two register sets swap
+//    roles without moves).
+//  * S^T MFMAs alternate between the two 32-key tiles (independent
+//    accumulators) with the K-fragment reads interleaved 1:1; the V^T
+//    fragment reads are interleaved 2:1 with the PV MFMAs.
+//  * softmax runs in the natural-log domain until the exponent:
+//    t = s*scale + mask (one FMA), p = exp2(t*log2e - m*log2e) (one FMA + exp).
+#define GCMI_GLB __attribute__((address_space(1)))
+
+struct FaFast {
+  uint32_t k_src[4], v_src[4]; // per-lane global byte offsets of this wave's DMA instructions (within a 64-key block)
+  uint32_t k_ld[8], v_ld[4];   // LDS fragment offsets
+  int wave_u;
+
+  __device__ __forceinline__ void issue_kv(char *__restrict__ stage, const char *kb_ptr, const char *vb_ptr) const {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(kb_ptr + k_src[i]),
+                                       (GCMI_LDS void *)(stage + (wave_u * 4 + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(vb_ptr + v_src[i]),
+                                       (GCMI_LDS void *)(stage + FA_TILE_BYTES + (wave_u * 4 + i) * 1024), 16, 0, 0);
+  }
+
+  // one 64-key block.  mk = this block's mask tile (already in registers).
+  template <bool HAS_MASK>
+  __device__ __forceinline__ void block(const char *__restrict__ st, const uint4 (&qf)[8], const f32x4_t (&mk)[8],
+                                        float scale, f32x16_t (&o)[4], float &m_run, float &l_run) const {
+    const char *sK = st, *sV = st + FA_TILE_BYTES;
+    // ---- S^T = K . Q^T, the two key tiles alternate
+    f32x16_t s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        s[kt][r] = 0.0f;
+#pragma unroll
+    for (int ds = 0; ds < 8; ds++) {
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++) {
+        uint4 kf = *reinterpret_cast<const uint4 *>(sK + k_ld[ds] + kt * 8192);
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf),
+                                                        __builtin_bit_cast(bf16x8_t, qf[ds]), s[kt], 0, 0, 0);
+      }
+    }
+    // ---- t = s*scale + mask ; block max
+    const float LOG2E = 1.4426950408889634f;
+    float m_blk = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          float v = HAS_MASK ? fmaf(s[kt][4 * q4 + e], scale, mk[kt * 4 + q4][e]) : s[kt][4 * q4 + e] * scale;
+          s[kt][4 * q4 + e] = v;
+          m_blk = fmaxf(m_blk, v);
+        }
+    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32));
+    // ---- online softmax update
+    const float m_new = fmaxf(m_run, m_blk);
+    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new; // fully masked so far: keep exp2 finite
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * LOG2E);
+    const float nm = -m_use * LOG2E;
+    m_run = m_new;
+    float l_blk = 0.0f;
+    uint32_t pk[2][8];
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        float p0 = __builtin_amdgcn_exp2f(fmaf(s[kt][r], LOG2E, nm));
+        float p1 = __builtin_amdgcn_exp2f(fmaf(s[kt][r + 1], LOG2E, nm));
+        l_blk += p0 + p1;
+        pk[kt][r >> 1] = pack_bf16x2(p0, p1);
+      }
+    l_run = l_run * alpha + l_blk;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          o[dt][r] *= alpha;
+    }
+    // ---- O^T += V^T . P^T
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int h2 = 0; h2 < 2; h2++) {
+        uint4 pf = make_uint4(pk[kt][4 * h2 + 0], pk[kt][4 * h2 + 1], pk[kt][4 * h2 + 2], pk[kt][4 * h2 + 3]);
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+          const char *vp = sV + v_ld[dt] + (kt * 32 + 16 * h2) * 256;
+          bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((GCMI_LDS bf16x4_t *)vp);
+          bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((GCMI_LDS bf16x4_t *)(vp + 8 * 256));
+          uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+          uint4 vf = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf),
+                                                          __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
+        }
+      }
+  }
+};
+
+template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fwd_fast_kernel(MhaParams p) {
+  __shared__ __align__(1024) char smem0[2 * FA_TILE_BYTES];
+  __shared__ __align__(1024) char smem1[2 * FA_TILE_BYTES];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, lh = lane >> 5;
+  const int nqb = p.Sq / FA_BQ;
+  const int qb = blockIdx.x % nqb, bh = blockIdx.x / nqb;
+  const int q_lane = qb * FA_BQ + wave * 32 + l32;
+
+  const char *Qb = reinterpret_cast<const char *>(p.Q) + (int64_t)bh * p.Sq * FA_D * 2;
+  const char *Kb = reinterpret_cast<const char *>(p.K) + (int64_t)bh * p.Sk * FA_D * 2;
+  const char *Vb = reinterpret_cast<const char *>(p.V) + (int64_t)bh * p.Sk * FA_D * 2;
+
+  uint4 qf[8];
+#pragma unroll
+  for (int ds = 0; ds < 8; ds++)
+    qf[ds] = *reinterpret_cast<const uint4 *>(Qb + (int64_t)q_lane * FA_D * 2 + ds * 32 + lh * 16);
+
+  FaFast g;
+  g.wave_u = wave;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    int key = (wave * 4 + i) * 4 + (lane >> 4), ph = lane & 15;
+    g.k_src[i] = (uint32_t)(key * 256 + ((ph ^ (key & 15)) << 4));
+    g.v_src[i] = (uint32_t)(key * 256 + ((ph ^ ((key & 3) << 2)) << 4));
+  }
+#pragma unroll
+  for (int ds = 0; ds < 8; ds++)
+    g.k_ld[ds] = l32 * 256 + (((ds * 2 + lh) ^ (l32 & 15)) << 4);
+  {
+    const int gq = lane >> 4, i16 = lane & 15, kk = i16 >> 2, cc = i16 & 3;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+      g.v_ld[dt] = (4 * lh + kk) * 256 + (((dt * 4 + 2 * (gq & 1) + (cc >> 1)) ^ (kk << 2)) << 4) + (cc & 1) * 8;
+  }
+
+  f32x16_t o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+      o[dt][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+  const int nkb = p.Sk / FA_BK;
+  const int64_t blk_bytes = (int64_t)FA_BK * FA_D * 2;
+  const float *mrow = HAS_MASK ? p.mask + (int64_t)q_lane * p.mask_ld + 4 * lh : nullptr;
+
+  f32x4_t mA[8], mB[8];
+  auto load_mask = [&](f32x4_t(&m)[8], int kb) {
+    if (HAS_MASK) {
+#pragma unroll
+      for (int t = 0; t < 8; t++) // t = kt*4 + q4 -> keys kb*64 + kt*32 + 8*q4 + 4*lh .. +3
+        m[t] = *reinterpret_cast<const f32x4_t *>(mrow + kb * FA_BK + (t >> 2) * 32 + (t & 3) * 8);
+    }
+  };
+
+  g.issue_kv(smem0, Kb, Vb);
+  load_mask(mA, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+
+  for (int kb = 0; kb < nkb; kb += 2) {
+    // even block: stage 0, mask set A; prefetch block kb+1 into stage 1 / set B
+    const bool n1 = kb + 1 < nkb;
+    if (n1) {
+      g.issue_kv(smem1, Kb + (kb + 1) * blk_bytes, Vb + (kb + 1) * blk_bytes);
+      load_mask(mB, kb + 1);
+    }
+    g.template block<HAS_MASK>(smem0, qf, mA, p.scale, o, m_run, l_run);
+    // the DMA was issued before the mask loads and loads retire in order: the
+    // mask tile (8 loads) may stay in flight across the barrier
+    if (n1 && HAS_MASK)
+      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    if (!n1)
+      break;
+    const bool n2 = kb + 2 < nkb;
+    if (n2) {
+      g.issue_kv(smem0, Kb + (kb + 2) * blk_bytes, Vb + (kb + 2) * blk_bytes);
+      load_mask(mA, kb + 2);
+    }
+    g.template block<HAS_MASK>(smem1, qf, mB, p.scale, o, m_run, l_run);
+    if (n2 && HAS_MASK)
+      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = 1.0f / l_tot;
+  char *Ob = reinterpret_cast<char *>(p.O) + ((int64_t)bh * p.Sq + q_lane) * FA_D * 2;
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; q4++) {
+      uint16_t h[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        h[e] = f32_to_bf16_bits(o[dt][4 * q4 + e] * inv);
+      *reinterpret_cast<uint2 *>(Ob + (dt * 32 + 8 * q4 + 4 * lh) * 2) =
+          make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+    }
+}
+
 } // namespace gcmi
 
 using namespace gcmi;
@@ -275,12 +497,12 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
   dim3 grid((unsigned)nblk), block(FA_THREADS);
   if (p.mask) {
     if (fast)
-      hipLaunchKernelGGL((mha_fwd_kernel<true, false>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((mha_fwd_fast_kernel<true>), grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL((mha_fwd_kernel<true, true>), grid, block, 0, stream, p);
   } else {
     if (fast)
-      hipLaunchKernelGGL((mha_fwd_kernel<false, false>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((mha_fwd_fast_kernel<false>), grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL((mha_fwd_kernel<false, true>), grid, block, 0, stream, p);
   }
