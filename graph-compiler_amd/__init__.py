@@ -21,7 +21,7 @@ ACT = {None: 0, "none": 0, "relu": 1, "gelu_erf": 2, "gelu_tanh": 3, "sigmoid": 
 # every symbol the public headers declare (checked by the CPU test-suite)
 EXPORTS = {
     "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_int8", "gcmi_colsum_s8",
-                         "gcmi_gemm_f32", "gcmi_mha_fwd_bf16"],
+                         "gcmi_gemm_f32", "gcmi_mha_fwd_bf16", "gcmi_mha_fwd_bf16_opt"],
     "gc_brgemm.h": ["dnnl_brgemm_dispatch", "dnnl_brgemm_tileconfig", "dnnl_brgemm_tilerelease",
                     "dnnl_brgemm_execute"],
 }
@@ -57,6 +57,8 @@ def lib():
     L.gcmi_gemm_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp, ci, vp]
     L.gcmi_mha_fwd_bf16.restype = ci
     L.gcmi_mha_fwd_bf16.argtypes = [vp, vp, vp, vp, i64, vp, i64, i64, i64, i64, f32, vp]
+    L.gcmi_mha_fwd_bf16_opt.restype = ci
+    L.gcmi_mha_fwd_bf16_opt.argtypes = [vp, vp, vp, vp, i64, vp, i64, i64, i64, i64, f32, ci, vp]
     L.dnnl_brgemm_dispatch.restype = i64
     L.dnnl_brgemm_dispatch.argtypes = [i64] * 8 + [f32, i64, i64]
     L.dnnl_brgemm_tileconfig.restype = None
@@ -147,7 +149,7 @@ def gemm_f32(A, B, bias=None, act=None, trans_a=False, trans_b=False, out=None):
     return out
 
 
-def mha_fwd_bf16(Q, K, V, mask=None, scale=None, out=None):
+def mha_fwd_bf16(Q, K, V, mask=None, scale=None, out=None, skip_masked=True):
     """Q [B,H,Sq,D], K,V [B,H,Sk,D] contiguous bf16; mask f32 [Sq,Sk] or None."""
     import torch
     Bn, H, Sq, D = Q.shape
@@ -158,6 +160,6 @@ def mha_fwd_bf16(Q, K, V, mask=None, scale=None, out=None):
     if out is None:
         out = torch.empty_like(Q)
     mld = 0 if mask is None else mask.stride(0)
-    check(lib().gcmi_mha_fwd_bf16(_ptr(Q), _ptr(K), _ptr(V), _ptr(mask), mld, _ptr(out), Bn * H, Sq, Sk, D,
-                                  float(scale), _stream()), "gcmi_mha_fwd_bf16")
+    check(lib().gcmi_mha_fwd_bf16_opt(_ptr(Q), _ptr(K), _ptr(V), _ptr(mask), mld, _ptr(out), Bn * H, Sq, Sk, D,
+                                      float(scale), int(bool(skip_masked)), _stream()), "gcmi_mha_fwd_bf16")
     return out

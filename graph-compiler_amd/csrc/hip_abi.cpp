@@ -153,6 +153,12 @@ extern "C" int gcmi_gemm_f32(const float *A, const float *B, float *C, int64_t M
 
 extern "C" int gcmi_mha_fwd_bf16(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld,
                                  void *O, int64_t BH, int64_t Sq, int64_t Sk, int64_t D, float scale, void *stream) {
+  return gcmi_mha_fwd_bf16_opt(Q, K, V, mask, mask_ld, O, BH, Sq, Sk, D, scale, 1, stream);
+}
+
+extern "C" int gcmi_mha_fwd_bf16_opt(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld,
+                                     void *O, int64_t BH, int64_t Sq, int64_t Sk, int64_t D, float scale,
+                                     int skip_masked, void *stream) {
   if (BH < 0 || Sq < 0 || Sk < 0)
     return fail(ST_INVALID, "mha_fwd: negative size");
   if (D != 128)
@@ -170,6 +176,7 @@ extern "C" int gcmi_mha_fwd_bf16(const void *Q, const void *K, const void *V, co
   MhaParams p{};
   p.Q = Q, p.K = K, p.V = V, p.O = O, p.mask = mask, p.mask_ld = mask_ld;
   p.BH = (int)BH, p.Sq = (int)Sq, p.Sk = (int)Sk, p.D = (int)D, p.scale = scale;
+  p.skip_masked = skip_masked ? 1 : 0;
   int rc = gcmi_launch_mha_fwd(&p, (hipStream_t)stream);
   if (rc == 2)
     return fail(ST_INVALID, "mha_fwd: Q/K/V/O must be 16-byte aligned");

@@ -270,6 +270,38 @@ template <bool HAS_MASK, bool EDGE> __global__ __launch_bounds__(FA_THREADS, 2) 
 //    t = s*scale + mask (one FMA), p = exp2(t*log2e - m*log2e) (one FMA + exp).
 #define GCMI_GLB __attribute__((address_space(1)))
 
+// Mask tile classes, found by one pass over the mask before the main kernel:
+// a tile that is constant 0 or constant -inf needs no mask traffic in the main
+// loop (the constant is put into the mask registers instead), and a -inf tile
+// may be skipped altogether: it contributes exp(-inf) = 0 to every sum and
+// leaves the running maximum unchanged.
+enum : uint8_t { FA_TILE_GENERAL = 0, FA_TILE_ZERO = 1, FA_TILE_NEG_INF = 2 };
+static constexpr int FA_MAX_TILES = 1 << 20;
+// Workspace of the classification pass.  One copy per device, shared by all
+// calls on that device: calls on different streams of one device must not
+// overlap (calls on one stream are ordered).
+static __device__ __align__(256) uint8_t fa_tile_class_ws[FA_MAX_TILES];
+
+__global__ __launch_bounds__(64) void mha_classify_mask_kernel(const float *mask, int64_t mask_ld, int n_kb, uint8_t *cls) {
+  const int qt = blockIdx.y, kb = blockIdx.x, lane = threadIdx.x;
+  // 32 rows x 64 floats: lane -> (row = it*4 + lane/16, 16 B chunk lane%16)
+  bool all_zero = true, all_ninf = true;
+#pragma unroll
+  for (int it = 0; it < 8; it++) {
+    f32x4_t v = *reinterpret_cast<const f32x4_t *>(mask + (int64_t)(qt * 32 + it * 4 + (lane >> 4)) * mask_ld + kb * 64 +
+                                                   (lane & 15) * 4);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      all_zero = all_zero && (__float_as_uint(v[e]) << 1) == 0; // +0 or -0
+      all_ninf = all_ninf && v[e] == -INFINITY;
+    }
+  }
+  all_zero = __all(all_zero);
+  all_ninf = __all(all_ninf);
+  if (lane == 0)
+    cls[qt * n_kb + kb] = all_zero ? FA_TILE_ZERO : (all_ninf ? FA_TILE_NEG_INF : FA_TILE_GENERAL);
+}
+
 struct FaFast {
   uint32_t k_src[4], v_src[4]; // per-lane global byte offsets of this wave's DMA instructions (within a 64-key block)
   uint32_t k_ld[8], v_ld[4];   // LDS fragment offsets
@@ -369,12 +401,25 @@ struct FaFast {
 template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fwd_fast_kernel(MhaParams p) {
   __shared__ __align__(1024) char smem0[2 * FA_TILE_BYTES];
   __shared__ __align__(1024) char smem1[2 * FA_TILE_BYTES];
+  __shared__ int s_last[4];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, lh = lane >> 5;
   const int nqb = p.Sq / FA_BQ;
-  const int qb = blockIdx.x % nqb, bh = blockIdx.x / nqb;
+  // Workgroup -> (head, query block).  Consecutive workgroup ids are dealt
+  // round-robin to the 8 XCDs; all query blocks of one (batch, head) are given to
+  // ONE XCD so that its K/V (Sk x 512 B) is fetched from HBM once and then served
+  // from that XCD's L2.  Long (late) query blocks first.
+  int qb, bh;
+  if ((p.BH & 7) == 0) {
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    bh = (idx / nqb) * 8 + xcd;
+    qb = nqb - 1 - idx % nqb;
+  } else {
+    qb = nqb - 1 - blockIdx.x % nqb;
+    bh = blockIdx.x / nqb;
+  }
   const int q_lane = qb * FA_BQ + wave * 32 + l32;
 
   const char *Qb = reinterpret_cast<const char *>(p.Q) + (int64_t)bh * p.Sq * FA_D * 2;
@@ -411,35 +456,78 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
     for (int r = 0; r < 16; r++)
       o[dt][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
-  const int nkb = p.Sk / FA_BK;
+  int nkb = p.Sk / FA_BK;
   const int64_t blk_bytes = (int64_t)FA_BK * FA_D * 2;
   const float *mrow = HAS_MASK ? p.mask + (int64_t)q_lane * p.mask_ld + 4 * lh : nullptr;
 
+  // classes of this wave's mask tiles, 64 key blocks at a time, as two lane masks
+  const uint8_t *cls_row = (HAS_MASK && p.tile_class) ? p.tile_class + (int64_t)(qb * 4 + wave) * nkb : nullptr;
+  uint64_t zero_bits = 0, ninf_bits = 0;
+  auto load_classes = [&](int kb0) {
+    uint8_t c = FA_TILE_GENERAL;
+    if (cls_row && kb0 + lane < nkb)
+      c = cls_row[kb0 + lane];
+    zero_bits = __ballot(c == FA_TILE_ZERO);
+    ninf_bits = __ballot(c == FA_TILE_NEG_INF);
+  };
+  if (HAS_MASK && cls_row && p.skip_masked) {
+    // trailing key blocks that are -inf for all 128 rows are never touched
+    int last = 0;
+    for (int kb0 = 0; kb0 < nkb; kb0 += 64) {
+      load_classes(kb0);
+      uint64_t live = ~ninf_bits & (nkb - kb0 >= 64 ? ~0ull : ((1ull << (nkb - kb0)) - 1));
+      if (live)
+        last = kb0 + 64 - __builtin_clzll(live);
+    }
+    if (lane == 0)
+      s_last[wave] = last;
+    __syncthreads();
+    nkb = max(max(s_last[0], s_last[1]), max(s_last[2], s_last[3]));
+  }
+  if (HAS_MASK)
+    load_classes(0);
+
   f32x4_t mA[8], mB[8];
-  auto load_mask = [&](f32x4_t(&m)[8], int kb) {
-    if (HAS_MASK) {
+  // returns true when global loads were issued (they then sit behind the DMA in the queue)
+  auto load_mask = [&](f32x4_t(&m)[8], int kb) -> bool {
+    if (!HAS_MASK)
+      return false;
+    const uint64_t bit = 1ull << (kb & 63);
+    if (!((zero_bits | ninf_bits) & bit)) {
 #pragma unroll
       for (int t = 0; t < 8; t++) // t = kt*4 + q4 -> keys kb*64 + kt*32 + 8*q4 + 4*lh .. +3
         m[t] = *reinterpret_cast<const f32x4_t *>(mrow + kb * FA_BK + (t >> 2) * 32 + (t & 3) * 8);
+      return true;
     }
+    const float c = (ninf_bits & bit) ? -INFINITY : 0.0f;
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+      m[t] = f32x4_t{c, c, c, c};
+    return false;
   };
+  auto skip = [&](int kb) -> bool { return HAS_MASK && p.skip_masked && ((ninf_bits >> (kb & 63)) & 1); };
 
-  g.issue_kv(smem0, Kb, Vb);
-  load_mask(mA, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __builtin_amdgcn_s_barrier();
+  if (nkb > 0) {
+    g.issue_kv(smem0, Kb, Vb);
+    load_mask(mA, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+  }
 
   for (int kb = 0; kb < nkb; kb += 2) {
     // even block: stage 0, mask set A; prefetch block kb+1 into stage 1 / set B
     const bool n1 = kb + 1 < nkb;
+    const bool sk0 = skip(kb);
+    bool pending = false;
     if (n1) {
       g.issue_kv(smem1, Kb + (kb + 1) * blk_bytes, Vb + (kb + 1) * blk_bytes);
-      load_mask(mB, kb + 1);
+      pending = load_mask(mB, kb + 1);
     }
-    g.template block<HAS_MASK>(smem0, qf, mA, p.scale, o, m_run, l_run);
+    if (!sk0)
+      g.template block<HAS_MASK>(smem0, qf, mA, p.scale, o, m_run, l_run);
     // the DMA was issued before the mask loads and loads retire in order: the
     // mask tile (8 loads) may stay in flight across the barrier
-    if (n1 && HAS_MASK)
+    if (pending)
       asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
     else
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -447,12 +535,17 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
     if (!n1)
       break;
     const bool n2 = kb + 2 < nkb;
+    const bool sk1 = skip(kb + 1);
+    if (HAS_MASK && n2 && ((kb + 2) & 63) == 0)
+      load_classes(kb + 2);
+    pending = false;
     if (n2) {
       g.issue_kv(smem0, Kb + (kb + 2) * blk_bytes, Vb + (kb + 2) * blk_bytes);
-      load_mask(mA, kb + 2);
+      pending = load_mask(mA, kb + 2);
     }
-    g.template block<HAS_MASK>(smem1, qf, mB, p.scale, o, m_run, l_run);
-    if (n2 && HAS_MASK)
+    if (!sk1)
+      g.template block<HAS_MASK>(smem1, qf, mB, p.scale, o, m_run, l_run);
+    if (pending)
       asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
     else
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -495,6 +588,18 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
   if (!(al16(p.Q) && al16(p.K) && al16(p.V) && al16(p.O)))
     return 2; // rows are 256 bytes: a 16-byte aligned base is required
   dim3 grid((unsigned)nblk), block(FA_THREADS);
+  p.tile_class = nullptr;
+  if (p.mask && fast) {
+    const int64_t n_qt = p.Sq / 32, n_kb = p.Sk / FA_BK;
+    if (n_qt * n_kb <= FA_MAX_TILES && n_qt <= 65535) {
+      uint8_t *ws = nullptr;
+      if (hipGetSymbolAddress((void **)&ws, HIP_SYMBOL(fa_tile_class_ws)) != hipSuccess)
+        return 5;
+      hipLaunchKernelGGL(mha_classify_mask_kernel, dim3((unsigned)n_kb, (unsigned)n_qt), dim3(64), 0, stream, p.mask,
+                         p.mask_ld, (int)n_kb, ws);
+      p.tile_class = ws;
+    }
+  }
   if (p.mask) {
     if (fast)
       hipLaunchKernelGGL((mha_fwd_fast_kernel<true>), grid, block, 0, stream, p);

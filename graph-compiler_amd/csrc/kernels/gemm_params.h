@@ -40,6 +40,9 @@ struct MhaParams {
   int64_t mask_ld;
   int32_t BH, Sq, Sk, D;
   float scale;
+  // fast path only: class of every (32 query rows x 64 keys) mask tile, [Sq/32][Sk/64], or null
+  const uint8_t *tile_class;
+  int32_t skip_masked; // 1: tiles whose mask is all -inf are not computed (the result is the same)
 };
 
 } // namespace gcmi
