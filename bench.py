@@ -43,24 +43,46 @@ def load_package():
 
 
 def time_launches(torch, fn, nsets, steps, warmup):
-    """fn(i) launches one step on buffer set i.  Returns (ms_per_step over the
-    whole timed region, mean and min per-launch ms from per-launch events)."""
+    """fn(i) launches one step on buffer set i.  Two passes of `steps` launches:
+    the first is bracketed by one event pair and the wall clock (ms_per_step,
+    the throughput figure); the second brackets every launch with its own
+    event pair (kernel_ms_*, the roofline figure -- an event pair around an
+    empty launch reads about 6 us on this runtime, so these run a few percent
+    above the kernel-trace durations)."""
     for i in range(warmup):
         fn(i % nsets)
     torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        fn(i % nsets)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    region_ms = e0.elapsed_time(e1)
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    t0 = time.perf_counter()
     for i in range(steps):
         starts[i].record()
         fn(i % nsets)
         stops[i].record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
     per = sorted(s.elapsed_time(e) for s, e in zip(starts, stops))
-    region_ms = starts[0].elapsed_time(stops[-1])
-    return {"ms_per_step": region_ms / steps, "wall_ms_per_step": wall_ms / steps,
+    return {"ms_per_step": max(region_ms, wall_ms) / steps, "wall_ms_per_step": wall_ms / steps,
+            "event_ms_per_step": region_ms / steps,
             "kernel_ms_mean": sum(per) / len(per), "kernel_ms_min": per[0], "kernel_ms_median": per[len(per) // 2]}
+
+
+# HBM-side bytes per launch (fabric reads + writes of the L2s), from
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script with
+# --copy-calibration: a 1 GiB copy reads FETCH_SIZE = 524304 KiB (scale 2.0)
+# and WRITE_SIZE = 1048580 KiB (scale 1.0).
+TRAFFIC = {
+    "gemm": int((98558.1 * 2.0 + 32768.0) * 1024),    # algorithmic 64 MiB read + 32 MiB written
+    "int8": int((144523.0 * 2.0 + 88064.0) * 1024),   # algorithmic 59 MiB read + 86 MiB written
+    "mha": int((104768.0 * 2.0 + 65536.1) * 1024),    # algorithmic 208 MiB read + 64 MiB written
+}
 
 
 def roofline(ops, ms, peak_tops, traffic=None):
@@ -76,7 +98,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32")
-    ap.add_argument("--cpu-rows", type=int, default=512, help="rows of the 4096^3 GEMM the CPU baseline computes")
+    ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the 4096^3 GEMM the CPU baseline computes")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch three 1 GiB device copies (known traffic: 1 GiB read + 1 GiB written each) so that "
+                         "FETCH_SIZE / WRITE_SIZE counter readings of the other kernels can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (no sharding, no collectives); --gpus %d is not supported. "
@@ -130,7 +155,7 @@ def main():
         others["int8_mlp_layer"] = {"workload": "u8[4096x4096] x s8[4096x11008] -> s32 -> dequant+bias+GELU -> bf16",
                                     "value": round(ops / t["ms_per_step"] / 1e9, 2), "unit": "TOP/s", "dtype": "int8",
                                     "ms_per_step": round(t["ms_per_step"], 5),
-                                    "roofline": roofline(ops, t["kernel_ms_mean"], PEAK["int8"]),
+                                    "roofline": roofline(ops, t["kernel_ms_mean"], PEAK["int8"], TRAFFIC["int8"]),
                                     "weight_colsum_precompute_ms": round(tc["kernel_ms_mean"], 5)}
         others["int8_mlp_layer"]["roofline"]["unit"] = "TOP/s"
         log("int8 mlp layer: %.4f ms  %.1f TOP/s" % (t["kernel_ms_mean"], ops / t["kernel_ms_mean"] / 1e9))
@@ -172,13 +197,24 @@ def main():
         for s in range(nsets):
             Q, Kk, V, mask, scale = wl.bf16_mha(seed=10 * s)
             sets.append((Q.to(dev), Kk.to(dev), V.to(dev), mask.to(dev), torch.empty(Bm, Hm, Sm, Dm, device=dev, dtype=torch.bfloat16)))
-        t = time_launches(torch, lambda i: gc.mha_fwd_bf16(sets[i][0], sets[i][1], sets[i][2], sets[i][3], scale, sets[i][4]),
-                          nsets, K, W)
+        def mha(skip):
+            return time_launches(torch, lambda i: gc.mha_fwd_bf16(sets[i][0], sets[i][1], sets[i][2], sets[i][3], scale,
+                                                                  sets[i][4], skip_masked=skip), nsets, K, W)
+
+        # default entry point: key blocks whose mask tile is all -inf for a whole
+        # query block are skipped (their softmax weight is exactly 0, so results
+        # are identical); "every_block" visits all of them.
+        t = mha(True)
+        td = mha(False)
         others["bf16_mha"] = {"workload": "B4 H32 S2048 D128, additive causal mask f32[2048,2048] read as data",
-                              "value": round(ops / t["ms_per_step"] / 1e9, 2), "unit": "TFLOP/s (dense 4*B*H*S*S*D)",
+                              "value": round(ops / t["ms_per_step"] / 1e9, 2), "unit": "TFLOP/s (dense count 4*B*H*S*S*D)",
                               "dtype": "bf16", "ms_per_step": round(t["ms_per_step"], 5),
-                              "roofline": roofline(ops, t["kernel_ms_mean"], PEAK["bf16"])}
-        log("bf16 mha: %.4f ms  %.1f TFLOP/s (dense count)" % (t["kernel_ms_mean"], ops / t["kernel_ms_mean"] / 1e9))
+                              "roofline": roofline(ops, t["kernel_ms_mean"], PEAK["bf16"], TRAFFIC["mha"]),
+                              "every_block": {"value": round(ops / td["ms_per_step"] / 1e9, 2),
+                                              "ms_per_step": round(td["ms_per_step"], 5),
+                                              "roofline": roofline(ops, td["kernel_ms_mean"], PEAK["bf16"])}}
+        log("bf16 mha: %.4f ms  %.1f TFLOP/s (dense count); visiting every block %.4f ms  %.1f TFLOP/s"
+            % (t["kernel_ms_mean"], ops / t["kernel_ms_mean"] / 1e9, td["kernel_ms_mean"], ops / td["kernel_ms_mean"] / 1e9))
         del sets
         torch.cuda.empty_cache()
 
@@ -192,6 +228,14 @@ def main():
                                           "ms_per_step": round(t["ms_per_step"], 5),
                                           "value": round(2.0 * 128 * 512 * 256 / t["kernel_ms_mean"] / 1e9, 4), "unit": "TFLOP/s"}
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---------------- CPU baseline: the oracle's deep-tile nest on a bounded sample
     cpu = None
     if not args.no_cpu and want("gemm"):
@@ -204,7 +248,7 @@ def main():
         orc.matmul_bf16(a16, b16)
         dt = time.perf_counter() - t0
         cpu = {"value": round(2.0 * rows * N * Kd / dt / 1e12, 5), "unit": "TFLOP/s", "cores": nt, "kind": "port",
-               "sample": "first %d of 4096 rows of the same bf16 4096^3 GEMM (deep-tile nest, 32^3 brgemm restatement, "
+               "sample": "%d of 4096 rows of the same bf16 4096^3 GEMM (deep-tile nest, 32^3 brgemm restatement, "
                          "gcc -O3 -march=native, OpenMP), %.2f s" % (rows, dt)}
         log("cpu baseline: %.4f TFLOP/s on %d threads (%.2f s)" % (cpu["value"], nt, dt))
 
@@ -218,7 +262,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "bf16 GEMM M=N=K=4096, row-major A and B, N(0,1)*0.1, f32 accumulate, bf16 out, no post-op",
                    "buffer_sets": 4},
-        "roofline": roofline(flops, res["kernel_ms_mean"], PEAK["bf16"]) if res else None,
+        "roofline": roofline(flops, res["kernel_ms_mean"], PEAK["bf16"], TRAFFIC["gemm"]) if res else None,
         "cpu_baseline": cpu,
         "kernel_ms": {k: round(v, 5) for k, v in res.items()} if res else None,
         "others": others,

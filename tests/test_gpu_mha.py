@@ -86,3 +86,18 @@ def test_mha_full_size_heads_and_invariants(gc, orc, wl, dev):
     ones = gc.mha_fwd_bf16(Qd, Kd, torch.ones_like(Vd), md, scale)
     torch.cuda.synchronize()
     assert (ones.float() - 1).abs().max().item() <= 2 ** -7
+
+
+@pytest.mark.parametrize("Sq,Sk,kind", [(512, 512, "causal"), (384, 640, "causal"), (256, 256, "neg1e9"), (300, 200, "random")])
+def test_skipping_masked_blocks_changes_no_bit(gc, dev, Sq, Sk, kind):
+    """Key blocks whose mask tile is -inf for a whole query block carry softmax
+    weight exactly 0: leaving them out must give the same bits as visiting them."""
+    torch.manual_seed(4)
+    Q = torch.randn(1, 8, Sq, 128).to(torch.bfloat16).to(dev)
+    K = torch.randn(1, 8, Sk, 128).to(torch.bfloat16).to(dev)
+    V = torch.randn(1, 8, Sk, 128).to(torch.bfloat16).to(dev)
+    mask = _mask(kind, Sq, Sk).to(dev)
+    a = gc.mha_fwd_bf16(Q, K, V, mask, 0.088, skip_masked=True)
+    b = gc.mha_fwd_bf16(Q, K, V, mask, 0.088, skip_masked=False)
+    torch.cuda.synchronize()
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
