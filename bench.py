@@ -97,7 +97,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32")
+    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32,api")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the 4096^3 GEMM the CPU baseline computes")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch three 1 GiB device copies (known traffic: 1 GiB read + 1 GiB written each) so that "
@@ -228,6 +228,41 @@ def main():
                                           "ms_per_step": round(t["ms_per_step"], 5),
                                           "value": round(2.0 * 128 * 512 * 256 / t["kernel_ms_mean"] / 1e9, 4), "unit": "TFLOP/s"}
 
+    # ---------------- the same GEMM through dnnl_graph_compiler_execute (the drop-in boundary)
+    if want("api"):
+        ga = importlib.import_module("graph_compiler_amd.graph_api")
+        A, B = wl.bf16_gemm(seed=0)
+        comp = ga.Compiler()
+        st, exe = comp.compile(ga.gemm_json(M, Kd, N, "bf16"))
+        if st:
+            log("bench.py: compile of the GEMM partition failed with status %d" % st)
+            sys.exit(4)
+        Ad, Bd = A.to(dev), B.to(dev)
+        Cd = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+        Ch = torch.empty(M, N, dtype=torch.bfloat16)
+
+        def wall(fn, n):
+            fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3 / n
+
+        t_dev = wall(lambda: exe.execute([(0, Ad), (1, Bd)], [(2, Cd)]), max(10, K // 2))
+        t_host = wall(lambda: exe.execute([(0, A), (1, B)], [(2, Ch)]), 5)
+        exe.close()
+        comp.close()
+        others["api_execute_bf16_gemm"] = {
+            "workload": "the headline GEMM as a one-MatMul JSON partition through dnnl_graph_compiler_execute "
+                        "(returns after completion; wall clock per call)",
+            "device_pointers": {"ms_per_call": round(t_dev, 4), "value": round(flops / t_dev / 1e9, 2), "unit": "TFLOP/s"},
+            "host_pointers_pcie_inclusive": {"ms_per_call": round(t_host, 3), "value": round(flops / t_host / 1e9, 2),
+                                             "unit": "TFLOP/s", "note": "pageable host buffers: 64 MiB in, 32 MiB out per call"}}
+        log("api execute: %.4f ms with device pointers, %.2f ms with host pointers" % (t_dev, t_host))
+        del Ad, Bd, Cd
+
     if args.copy_calibration:
         src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()
         dst = torch.empty_like(src)
@@ -251,6 +286,18 @@ def main():
                "sample": "%d of 4096 rows of the same bf16 4096^3 GEMM (deep-tile nest, 32^3 brgemm restatement, "
                          "gcc -O3 -march=native, OpenMP), %.2f s" % (rows, dt)}
         log("cpu baseline: %.4f TFLOP/s on %d threads (%.2f s)" % (cpu["value"], nt, dt))
+        # second CPU figure: torch's bundled oneDNN kernels on the same operands
+        # (the closest stand-in here for the reference's tiling + oneDNN brgemm)
+        torch.mm(A[:128], B)
+        t0 = time.perf_counter()
+        reps = 0
+        while reps < 1 or (time.perf_counter() - t0 < 5.0 and reps < 20):
+            torch.mm(A, B)
+            reps += 1
+        dt2 = (time.perf_counter() - t0) / reps
+        cpu["torch_mm_bf16"] = {"value": round(2.0 * rows * N * Kd / dt2 / 1e12, 5), "unit": "TFLOP/s",
+                                "cores": torch.get_num_threads(), "sample": "torch.mm on the same operands, mean of %d" % reps}
+        log("cpu torch.mm bf16: %.4f TFLOP/s on %d threads" % (cpu["torch_mm_bf16"]["value"], torch.get_num_threads()))
 
     line = {
         "metric": "TFLOPS/TOPS + % of MI355X MFMA peak: bf16 4096^3 GEMM, int8 MLP, bf16 MHA",
