@@ -319,9 +319,18 @@ struct FaFast {
   }
 
   // one 64-key block.  mk = this block's mask tile (already in registers).
-  template <bool HAS_MASK>
-  __device__ __forceinline__ void block(const char *__restrict__ st, const uint4 (&qf)[8], const f32x4_t (&mk)[8],
+  // MK: 0 = no mask term, 1 = mask tile in mk, 2 = the tile is -inf throughout
+  // mtile: this lane's 8 x 16 B pieces of the block's mask tile (MK == 1), requested
+  // before the S MFMAs are issued and consumed after them.
+  template <int MK>
+  __device__ __forceinline__ void block(const char *__restrict__ st, const uint4 (&qf)[8], const float *mtile,
                                         float scale, f32x16_t (&o)[4], float &m_run, float &l_run) const {
+    f32x4_t mk[8];
+    if (MK == 1) {
+#pragma unroll
+      for (int t = 0; t < 8; t++) // t = kt*4 + q4 -> keys kt*32 + 8*q4 + 4*(lane/32) .. +3
+        mk[t] = *reinterpret_cast<const f32x4_t *>(mtile + (t >> 2) * 32 + (t & 3) * 8);
+    }
     const char *sK = st, *sV = st + FA_TILE_BYTES;
     // ---- S^T = K . Q^T, the two key tiles alternate
     f32x16_t s[2];
@@ -339,25 +348,37 @@ struct FaFast {
                                                         __builtin_bit_cast(bf16x8_t, qf[ds]), s[kt], 0, 0, 0);
       }
     }
-    // ---- t = s*scale + mask ; block max
     const float LOG2E = 1.4426950408889634f;
     float m_blk = -INFINITY;
+    if (MK != 0) {
+      // ---- t = s*scale + mask ; block max over t
 #pragma unroll
-    for (int kt = 0; kt < 2; kt++)
+      for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-      for (int q4 = 0; q4 < 4; q4++)
+        for (int q4 = 0; q4 < 4; q4++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-          float v = HAS_MASK ? fmaf(s[kt][4 * q4 + e], scale, mk[kt * 4 + q4][e]) : s[kt][4 * q4 + e] * scale;
-          s[kt][4 * q4 + e] = v;
-          m_blk = fmaxf(m_blk, v);
-        }
+          for (int e = 0; e < 4; e++) {
+            float v = fmaf(s[kt][4 * q4 + e], scale, MK == 1 ? mk[kt * 4 + q4][e] : -INFINITY);
+            s[kt][4 * q4 + e] = v;
+            m_blk = fmaxf(m_blk, v);
+          }
+    } else {
+      // ---- no mask term: the maximum of t = s*scale is scale * max(s) (scale > 0),
+      // and the scale folds into the exponent's multiplier
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2)
+          m_blk = fmaxf(fmaxf(m_blk, s[kt][r]), s[kt][r + 1]);
+      m_blk *= scale;
+    }
     m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32));
     // ---- online softmax update
     const float m_new = fmaxf(m_run, m_blk);
     const float m_use = (m_new == -INFINITY) ? 0.0f : m_new; // fully masked so far: keep exp2 finite
     const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * LOG2E);
     const float nm = -m_use * LOG2E;
+    const float c = MK != 0 ? LOG2E : scale * LOG2E;
     m_run = m_new;
     float l_blk = 0.0f;
     uint32_t pk[2][8];
@@ -365,8 +386,8 @@ struct FaFast {
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
-        float p0 = __builtin_amdgcn_exp2f(fmaf(s[kt][r], LOG2E, nm));
-        float p1 = __builtin_amdgcn_exp2f(fmaf(s[kt][r + 1], LOG2E, nm));
+        float p0 = __builtin_amdgcn_exp2f(fmaf(s[kt][r], c, nm));
+        float p1 = __builtin_amdgcn_exp2f(fmaf(s[kt][r + 1], c, nm));
         l_blk += p0 + p1;
         pk[kt][r >> 1] = pack_bf16x2(p0, p1);
       }
@@ -410,16 +431,22 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
   // Workgroup -> (head, query block).  Consecutive workgroup ids are dealt
   // round-robin to the 8 XCDs; all query blocks of one (batch, head) are given to
   // ONE XCD so that its K/V (Sk x 512 B) is fetched from HBM once and then served
-  // from that XCD's L2.  Long (late) query blocks first.
-  int qb, bh;
+  // from that XCD's L2.  Long (late) query blocks first.  With pair_q a workgroup
+  // takes block n-1-j and then block j: under a triangular mask with skipping
+  // every workgroup then has the same amount of work.
+  const int per_head = p.pair_q ? (nqb + 1) / 2 : nqb;
+  int qj, bh;
   if ((p.BH & 7) == 0) {
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    bh = (idx / nqb) * 8 + xcd;
-    qb = nqb - 1 - idx % nqb;
+    bh = (idx / per_head) * 8 + xcd;
+    qj = idx % per_head;
   } else {
-    qb = nqb - 1 - blockIdx.x % nqb;
-    bh = blockIdx.x / nqb;
+    qj = blockIdx.x % per_head;
+    bh = blockIdx.x / per_head;
   }
+  const int n_pass = (p.pair_q && qj != nqb - 1 - qj) ? 2 : 1;
+  for (int pass = 0; pass < n_pass; pass++) {
+  const int qb = pass == 0 ? nqb - 1 - qj : qj;
   const int q_lane = qb * FA_BQ + wave * 32 + l32;
 
   const char *Qb = reinterpret_cast<const char *>(p.Q) + (int64_t)bh * p.Sq * FA_D * 2;
@@ -487,69 +514,47 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
   if (HAS_MASK)
     load_classes(0);
 
-  f32x4_t mA[8], mB[8];
-  // returns true when global loads were issued (they then sit behind the DMA in the queue)
-  auto load_mask = [&](f32x4_t(&m)[8], int kb) -> bool {
-    if (!HAS_MASK)
-      return false;
-    const uint64_t bit = 1ull << (kb & 63);
-    if (!((zero_bits | ninf_bits) & bit)) {
-#pragma unroll
-      for (int t = 0; t < 8; t++) // t = kt*4 + q4 -> keys kb*64 + kt*32 + 8*q4 + 4*lh .. +3
-        m[t] = *reinterpret_cast<const f32x4_t *>(mrow + kb * FA_BK + (t >> 2) * 32 + (t & 3) * 8);
-      return true;
-    }
-    const float c = (ninf_bits & bit) ? -INFINITY : 0.0f;
-#pragma unroll
-    for (int t = 0; t < 8; t++)
-      m[t] = f32x4_t{c, c, c, c};
-    return false;
-  };
-  auto skip = [&](int kb) -> bool { return HAS_MASK && p.skip_masked && ((ninf_bits >> (kb & 63)) & 1); };
-
   if (nkb > 0) {
     g.issue_kv(smem0, Kb, Vb);
-    load_mask(mA, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
   }
 
+  // One key block: start the DMA of the next K/V block into the other stage
+  // (the last block re-fetches itself into the free stage), then compute.
+  auto step = [&](const char *cur, char *nxt, int kb) {
+    const uint64_t bit = 1ull << (kb & 63);
+    const bool is_zero = !HAS_MASK || (zero_bits & bit);
+    const bool is_ninf = HAS_MASK && (ninf_bits & bit);
+    const bool is_skip = is_ninf && p.skip_masked;
+    const int kbn = min(kb + 1, nkb - 1);
+    if (HAS_MASK && ((kb + 1) & 63) == 0 && kb + 1 < nkb)
+      load_classes(kb + 1);
+    // the DMA is issued inside each arm, in the basic block of the LDS reads it
+    // must not be ordered against
+    const char *kn = Kb + kbn * blk_bytes, *vn = Vb + kbn * blk_bytes;
+    if (is_skip) {
+      g.issue_kv(nxt, kn, vn);
+    } else if (is_zero) {
+      asm volatile("; arm: no mask term" ::: "memory"); // distinct text: keeps the DMA from being hoisted out of the arm
+      g.issue_kv(nxt, kn, vn);
+      g.template block<0>(cur, qf, nullptr, p.scale, o, m_run, l_run);
+    } else if (is_ninf) {
+      asm volatile("; arm: -inf tile" ::: "memory");
+      g.issue_kv(nxt, kn, vn);
+      g.template block<2>(cur, qf, nullptr, p.scale, o, m_run, l_run);
+    } else {
+      asm volatile("; arm: mask tile" ::: "memory");
+      g.issue_kv(nxt, kn, vn);
+      g.template block<1>(cur, qf, mrow + kb * FA_BK, p.scale, o, m_run, l_run);
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+  };
   for (int kb = 0; kb < nkb; kb += 2) {
-    // even block: stage 0, mask set A; prefetch block kb+1 into stage 1 / set B
-    const bool n1 = kb + 1 < nkb;
-    const bool sk0 = skip(kb);
-    bool pending = false;
-    if (n1) {
-      g.issue_kv(smem1, Kb + (kb + 1) * blk_bytes, Vb + (kb + 1) * blk_bytes);
-      pending = load_mask(mB, kb + 1);
-    }
-    if (!sk0)
-      g.template block<HAS_MASK>(smem0, qf, mA, p.scale, o, m_run, l_run);
-    // the DMA was issued before the mask loads and loads retire in order: the
-    // mask tile (8 loads) may stay in flight across the barrier
-    if (pending)
-      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    if (!n1)
-      break;
-    const bool n2 = kb + 2 < nkb;
-    const bool sk1 = skip(kb + 1);
-    if (HAS_MASK && n2 && ((kb + 2) & 63) == 0)
-      load_classes(kb + 2);
-    pending = false;
-    if (n2) {
-      g.issue_kv(smem0, Kb + (kb + 2) * blk_bytes, Vb + (kb + 2) * blk_bytes);
-      pending = load_mask(mA, kb + 2);
-    }
-    if (!sk1)
-      g.template block<HAS_MASK>(smem1, qf, mB, p.scale, o, m_run, l_run);
-    if (pending)
-      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
+    step(smem0, smem1, kb);
+    if (kb + 1 < nkb)
+      step(smem1, smem0, kb + 1);
   }
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);
@@ -566,11 +571,27 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
       *reinterpret_cast<uint2 *>(Ob + (dt * 32 + 8 * q4 + 4 * lh) * 2) =
           make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
     }
+  } // pass
 }
 
 } // namespace gcmi
 
 using namespace gcmi;
+
+// compute units of the current device (cached per device)
+static int gcmi_num_cus() {
+  static int cache[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    return 256;
+  if (cache[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cache[dev] = n;
+  }
+  return cache[dev];
+}
 
 extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
   MhaParams p = *pp;
@@ -579,16 +600,17 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
   if (p.BH <= 0 || p.Sq <= 0 || p.Sk <= 0)
     return 0;
   const int nqb = (p.Sq + FA_BQ - 1) / FA_BQ;
-  const int64_t nblk = (int64_t)nqb * p.BH;
+  int64_t nblk = (int64_t)nqb * p.BH;
   if (nblk > 0x7fffffff)
     return 2;
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
-  bool fast = p.Sq % FA_BQ == 0 && p.Sk % FA_BK == 0 && al16(p.Q) && al16(p.K) && al16(p.V) && al16(p.O) &&
+  // the fast kernel takes max(s*scale) as scale*max(s): it needs scale > 0
+  bool fast = p.scale > 0.0f && p.Sq % FA_BQ == 0 && p.Sk % FA_BK == 0 && al16(p.Q) && al16(p.K) && al16(p.V) && al16(p.O) &&
               (!p.mask || (al16(p.mask) && p.mask_ld % 4 == 0));
   if (!(al16(p.Q) && al16(p.K) && al16(p.V) && al16(p.O)))
     return 2; // rows are 256 bytes: a 16-byte aligned base is required
-  dim3 grid((unsigned)nblk), block(FA_THREADS);
   p.tile_class = nullptr;
+  p.pair_q = 0;
   if (p.mask && fast) {
     const int64_t n_qt = p.Sq / 32, n_kb = p.Sk / FA_BK;
     if (n_qt * n_kb <= FA_MAX_TILES && n_qt <= 65535) {
@@ -600,6 +622,12 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
       p.tile_class = ws;
     }
   }
+  // pairing halves the number of workgroups: only when the GPU stays full (2 per CU)
+  if (fast && p.tile_class && p.skip_masked && (int64_t)((nqb + 1) / 2) * p.BH >= 2 * gcmi_num_cus()) {
+    p.pair_q = 1;
+    nblk = (int64_t)((nqb + 1) / 2) * p.BH;
+  }
+  dim3 grid((unsigned)nblk), block(FA_THREADS);
   if (p.mask) {
     if (fast)
       hipLaunchKernelGGL((mha_fwd_fast_kernel<true>), grid, block, 0, stream, p);
