@@ -302,6 +302,10 @@ __global__ __launch_bounds__(64) void mha_classify_mask_kernel(const float *mask
     cls[qt * n_kb + kb] = all_zero ? FA_TILE_ZERO : (all_ninf ? FA_TILE_NEG_INF : FA_TILE_GENERAL);
 }
 
+// how far (natural-log units) a block maximum may exceed the softmax reference
+// before the reference is moved: p stays below e^5 = 148
+constexpr float FA_REF_SLACK = 5.0f;
+
 struct FaFast {
   uint32_t k_src[4], v_src[4]; // per-lane global byte offsets of this wave's DMA instructions (within a 64-key block)
   uint32_t k_ld[8], v_ld[4];   // LDS fragment offsets
@@ -373,38 +377,42 @@ struct FaFast {
       m_blk *= scale;
     }
     m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32));
-    // ---- online softmax update
-    const float m_new = fmaxf(m_run, m_blk);
-    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new; // fully masked so far: keep exp2 finite
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * LOG2E);
-    const float nm = -m_use * LOG2E;
-    const float c = MK != 0 ? LOG2E : scale * LOG2E;
-    m_run = m_new;
-    float l_blk = 0.0f;
-    uint32_t pk[2][8];
-#pragma unroll
-    for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        float p0 = __builtin_amdgcn_exp2f(fmaf(s[kt][r], c, nm));
-        float p1 = __builtin_amdgcn_exp2f(fmaf(s[kt][r + 1], c, nm));
-        l_blk += p0 + p1;
-        pk[kt][r >> 1] = pack_bf16x2(p0, p1);
-      }
-    l_run = l_run * alpha + l_blk;
-    if (__any(alpha != 1.0f)) {
+    // ---- online softmax with a lazily moved reference.  m_run is the value
+    // subtracted in the exponent; it only moves (and O, l are only rescaled) when
+    // the block maximum exceeds it by more than FA_REF_SLACK, so p <= e^FA_REF_SLACK
+    // and after the first blocks of a row the rescale branch is hardly taken.
+    const bool grow = m_blk > m_run + FA_REF_SLACK;
+    if (__any(grow)) {
+      const float m_new = grow ? m_blk : m_run;
+      const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E) : 1.0f;
+      m_run = m_new;
+      l_run *= alpha;
 #pragma unroll
       for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int r = 0; r < 16; r++)
           o[dt][r] *= alpha;
     }
-    // ---- O^T += V^T . P^T
+    const float m_use = (m_run == -INFINITY) ? 0.0f : m_run; // fully masked so far: keep exp2 finite
+    const float nm = -m_use * LOG2E;
+    const float c = MK != 0 ? LOG2E : scale * LOG2E;
+    // ---- p = exp2(t*log2e - m*log2e), O^T += V^T . P^T, 16 keys at a time: the
+    // exponentials of one chunk are independent of the MFMAs of the previous one
+    float l_blk = 0.0f;
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
       for (int h2 = 0; h2 < 2; h2++) {
-        uint4 pf = make_uint4(pk[kt][4 * h2 + 0], pk[kt][4 * h2 + 1], pk[kt][4 * h2 + 2], pk[kt][4 * h2 + 3]);
+        uint32_t pk[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const int r = 8 * h2 + 2 * j;
+          float p0 = __builtin_amdgcn_exp2f(fmaf(s[kt][r], c, nm));
+          float p1 = __builtin_amdgcn_exp2f(fmaf(s[kt][r + 1], c, nm));
+          l_blk += p0 + p1;
+          pk[j] = pack_bf16x2(p0, p1);
+        }
+        uint4 pf = make_uint4(pk[0], pk[1], pk[2], pk[3]);
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) {
           const char *vp = sV + v_ld[dt] + (kt * 32 + 16 * h2) * 256;
@@ -416,6 +424,17 @@ struct FaFast {
                                                           __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
         }
       }
+    l_run += l_blk;
+    // issue order for the region above: the first chunk's exponentials, then every
+    // MFMA followed by its share of the next chunk's VALU work, so that the vector
+    // ALU runs in the shadow of the matrix pipe (0x2 VALU, 0x400 transcendental, 0x8 MFMA)
+    __builtin_amdgcn_sched_group_barrier(0x002, 28, 0);
+#pragma unroll
+    for (int i = 0; i < 12; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
   }
 };
 
