@@ -169,3 +169,18 @@ def test_mlp_chain_bf16_reduced(gc, orc, wl, dev):
     assert_close(orc.bf16_to_f32(href), h.float().cpu().numpy(), 1e-2, "mlp hidden")
     mm = orc.bf16_to_f32(orc.matmul_bf16(href, wl.bf16_bits(W2)))
     assert_close(orc.bf16_to_f32(yref), y.float().cpu().numpy(), 2e-2, "mlp out (two rounding points)", mag=mm)
+
+
+def test_gelu_erf_epilogue_absolute_accuracy(gc, dev):
+    """The epilogue's erf is a rational approximation with absolute error < 5e-7
+    (the reference's own erf is an approximation of that class): GELU over a
+    dense grid of x, computed as a [M,1]x[1,1] matmul with the activation fused,
+    against float64."""
+    from scipy.special import erf
+    x = torch.linspace(-8, 8, 200001, dtype=torch.float32).reshape(-1, 1)
+    one = torch.ones(1, 1, dtype=torch.float32)
+    out = gc.gemm_f32(x.to(dev), one.to(dev), act="gelu_erf").cpu().numpy().astype(np.float64).ravel()
+    xd = x.numpy().astype(np.float64).ravel()
+    ref = 0.5 * xd * (1 + erf(xd * 0.7071067811865476))
+    assert np.abs(out - ref).max() <= 1e-6 * 4  # |x| <= 8: 0.5 * 8 * 5e-7 + f32 rounding
+    assert (out[xd < -5.7] == 0).all()  # erf saturates to exactly -1, as libm's does
