@@ -245,7 +245,9 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
     for (int it = 0; it < 16; it++) {
       const int row = it * 8 + r8;
       uint4 v = *reinterpret_cast<const uint4 *>(stg + row * G_STG_PITCH + c8 * 16);
-      *reinterpret_cast<uint4 *>(Cb + ((m0 + wm * 128 + row) * p.ldc + n0 + wn * 64 + c8 * 8) * 2) = v;
+      typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+      u32x4_t vv = {v.x, v.y, v.z, v.w};
+      __builtin_nontemporal_store(vv, reinterpret_cast<u32x4_t *>(Cb + ((m0 + wm * 128 + row) * p.ldc + n0 + wn * 64 + c8 * 8) * 2));
     }
   }
 }
