@@ -305,6 +305,10 @@ __global__ __launch_bounds__(64) void mha_classify_mask_kernel(const float *mask
 // how far (natural-log units) a block maximum may exceed the softmax reference
 // before the reference is moved: p stays below e^5 = 148
 constexpr float FA_REF_SLACK = 5.0f;
+// K fragment reads kept in flight ahead of the S MFMAs
+constexpr int FA_K_AHEAD = 6;
+// the set of visited key blocks is kept for up to 64 * FA_MAX_GROUPS blocks (65536 keys)
+constexpr int FA_MAX_GROUPS = 16;
 
 struct FaFast {
   uint32_t k_src[4], v_src[4]; // per-lane global byte offsets of this wave's DMA instructions (within a 64-key block)
@@ -322,19 +326,14 @@ struct FaFast {
                                        (GCMI_LDS void *)(stage + FA_TILE_BYTES + (wave_u * 4 + i) * 1024), 16, 0, 0);
   }
 
-  // one 64-key block.  mk = this block's mask tile (already in registers).
-  // MK: 0 = no mask term, 1 = mask tile in mk, 2 = the tile is -inf throughout
-  // mtile: this lane's 8 x 16 B pieces of the block's mask tile (MK == 1), requested
-  // before the S MFMAs are issued and consumed after them.
-  template <int MK>
-  __device__ __forceinline__ void block(const char *__restrict__ st, const uint4 (&qf)[8], const float *mtile,
-                                        float scale, f32x16_t (&o)[4], float &m_run, float &l_run) const {
-    f32x4_t mk[8];
-    if (MK == 1) {
-#pragma unroll
-      for (int t = 0; t < 8; t++) // t = kt*4 + q4 -> keys kt*32 + 8*q4 + 4*(lane/32) .. +3
-        mk[t] = *reinterpret_cast<const f32x4_t *>(mtile + (t >> 2) * 32 + (t & 3) * 8);
-    }
+  // One 64-key block.  kind (wave-uniform): 0 the mask tile adds nothing, 1 read it
+  // (mtile: this lane's 8 x 16 B pieces of it), 2 it is -inf throughout.  The mask joins the raw
+  // scores as s + mask/scale, so that one code path (maximum of the raw scores,
+  // scale folded into the exponent's multiplier) serves both cases; scale > 0.
+  template <bool HAS_MASK>
+  __device__ __forceinline__ void block(const char *__restrict__ st, const uint4 (&qf)[8], int kind, const float *mtile,
+                                        float scale, float inv_scale, f32x16_t (&o)[4], float &m_run,
+                                        float &l_run) const {
     const char *sK = st, *sV = st + FA_TILE_BYTES;
     // ---- S^T = K . Q^T, the two key tiles alternate
     f32x16_t s[2];
@@ -352,30 +351,52 @@ struct FaFast {
                                                         __builtin_bit_cast(bf16x8_t, qf[ds]), s[kt], 0, 0, 0);
       }
     }
+    // fragments of V for the first 16 keys are requested here, long before the
+    // first PV MFMA needs them
+    auto load_v = [&](int chunk, uint4 (&vf)[4]) {
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++) {
+        const char *vp = sV + v_ld[dt] + chunk * 16 * 256;
+        bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((GCMI_LDS bf16x4_t *)vp);
+        bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((GCMI_LDS bf16x4_t *)(vp + 8 * 256));
+        uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+        vf[dt] = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+      }
+    };
+    uint4 vcur[4];
+    load_v(0, vcur);
+    // issue order of the S phase: K fragments run FA_K_AHEAD reads ahead of the MFMAs
+    __builtin_amdgcn_sched_group_barrier(0x100, FA_K_AHEAD, 0);
+#pragma unroll
+    for (int i = 0; i < 16 - FA_K_AHEAD; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, FA_K_AHEAD, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+    if (HAS_MASK && kind == 2) {
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          s[kt][r] = -INFINITY;
+    } else if (HAS_MASK && kind == 1) {
+#pragma unroll
+      for (int t = 0; t < 8; t++) { // t = kt*4 + q4 -> keys kt*32 + 8*q4 + 4*(lane/32) .. +3
+        const f32x4_t mk = *reinterpret_cast<const f32x4_t *>(mtile + (t >> 2) * 32 + (t & 3) * 8);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          s[t >> 2][4 * (t & 3) + e] = fmaf(mk[e], inv_scale, s[t >> 2][4 * (t & 3) + e]);
+      }
+    }
     const float LOG2E = 1.4426950408889634f;
     float m_blk = -INFINITY;
-    if (MK != 0) {
-      // ---- t = s*scale + mask ; block max over t
 #pragma unroll
-      for (int kt = 0; kt < 2; kt++)
+    for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-        for (int q4 = 0; q4 < 4; q4++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            float v = fmaf(s[kt][4 * q4 + e], scale, MK == 1 ? mk[kt * 4 + q4][e] : -INFINITY);
-            s[kt][4 * q4 + e] = v;
-            m_blk = fmaxf(m_blk, v);
-          }
-    } else {
-      // ---- no mask term: the maximum of t = s*scale is scale * max(s) (scale > 0),
-      // and the scale folds into the exponent's multiplier
-#pragma unroll
-      for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2)
-          m_blk = fmaxf(fmaxf(m_blk, s[kt][r]), s[kt][r + 1]);
-      m_blk *= scale;
-    }
+      for (int r = 0; r < 16; r += 2)
+        m_blk = fmaxf(fmaxf(m_blk, s[kt][r]), s[kt][r + 1]);
+    m_blk *= scale;
     m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32));
     // ---- online softmax with a lazily moved reference.  m_run is the value
     // subtracted in the exponent; it only moves (and O, l are only rescaled) when
@@ -395,7 +416,7 @@ struct FaFast {
     }
     const float m_use = (m_run == -INFINITY) ? 0.0f : m_run; // fully masked so far: keep exp2 finite
     const float nm = -m_use * LOG2E;
-    const float c = MK != 0 ? LOG2E : scale * LOG2E;
+    const float c = scale * LOG2E;
     // ---- p = exp2(t*log2e - m*log2e), O^T += V^T . P^T, 16 keys at a time: the
     // exponentials of one chunk are independent of the MFMAs of the previous one
     float l_blk = 0.0f;
@@ -413,15 +434,17 @@ struct FaFast {
           pk[j] = pack_bf16x2(p0, p1);
         }
         uint4 pf = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        uint4 vnext[4];
+        if (kt * 2 + h2 < 3)
+          load_v(kt * 2 + h2 + 1, vnext);
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-          const char *vp = sV + v_ld[dt] + (kt * 32 + 16 * h2) * 256;
-          bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((GCMI_LDS bf16x4_t *)vp);
-          bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((GCMI_LDS bf16x4_t *)(vp + 8 * 256));
-          uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
-          uint4 vf = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf),
+        for (int dt = 0; dt < 4; dt++)
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vcur[dt]),
                                                           __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
+        if (kt * 2 + h2 < 3) {
+#pragma unroll
+          for (int dt = 0; dt < 4; dt++)
+            vcur[dt] = vnext[dt];
         }
       }
     l_run += l_blk;
@@ -441,7 +464,8 @@ struct FaFast {
 template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fwd_fast_kernel(MhaParams p) {
   __shared__ __align__(1024) char smem0[2 * FA_TILE_BYTES];
   __shared__ __align__(1024) char smem1[2 * FA_TILE_BYTES];
-  __shared__ int s_last[4];
+  __shared__ uint64_t s_ninf[4];          // per wave: -inf classes of the current group of 64 key blocks
+  __shared__ uint64_t s_live[FA_MAX_GROUPS]; // per group of 64 key blocks: the ones the workgroup visits
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -502,78 +526,89 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
     for (int r = 0; r < 16; r++)
       o[dt][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
-  int nkb = p.Sk / FA_BK;
+  const int nkb = p.Sk / FA_BK;
   const int64_t blk_bytes = (int64_t)FA_BK * FA_D * 2;
   const float *mrow = HAS_MASK ? p.mask + (int64_t)q_lane * p.mask_ld + 4 * lh : nullptr;
 
   // classes of this wave's mask tiles, 64 key blocks at a time, as two lane masks
   const uint8_t *cls_row = (HAS_MASK && p.tile_class) ? p.tile_class + (int64_t)(qb * 4 + wave) * nkb : nullptr;
   uint64_t zero_bits = 0, ninf_bits = 0;
-  auto load_classes = [&](int kb0) {
+  int cls_group = -1;
+  auto load_classes = [&](int group) {
     uint8_t c = FA_TILE_GENERAL;
-    if (cls_row && kb0 + lane < nkb)
-      c = cls_row[kb0 + lane];
+    if (cls_row && group * 64 + lane < nkb)
+      c = cls_row[group * 64 + lane];
     zero_bits = __ballot(c == FA_TILE_ZERO);
     ninf_bits = __ballot(c == FA_TILE_NEG_INF);
+    cls_group = group;
   };
-  if (HAS_MASK && cls_row && p.skip_masked) {
-    // trailing key blocks that are -inf for all 128 rows are never touched
-    int last = 0;
-    for (int kb0 = 0; kb0 < nkb; kb0 += 64) {
-      load_classes(kb0);
-      uint64_t live = ~ninf_bits & (nkb - kb0 >= 64 ? ~0ull : ((1ull << (nkb - kb0)) - 1));
-      if (live)
-        last = kb0 + 64 - __builtin_clzll(live);
+  // Key blocks whose tiles are -inf for all four waves are left out: their set is
+  // built once (one bit per block), and the main loop walks its bits, so there is
+  // no branch around a block.  A wave whose own tile is -inf inside a visited
+  // block fills its scores with -inf (every weight comes out 0).
+  const bool use_list = HAS_MASK && cls_row && p.skip_masked && nkb <= 64 * FA_MAX_GROUPS;
+  int n_live = nkb;
+  if (use_list) {
+    n_live = 0;
+    for (int group = 0; group * 64 < nkb; group++) {
+      load_classes(group);
+      __syncthreads(); // the previous group's s_ninf has been read
+      if (lane == 0)
+        s_ninf[wave] = ninf_bits;
+      __syncthreads();
+      const int left = nkb - group * 64;
+      const uint64_t live = ~(s_ninf[0] & s_ninf[1] & s_ninf[2] & s_ninf[3]) & (left >= 64 ? ~0ull : ((1ull << left) - 1));
+      if (tid == 0)
+        s_live[group] = live;
+      n_live += __builtin_popcountll(live);
     }
-    if (lane == 0)
-      s_last[wave] = last;
     __syncthreads();
-    nkb = max(max(s_last[0], s_last[1]), max(s_last[2], s_last[3]));
   }
-  if (HAS_MASK)
-    load_classes(0);
+  // walks the visited blocks in order (all scalar); called at most n_live times
+  int walk_group = -1;
+  uint64_t walk_bits = 0;
+  auto next_block = [&](int ordinal) -> int {
+    if (!use_list)
+      return ordinal;
+    while (walk_bits == 0) {
+      walk_group++;
+      const uint64_t v = s_live[walk_group];
+      walk_bits = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(v >> 32)) << 32) |
+                  __builtin_amdgcn_readfirstlane((uint32_t)v);
+    }
+    const int kb = walk_group * 64 + __builtin_ctzll(walk_bits);
+    walk_bits &= walk_bits - 1;
+    return kb;
+  };
 
-  if (nkb > 0) {
-    g.issue_kv(smem0, Kb, Vb);
+  int kb_cur = 0;
+  if (n_live > 0) {
+    kb_cur = next_block(0);
+    g.issue_kv(smem0, Kb + kb_cur * blk_bytes, Vb + kb_cur * blk_bytes);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
   }
 
-  // One key block: start the DMA of the next K/V block into the other stage
-  // (the last block re-fetches itself into the free stage), then compute.
-  auto step = [&](const char *cur, char *nxt, int kb) {
-    const uint64_t bit = 1ull << (kb & 63);
-    const bool is_zero = !HAS_MASK || (zero_bits & bit);
-    const bool is_ninf = HAS_MASK && (ninf_bits & bit);
-    const bool is_skip = is_ninf && p.skip_masked;
-    const int kbn = min(kb + 1, nkb - 1);
-    if (HAS_MASK && ((kb + 1) & 63) == 0 && kb + 1 < nkb)
-      load_classes(kb + 1);
-    // the DMA is issued inside each arm, in the basic block of the LDS reads it
-    // must not be ordered against
-    const char *kn = Kb + kbn * blk_bytes, *vn = Vb + kbn * blk_bytes;
-    if (is_skip) {
-      g.issue_kv(nxt, kn, vn);
-    } else if (is_zero) {
-      asm volatile("; arm: no mask term" ::: "memory"); // distinct text: keeps the DMA from being hoisted out of the arm
-      g.issue_kv(nxt, kn, vn);
-      g.template block<0>(cur, qf, nullptr, p.scale, o, m_run, l_run);
-    } else if (is_ninf) {
-      asm volatile("; arm: -inf tile" ::: "memory");
-      g.issue_kv(nxt, kn, vn);
-      g.template block<2>(cur, qf, nullptr, p.scale, o, m_run, l_run);
-    } else {
-      asm volatile("; arm: mask tile" ::: "memory");
-      g.issue_kv(nxt, kn, vn);
-      g.template block<1>(cur, qf, mrow + kb * FA_BK, p.scale, o, m_run, l_run);
-    }
+  const float inv_scale = 1.0f / p.scale;
+  // One visited key block: start the DMA of the next one into the other stage
+  // (the last re-fetches itself into the free stage), then compute.
+  auto step = [&](const char *cur, char *nxt, int i) {
+    const int kb = kb_cur;
+    const int kbn = i + 1 < n_live ? next_block(i + 1) : kb;
+    kb_cur = kbn;
+    if (HAS_MASK && (kb >> 6) != cls_group)
+      load_classes(kb >> 6);
+    // 0: the tile adds nothing, 1: read it, 2: -inf throughout
+    const int kind = !HAS_MASK ? 0 : ((zero_bits >> (kb & 63)) & 1) ? 0 : ((ninf_bits >> (kb & 63)) & 1) ? 2 : 1;
+    g.issue_kv(nxt, Kb + kbn * blk_bytes, Vb + kbn * blk_bytes);
+    g.template block<HAS_MASK>(cur, qf, kind, mrow + kb * FA_BK, p.scale, inv_scale, o, m_run, l_run);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
   };
-  for (int kb = 0; kb < nkb; kb += 2) {
-    step(smem0, smem1, kb);
-    if (kb + 1 < nkb)
-      step(smem1, smem0, kb + 1);
+  for (int i = 0; i < n_live; i += 2) {
+    step(smem0, smem1, i);
+    if (i + 1 < n_live)
+      step(smem1, smem0, i + 1);
   }
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);

@@ -100,11 +100,13 @@ int gcmi_mha_fwd_bf16(const void *Q, const void *K, const void *V, const float *
  * The same with the block-skipping switch exposed.  When a mask is given, one
  * pass over it classifies every (32 query rows x 64 keys) tile as all 0, all
  * -inf or general; constant tiles cost no mask traffic in the main kernel.
- * skip_masked != 0 (what gcmi_mha_fwd_bf16 uses): tiles that are all -inf are
- * not computed at all -- they contribute exp(-inf) = 0 to every sum, so the
- * result is bit-identical.  skip_masked == 0: every tile is computed (the dense
- * 4*BH*Sq*Sk*D operation count).  The tile classes live in a per-device static
- * buffer: calls on different streams of one device must not overlap.
+ * skip_masked != 0 (what gcmi_mha_fwd_bf16 uses): a block of 64 keys whose
+ * tiles are -inf for all 128 query rows of a workgroup is not visited at all --
+ * it contributes exp(-inf) = 0 to every sum, so the result is bit-identical.
+ * skip_masked == 0: every block is computed (the dense 4*BH*Sq*Sk*D operation
+ * count).  scale must be > 0 for the fast kernel (otherwise a slower, general
+ * kernel runs).  The tile classes live in a per-device static buffer: calls on
+ * different streams of one device must not overlap.
  * No counterpart in the reference.
  */
 int gcmi_mha_fwd_bf16_opt(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld, void *O,
