@@ -4,8 +4,8 @@
 // gemm_f32_kernel: C[M,N] = act(beta*C + A.B + bias), arbitrary element strides
 // on A and B so that transpose_a / transpose_b of onednn_graph.matmul
 // (lib/gc/Transforms/OneDNNGraphToLinalg.cpp:421-499) need no copy.
-// 64x64 workgroup tile, 16-deep K slices through LDS, 4x4 outputs per thread,
-// k ascending per output element.
+// 64/32/16-square workgroup tiles, 32-deep K slices through LDS with register
+// prefetch, k ascending per output element.
 //
 // brgemm_kernel: C[m*LDC+n] (+)= sum_i sum_k a(i,m,k) * b(i,k,n) with
 //   f32 : b at i*stride_b + k*LDB + n
@@ -19,58 +19,83 @@
 
 namespace gcmi {
 
-__global__ __launch_bounds__(256) void gemm_f32_kernel(F32GemmParams p) {
-  __shared__ float As[16][64 + 4];
-  __shared__ float Bs[16][64 + 4];
+// BT x BT workgroup tile (BT = 64, 32 or 16: small problems take small tiles so
+// that more compute units take part), 256 threads, (BT/16)^2 outputs per thread,
+// 32-deep K slices through LDS.  The next slice is fetched into registers while
+// the current one is multiplied, so global latency is paid once, not per slice.
+template <int BT> __global__ __launch_bounds__(256) void gemm_f32_kernel(F32GemmParams p) {
+  constexpr int BK = 32, MT = BT / 16, PER = BT * BK / 256; // elements per thread per operand slice
+  __shared__ float As[BK][BT + 4];
+  __shared__ float Bs[BK][BT + 4];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-  const int64_t m0 = (int64_t)blockIdx.y * 64, n0 = (int64_t)blockIdx.x * 64;
-  float acc[4][4] = {};
-  for (int64_t k0 = 0; k0 < p.K; k0 += 16) {
-    // 64x16 of A and 16x64 of B: 1024 elements each, 4 per thread
+  const int64_t m0 = (int64_t)blockIdx.y * BT, n0 = (int64_t)blockIdx.x * BT;
+  // slice element e of this thread: (row/col within the tile, k within the slice);
+  // the contiguous direction of each operand runs along consecutive threads
+  int am[PER], ak[PER], bn[PER], bk[PER];
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-      int idx = threadIdx.x + 256 * e;
-      int am = idx & 63, ak = idx >> 6; // consecutive threads along m
-      if (p.a_cs == 1) {                // k contiguous: walk k fastest instead
-        ak = idx & 15;
-        am = idx >> 4;
-      }
-      int64_t gm = m0 + am, gk = k0 + ak;
-      As[ak][am] = (gm < p.M && gk < p.K) ? p.A[gm * p.a_rs + gk * p.a_cs] : 0.0f;
-      int bn = idx & 63, bk = idx >> 6;
-      if (p.b_rs == 1 && p.b_cs != 1) {
-        bk = idx & 15;
-        bn = idx >> 4;
-      }
-      int64_t gn = n0 + bn, gk2 = k0 + bk;
-      Bs[bk][bn] = (gn < p.N && gk2 < p.K) ? p.B[gk2 * p.b_rs + gn * p.b_cs] : 0.0f;
+  for (int e = 0; e < PER; e++) {
+    const int idx = threadIdx.x + 256 * e;
+    if (p.a_cs == 1) {
+      ak[e] = idx % BK;
+      am[e] = idx / BK;
+    } else {
+      am[e] = idx % BT;
+      ak[e] = idx / BT;
+    }
+    if (p.b_rs == 1 && p.b_cs != 1) {
+      bk[e] = idx % BK;
+      bn[e] = idx / BK;
+    } else {
+      bn[e] = idx % BT;
+      bk[e] = idx / BT;
+    }
+  }
+  float ra[PER], rb[PER];
+  auto fetch = [&](int64_t k0) {
+#pragma unroll
+    for (int e = 0; e < PER; e++) {
+      const int64_t gm = m0 + am[e], gk = k0 + ak[e];
+      ra[e] = (gm < p.M && gk < p.K) ? p.A[gm * p.a_rs + gk * p.a_cs] : 0.0f;
+      const int64_t gn = n0 + bn[e], gk2 = k0 + bk[e];
+      rb[e] = (gn < p.N && gk2 < p.K) ? p.B[gk2 * p.b_rs + gn * p.b_cs] : 0.0f;
+    }
+  };
+  float acc[MT][MT] = {};
+  fetch(0);
+  for (int64_t k0 = 0; k0 < p.K; k0 += BK) {
+#pragma unroll
+    for (int e = 0; e < PER; e++) {
+      As[ak[e]][am[e]] = ra[e];
+      Bs[bk[e]][bn[e]] = rb[e];
     }
     __syncthreads();
+    if (k0 + BK < p.K)
+      fetch(k0 + BK);
 #pragma unroll
-    for (int k = 0; k < 16; k++) {
-      float a[4], b[4];
+    for (int k = 0; k < BK; k++) { // k ascending per output element
+      float a[MT], b[MT];
 #pragma unroll
-      for (int i = 0; i < 4; i++)
-        a[i] = As[k][ty * 4 + i];
+      for (int i = 0; i < MT; i++)
+        a[i] = As[k][ty * MT + i];
 #pragma unroll
-      for (int j = 0; j < 4; j++)
-        b[j] = Bs[k][tx * 4 + j];
+      for (int j = 0; j < MT; j++)
+        b[j] = Bs[k][tx * MT + j];
 #pragma unroll
-      for (int i = 0; i < 4; i++)
+      for (int i = 0; i < MT; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < MT; j++)
           acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
     }
     __syncthreads();
   }
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    int64_t m = m0 + ty * 4 + i;
+  for (int i = 0; i < MT; i++) {
+    int64_t m = m0 + ty * MT + i;
     if (m >= p.M)
       continue;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      int64_t n = n0 + tx * 4 + j;
+    for (int j = 0; j < MT; j++) {
+      int64_t n = n0 + tx * MT + j;
       if (n >= p.N)
         continue;
       float x = acc[i][j];
@@ -136,8 +161,18 @@ extern "C" int gcmi_launch_gemm_f32(const F32GemmParams *pp, hipStream_t stream)
   F32GemmParams p = *pp;
   if (p.M <= 0 || p.N <= 0)
     return 0;
-  dim3 grid((unsigned)((p.N + 63) / 64), (unsigned)((p.M + 63) / 64)), block(256);
-  hipLaunchKernelGGL(gemm_f32_kernel, grid, block, 0, stream, p);
+  // the largest tile that still gives every compute unit a workgroup
+  auto tiles = [&](int bt) { return ((p.N + bt - 1) / bt) * ((p.M + bt - 1) / bt); };
+  const int bt = tiles(64) >= 256 ? 64 : tiles(32) >= 256 ? 32 : 16;
+  dim3 grid((unsigned)((p.N + bt - 1) / bt), (unsigned)((p.M + bt - 1) / bt)), block(256);
+  if (grid.y > 65535)
+    return 2;
+  if (bt == 64)
+    hipLaunchKernelGGL(gemm_f32_kernel<64>, grid, block, 0, stream, p);
+  else if (bt == 32)
+    hipLaunchKernelGGL(gemm_f32_kernel<32>, grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL(gemm_f32_kernel<16>, grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 
