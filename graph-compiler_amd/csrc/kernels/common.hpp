@@ -84,3 +84,18 @@ __device__ __forceinline__ float apply_act(float x, int act) {
 }
 
 } // namespace gcmi
+
+// compute units of the current device (host side, cached per device)
+static inline int gcmi_num_cus() {
+  static int cache[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    return 256;
+  if (cache[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cache[dev] = n;
+  }
+  return cache[dev];
+}

@@ -632,21 +632,6 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
 
 using namespace gcmi;
 
-// compute units of the current device (cached per device)
-static int gcmi_num_cus() {
-  static int cache[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
-    return 256;
-  if (cache[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    cache[dev] = n;
-  }
-  return cache[dev];
-}
-
 extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
   MhaParams p = *pp;
   if (p.D != FA_D)
