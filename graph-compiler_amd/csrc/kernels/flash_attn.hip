@@ -473,23 +473,25 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
   const int nqb = p.Sq / FA_BQ;
   // Workgroup -> (head, query block).  Consecutive workgroup ids are dealt
   // round-robin to the 8 XCDs; all query blocks of one (batch, head) are given to
-  // ONE XCD so that its K/V (Sk x 512 B) is fetched from HBM once and then served
-  // from that XCD's L2.  Long (late) query blocks first.  With pair_q a workgroup
-  // takes block n-1-j and then block j: under a triangular mask with skipping
-  // every workgroup then has the same amount of work.
-  const int per_head = p.pair_q ? (nqb + 1) / 2 : nqb;
-  int qj, bh;
+  // ONE XCD so that its K/V (Sk x 512 B) is fetched once and then served from that
+  // XCD's L2.  An XCD works on four heads at a time (4 MiB of K and V at 2048
+  // keys) and takes their long (late) query blocks first, so that under a
+  // triangular mask with skipping the short blocks fill the gaps at the end.
+  int qb, bh;
   if ((p.BH & 7) == 0) {
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    bh = (idx / per_head) * 8 + xcd;
-    qj = idx % per_head;
+    if (((p.BH >> 3) & 3) == 0) {
+      const int grp = idx / (4 * nqb), r = idx % (4 * nqb);
+      bh = (grp * 4 + (r & 3)) * 8 + xcd;
+      qb = nqb - 1 - (r >> 2);
+    } else {
+      bh = (idx / nqb) * 8 + xcd;
+      qb = nqb - 1 - idx % nqb;
+    }
   } else {
-    qj = blockIdx.x % per_head;
-    bh = blockIdx.x / per_head;
+    qb = nqb - 1 - blockIdx.x % nqb;
+    bh = blockIdx.x / nqb;
   }
-  const int n_pass = (p.pair_q && qj != nqb - 1 - qj) ? 2 : 1;
-  for (int pass = 0; pass < n_pass; pass++) {
-  const int qb = pass == 0 ? nqb - 1 - qj : qj;
   const int q_lane = qb * FA_BQ + wave * 32 + l32;
 
   const char *Qb = reinterpret_cast<const char *>(p.Q) + (int64_t)bh * p.Sq * FA_D * 2;
@@ -625,7 +627,6 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
       *reinterpret_cast<uint2 *>(Ob + (dt * 32 + 8 * q4 + 4 * lh) * 2) =
           make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
     }
-  } // pass
 }
 
 } // namespace gcmi
@@ -639,7 +640,7 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
   if (p.BH <= 0 || p.Sq <= 0 || p.Sk <= 0)
     return 0;
   const int nqb = (p.Sq + FA_BQ - 1) / FA_BQ;
-  int64_t nblk = (int64_t)nqb * p.BH;
+  const int64_t nblk = (int64_t)nqb * p.BH;
   if (nblk > 0x7fffffff)
     return 2;
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
@@ -649,7 +650,6 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
   if (!(al16(p.Q) && al16(p.K) && al16(p.V) && al16(p.O)))
     return 2; // rows are 256 bytes: a 16-byte aligned base is required
   p.tile_class = nullptr;
-  p.pair_q = 0;
   if (p.mask && fast) {
     const int64_t n_qt = p.Sq / 32, n_kb = p.Sk / FA_BK;
     if (n_qt * n_kb <= FA_MAX_TILES && n_qt <= 65535) {
@@ -660,11 +660,6 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
                          p.mask_ld, (int)n_kb, ws);
       p.tile_class = ws;
     }
-  }
-  // pairing halves the number of workgroups: only when the GPU stays full (2 per CU)
-  if (fast && p.tile_class && p.skip_masked && (int64_t)((nqb + 1) / 2) * p.BH >= 2 * gcmi_num_cus()) {
-    p.pair_q = 1;
-    nblk = (int64_t)((nqb + 1) / 2) * p.BH;
   }
   dim3 grid((unsigned)nblk), block(FA_THREADS);
   if (p.mask) {

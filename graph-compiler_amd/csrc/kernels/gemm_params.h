@@ -43,7 +43,6 @@ struct MhaParams {
   // fast path only: class of every (32 query rows x 64 keys) mask tile, [Sq/32][Sk/64], or null
   const uint8_t *tile_class;
   int32_t skip_masked; // 1: tiles whose mask is all -inf are not computed (the result is the same)
-  int32_t pair_q;      // 1: a workgroup takes query blocks j and n-1-j in turn (evens out triangular masks)
 };
 
 } // namespace gcmi
