@@ -101,3 +101,43 @@ def test_skipping_masked_blocks_changes_no_bit(gc, dev, Sq, Sk, kind):
     b = gc.mha_fwd_bf16(Q, K, V, mask, 0.088, skip_masked=False)
     torch.cuda.synchronize()
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+@pytest.mark.parametrize("skip", [True, False])
+def test_band_mask_over_many_key_blocks(gc, orc, wl, dev, skip):
+    """8192 keys = 128 key blocks (two groups of 64 in the kernel's bookkeeping).
+    A band mask leaves -inf blocks before and after the band, and the band
+    crosses the group boundary: the set of visited blocks has gaps on both
+    sides and spans both groups."""
+    torch.manual_seed(5)
+    H, Sq, Sk, D = 8, 256, 8192, 128
+    Q = torch.randn(1, H, Sq, D).to(torch.bfloat16)
+    K = torch.randn(1, H, Sk, D).to(torch.bfloat16)
+    V = torch.randn(1, H, Sk, D).to(torch.bfloat16)
+    qi = torch.arange(Sq).reshape(-1, 1)
+    kj = torch.arange(Sk).reshape(1, -1)
+    lo = 3000 + 4 * qi            # band start moves with the query row
+    mask = torch.where((kj >= lo) & (kj < lo + 1500), 0.0, float("-inf")).float()
+    mask[:, 7000:7003] = -2.5      # a few finite entries far from the band: one more visited block
+    scale = 1 / np.sqrt(D)
+    out = gc.mha_fwd_bf16(Q.to(dev), K.to(dev), V.to(dev), mask.to(dev), scale, skip_masked=skip)
+    torch.cuda.synchronize()
+    for h in (0, 5):
+        ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q[:, h:h + 1]), wl.bf16_bits(K[:, h:h + 1]),
+                                           wl.bf16_bits(V[:, h:h + 1]), mask.numpy(), scale))
+        assert_close(ref, out[:, h:h + 1].float().cpu().numpy(), 1e-2, "band mask head %d" % h,
+                     mag=_pv_mag(Q[:, h:h + 1], K[:, h:h + 1], V[:, h:h + 1], mask, scale))
+
+
+def test_negative_scale_takes_the_general_kernel(gc, orc, wl, dev):
+    """The fast kernel folds the scale into the maximum (needs scale > 0); a
+    negative scale must still give the reference result."""
+    torch.manual_seed(6)
+    Q = torch.randn(1, 2, 128, 128).to(torch.bfloat16)
+    K = torch.randn(1, 2, 128, 128).to(torch.bfloat16)
+    V = torch.randn(1, 2, 128, 128).to(torch.bfloat16)
+    mask = _mask("causal", 128, 128)
+    ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q), wl.bf16_bits(K), wl.bf16_bits(V), mask.numpy(), -0.05))
+    out = gc.mha_fwd_bf16(Q.to(dev), K.to(dev), V.to(dev), mask.to(dev), -0.05)
+    torch.cuda.synchronize()
+    assert_close(ref, out.float().cpu().numpy(), 1e-2, "negative scale", mag=_pv_mag(Q, K, V, mask, -0.05))
