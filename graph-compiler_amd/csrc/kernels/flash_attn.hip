@@ -310,20 +310,46 @@ constexpr int FA_K_AHEAD = 6;
 // the set of visited key blocks is kept for up to 64 * FA_MAX_GROUPS blocks (65536 keys)
 constexpr int FA_MAX_GROUPS = 16;
 
-struct FaFast {
-  uint32_t k_src[4], v_src[4]; // per-lane global byte offsets of this wave's DMA instructions (within a 64-key block)
+// NW waves per workgroup (4 or 8); each takes 32 query rows and 16/NW of the 16 DMA
+// instructions that bring a K (or V) tile in.
+template <int NW> struct FaFast {
+  static constexpr int NDMA = 16 / NW;
+  uint32_t k_src[NDMA], v_src[NDMA]; // per-lane global byte offsets of this wave's DMA instructions (within a 64-key block)
   uint32_t k_ld[8], v_ld[4];   // LDS fragment offsets
   int wave_u;
 
+  // One 1 KiB piece: lane l's 16 bytes land at lds_addr + 16*l.  For the three-stage
+  // ring (NW == 8) written as inline
+  // assembly (M0 = LDS destination, as the instruction wants it) so that these
+  // requests stay outside the compiler's own memory-counter bookkeeping: it would
+  // otherwise make every later LDS read wait for all of them, and the point is to
+  // keep them in flight across one or two key blocks.  The waits are the explicit
+  // s_waitcnt vmcnt(..) in the main loop; nothing else in this kernel uses M0.
+  static __device__ __forceinline__ void dma_1k(const char *src, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr)
+                 : "memory", "m0");
+  }
   __device__ __forceinline__ void issue_kv(char *__restrict__ stage, const char *kb_ptr, const char *vb_ptr) const {
+    if constexpr (NW == 8) {
+      const uint32_t base = (uint32_t)(uintptr_t)(GCMI_LDS char *)stage + (uint32_t)(wave_u * NDMA) * 1024u;
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(kb_ptr + k_src[i]),
-                                       (GCMI_LDS void *)(stage + (wave_u * 4 + i) * 1024), 16, 0, 0);
+      for (int i = 0; i < NDMA; i++)
+        dma_1k(kb_ptr + k_src[i], base + i * 1024u);
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(vb_ptr + v_src[i]),
-                                       (GCMI_LDS void *)(stage + FA_TILE_BYTES + (wave_u * 4 + i) * 1024), 16, 0, 0);
+      for (int i = 0; i < NDMA; i++)
+        dma_1k(vb_ptr + v_src[i], base + FA_TILE_BYTES + i * 1024u);
+    } else {
+      // two stages, one block ahead: the compiler's own counting is exact enough here,
+      // and it may spread these requests between the MFMAs
+#pragma unroll
+      for (int i = 0; i < NDMA; i++)
+        __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(kb_ptr + k_src[i]),
+                                         (GCMI_LDS void *)(stage + (wave_u * NDMA + i) * 1024), 16, 0, 0);
+#pragma unroll
+      for (int i = 0; i < NDMA; i++)
+        __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(vb_ptr + v_src[i]),
+                                         (GCMI_LDS void *)(stage + FA_TILE_BYTES + (wave_u * NDMA + i) * 1024), 16, 0, 0);
+    }
   }
 
   // One 64-key block.  kind (wave-uniform): 0 the mask tile adds nothing, 1 read it
@@ -461,16 +487,26 @@ struct FaFast {
   }
 };
 
-template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fwd_fast_kernel(MhaParams p) {
+// NW = 4: 128 query rows per workgroup, two workgroups per compute unit.
+// NW = 8: 256 query rows, one workgroup per compute unit -- every K/V tile then
+// serves twice as many rows, which halves the DMA traffic into LDS.
+template <bool HAS_MASK, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void mha_fwd_fast_kernel(MhaParams p) {
+  constexpr int BQ = NW * 32;
   __shared__ __align__(1024) char smem0[2 * FA_TILE_BYTES];
   __shared__ __align__(1024) char smem1[2 * FA_TILE_BYTES];
-  __shared__ uint64_t s_ninf[4];          // per wave: -inf classes of the current group of 64 key blocks
+  // the 8-wave kernel (one workgroup per compute unit) has room for a third stage:
+  // the DMA then runs two key blocks ahead
+  constexpr int NST = NW == 8 ? 3 : 2;
+  __shared__ __align__(1024) char smem2[NST == 3 ? 2 * FA_TILE_BYTES : 1024];
+  __shared__ uint64_t s_zero[NW][FA_MAX_GROUPS], s_ninf[NW][FA_MAX_GROUPS]; // per wave and group of 64 key blocks: tile classes
+         // per wave: -inf classes of the current group of 64 key blocks
   __shared__ uint64_t s_live[FA_MAX_GROUPS]; // per group of 64 key blocks: the ones the workgroup visits
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, lh = lane >> 5;
-  const int nqb = p.Sq / FA_BQ;
+  const int nqb = p.Sq / BQ;
   // Workgroup -> (head, query block).  Consecutive workgroup ids are dealt
   // round-robin to the 8 XCDs; all query blocks of one (batch, head) are given to
   // ONE XCD so that its K/V (Sk x 512 B) is fetched once and then served from that
@@ -492,7 +528,7 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
     qb = nqb - 1 - blockIdx.x % nqb;
     bh = blockIdx.x / nqb;
   }
-  const int q_lane = qb * FA_BQ + wave * 32 + l32;
+  const int q_lane = qb * BQ + wave * 32 + l32;
 
   const char *Qb = reinterpret_cast<const char *>(p.Q) + (int64_t)bh * p.Sq * FA_D * 2;
   const char *Kb = reinterpret_cast<const char *>(p.K) + (int64_t)bh * p.Sk * FA_D * 2;
@@ -503,11 +539,11 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
   for (int ds = 0; ds < 8; ds++)
     qf[ds] = *reinterpret_cast<const uint4 *>(Qb + (int64_t)q_lane * FA_D * 2 + ds * 32 + lh * 16);
 
-  FaFast g;
+  FaFast<NW> g;
   g.wave_u = wave;
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    int key = (wave * 4 + i) * 4 + (lane >> 4), ph = lane & 15;
+  for (int i = 0; i < FaFast<NW>::NDMA; i++) {
+    int key = (wave * FaFast<NW>::NDMA + i) * 4 + (lane >> 4), ph = lane & 15;
     g.k_src[i] = (uint32_t)(key * 256 + ((ph ^ (key & 15)) << 4));
     g.v_src[i] = (uint32_t)(key * 256 + ((ph ^ ((key & 3) << 2)) << 4));
   }
@@ -532,39 +568,61 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
   const int64_t blk_bytes = (int64_t)FA_BK * FA_D * 2;
   const float *mrow = HAS_MASK ? p.mask + (int64_t)q_lane * p.mask_ld + 4 * lh : nullptr;
 
-  // classes of this wave's mask tiles, 64 key blocks at a time, as two lane masks
-  const uint8_t *cls_row = (HAS_MASK && p.tile_class) ? p.tile_class + (int64_t)(qb * 4 + wave) * nkb : nullptr;
+  // Classes of this wave's mask tiles, one bit per key block in groups of 64,
+  // read from memory once and kept in LDS: the main loop must not issue vector
+  // memory loads of its own next to the K/V DMA it counts.
+  const bool have_cls = HAS_MASK && p.tile_class && nkb <= 64 * FA_MAX_GROUPS;
+  const int n_groups = (nkb + 63) >> 6;
+  if (have_cls) {
+    const uint8_t *cls_row = p.tile_class + (int64_t)(qb * NW + wave) * nkb;
+    for (int group = 0; group < n_groups; group++) {
+      uint8_t c = FA_TILE_GENERAL;
+      if (group * 64 + lane < nkb)
+        c = cls_row[group * 64 + lane];
+      const uint64_t zb = __ballot(c == FA_TILE_ZERO), nb = __ballot(c == FA_TILE_NEG_INF);
+      if (lane == 0) {
+        s_zero[wave][group] = zb;
+        s_ninf[wave][group] = nb;
+      }
+    }
+  }
+  __syncthreads();
   uint64_t zero_bits = 0, ninf_bits = 0;
   int cls_group = -1;
+  auto bcast64 = [](uint64_t v) -> uint64_t {
+    // readfirstlane returns int: widen through uint32_t, or bit 31 smears over the upper half
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)v);
+    return ((uint64_t)hi << 32) | lo;
+  };
   auto load_classes = [&](int group) {
-    uint8_t c = FA_TILE_GENERAL;
-    if (cls_row && group * 64 + lane < nkb)
-      c = cls_row[group * 64 + lane];
-    zero_bits = __ballot(c == FA_TILE_ZERO);
-    ninf_bits = __ballot(c == FA_TILE_NEG_INF);
+    if (have_cls) {
+      zero_bits = bcast64(s_zero[wave][group]);
+      ninf_bits = bcast64(s_ninf[wave][group]);
+    }
     cls_group = group;
   };
-  // Key blocks whose tiles are -inf for all four waves are left out: their set is
+  // Key blocks whose tiles are -inf for all waves of the workgroup are left out: their set is
   // built once (one bit per block), and the main loop walks its bits, so there is
   // no branch around a block.  A wave whose own tile is -inf inside a visited
   // block fills its scores with -inf (every weight comes out 0).
-  const bool use_list = HAS_MASK && cls_row && p.skip_masked && nkb <= 64 * FA_MAX_GROUPS;
+  const bool use_list = have_cls && p.skip_masked;
   int n_live = nkb;
   if (use_list) {
     n_live = 0;
-    for (int group = 0; group * 64 < nkb; group++) {
-      load_classes(group);
-      __syncthreads(); // the previous group's s_ninf has been read
-      if (lane == 0)
-        s_ninf[wave] = ninf_bits;
-      __syncthreads();
+    for (int group = 0; group < n_groups; group++) {
       const int left = nkb - group * 64;
-      const uint64_t live = ~(s_ninf[0] & s_ninf[1] & s_ninf[2] & s_ninf[3]) & (left >= 64 ? ~0ull : ((1ull << left) - 1));
+      uint64_t all_ninf = s_ninf[0][group];
+#pragma unroll
+      for (int w = 1; w < NW; w++)
+        all_ninf &= s_ninf[w][group];
+      const uint64_t live = bcast64(~all_ninf & (left >= 64 ? ~0ull : ((1ull << left) - 1)));
       if (tid == 0)
         s_live[group] = live;
       n_live += __builtin_popcountll(live);
     }
     __syncthreads();
+    n_live = min(n_live, nkb);
   }
   // walks the visited blocks in order (all scalar); called at most n_live times
   int walk_group = -1;
@@ -572,46 +630,70 @@ template <bool HAS_MASK> __global__ __launch_bounds__(FA_THREADS, 2) void mha_fw
   auto next_block = [&](int ordinal) -> int {
     if (!use_list)
       return ordinal;
-    while (walk_bits == 0) {
+    while (walk_bits == 0 && walk_group + 1 < n_groups) {
       walk_group++;
-      const uint64_t v = s_live[walk_group];
-      walk_bits = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(v >> 32)) << 32) |
-                  __builtin_amdgcn_readfirstlane((uint32_t)v);
+      walk_bits = bcast64(s_live[walk_group]);
     }
+    if (walk_bits == 0)
+      return nkb - 1; // not reached: next_block is called once per visited block
     const int kb = walk_group * 64 + __builtin_ctzll(walk_bits);
     walk_bits &= walk_bits - 1;
-    return kb;
+    return min(kb, nkb - 1); // the set only holds blocks below nkb; the clamp keeps every K/V address in range regardless
   };
 
-  int kb_cur = 0;
+  // kb_q[0] is the block being computed, kb_q[1..] the ones already requested
+  int kb_q[NST - 1] = {};
   if (n_live > 0) {
-    kb_cur = next_block(0);
-    g.issue_kv(smem0, Kb + kb_cur * blk_bytes, Vb + kb_cur * blk_bytes);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    kb_q[0] = next_block(0);
+    g.issue_kv(smem0, Kb + kb_q[0] * blk_bytes, Vb + kb_q[0] * blk_bytes);
+    if (NST == 3) {
+      kb_q[NST - 2] = n_live > 1 ? next_block(1) : kb_q[0];
+      g.issue_kv(smem1, Kb + kb_q[NST - 2] * blk_bytes, Vb + kb_q[NST - 2] * blk_bytes);
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * FaFast<NW>::NDMA) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     __builtin_amdgcn_s_barrier();
   }
 
   const float inv_scale = 1.0f / p.scale;
-  // One visited key block: start the DMA of the next one into the other stage
-  // (the last re-fetches itself into the free stage), then compute.
-  auto step = [&](const char *cur, char *nxt, int i) {
-    const int kb = kb_cur;
-    const int kbn = i + 1 < n_live ? next_block(i + 1) : kb;
-    kb_cur = kbn;
+  // One visited key block: request the block NST-1 ahead into the stage that was
+  // computed from last (past the end the last block is fetched again: the order
+  // of requests stays unconditional), compute, wait for the next block only.
+  auto step = [&](const char *cur, char *fill, int i) {
+    const int kb = kb_q[0];
+    const int kbf = i + NST - 1 < n_live ? next_block(i + NST - 1) : kb_q[NST - 2];
+    if (NST == 3)
+      kb_q[0] = kb_q[1];
+    kb_q[NST - 2] = kbf;
     if (HAS_MASK && (kb >> 6) != cls_group)
       load_classes(kb >> 6);
     // 0: the tile adds nothing, 1: read it, 2: -inf throughout
     const int kind = !HAS_MASK ? 0 : ((zero_bits >> (kb & 63)) & 1) ? 0 : ((ninf_bits >> (kb & 63)) & 1) ? 2 : 1;
-    g.issue_kv(nxt, Kb + kbn * blk_bytes, Vb + kbn * blk_bytes);
+    g.issue_kv(fill, Kb + kbf * blk_bytes, Vb + kbf * blk_bytes);
     g.template block<HAS_MASK>(cur, qf, kind, mrow + kb * FA_BK, p.scale, inv_scale, o, m_run, l_run);
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    if (NST == 3)
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * FaFast<NW>::NDMA) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
   };
-  for (int i = 0; i < n_live; i += 2) {
-    step(smem0, smem1, i);
-    if (i + 1 < n_live)
-      step(smem1, smem0, i + 1);
+  if (NST == 3) {
+    for (int i = 0; i < n_live; i += 3) {
+      step(smem0, smem2, i);
+      if (i + 1 < n_live)
+        step(smem1, smem0, i + 1);
+      if (i + 2 < n_live)
+        step(smem2, smem1, i + 2);
+    }
+  } else {
+    for (int i = 0; i < n_live; i += 2) {
+      step(smem0, smem1, i);
+      if (i + 1 < n_live)
+        step(smem1, smem0, i + 1);
+    }
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // requests past the end have landed before the stages go away
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = 1.0f / l_tot;
@@ -639,8 +721,8 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
     return 3;
   if (p.BH <= 0 || p.Sq <= 0 || p.Sk <= 0)
     return 0;
-  const int nqb = (p.Sq + FA_BQ - 1) / FA_BQ;
-  const int64_t nblk = (int64_t)nqb * p.BH;
+  int nqb = (p.Sq + FA_BQ - 1) / FA_BQ;
+  int64_t nblk = (int64_t)nqb * p.BH;
   if (nblk > 0x7fffffff)
     return 2;
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
@@ -661,15 +743,27 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
       p.tile_class = ws;
     }
   }
-  dim3 grid((unsigned)nblk), block(FA_THREADS);
+  // 256-row workgroups when they still fill the GPU.  Measured at 4 x 32 heads, 2048 x 2048: 2-3 % faster
+  // without a mask, slower with a triangular mask (block skipping is coarser, fewer workgroups
+  // to even out), so masked calls keep the 128-row kernel.
+  const bool wide = fast && !p.mask && p.Sq % 256 == 0 && (int64_t)(p.Sq / 256) * p.BH >= gcmi_num_cus();
+  if (wide) {
+    nqb = p.Sq / 256;
+    nblk = (int64_t)nqb * p.BH;
+  }
+  dim3 grid((unsigned)nblk), block(wide ? 512 : FA_THREADS);
   if (p.mask) {
-    if (fast)
-      hipLaunchKernelGGL((mha_fwd_fast_kernel<true>), grid, block, 0, stream, p);
+    if (wide)
+      hipLaunchKernelGGL((mha_fwd_fast_kernel<true, 8>), grid, block, 0, stream, p);
+    else if (fast)
+      hipLaunchKernelGGL((mha_fwd_fast_kernel<true, 4>), grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL((mha_fwd_kernel<true, true>), grid, block, 0, stream, p);
   } else {
-    if (fast)
-      hipLaunchKernelGGL((mha_fwd_fast_kernel<false>), grid, block, 0, stream, p);
+    if (wide)
+      hipLaunchKernelGGL((mha_fwd_fast_kernel<false, 8>), grid, block, 0, stream, p);
+    else if (fast)
+      hipLaunchKernelGGL((mha_fwd_fast_kernel<false, 4>), grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL((mha_fwd_kernel<false, true>), grid, block, 0, stream, p);
   }

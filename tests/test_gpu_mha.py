@@ -141,3 +141,28 @@ def test_negative_scale_takes_the_general_kernel(gc, orc, wl, dev):
     out = gc.mha_fwd_bf16(Q.to(dev), K.to(dev), V.to(dev), mask.to(dev), -0.05)
     torch.cuda.synchronize()
     assert_close(ref, out.float().cpu().numpy(), 1e-2, "negative scale", mag=_pv_mag(Q, K, V, mask, -0.05))
+
+
+@pytest.mark.parametrize("kind", ["causal", "random", "none"])
+def test_wide_workgroups_many_heads(gc, orc, wl, dev, kind):
+    """256 (batch, head) pairs x 256 query rows: enough 256-row workgroups to fill
+    the GPU, so the 8-wave kernel runs.  A few heads against the oracle, and the
+    skip / no-skip modes against each other."""
+    torch.manual_seed(7)
+    B, H, Sq, Sk, D = 8, 32, 256, 320, 128
+    Q = torch.randn(B, H, Sq, D).to(torch.bfloat16)
+    K = torch.randn(B, H, Sk, D).to(torch.bfloat16)
+    V = torch.randn(B, H, Sk, D).to(torch.bfloat16)
+    mask = _mask(kind, Sq, Sk)
+    md = None if mask is None else mask.to(dev)
+    scale = 1 / np.sqrt(D)
+    out = gc.mha_fwd_bf16(Q.to(dev), K.to(dev), V.to(dev), md, scale)
+    out2 = gc.mha_fwd_bf16(Q.to(dev), K.to(dev), V.to(dev), md, scale, skip_masked=False)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+    for (b, h) in [(0, 0), (3, 17), (7, 31)]:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q[sl]), wl.bf16_bits(K[sl]), wl.bf16_bits(V[sl]),
+                                           None if mask is None else mask.numpy(), scale))
+        assert_close(ref, out[sl].float().cpu().numpy(), 1e-2, "wide %s (%d,%d)" % (kind, b, h),
+                     mag=_pv_mag(Q[sl], K[sl], V[sl], mask, scale))
