@@ -101,6 +101,8 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the 4096^3 GEMM the CPU baseline computes")
     ap.add_argument("--mha-mode", default="both", choices=["both", "skip", "every"],
                     help="attention: time the default entry point (masked key blocks skipped), the every-block mode, or both")
+    ap.add_argument("--no-vendor", action="store_true",
+                    help="skip the torch.mm (hipBLASLt) / torch SDPA timings reported under others.vendor_libraries")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch three 1 GiB device copies (known traffic: 1 GiB read + 1 GiB written each) so that "
                          "FETCH_SIZE / WRITE_SIZE counter readings of the other kernels can be scaled")
@@ -231,6 +233,34 @@ def main():
         others["f32_matmul_bias_relu"] = {"workload": "A[128x512].B[512x256]+bias+ReLU f32 (launch bound)",
                                           "ms_per_step": round(t["ms_per_step"], 5),
                                           "value": round(2.0 * 128 * 512 * 256 / t["kernel_ms_mean"] / 1e9, 4), "unit": "TFLOP/s"}
+
+    # ---------------- the vendor libraries on the same shapes, same process, same timing code (context only)
+    if not args.no_vendor and not only:
+        import torch.nn.functional as F
+        vend = {}
+        sets = []
+        for s in range(4):
+            A, B = wl.bf16_gemm(seed=10 * s)
+            sets.append((A.to(dev), B.to(dev), torch.empty(M, N, device=dev, dtype=torch.bfloat16)))
+        t = time_launches(torch, lambda i: torch.mm(sets[i][0], sets[i][1], out=sets[i][2]), 4, K, W)
+        vend["torch_mm_bf16_4096"] = {"kernel_ms_mean": round(t["kernel_ms_mean"], 5),
+                                      "value": round(flops / t["kernel_ms_mean"] / 1e9, 1), "unit": "TFLOP/s"}
+        del sets
+        Q, Kk, V, mask, scale = wl.bf16_mha(seed=0)
+        Qv, Kv, Vv = Q.to(dev), Kk.to(dev), V.to(dev)
+        mops = 4.0 * 4 * 32 * 2048 * 2048 * 128
+        try:
+            t = time_launches(torch, lambda i: F.scaled_dot_product_attention(Qv, Kv, Vv, is_causal=True, scale=scale), 1,
+                              max(10, K // 4), 5)
+            vend["torch_sdpa_is_causal"] = {"kernel_ms_mean": round(t["kernel_ms_mean"], 5),
+                                            "value": round(mops / t["kernel_ms_mean"] / 1e9, 1),
+                                            "unit": "TFLOP/s (dense count)"}
+        except Exception as e:  # the library may lack a kernel for this build
+            vend["torch_sdpa_is_causal"] = {"error": str(e)[:120]}
+        others["vendor_libraries"] = vend
+        log("vendor libraries: %s" % json.dumps(vend))
+        del Qv, Kv, Vv
+        torch.cuda.empty_cache()
 
     # ---------------- the same GEMM through dnnl_graph_compiler_execute (the drop-in boundary)
     if want("api"):
