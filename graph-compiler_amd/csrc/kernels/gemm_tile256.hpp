@@ -42,6 +42,12 @@ namespace gcmi {
 static constexpr int G_BM = 256, G_BN = 256, G_KBYTES = 128;
 static constexpr int G_THREADS = 512;
 static constexpr int G_STAGE_BYTES = 65536; // A 32 KiB + B 32 KiB
+#ifndef G_FAST_WJ
+// wave layout of the fast path: 2 = 8 waves of 128 x 64 (two per SIMD), 4 = 4 waves of 128 x 128 (one per
+// SIMD, a third less LDS read traffic).  Measured on MI355X: the 4-wave layout is 5-7 % slower on bf16
+// 4096^3 / 8192^3 and 19 % slower on the int8 MLP layer (nothing overlaps its epilogue), so 2 it is.
+#define G_FAST_WJ 2
+#endif
 #ifndef G_FAST_KS
 #define G_FAST_KS 2 // MFMA k-steps per LDS stage of the fast path: 2 (4-stage ring) or 4 (2-stage ring)
 #endif
@@ -138,17 +144,20 @@ template <int ACT> __device__ __forceinline__ float act_const(float x) { return 
 static constexpr int G_STG_PITCH = 144;
 static constexpr int G_STG_WAVE_BYTES = 128 * G_STG_PITCH; // 18 KiB per wave
 
-template <int ES, bool EDGE, int ACT, bool STAGED>
-__device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[2][4],
+// WJ = MFMA tiles along n per wave: 2 (8 waves as 2 x 4, wave tile 128 x 64) or 4
+// (4 waves as 2 x 2, wave tile 128 x 128).
+template <int ES, bool EDGE, int ACT, bool STAGED, int WJ = 2>
+__device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[WJ][4],
                                                   int64_t m0, int64_t n0, int wm, int wn, int l32, int lh,
                                                   char *stg) {
+  constexpr int PITCH = 64 * WJ + 16; // staging row: 32*WJ bf16 + 16 bytes of padding
   const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
   char *Cb = reinterpret_cast<char *>(p.C);
-  static_for<0, 2>([&](auto jc) {
+  static_for<0, WJ>([&](auto jc) {
     constexpr int j = decltype(jc)::value;
     static_for<0, 4>([&](auto qc) {
       constexpr int q = decltype(qc)::value;
-      const int64_t n = n0 + wn * 64 + j * 32 + 8 * q + 4 * lh;
+      const int64_t n = n0 + wn * (32 * WJ) + j * 32 + 8 * q + 4 * lh;
       float bias4[4] = {0.f, 0.f, 0.f, 0.f}, scale4[4] = {1.f, 1.f, 1.f, 1.f};
       int cs4[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -211,7 +220,7 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
           }
         }
         if (STAGED) {
-          *reinterpret_cast<uint2 *>(stg + (i * 32 + l32) * G_STG_PITCH + j * 64 + q * 16 + lh * 8) =
+          *reinterpret_cast<uint2 *>(stg + (i * 32 + l32) * PITCH + j * 64 + q * 16 + lh * 8) =
               make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
           return;
         }
@@ -240,36 +249,37 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
     // wave-private region: only this wave's own LDS writes have to land
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     const int lane = lh * 32 + l32;
-    const int r8 = lane >> 3, c8 = lane & 7;
+    constexpr int LPR = 4 * WJ, RPP = 64 / LPR; // lanes per row (16 B each), rows per pass
+    const int rr = lane / LPR, cc = lane % LPR;
 #pragma unroll
-    for (int it = 0; it < 16; it++) {
-      const int row = it * 8 + r8;
-      uint4 v = *reinterpret_cast<const uint4 *>(stg + row * G_STG_PITCH + c8 * 16);
+    for (int it = 0; it < 128 / RPP; it++) {
+      const int row = it * RPP + rr;
+      uint4 v = *reinterpret_cast<const uint4 *>(stg + row * PITCH + cc * 16);
       typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
       u32x4_t vv = {v.x, v.y, v.z, v.w};
-      __builtin_nontemporal_store(vv, reinterpret_cast<u32x4_t *>(Cb + ((m0 + wm * 128 + row) * p.ldc + n0 + wn * 64 + c8 * 8) * 2));
+      __builtin_nontemporal_store(vv, reinterpret_cast<u32x4_t *>(Cb + ((m0 + wm * 128 + row) * p.ldc + n0 + wn * (32 * WJ) + cc * 8) * 2));
     }
   }
 }
 
-template <int ES, bool EDGE, bool STAGED>
-__device__ __forceinline__ void gemm_epilogue(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[2][4], int64_t m0,
+template <int ES, bool EDGE, bool STAGED, int WJ = 2>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[WJ][4], int64_t m0,
                                               int64_t n0, int wm, int wn, int l32, int lh, char *stg) {
   switch (p.act) {
   case ACT_RELU:
-    gemm_epilogue_act<ES, EDGE, ACT_RELU, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_RELU, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   case ACT_GELU_ERF:
-    gemm_epilogue_act<ES, EDGE, ACT_GELU_ERF, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_ERF, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   case ACT_GELU_TANH:
-    gemm_epilogue_act<ES, EDGE, ACT_GELU_TANH, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_TANH, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   case ACT_SIGMOID:
-    gemm_epilogue_act<ES, EDGE, ACT_SIGMOID, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_SIGMOID, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   default:
-    gemm_epilogue_act<ES, EDGE, ACT_NONE, STAGED>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_NONE, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
     break;
   }
 }
@@ -429,7 +439,8 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
 //  * The stage loop is unrolled over the ring, so every LDS address is static.
 #define GCMI_GLB __attribute__((address_space(1)))
 
-template <int ES, int KS> struct FastGemm {
+template <int ES, int KS, int WJ = 2> struct FastGemm {
+  static constexpr int NWAVES = 16 / WJ; // 8 or 4
   typedef MfmaOp<ES> Op;
   typedef typename Op::acc_t acc_t;
   static constexpr int NST = 8 / KS;                  // stages in the LDS ring
@@ -444,12 +455,12 @@ template <int ES, int KS> struct FastGemm {
   static constexpr int CW = ES == 2 ? 4 : 2;
   static constexpr int B_ROWS_PER_DMA = 1024 / B_ROW_BYTES; // 2 (bf16) or 4 (int8)
   static constexpr int B_CPR = B_ROW_BYTES / 16;
-  static constexpr int NDMA = KS;                     // DMA instructions per operand per wave per stage
+  static constexpr int NDMA = KS * 8 / NWAVES;        // DMA instructions per operand per wave per stage
 
   static __device__ __forceinline__ int a_swz(int row) { return KS == 4 ? ((row >> 1) & 7) : ((row >> 2) & 3); }
 
   uint32_t a_src[NDMA], b_src[NDMA]; // per-lane byte offsets of this wave's DMA instructions
-  uint32_t a_ld[KS], b_ld[2];        // fragment read offsets
+  uint32_t a_ld[KS], b_ld[WJ];       // fragment read offsets
   uint32_t a_xor;
   int wave_u; // wave id, wave-uniform
 
@@ -464,7 +475,7 @@ template <int ES, int KS> struct FastGemm {
                                        (GCMI_LDS void *)(stage + A_BYTES + (wave_u * NDMA + i) * 1024), 16, 0, 0);
   }
 
-  __device__ __forceinline__ void load_frags(const char *__restrict__ s, int ks, uint4 (&af)[4], uint4 (&bf)[2]) const {
+  __device__ __forceinline__ void load_frags(const char *__restrict__ s, int ks, uint4 (&af)[4], uint4 (&bf)[WJ]) const {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       uint4 v = *reinterpret_cast<const uint4 *>(s + a_ld[ks] + i * 32 * KB);
@@ -473,16 +484,16 @@ template <int ES, int KS> struct FastGemm {
       af[i] = v;
     }
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int j = 0; j < WJ; j++) {
       uint2 lo = Op::tr_read(s + b_ld[j] + ks * 8192);
       uint2 hi = Op::tr_read(s + b_ld[j] + ks * 8192 + 2048);
       bf[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
     }
   }
 
-  static __device__ __forceinline__ void mfma_all(acc_t (&acc)[2][4], const uint4 (&af)[4], const uint4 (&bf)[2]) {
+  static __device__ __forceinline__ void mfma_all(acc_t (&acc)[WJ][4], const uint4 (&af)[4], const uint4 (&bf)[WJ]) {
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < WJ; j++)
 #pragma unroll
       for (int i = 0; i < 4; i++)
         acc[j][i] = Op::run(bf[j], af[i], acc[j][i]);
@@ -491,7 +502,7 @@ template <int ES, int KS> struct FastGemm {
   // ask the scheduler for MFMA, DS read, MFMA, DS read, ... over the region
   static __device__ __forceinline__ void interleave_hint() {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < 4 * WJ; i++) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // 1 DS read
     }
@@ -509,8 +520,8 @@ template <int ES, int KS> struct FastGemm {
   // k-block kt+1, behind which BEHIND more blocks are in flight.
   template <bool HAS_FILL, bool HAS_NEXT, int BEHIND>
   __device__ __forceinline__ void stage(char *__restrict__ cur, char *__restrict__ nxt, char *__restrict__ fill,
-                                        const char *a_fill, const char *b_fill, acc_t (&acc)[2][4], uint4 (&a0)[4],
-                                        uint4 (&b0)[2], uint4 (&a1)[4], uint4 (&b1)[2]) const {
+                                        const char *a_fill, const char *b_fill, acc_t (&acc)[WJ][4], uint4 (&a0)[4],
+                                        uint4 (&b0)[WJ], uint4 (&a1)[4], uint4 (&b1)[WJ]) const {
     if (HAS_FILL)
       issue_loads(fill, a_fill, b_fill);
 #pragma unroll
@@ -537,8 +548,9 @@ template <int ES, int KS> struct FastGemm {
   }
 };
 
-template <int ES, int KS> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_fast_kernel(GemmParams p) {
-  typedef FastGemm<ES, KS> FG;
+template <int ES, int KS, int WJ>
+__global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmParams p) {
+  typedef FastGemm<ES, KS, WJ> FG;
   typedef typename FG::acc_t acc_t;
   constexpr int NST = FG::NST;
   // ring of NST stages (128 KiB); the epilogue reuses the whole array as 8 x 18 KiB staging regions
@@ -547,7 +559,7 @@ template <int ES, int KS> __global__ __launch_bounds__(G_THREADS) void gemm_tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = WJ == 2 ? wave >> 2 : wave >> 1, wn = WJ == 2 ? wave & 3 : wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
 
   const int tiles_m = (int)(p.M / G_BM), tiles_n = (int)(p.N / G_BN);
@@ -580,17 +592,18 @@ template <int ES, int KS> __global__ __launch_bounds__(G_THREADS) void gemm_tile
     const int kk = ES == 2 ? (i16 >> 2) : (i16 >> 1);
     const int cc = ES == 2 ? (i16 & 3) : (i16 & 1);
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      int chunk = ES == 2 ? (wn * 8 + j * 4 + 2 * (gq & 1) + (cc >> 1)) : (wn * 4 + j * 2 + (gq & 1));
+    for (int j = 0; j < WJ; j++) {
+      const int nb = wn * WJ + j; // 32-column block of the tile
+      int chunk = ES == 2 ? (nb * 4 + 2 * (gq & 1) + (cc >> 1)) : (nb * 2 + (gq & 1));
       int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
       int krow_lane = (ES == 2 ? 8 : 16) * (gq >> 1) + kk;
       g.b_ld[j] = FG::A_BYTES + krow_lane * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + sub;
     }
   }
 
-  acc_t acc[2][4];
+  acc_t acc[WJ][4];
 #pragma unroll
-  for (int j = 0; j < 2; j++)
+  for (int j = 0; j < WJ; j++)
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -602,7 +615,7 @@ template <int ES, int KS> __global__ __launch_bounds__(G_THREADS) void gemm_tile
   const int64_t b_step = (int64_t)FG::BK * ldb_b;
   const int KT = (int)(p.K / FG::BK);
 
-  uint4 a0[4], b0[2], a1[4], b1[2];
+  uint4 a0[4], b0[WJ], a1[4], b1[WJ];
   // prologue: request k-blocks 0 .. NST-2 (KT is a positive multiple of NST), wait for block 0
 #pragma unroll
   for (int d = 0; d < NST - 1; d++)
@@ -637,9 +650,9 @@ template <int ES, int KS> __global__ __launch_bounds__(G_THREADS) void gemm_tile
   // no wave reads fragments any more (the last stage's barrier came after its
   // final fragment reads), so the stage buffers can be overwritten
   if (p.out_dt == DT_BF16)
-    gemm_epilogue<ES, false, true>(p, acc, m0, n0, wm, wn, l32, lh, smem + wave * G_STG_WAVE_BYTES);
+    gemm_epilogue<ES, false, true, WJ>(p, acc, m0, n0, wm, wn, l32, lh, smem + wave * (128 * (64 * WJ + 16)));
   else
-    gemm_epilogue<ES, false, false>(p, acc, m0, n0, wm, wn, l32, lh, nullptr);
+    gemm_epilogue<ES, false, false, WJ>(p, acc, m0, n0, wm, wn, l32, lh, nullptr);
 }
 
 // Host-side launch of the 256x256 tile kernels for one element size.
@@ -661,7 +674,7 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
     p.group_m = 4;
   dim3 grid((unsigned)nblk), block(G_THREADS);
   if (fast)
-    hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ>), grid, dim3(1024 / G_FAST_WJ), 0, stream, p);
   else
     hipLaunchKernelGGL((gemm_tile256_kernel<ES, true>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 5;
