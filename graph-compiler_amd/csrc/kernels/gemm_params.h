@@ -19,6 +19,11 @@ struct GemmParams {
   int32_t out_dt;        // gcmi::DType of C
   int32_t bias_dt;       // gcmi::DType of bias
   int32_t group_m;       // tile-order group height (XCD/L2 locality), 0 = default
+  // split-K (set by the launcher; one tile row, M <= 256): workgroup b takes tile b % tiles and K slice b / tiles,
+  // and writes its f32 partial sums [M x N] to partial + slice * M * N; a second kernel sums the slices and
+  // runs the epilogue
+  int32_t splits;        // 0 or 1: off
+  float *partial;
 };
 
 struct F32GemmParams {

@@ -439,8 +439,11 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
 //  * The stage loop is unrolled over the ring, so every LDS address is static.
 #define GCMI_GLB __attribute__((address_space(1)))
 
-template <int ES, int KS, int WJ = 2> struct FastGemm {
+// SPLIT (split-K on a short A): only the first `mi` 32-row tiles of a wave hold rows of A; the others are
+// neither read from LDS nor multiplied.
+template <int ES, int KS, int WJ = 2, bool SPLIT = false> struct FastGemm {
   static constexpr int NWAVES = 16 / WJ; // 8 or 4
+  int mi = 4;
   typedef MfmaOp<ES> Op;
   typedef typename Op::acc_t acc_t;
   static constexpr int NST = 8 / KS;                  // stages in the LDS ring
@@ -476,8 +479,12 @@ template <int ES, int KS, int WJ = 2> struct FastGemm {
   }
 
   __device__ __forceinline__ void load_frags(const char *__restrict__ s, int ks, uint4 (&af)[4], uint4 (&bf)[WJ]) const {
+    if (SPLIT && mi == 0)
+      return;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
+      if (SPLIT && i >= mi)
+        break;
       uint4 v = *reinterpret_cast<const uint4 *>(s + a_ld[ks] + i * 32 * KB);
       if (ES == 1) // u8 activations: a - 128 as s8 == a ^ 0x80
         v = make_uint4(v.x ^ a_xor, v.y ^ a_xor, v.z ^ a_xor, v.w ^ a_xor);
@@ -491,16 +498,19 @@ template <int ES, int KS, int WJ = 2> struct FastGemm {
     }
   }
 
-  static __device__ __forceinline__ void mfma_all(acc_t (&acc)[WJ][4], const uint4 (&af)[4], const uint4 (&bf)[WJ]) {
+  __device__ __forceinline__ void mfma_all(acc_t (&acc)[WJ][4], const uint4 (&af)[4], const uint4 (&bf)[WJ]) const {
 #pragma unroll
     for (int j = 0; j < WJ; j++)
 #pragma unroll
       for (int i = 0; i < 4; i++)
-        acc[j][i] = Op::run(bf[j], af[i], acc[j][i]);
+        if (!SPLIT || i < mi)
+          acc[j][i] = Op::run(bf[j], af[i], acc[j][i]);
   }
 
   // ask the scheduler for MFMA, DS read, MFMA, DS read, ... over the region
   static __device__ __forceinline__ void interleave_hint() {
+    if (SPLIT)
+      return;
 #pragma unroll
     for (int i = 0; i < 4 * WJ; i++) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
@@ -548,9 +558,9 @@ template <int ES, int KS, int WJ = 2> struct FastGemm {
   }
 };
 
-template <int ES, int KS, int WJ>
+template <int ES, int KS, int WJ, bool SPLIT = false>
 __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmParams p) {
-  typedef FastGemm<ES, KS, WJ> FG;
+  typedef FastGemm<ES, KS, WJ, SPLIT> FG;
   typedef typename FG::acc_t acc_t;
   constexpr int NST = FG::NST;
   // ring of NST stages (128 KiB); the epilogue reuses the whole array as 8 x 18 KiB staging regions
@@ -562,21 +572,33 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
   const int wm = WJ == 2 ? wave >> 2 : wave >> 1, wn = WJ == 2 ? wave & 3 : wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  const int tiles_m = (int)(p.M / G_BM), tiles_n = (int)(p.N / G_BN);
-  int tm, tn;
-  tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
+  const int tiles_m = (int)((p.M + G_BM - 1) / G_BM), tiles_n = (int)(p.N / G_BN);
+  int tm, tn, slice = 0;
+  if (SPLIT) { // one tile row: tile = column block, K slice = blockIdx / tiles
+    tm = 0;
+    tn = (int)blockIdx.x % tiles_n;
+    slice = (int)blockIdx.x / tiles_n;
+  } else {
+    tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
+  }
   const int64_t m0 = (int64_t)tm * G_BM, n0 = (int64_t)tn * G_BN;
   const int64_t lda_b = p.lda * ES, ldb_b = p.ldb * ES;
 
   FG g;
   g.wave_u = wave;
+  if (SPLIT) { // 32-row tiles of this wave that hold rows of A
+    const int64_t left = p.M - m0 - wm * 128;
+    g.mi = left <= 0 ? 0 : (int)min((int64_t)4, (left + 31) / 32);
+  }
   g.a_xor = p.a_xor;
 #pragma unroll
   for (int i = 0; i < FG::NDMA; i++) {
     // A: this instruction fills 1 KiB = A_ROWS_PER_DMA rows; lane -> (row, physical chunk)
     int row = (wave * FG::NDMA + i) * FG::A_ROWS_PER_DMA + lane / FG::A_CPR;
     int c = (lane % FG::A_CPR) ^ FG::a_swz(row);
-    g.a_src[i] = (uint32_t)(row * lda_b + c * 16);
+    // rows past M (split-K on a short A): fetch the last row instead, its results are dropped
+    const int row_src = (int)min((int64_t)row, p.M - 1 - m0);
+    g.a_src[i] = (uint32_t)(row_src * lda_b + c * 16);
     // B: B_ROWS_PER_DMA k-rows; lane -> (krow, physical chunk)
     int krow = (wave * FG::NDMA + i) * FG::B_ROWS_PER_DMA + lane / FG::B_CPR;
     int cb = (lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW);
@@ -610,10 +632,13 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
       for (int r = 0; r < 16; r++)
         acc[j][i][r] = 0;
 
-  const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b; // k-block 0; KB bytes per k-block
-  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * ES;    // k-block 0; BK rows per k-block
   const int64_t b_step = (int64_t)FG::BK * ldb_b;
-  const int KT = (int)(p.K / FG::BK);
+  // K slice of this workgroup in ring groups (NST stages each): slices differ by at most one group
+  const int groups = (int)(p.K / FG::BK) / NST, nsl = SPLIT ? p.splits : 1;
+  const int g0 = (int)((int64_t)slice * groups / nsl), g1 = (int)((int64_t)(slice + 1) * groups / nsl);
+  const int KT = (g1 - g0) * NST;
+  const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b + (int64_t)g0 * NST * FG::KB; // first k-block; KB bytes each
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * ES + (int64_t)g0 * NST * b_step;   // BK rows per k-block
 
   uint4 a0[4], b0[WJ], a1[4], b1[WJ];
   // prologue: request k-blocks 0 .. NST-2 (KT is a positive multiple of NST), wait for block 0
@@ -649,11 +674,95 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
 
   // no wave reads fragments any more (the last stage's barrier came after its
   // final fragment reads), so the stage buffers can be overwritten
+  if constexpr (SPLIT) {
+    // f32 partial sums of the rows that exist, 16 bytes per lane (4 consecutive n of one m)
+    float *part = p.partial + (int64_t)slice * p.M * p.N;
+    static_for<0, WJ>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      static_for<0, 4>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        const int64_t m = m0 + wm * 128 + i * 32 + l32;
+        if (m < p.M) {
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const int64_t n = n0 + wn * (32 * WJ) + j * 32 + 8 * q + 4 * lh;
+            f32x4_t v = {(float)acc[j][i][4 * q], (float)acc[j][i][4 * q + 1], (float)acc[j][i][4 * q + 2],
+                         (float)acc[j][i][4 * q + 3]};
+            *reinterpret_cast<f32x4_t *>(part + m * p.N + n) = v;
+          }
+        }
+      });
+    });
+    return; // the sum over slices and the epilogue are the second kernel's (a kernel boundary is the cheapest
+            // way to make partial sums visible across XCDs: device-scope fences write back and invalidate whole L2s)
+  }
   if (p.out_dt == DT_BF16)
     gemm_epilogue<ES, false, true, WJ>(p, acc, m0, n0, wm, wn, l32, lh, smem + wave * (128 * (64 * WJ + 16)));
   else
     gemm_epilogue<ES, false, false, WJ>(p, acc, m0, n0, wm, wn, l32, lh, nullptr);
 }
+
+// Second pass of split-K: out = epilogue(sum over slices of the f32 partials), slices added in ascending
+// order (deterministic), the same rounding points as the fused epilogue.  One thread per 4 columns; the
+// loads of eight slices are in flight together.
+template <int ACT> __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmParams p) {
+  const int64_t n4 = p.N / 4, idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.M * n4)
+    return;
+  const int64_t m = idx / n4, n = (idx % n4) * 4, sl = p.M * p.N;
+  const float *src = p.partial + m * p.N + n;
+  f32x4_t a = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = 0; s0 < p.splits; s0 += 8) {
+    f32x4_t b[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++)
+      b[u] = s0 + u < p.splits ? *reinterpret_cast<const f32x4_t *>(src + (s0 + u) * sl) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < 8; u++)
+      if (s0 + u < p.splits) {
+        if (s0 + u == 0)
+          a = b[u];
+        else
+          a[0] += b[u][0], a[1] += b[u][1], a[2] += b[u][2], a[3] += b[u][3];
+      }
+  }
+  float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+  if (p.bias) {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      bias4[e] = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n + e])
+                                      : reinterpret_cast<const float *>(p.bias)[n + e];
+  }
+  uint16_t o16[4];
+  float o32[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    float x = a[e];
+    if (p.out_dt == DT_BF16) { // bf16 graph: round after the matmul and after every bf16 op
+      x = round_bf16(x);
+      if (p.bias)
+        x = round_bf16(x + bias4[e]);
+      if (ACT != ACT_NONE)
+        x = round_bf16(act_const<ACT>(x));
+    } else {
+      if (p.bias)
+        x = x + bias4[e];
+      x = act_const<ACT>(x);
+    }
+    o32[e] = x;
+    o16[e] = f32_to_bf16_bits(x);
+  }
+  if (p.out_dt == DT_BF16)
+    *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.C) + m * p.ldc + n) =
+        make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
+  else
+    *reinterpret_cast<f32x4_t *>(reinterpret_cast<float *>(p.C) + m * p.ldc + n) = f32x4_t{o32[0], o32[1], o32[2], o32[3]};
+}
+
+// Workspace of the split-K partial sums.  One copy per device, shared by all calls: calls on different
+// streams of one device must not overlap.
+static constexpr int64_t G_SPLITK_WS_FLOATS = (int64_t)8 << 20; // 32 MiB
+static __device__ __align__(256) float gemm_splitk_ws[G_SPLITK_WS_FLOATS];
 
 // Host-side launch of the 256x256 tile kernels for one element size.
 template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t stream) {
@@ -667,9 +776,51 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   const int BK = G_KBYTES / ES;
   // fast path: whole tiles, 16-byte aligned rows, and a tile's rows reachable with 32-bit byte offsets
   const int KGROUP = 256 / ES; // K elements of one trip round the LDS ring
-  bool fast = p.M % G_BM == 0 && p.N % G_BN == 0 && p.K % KGROUP == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
-              (p.lda * ES) % 16 == 0 && (p.ldb * ES) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
-              p.lda * ES * G_BM < (int64_t)1 << 31 && p.ldb * ES * BK < (int64_t)1 << 31;
+  const bool fast_but_m = p.N % G_BN == 0 && p.K % KGROUP == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
+                          (p.lda * ES) % 16 == 0 && (p.ldb * ES) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
+                          p.lda * ES * G_BM < (int64_t)1 << 31 && p.ldb * ES * BK < (int64_t)1 << 31;
+  bool fast = fast_but_m && p.M % G_BM == 0;
+  p.splits = 0;
+  p.partial = nullptr;
+  // One tile row and too few column tiles to fill the GPU (decode-style shapes such as 32 x 4096 x 4096): the
+  // weights have to stream from HBM through all compute units, so K is cut into slices, one workgroup per
+  // (column tile, slice); partial sums go through the workspace and a small second kernel.
+  if (ES == 2 && fast_but_m && tiles_m == 1 && p.out_dt != DT_S32) {
+    const int n_cu = gcmi_num_cus();
+    const int groups = (int)(p.K / KGROUP);
+    int splits = (n_cu + tiles_n - 1) / tiles_n;
+    splits = splits < groups ? splits : groups;
+    while (splits > 1 && (int64_t)splits * p.M * p.N > G_SPLITK_WS_FLOATS)
+      splits--;
+    if (splits > 1 && tiles_n * 2 <= n_cu) {
+      float *ws = nullptr;
+      if (hipGetSymbolAddress((void **)&ws, HIP_SYMBOL(gemm_splitk_ws)) != hipSuccess)
+        return 5;
+      p.splits = splits;
+      p.partial = ws;
+      hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true>), dim3((unsigned)(tiles_n * splits)),
+                         dim3(1024 / G_FAST_WJ), 0, stream, p);
+      const unsigned rblocks = (unsigned)((p.M * (p.N / 4) + 255) / 256);
+      switch (p.act) {
+      case ACT_RELU:
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_RELU>, dim3(rblocks), dim3(256), 0, stream, p);
+        break;
+      case ACT_GELU_ERF:
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_GELU_ERF>, dim3(rblocks), dim3(256), 0, stream, p);
+        break;
+      case ACT_GELU_TANH:
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_GELU_TANH>, dim3(rblocks), dim3(256), 0, stream, p);
+        break;
+      case ACT_SIGMOID:
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_SIGMOID>, dim3(rblocks), dim3(256), 0, stream, p);
+        break;
+      default:
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_NONE>, dim3(rblocks), dim3(256), 0, stream, p);
+        break;
+      }
+      return hipGetLastError() == hipSuccess ? 0 : 5;
+    }
+  }
   if (p.group_m <= 0)
     p.group_m = 4;
   dim3 grid((unsigned)nblk), block(G_THREADS);

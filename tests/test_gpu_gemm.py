@@ -184,3 +184,34 @@ def test_gelu_erf_epilogue_absolute_accuracy(gc, dev):
     ref = 0.5 * xd * (1 + erf(xd * 0.7071067811865476))
     assert np.abs(out - ref).max() <= 1e-6 * 4  # |x| <= 8: 0.5 * 8 * 5e-7 + f32 rounding
     assert (out[xd < -5.7] == 0).all()  # erf saturates to exactly -1, as libm's does
+
+
+@pytest.mark.parametrize("M,N,K,act,with_bias,out_f32", [(32, 4096, 4096, None, False, False), (1, 4096, 4096, "relu", True, False),
+                                                         (100, 11008, 4096, "gelu_erf", True, False),
+                                                         (32, 4096, 11008, None, True, True), (256, 2048, 1024, "sigmoid", False, False),
+                                                         (7, 256, 128, None, False, False)])
+def test_short_a_takes_split_k(gc, orc, wl, dev, M, N, K, act, with_bias, out_f32):
+    """One tile row of A (M <= 256) against a wide weight: the K range is cut over workgroups and the f32
+    partial sums are reduced by a second kernel.  Same rounding points as the one-pass kernel."""
+    torch.manual_seed(M + N)
+    A = (torch.randn(M, K) * 0.5).to(torch.bfloat16)
+    torch.manual_seed(K)
+    B = (torch.randn(K, N) * 0.05).to(torch.bfloat16)
+    torch.manual_seed(3)
+    bias = torch.randn(N).to(torch.bfloat16) if with_bias else None
+    out = gc.gemm_bf16(A.to(dev), B.to(dev), None if bias is None else bias.to(dev), act,
+                       out_dtype=gc.F32 if out_f32 else gc.BF16)
+    torch.cuda.synchronize()
+    if out_f32:
+        ref = A.float().double() @ B.float().double()
+        if bias is not None:
+            ref = ref + bias.double()
+        assert_close(ref.float().numpy(), out.cpu().numpy(), 1e-4, "split-k f32 out")
+    else:
+        ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B), None if bias is None else wl.bf16_bits(bias), act))
+        mm = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B)))
+        assert_close(ref, out.float().cpu().numpy(), 2e-2 if (with_bias or act) else 1e-2, "split-k", mag=mm)
+    again = gc.gemm_bf16(A.to(dev), B.to(dev), None if bias is None else bias.to(dev), act,
+                         out_dtype=gc.F32 if out_f32 else gc.BF16)
+    torch.cuda.synchronize()
+    assert torch.equal(out, again)  # fixed summation order: reruns agree bit for bit
