@@ -97,7 +97,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32,api")
+    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32,decode,api")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the 4096^3 GEMM the CPU baseline computes")
     ap.add_argument("--mha-mode", default="both", choices=["both", "skip", "every"],
                     help="attention: time the default entry point (masked key blocks skipped), the every-block mode, or both")
@@ -223,6 +223,30 @@ def main():
         others["bf16_mha"] = entry
         del sets
         torch.cuda.empty_cache()
+
+    # ---------------- decode-style GEMM: 32 rows against Llama-7B FFN weights (split-K path, HBM bound)
+    if want("decode"):
+        dec = {}
+        for (Md, Nd, Kdd) in [(32, 4096, 4096), (32, 11008, 4096), (32, 4096, 11008)]:
+            nsets = 4  # 4 x 32..90 MB of weights: beyond the Infinity Cache in rotation
+            sets = []
+            for s in range(nsets):
+                torch.manual_seed(100 + s)
+                sets.append(((torch.randn(Md, Kdd) * 0.1).to(torch.bfloat16).to(dev),
+                             (torch.randn(Kdd, Nd) * 0.02).to(torch.bfloat16).to(dev),
+                             torch.empty(Md, Nd, device=dev, dtype=torch.bfloat16)))
+            t = time_launches(torch, lambda i: gc.gemm_bf16(sets[i][0], sets[i][1], out=sets[i][2]), nsets, K, W)
+            byts = 2.0 * (Md * Kdd + Kdd * Nd + Md * Nd)
+            gbs = byts / (t["kernel_ms_mean"] * 1e-3) / 1e9
+            dec["%dx%dx%d" % (Md, Nd, Kdd)] = {
+                "ms_per_step": round(t["ms_per_step"], 5), "kernel_ms_mean": round(t["kernel_ms_mean"], 5),
+                "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
+            log("bf16 decode gemm %dx%dx%d: %.4f ms  %.0f GB/s of operands" % (Md, Nd, Kdd, t["kernel_ms_mean"], gbs))
+            del sets
+            torch.cuda.empty_cache()
+        others["bf16_decode_gemm"] = {"workload": "A[32 x K] . W[K x N] bf16, two launches (K slices, then reduction + epilogue); "
+                                                  "algorithmic bytes = A + W + C once", "shapes": dec}
 
     # ---------------- f32 plumbing case (configs[0])
     if want("f32"):

@@ -46,6 +46,11 @@ const char *gcmi_last_error(void);
  * activation (lib/gc/Transforms/Pipeline.cpp:79-95).  out_dtype GCMI_F32: no
  * intermediate rounding.  bias: [N] of bias_dtype (GCMI_BF16 or GCMI_F32) or
  * NULL.
+ * When A has at most 256 rows and N is narrow (fewer column tiles than half the
+ * compute units), K is cut into slices over workgroups and a second kernel adds
+ * the f32 partial sums in a fixed order (results do not vary from run to run).
+ * The partial sums live in a 32 MiB per-device static buffer: such calls on
+ * different streams of one device must not overlap.
  */
 int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                    int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
