@@ -446,7 +446,9 @@ void Executable::plan() {
       DT out_dt = T(mm.out[0]).dt;
       if (A.dt == DT::bf16 && (tA || tB)) {
         // the bf16 kernel reads row-major [M,K] and [K,N]: materialise the transposes
-        auto transposed = [&](int slot, std::vector<int64_t> &shp) {
+        // (once per executable when the operand is a constant: the analogue of the reference's weight
+        // pre-packing of constant tensors, docs/CPU_pipeline_overview.md:58)
+        auto transposed = [&](int slot, std::vector<int64_t> &shp, bool constant) {
           std::vector<int64_t> st = dense_strides(shp), d = shp;
           std::swap(d[d.size() - 1], d[d.size() - 2]);
           std::swap(st[st.size() - 1], st[st.size() - 2]);
@@ -454,16 +456,17 @@ void Executable::plan() {
           if (d.size() > (size_t)gcmi::ELT_MAX_RANK)
             throw std::logic_error("tensor rank above 6 is not supported");
           Step cp;
-          cp.kind = Step::Elt, cp.note = "transpose copy", cp.op = gcmi::ELT_COPY, cp.a = slot, cp.out = t;
+          cp.kind = Step::Elt, cp.note = constant ? "transpose copy, once: the operand is constant" : "transpose copy";
+          cp.once = constant, cp.op = gcmi::ELT_COPY, cp.a = slot, cp.out = t;
           cp.a_dt = cp.out_dt = GCMI_BF16, cp.dims = d, cp.sa = st;
           v.push_back(cp);
           shp = d;
           return t;
         };
         if (tA)
-          sa_slot = transposed(sa_slot, as), tA = false;
+          sa_slot = transposed(sa_slot, as, A.constant), tA = false;
         if (tB)
-          sb_slot = transposed(sb_slot, bs), tB = false;
+          sb_slot = transposed(sb_slot, bs, B.constant), tB = false;
       }
       std::vector<int64_t> ba(as.begin(), as.end() - 2), bb(bs.begin(), bs.end() - 2), bo;
       broadcast_shape(ba, bb, bo);
@@ -741,10 +744,18 @@ void Executable::execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler
         slot = (int)s;
     if (slot < 0 || !t->data)
       continue;
-    if (is_device_pointer(t->data))
+    if (is_device_pointer(t->data)) {
       ptr_[(size_t)slot] = t->data;
-    else
+    } else {
+      // a constant keeps its first contents: staged once
+      const bool constant = g_.tensors.at(id).constant;
+      if (const_staged_.size() < slots_.size())
+        const_staged_.resize(slots_.size(), 0);
+      if (constant && const_staged_[(size_t)slot])
+        continue;
       hip_check(hipMemcpyAsync(ptr_[(size_t)slot], t->data, slots_[(size_t)slot].bytes, hipMemcpyHostToDevice, stream_), "stage input");
+      const_staged_[(size_t)slot] = constant;
+    }
   }
   std::vector<std::pair<void *, int>> copy_back;
   for (size_t i = 0; i < g_.output_ids.size(); i++) {
@@ -761,8 +772,14 @@ void Executable::execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler
     else
       copy_back.emplace_back(t->data, slot);
   }
-  for (auto &s : steps_)
-    launch(s);
+  if (step_done_.size() < steps_.size())
+    step_done_.resize(steps_.size(), 0);
+  for (size_t i = 0; i < steps_.size(); i++) {
+    if (steps_[i].once && step_done_[i])
+      continue;
+    launch(steps_[i]);
+    step_done_[i] = steps_[i].once;
+  }
   for (auto &cb : copy_back) {
     hipMemcpyKind kind = is_device_pointer(cb.first) ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost;
     hip_check(hipMemcpyAsync(cb.first, ptr_[(size_t)cb.second], slots_[(size_t)cb.second].bytes, kind, stream_), "copy result");

@@ -28,6 +28,7 @@ namespace gcapi {
 struct Step {
   enum Kind { GemmF32, GemmBf16, GemmInt8, ColSum, Mha, Elt, Reduce, Softmax } kind;
   std::string note; // what was fused, for introspection
+  bool once = false; // depends on constant tensors only: runs in the first execute, its result is kept
   // operands are arena slot indices (-1 = none)
   int a = -1, b = -1, c = -1, out = -1, bias = -1, mask = -1, aux = -1;
   int64_t M = 0, N = 0, K = 0, lda = 0, ldb = 0, ldc = 0;
@@ -85,6 +86,8 @@ private:
   size_t arena_bytes_ = 0;
   hipStream_t stream_ = nullptr;
   std::unordered_map<int, bool> colsum_valid_; // ColSum results of constant weights are computed once
+  std::vector<char> step_done_;                // per step: a `once` step has run
+  std::vector<char> const_staged_;             // per slot: a constant host input has been copied to the device
 
   int new_slot(size_t bytes, long tensor_id = -1);
   int slot_for(size_t tensor_id);

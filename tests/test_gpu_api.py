@@ -197,3 +197,37 @@ def test_attention_partition(ga, orc, wl, dev, D, with_mask, scale_op):
     Sd = Q.double() @ K.double().transpose(-1, -2) * scale + (mask.double() if with_mask else 0)
     mag = (torch.softmax(Sd, -1) @ V.double().abs()).numpy()
     assert_close(ref, out.float().numpy(), 1e-2, "attention partition", mag=mag)
+
+
+def test_constant_transposed_weight_is_prepared_once(ga, orc, wl, dev):
+    """x[32,512] . W^T with W stored [N,K] (transpose_b, as the reference's llama2 case stores its weights).
+    With property_type "constant" the row-major copy of W is made in the first execute only: a second execute
+    that is handed a different buffer under the same id still multiplies by the first contents.  Without the
+    property the copy is redone every time."""
+    M, K, N = 32, 512, 768
+    torch.manual_seed(21)
+    x = (torch.randn(M, K) * 0.5).to(torch.bfloat16)
+    W = (torch.randn(N, K) * 0.05).to(torch.bfloat16)
+    W2 = (torch.randn(N, K) * 0.05).to(torch.bfloat16)
+
+    def graph(prop):
+        return ga._graph([{"kind": "MatMul", "attrs": {"transpose_b": {"type": "bool", "value": 1}},
+                           "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [N, K], property_type=prop)],
+                           "outputs": [ga._t(2, "bf16", [M, N])]}], [0, 1], [2])
+
+    ref1 = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(x), wl.bf16_bits(W.t().contiguous())))
+    ref2 = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(x), wl.bf16_bits(W2.t().contiguous())))
+    for prop, second in (("constant", ref1), ("variable", ref2)):
+        comp = ga.Compiler()
+        st, exe = comp.compile(graph(prop))
+        assert st == 0, ga.api().dnnl_graph_compiler_last_error().decode()
+        st, plan = ga.explain(graph(prop))
+        assert ("once" in plan) == (prop == "constant")
+        out = torch.zeros(M, N, dtype=torch.bfloat16)
+        for Wt, ref in ((W, ref1), (W2, second)):
+            for pass_device in (False, True):
+                xs, ws = (x.to(dev), Wt.to(dev)) if pass_device else (x, Wt)
+                assert exe.execute([(0, xs), (1, ws)], [(2, out)]) == 0
+                assert_close(ref, out.float().numpy(), 1e-2, "transpose_b %s" % prop)
+        exe.close()
+        comp.close()
