@@ -131,21 +131,80 @@ void Executable::add_copy(int src, DT sdt, const std::vector<int64_t> &dims, con
 Executable::Executable(const char *json, bool dry) : g_(parse_graph(json)) {
   verify_graph(g_);
   plan();
+  layout_arena();
   if (dry)
     return;
-  // arena layout
-  size_t off = 0;
-  for (auto &s : slots_) {
-    s.offset = off;
-    off += align256(s.bytes);
-  }
-  arena_bytes_ = off ? off : 256;
   hip_check(hipMalloc((void **)&arena_, arena_bytes_), "hipMalloc(arena)");
   hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
   for (auto &s : slots_)
     if (!s.init.empty())
       hip_check(hipMemcpy(arena_ + s.offset, s.init.data(), s.init.size(), hipMemcpyHostToDevice), "upload constants");
   ptr_.resize(slots_.size());
+}
+
+// One allocation per executable, temporaries with disjoint lifetimes share memory: the tick-based merge
+// of the reference (lib/gc/Transforms/MergeAllocTickBased.cpp, docs/memref_schedule.md) with the step
+// index as the tick.  A slot lives from the first step that names it to the last; graph inputs and
+// outputs, constants and the results of once-only steps live for the whole executable.  Temporaries
+// are placed in order of their first tick at the lowest offset that is free for their whole lifetime.
+void Executable::layout_arena() {
+  const int n = (int)slots_.size();
+  std::vector<int> first(n, -1), last(n, -1);
+  std::vector<char> pinned(n, 0);
+  auto touch = [&](int slot, int tick) {
+    if (slot < 0)
+      return;
+    if (first[slot] < 0)
+      first[slot] = tick;
+    last[slot] = tick;
+  };
+  for (int i = 0; i < (int)steps_.size(); i++) {
+    const Step &s = steps_[i];
+    for (int slot : {s.a, s.b, s.c, s.out, s.bias, s.mask, s.aux, s.scale_slot, s.scales_slot, s.zps_slot})
+      touch(slot, i);
+    if (s.once || (s.kind == Step::ColSum && s.op == 1))
+      if (s.out >= 0)
+        pinned[s.out] = 1;
+  }
+  for (int i = 0; i < n; i++)
+    if (slots_[i].is_input || slots_[i].is_output || !slots_[i].init.empty() || first[i] < 0)
+      pinned[i] = 1;
+  size_t off = 0, naive = 0;
+  for (int i = 0; i < n; i++) {
+    naive += align256(slots_[i].bytes);
+    if (pinned[i]) {
+      slots_[i].offset = off;
+      off += align256(slots_[i].bytes);
+    }
+  }
+  const size_t temp_base = off;
+  std::vector<int> order;
+  for (int i = 0; i < n; i++)
+    if (!pinned[i])
+      order.push_back(i);
+  std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return first[x] < first[y]; });
+  std::vector<int> placed;
+  size_t top = temp_base;
+  for (int i : order) {
+    // regions of already placed temporaries whose lifetimes overlap this one, by offset
+    std::vector<std::pair<size_t, size_t>> busy;
+    for (int j : placed)
+      if (!(last[j] < first[i] || last[i] < first[j]))
+        busy.emplace_back(slots_[j].offset, slots_[j].offset + align256(slots_[j].bytes));
+    std::sort(busy.begin(), busy.end());
+    size_t at = temp_base;
+    const size_t need = align256(slots_[i].bytes);
+    for (auto &b : busy) {
+      if (at + need <= b.first)
+        break;
+      at = std::max(at, b.second);
+    }
+    slots_[i].offset = at;
+    top = std::max(top, at + need);
+    placed.push_back(i);
+  }
+  arena_bytes_ = top ? top : 256;
+  arena_bytes_no_reuse_ = naive ? naive : 256;
 }
 
 Executable::~Executable() {
@@ -792,6 +851,7 @@ std::string Executable::describe() const {
   std::ostringstream os;
   for (auto &s : steps_)
     os << names[(int)s.kind] << ": " << s.note << "\n";
+  os << "arena: " << arena_bytes_ << " bytes (" << arena_bytes_no_reuse_ << " with one region per buffer)\n";
   return os.str();
 }
 

@@ -84,6 +84,7 @@ private:
   std::vector<void *> ptr_; // per-slot device pointer during execute
   char *arena_ = nullptr;
   size_t arena_bytes_ = 0;
+  size_t arena_bytes_no_reuse_ = 0; // what one region per slot would take
   hipStream_t stream_ = nullptr;
   std::unordered_map<int, bool> colsum_valid_; // ColSum results of constant weights are computed once
   std::vector<char> step_done_;                // per step: a `once` step has run
@@ -93,6 +94,7 @@ private:
   int slot_for(size_t tensor_id);
   int const_slot(const void *data, size_t bytes);
   void plan();
+  void layout_arena();
   void plan_generic(const Op &op);
   void plan_matmul(size_t op_index, std::vector<bool> &done);
   bool try_int8(size_t op_index, std::vector<bool> &done);

@@ -46,21 +46,26 @@ def test_every_reference_fixture_parses_and_plans(ga, name):
     assert plan.strip()
 
 
+def _steps(plan):
+    """The launch lines of a plan (the last line reports the arena size)."""
+    return [ln for ln in plan.splitlines() if not ln.startswith("arena:")]
+
+
 def test_fusion_plan_of_reference_mlp(ga):
     """mpl.json (test/dnnl/resources): MatMul+bias -> ReLU -> MatMul -> Add -> ReLU
     becomes two GEMM launches with everything else in the epilogues."""
     st, plan = ga.explain(_res("mpl.json"))
     assert st == OK
-    assert plan.splitlines() == ["gemm_bf16: MatMul+bias+act", "gemm_bf16: MatMul+bias+act"]
+    assert _steps(plan) == ["gemm_bf16: MatMul+bias+act", "gemm_bf16: MatMul+bias+act"]
 
 
 def test_fusion_plans_of_benchmark_partitions(ga):
-    assert ga.explain(ga.matmul_bias_relu_json(128, 512, 256))[1].splitlines() == ["gemm_f32: MatMul+bias+act"]
-    assert ga.explain(_res("matmul.json"))[1].splitlines() == ["gemm_f32: MatMul+bias"]  # transpose_a folds into strides
+    assert _steps(ga.explain(ga.matmul_bias_relu_json(128, 512, 256))[1]) == ["gemm_f32: MatMul+bias+act"]
+    assert _steps(ga.explain(_res("matmul.json"))[1]) == ["gemm_f32: MatMul+bias"]  # transpose_a folds into strides
     j, _ = ga.int8_mlp_json(256, 256, 512, 0.02, 128, [0.01] * 512)
-    lines = ga.explain(j)[1].splitlines()
+    lines = _steps(ga.explain(j)[1])
     assert lines[0].startswith("colsum") and lines[1].startswith("gemm_int8: Dequantize x2 + MatMul+bias+act+cast") and len(lines) == 2
-    assert ga.explain(ga.mlp_chain_json(256, 256, 512))[1].splitlines() == ["gemm_bf16: MatMul+act", "gemm_bf16: MatMul+bias"]
+    assert _steps(ga.explain(ga.mlp_chain_json(256, 256, 512))[1]) == ["gemm_bf16: MatMul+act", "gemm_bf16: MatMul+bias"]
     assert ga.explain(ga.mha_json(2, 2, 128, 128, 128))[1].startswith("attention:")
     assert ga.explain(ga.mha_json(2, 2, 128, 128, 128, with_mask=False, scale_op="Divide"))[1].startswith("attention:")
     # head_dim 64 has no fused kernel: falls back to per-op kernels, still a valid plan
@@ -72,7 +77,7 @@ def test_intermediate_that_is_an_output_is_not_fused_away(ga):
     g = json.loads(ga.matmul_bias_relu_json(64, 64, 64))
     g["output_ports"] = [3, 4]  # the pre-activation tensor is wanted too
     st, plan = ga.explain(json.dumps(g))
-    assert st == OK and plan.splitlines() == ["gemm_f32: MatMul+bias", "eltwise: ReLU"]
+    assert st == OK and _steps(plan) == ["gemm_f32: MatMul+bias", "eltwise: ReLU"]
 
 
 def _mutate(fn):
@@ -144,3 +149,24 @@ def test_tensor_struct_layout_matches_the_reference_initialisers(ga):
     T = ga.Tensor
     assert (T.id.offset, T.ndims.offset, T.dims.offset, T.data.offset, C.sizeof(T)) == (0, 8, 16, 24, 32)
     assert C.sizeof(ga.Context) == 4
+
+
+def test_arena_shares_memory_between_temporaries_with_disjoint_lifetimes(ga):
+    """Four chained matmuls: t1 is dead once t2 exists, so t3 can take its place (the reference merges
+    allocations by lifetime ticks, lib/gc/Transforms/MergeAllocTickBased.cpp).  The plan reports both sizes."""
+    import json
+    import re
+    M = 256
+    ops = []
+    for i in range(4):
+        src = 0 if i == 0 else 10 + i - 1
+        ops.append({"kind": "MatMul", "inputs": [ga._t(src, "bf16", [M, M]), ga._t(1 + i, "bf16", [M, M])],
+                    "outputs": [ga._t(10 + i, "bf16", [M, M])]})
+    st, plan = ga.explain(ga._graph(ops, [0, 1, 2, 3, 4], [13]))
+    assert st == 0, plan
+    m = re.search(r"arena: (\d+) bytes \((\d+) with one region per buffer\)", plan)
+    assert m, plan
+    shared, naive = int(m.group(1)), int(m.group(2))
+    one = M * M * 2
+    assert naive == 9 * one          # 5 inputs + 3 temporaries + 1 output
+    assert shared == 8 * one         # t3 reuses t1's region

@@ -231,3 +231,23 @@ def test_constant_transposed_weight_is_prepared_once(ga, orc, wl, dev):
                 assert_close(ref, out.float().numpy(), 1e-2, "transpose_b %s" % prop)
         exe.close()
         comp.close()
+
+
+def test_chain_of_four_matmuls_with_shared_temporaries(ga, orc, wl, dev):
+    """The third temporary lives in the first one's memory (lifetimes do not overlap): results must not care."""
+    M = 256
+    torch.manual_seed(31)
+    x = (torch.randn(M, M) * 0.5).to(torch.bfloat16)
+    Ws = [(torch.randn(M, M) * 0.08).to(torch.bfloat16) for _ in range(4)]
+    ops = []
+    for i in range(4):
+        src = 0 if i == 0 else 10 + i - 1
+        ops.append({"kind": "MatMul", "inputs": [ga._t(src, "bf16", [M, M]), ga._t(1 + i, "bf16", [M, M])],
+                    "outputs": [ga._t(10 + i, "bf16", [M, M])]})
+    js = ga._graph(ops, [0, 1, 2, 3, 4], [13])
+    out = torch.zeros(M, M, dtype=torch.bfloat16)
+    _run(ga, js, [(0, x)] + [(1 + i, Ws[i]) for i in range(4)], [(13, out)])
+    cur = wl.bf16_bits(x)
+    for W in Ws:
+        cur = orc.matmul_bf16(cur, wl.bf16_bits(W))
+    assert_close(orc.bf16_to_f32(cur), out.float().numpy(), 4e-2, "four chained matmuls (four rounding points)")
