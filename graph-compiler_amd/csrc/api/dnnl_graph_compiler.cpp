@@ -16,6 +16,7 @@
 #include "gc-c/Dialects.h"
 #include "gc-c/Passes.h"
 #include "gc_hip_kernels.h"
+#include "mlir_text.h"
 
 struct dnnl_graph_compiler {
   uint32_t num_threads = 0;
@@ -25,6 +26,7 @@ struct dnnl_graph_compiler {
 struct dnnl_graph_compiler_executable {
   gcapi::Executable impl;
   explicit dnnl_graph_compiler_executable(const char *json) : impl(json) {}
+  explicit dnnl_graph_compiler_executable(gcapi::Graph g) : impl(std::move(g)) {}
 };
 
 namespace {
@@ -68,6 +70,33 @@ extern "C" dnnl_status_t dnnl_graph_compiler_compile(const dnnl_graph_compiler *
     return dnnl_invalid_arguments;
   try {
     *exe = new dnnl_graph_compiler_executable(graph_json);
+    return dnnl_success;
+  } catch (const std::invalid_argument &e) {
+    remember(e.what());
+    return dnnl_invalid_graph;
+  } catch (const std::logic_error &e) {
+    remember(e.what());
+    return dnnl_unimplemented;
+  } catch (const std::bad_alloc &) {
+    remember("out of memory");
+    return dnnl_out_of_memory;
+  } catch (const std::exception &e) {
+    remember(e.what());
+    return dnnl_runtime_error;
+  } catch (...) {
+    remember("unknown error");
+    return dnnl_runtime_error;
+  }
+}
+
+// The same for a module in MLIR's textual form (what the reference's gc-cpu-runner and benchgc's
+// `--driver mlir` take, test/benchgc/cases/*.mlir); see mlir_text.h for the accepted subset.
+extern "C" dnnl_status_t dnnl_graph_compiler_compile_mlir(const dnnl_graph_compiler *gc, const char *module_text,
+                                                          const dnnl_graph_compiler_executable **exe) {
+  if (!gc || !exe)
+    return dnnl_invalid_arguments;
+  try {
+    *exe = new dnnl_graph_compiler_executable(gcapi::parse_mlir(module_text));
     return dnnl_success;
   } catch (const std::invalid_argument &e) {
     remember(e.what());
@@ -131,6 +160,32 @@ extern "C" __attribute__((visibility("default"))) size_t gc_executable_describe(
 extern "C" dnnl_status_t dnnl_graph_compiler_explain(const char *graph_json, char *buf, size_t len) {
   try {
     gcapi::Executable e(graph_json, true);
+    std::string d = e.describe();
+    if (buf && len) {
+      size_t n = d.size() < len - 1 ? d.size() : len - 1;
+      memcpy(buf, d.data(), n);
+      buf[n] = 0;
+    }
+    return dnnl_success;
+  } catch (const std::invalid_argument &e) {
+    remember(e.what());
+    return dnnl_invalid_graph;
+  } catch (const std::logic_error &e) {
+    remember(e.what());
+    return dnnl_unimplemented;
+  } catch (const std::bad_alloc &) {
+    return dnnl_out_of_memory;
+  } catch (const std::exception &e) {
+    remember(e.what());
+    return dnnl_runtime_error;
+  } catch (...) {
+    return dnnl_runtime_error;
+  }
+}
+
+extern "C" dnnl_status_t dnnl_graph_compiler_explain_mlir(const char *module_text, char *buf, size_t len) {
+  try {
+    gcapi::Executable e(gcapi::parse_mlir(module_text), true);
     std::string d = e.describe();
     if (buf && len) {
       size_t n = d.size() < len - 1 ? d.size() : len - 1;

@@ -102,6 +102,26 @@ int Executable::slot_for(size_t tid) {
   int es = dt_size(t.dt);
   if (es == 0)
     throw std::logic_error(std::string("Unsupported tensor dtype on this path: ") + dt_name(t.dt));
+  if (t.alias_of >= 0) { // a reshape view: the storage of the tensor it views
+    int s = slot_for((size_t)t.alias_of);
+    slot_of_tensor_[tid] = s;
+    return s;
+  }
+  if (t.has_splat) { // one element, read with stride 0
+    uint32_t bits = 0;
+    float f = (float)t.splat;
+    if (t.dt == DT::f32)
+      memcpy(&bits, &f, 4);
+    else if (t.dt == DT::bf16) {
+      uint32_t u;
+      memcpy(&u, &f, 4);
+      bits = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+    } else
+      throw std::logic_error(std::string("Constant of this dtype is not supported: ") + dt_name(t.dt));
+    int s = const_slot(&bits, (size_t)es);
+    slot_of_tensor_[tid] = s;
+    return s;
+  }
   int s = new_slot((size_t)t.numel() * es, (long)tid);
   slot_of_tensor_[tid] = s;
   return s;
@@ -128,7 +148,10 @@ void Executable::add_copy(int src, DT sdt, const std::vector<int64_t> &dims, con
 }
 
 // ---------------------------------------------------------------------------
-Executable::Executable(const char *json, bool dry) : g_(parse_graph(json)) {
+Executable::Executable(const char *json, bool dry) : g_(parse_graph(json)) { init(dry); }
+Executable::Executable(Graph g, bool dry) : g_(std::move(g)) { init(dry); }
+
+void Executable::init(bool dry) {
   verify_graph(g_);
   plan();
   layout_arena();
@@ -296,7 +319,9 @@ void Executable::plan() {
             }
             const LTensor &st = T(other);
             bool is_in = std::find(g_.input_ids.begin(), g_.input_ids.end(), other) != g_.input_ids.end();
-            if (st.numel() != 1 || !is_in || !(st.dt == DT::f32 || st.dt == DT::bf16)) {
+            // a one-element input tensor, or a constant of one repeated value (MLIR's dense<x> splat)
+            bool one_input = st.numel() == 1 && is_in && (st.dt == DT::f32 || st.dt == DT::bf16);
+            if (!one_input && !st.has_splat) {
               ok = false;
               break;
             }
@@ -370,7 +395,10 @@ void Executable::plan() {
           s.mask = mask_slot, s.mask_ld = mask_ld;
           s.BH = prod(q.shape, 0, r - 2), s.Sq = Sq, s.Sk = Sk, s.D = 128;
           s.scale = 1.0f;
-          if (scale_t >= 0) {
+          if (scale_t >= 0 && T((size_t)scale_t).has_splat) {
+            const float x = (float)T((size_t)scale_t).splat;
+            s.scale = scale_div ? 1.0f / x : x;
+          } else if (scale_t >= 0) {
             s.scale_slot = slot_for((size_t)scale_t);
             s.scale_div = scale_div;
             s.a_dt = dt_dnnl(T((size_t)scale_t).dt);
@@ -615,6 +643,8 @@ void Executable::plan_generic(const Op &op) {
     throw std::logic_error("tensor rank above 6 is not supported");
   auto bstrides = [&](const LTensor &t) {
     std::vector<int64_t> st = dense_strides(t.shape), full(out.shape.size(), 0);
+    if (t.has_splat)
+      return full;
     for (size_t d = 0; d < t.shape.size(); d++) {
       size_t od = out.shape.size() - t.shape.size() + d;
       full[od] = t.shape[d] == 1 ? 0 : st[d];
@@ -624,13 +654,43 @@ void Executable::plan_generic(const Op &op) {
   Step s;
   s.kind = Step::Elt;
   s.note = k;
-  if (k == "Add" || k == "Subtract" || k == "Multiply" || k == "Divide") {
-    s.op = k == "Add" ? gcmi::ELT_ADD : k == "Subtract" ? gcmi::ELT_SUB : k == "Multiply" ? gcmi::ELT_MUL : gcmi::ELT_DIV;
+  if (k == "Reshape") {
+    (void)slot_for(op.out[0]); // a view: no work
+    return;
+  }
+  if (k == "Transpose" || k == "BroadcastTo") {
+    const LTensor &in = T(op.in[0]);
+    std::vector<int64_t> ist = dense_strides(in.shape), st(out.shape.size(), 0);
+    if (k == "Transpose") {
+      const auto &perm = op.attrs.at("perm").ia;
+      for (size_t d = 0; d < perm.size(); d++)
+        st[d] = ist[(size_t)perm[d]];
+    } else {
+      const auto &added = op.attrs.at("dims").ia;
+      size_t src = 0;
+      for (size_t d = 0; d < out.shape.size(); d++)
+        if (std::find(added.begin(), added.end(), (int64_t)d) == added.end())
+          st[d] = in.has_splat ? 0 : ist[src++];
+    }
+    s.note = k == "Transpose" ? "Transpose (strided copy)" : "BroadcastTo (stride-0 copy)";
+    s.op = gcmi::ELT_COPY;
+    s.a = slot_for(op.in[0]), s.out = slot_for(op.out[0]);
+    s.a_dt = dt_dnnl(in.dt), s.out_dt = dt_dnnl(out.dt);
+    s.dims = out.shape, s.sa = st;
+    steps_.push_back(std::move(s));
+    return;
+  }
+  if (k == "Add" || k == "Subtract" || k == "Multiply" || k == "Divide" || k == "Maximum") {
+    s.op = k == "Add" ? gcmi::ELT_ADD : k == "Subtract" ? gcmi::ELT_SUB : k == "Multiply" ? gcmi::ELT_MUL
+           : k == "Divide" ? gcmi::ELT_DIV : gcmi::ELT_MAX;
     s.a = slot_for(op.in[0]), s.b = slot_for(op.in[1]), s.out = slot_for(op.out[0]);
     s.a_dt = dt_dnnl(T(op.in[0]).dt), s.b_dt = dt_dnnl(T(op.in[1]).dt), s.out_dt = dt_dnnl(out.dt);
     s.dims = out.shape, s.sa = bstrides(T(op.in[0])), s.sb = bstrides(T(op.in[1]));
-  } else if (k == "ReLU" || k == "Sigmoid" || k == "GELU" || k == "Pow" || k == "Typecast" || k == "TypeCast") {
+  } else if (k == "ReLU" || k == "Sigmoid" || k == "GELU" || k == "Pow" || k == "Typecast" || k == "TypeCast" ||
+             k == "Exp" || k == "Neg") {
     s.op = k == "ReLU" ? gcmi::ELT_RELU
+           : k == "Exp" ? gcmi::ELT_EXP
+           : k == "Neg" ? gcmi::ELT_NEG
            : k == "Sigmoid" ? gcmi::ELT_SIGMOID
            : k == "GELU" ? (act_of(op) == GCMI_ACT_GELU_TANH ? gcmi::ELT_GELU_TANH : gcmi::ELT_GELU_ERF)
            : k == "Pow" ? gcmi::ELT_POW
@@ -851,6 +911,12 @@ std::string Executable::describe() const {
   std::ostringstream os;
   for (auto &s : steps_)
     os << names[(int)s.kind] << ": " << s.note << "\n";
+  if (!g_.target_hints.empty()) {
+    os << "target hints (CPU, not used):";
+    for (auto &h : g_.target_hints)
+      os << " " << h.first << "=" << h.second;
+    os << "\n";
+  }
   os << "arena: " << arena_bytes_ << " bytes (" << arena_bytes_no_reuse_ << " with one region per buffer)\n";
   return os.str();
 }

@@ -66,6 +66,8 @@ class Executable {
 public:
   // dry = plan only: no device memory, no stream (host-side tests and explain)
   explicit Executable(const char *json, bool dry = false);
+  // from a graph built by another front end (mlir_text.h)
+  explicit Executable(Graph g, bool dry = false);
   ~Executable();
   Executable(const Executable &) = delete;
   Executable &operator=(const Executable &) = delete;
@@ -93,6 +95,7 @@ private:
   int new_slot(size_t bytes, long tensor_id = -1);
   int slot_for(size_t tensor_id);
   int const_slot(const void *data, size_t bytes);
+  void init(bool dry);
   void plan();
   void layout_arena();
   void plan_generic(const Op &op);

@@ -84,6 +84,10 @@ static const std::set<std::string> &extension_ops() {
 }
 bool is_known_op(const std::string &k) { return reference_ops().count(k) || extension_ops().count(k); }
 bool is_extension_op(const std::string &k) { return extension_ops().count(k) != 0; }
+bool is_internal_op(const std::string &k) {
+  static const std::set<std::string> s = {"Maximum", "Exp", "Neg", "Reshape", "Transpose", "BroadcastTo"};
+  return s.count(k) != 0;
+}
 
 namespace {
 
@@ -384,7 +388,7 @@ void verify_graph(const Graph &g) {
       if (T(id).unranked)
         vfail(op, "unranked result");
     const std::string &k = op.kind;
-    if (k == "Add" || k == "Subtract" || k == "Multiply" || k == "Divide") {
+    if (k == "Add" || k == "Subtract" || k == "Multiply" || k == "Divide" || k == "Maximum") {
       if (op.in.size() != 2 || op.out.size() != 1)
         vfail(op, "expects 2 operands and 1 result");
       std::vector<int64_t> o;
@@ -394,13 +398,42 @@ void verify_graph(const Graph &g) {
         vfail(op, "operand shapes do not broadcast to the result shape");
       if (!op.attr_bool("auto_broadcast", true) && T(op.in[0]).shape != T(op.in[1]).shape)
         vfail(op, "auto_broadcast is none but shapes differ");
-    } else if (k == "ReLU" || k == "Sigmoid" || k == "Pow" || k == "GELU") {
+    } else if (k == "ReLU" || k == "Sigmoid" || k == "Pow" || k == "GELU" || k == "Exp" || k == "Neg") {
       if (op.in.size() != 1 || op.out.size() != 1)
         vfail(op, "expects 1 operand and 1 result");
       if (T(op.in[0]).shape != T(op.out[0]).shape || T(op.in[0]).dt != T(op.out[0]).dt || !is_float(T(op.in[0]).dt))
         vfail(op, "operand and result types differ");
       if (k == "Pow" && !op.attrs.count("beta"))
         vfail(op, "attribute beta is required");
+    } else if (k == "Reshape") {
+      if (op.in.size() != 1 || op.out.size() != 1 || T(op.in[0]).numel() != T(op.out[0]).numel() ||
+          T(op.in[0]).dt != T(op.out[0]).dt)
+        vfail(op, "a reshape keeps the element count and type");
+    } else if (k == "Transpose") {
+      const auto &in = T(op.in[0]), &out = T(op.out[0]);
+      auto it = op.attrs.find("perm");
+      if (op.in.size() != 1 || op.out.size() != 1 || it == op.attrs.end() || it->second.ia.size() != in.shape.size() ||
+          out.shape.size() != in.shape.size() || in.dt != out.dt)
+        vfail(op, "permutation does not fit the operand");
+      std::vector<char> seen(in.shape.size(), 0);
+      for (size_t d = 0; d < in.shape.size(); d++) {
+        int64_t q = it->second.ia[d];
+        if (q < 0 || q >= (int64_t)in.shape.size() || seen[(size_t)q] || out.shape[d] != in.shape[(size_t)q])
+          vfail(op, "permutation does not fit the operand");
+        seen[(size_t)q] = 1;
+      }
+    } else if (k == "BroadcastTo") {
+      const auto &in = T(op.in[0]), &out = T(op.out[0]);
+      auto it = op.attrs.find("dims");
+      if (op.in.size() != 1 || op.out.size() != 1 || it == op.attrs.end() || in.dt != out.dt ||
+          in.shape.size() + it->second.ia.size() != out.shape.size())
+        vfail(op, "broadcast dimensions do not fit");
+      size_t src = 0;
+      for (size_t d = 0; d < out.shape.size(); d++) {
+        bool added = std::find(it->second.ia.begin(), it->second.ia.end(), (int64_t)d) != it->second.ia.end();
+        if (!added && (src >= in.shape.size() || in.shape[src++] != out.shape[d]))
+          vfail(op, "broadcast dimensions do not fit");
+      }
     } else if (k == "Typecast" || k == "TypeCast") {
       if (op.in.size() != 1 || op.out.size() != 1 || T(op.in[0]).shape != T(op.out[0]).shape)
         vfail(op, "operand and result shapes differ");

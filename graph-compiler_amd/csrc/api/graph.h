@@ -8,6 +8,7 @@
 #include <map>
 #include <string>
 #include <unordered_map>
+#include <utility>
 #include <vector>
 
 namespace gcapi {
@@ -25,6 +26,10 @@ struct LTensor {
   bool strided = false;
   std::vector<int64_t> stride; // elements; only meaningful when strided
   bool constant = false;       // property_type == "constant"
+  // set by the MLIR front end only:
+  long alias_of = -1;          // id of the tensor whose storage this one shares (reshape views); same numel
+  bool has_splat = false;      // every element equals `splat` (arith.constant dense<c>, linalg.fill of a constant)
+  double splat = 0.0;
   int64_t numel() const {
     int64_t n = 1;
     for (auto d : shape)
@@ -58,6 +63,10 @@ struct Graph {
   std::unordered_map<size_t, LTensor> tensors;
   std::vector<size_t> input_ids;  // order of first use = argument order (JsonParser.cpp:183-199)
   std::vector<size_t> output_ids; // output_ports, or the last op's outputs (:91-94)
+  // entries of a module's dlti.target_system_spec ("CPU" device: cache sizes, num_threads, max_vector_width, as
+  // benchgc attaches them, test/benchgc/src/benchgc/mlir/util.py:187-197).  Read and reported; tiling on the GPU
+  // follows the GPU's own parameters, so they steer nothing.
+  std::vector<std::pair<std::string, int64_t>> target_hints;
 };
 
 // op kinds the reference front end accepts (src/dnnl/JsonParser.h:152-164) plus
@@ -66,6 +75,10 @@ bool is_known_op(const std::string &kind);
 bool is_extension_op(const std::string &kind);
 
 Graph parse_graph(const char *json);
+
+// ops only the MLIR front end produces (mlir_text.h): Maximum, Exp, Neg (element-wise), Reshape (a view),
+// Transpose {perm}, BroadcastTo {dims: the result dimensions that are added}
+bool is_internal_op(const std::string &kind);
 
 // Checks every op's operand/result shapes and dtypes (the role of the MLIR op
 // verifiers, include/gc/Dialect/OneDNNGraph/OneDNNGraphOps.td and

@@ -6,6 +6,7 @@
 // (lib/gc/Transforms/Pipeline.cpp:79-95).  Semantics per op:
 //   Add/Subtract/Multiply/Divide  numpy broadcasting
 //                                 (lib/gc/Transforms/OneDNNGraphToLinalg.cpp:64-118)
+//   Maximum / Exp / Neg           linalg.max, linalg.exp, linalg.negf of the MLIR front end
 //   ReLU max(x,0), Sigmoid 1/(1+exp(-x)), Pow x^beta, Typecast = copy with rounding
 //                                 (OneDNNGraphToLinalg.cpp:331-358)
 //   ReduceSum / ReduceMean        sum over axes, mean divides by the count (:505-559)
@@ -62,6 +63,9 @@ __global__ void eltwise_kernel(EltParams p) {
     case ELT_SUB: r = x - y; break;
     case ELT_MUL: r = x * y; break;
     case ELT_DIV: r = x / y; break;
+    case ELT_MAX: r = (x != x || y != y) ? x + y : fmaxf(x, y); break; // arith.maximumf: NaN propagates
+    case ELT_EXP: r = expf(x); break;
+    case ELT_NEG: r = -x; break;
     case ELT_RELU: r = apply_act(x, ACT_RELU); break;
     case ELT_SIGMOID: r = apply_act(x, ACT_SIGMOID); break;
     case ELT_GELU_ERF: r = apply_act(x, ACT_GELU_ERF); break;

@@ -8,7 +8,7 @@ static constexpr int ELT_MAX_RANK = 6;
 
 enum EltOp : int {
   ELT_COPY = 0, ELT_ADD, ELT_SUB, ELT_MUL, ELT_DIV, ELT_RELU, ELT_SIGMOID, ELT_GELU_ERF, ELT_GELU_TANH, ELT_POW,
-  ELT_DEQUANT, ELT_QUANT
+  ELT_DEQUANT, ELT_QUANT, ELT_MAX, ELT_EXP, ELT_NEG
 };
 
 struct EltParams {

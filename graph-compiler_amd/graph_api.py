@@ -14,7 +14,8 @@ from . import lib, EXPORTS
 EXPORTS["dnnl_graph_compiler.h"] = [
     "dnnl_graph_compiler_get_version", "dnnl_graph_compiler_create", "dnnl_graph_compiler_destroy",
     "dnnl_graph_compiler_compile", "dnnl_graph_compiler_destroy_executable", "dnnl_graph_compiler_execute",
-    "dnnl_graph_compiler_explain", "dnnl_graph_compiler_last_error"]
+    "dnnl_graph_compiler_explain", "dnnl_graph_compiler_last_error",
+    "dnnl_graph_compiler_compile_mlir", "dnnl_graph_compiler_explain_mlir"]
 
 SUCCESS, OUT_OF_MEMORY, INVALID_ARGUMENTS, UNIMPLEMENTED, RUNTIME_ERROR, INVALID_GRAPH = 0, 1, 2, 3, 5, 7
 
@@ -54,6 +55,10 @@ def api():
         L.dnnl_graph_compiler_explain.restype = C.c_int
         L.dnnl_graph_compiler_explain.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t]
         L.dnnl_graph_compiler_last_error.restype = C.c_char_p
+        L.dnnl_graph_compiler_compile_mlir.restype = C.c_int
+        L.dnnl_graph_compiler_compile_mlir.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
+        L.dnnl_graph_compiler_explain_mlir.restype = C.c_int
+        L.dnnl_graph_compiler_explain_mlir.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t]
         _bound = True
     return L
 
@@ -62,6 +67,13 @@ def explain(graph_json):
     """(status, plan text or error text) from the host-side stages; needs no GPU."""
     buf = C.create_string_buffer(1 << 16)
     st = api().dnnl_graph_compiler_explain(graph_json.encode(), buf, len(buf))
+    return st, (buf.value.decode() if st == 0 else api().dnnl_graph_compiler_last_error().decode())
+
+
+def explain_mlir(module_text):
+    """explain() for a module in MLIR's textual form."""
+    buf = C.create_string_buffer(1 << 16)
+    st = api().dnnl_graph_compiler_explain_mlir(module_text.encode(), buf, len(buf))
     return st, (buf.value.decode() if st == 0 else api().dnnl_graph_compiler_last_error().decode())
 
 
@@ -86,6 +98,12 @@ class Compiler:
     def compile(self, graph_json):
         exe = C.c_void_p()
         st = api().dnnl_graph_compiler_compile(self.h, graph_json.encode(), C.byref(exe))
+        return st, (Executable(exe) if st == 0 else None)
+
+    def compile_mlir(self, module_text):
+        """Function argument i has tensor id i, result j has id (number of arguments) + j."""
+        exe = C.c_void_p()
+        st = api().dnnl_graph_compiler_compile_mlir(self.h, module_text.encode(), C.byref(exe))
         return st, (Executable(exe) if st == 0 else None)
 
     def close(self):

@@ -109,6 +109,21 @@ dnnl_status_t dnnl_graph_compiler_execute(const struct dnnl_graph_compiler_execu
  * printing the IR after the pass pipeline (gc-opt --gc-cpu-pipeline). */
 dnnl_status_t dnnl_graph_compiler_explain(const char *graph_json, char *buf, size_t len);
 
+/* compile / explain for a module in MLIR's textual form: one func.func over
+ * ranked tensors made of tensor.empty, arith.constant, linalg.{fill, matmul,
+ * matmul_transpose_a/b, batch_matmul, batch_matmul_transpose_b, add, sub, mul,
+ * div, max, powf, negf, exp, copy, broadcast, transpose, softmax, reduce(addf)}
+ * and tensor.{collapse,expand}_shape -- the subset of the reference's benchgc
+ * cases (test/benchgc/cases/llama2.mlir) and MLP/matmul patterns
+ * (test/benchgc/src/benchgc/pattern/mlp.py).  Takes over what gc-cpu-runner /
+ * benchgc `--driver mlir` do with such a module on the CPU
+ * (src/gc-cpu-runner/gc-cpu-runner.cpp, test/benchgc/src/benchgc/runner.py).
+ * Tensor ids for execute: function argument i has id i, result j has id
+ * (number of arguments) + j.  Anything outside the subset: dnnl_unimplemented. */
+dnnl_status_t dnnl_graph_compiler_compile_mlir(const struct dnnl_graph_compiler *gc, const char *module_text,
+                                               const struct dnnl_graph_compiler_executable **exe);
+dnnl_status_t dnnl_graph_compiler_explain_mlir(const char *module_text, char *buf, size_t len);
+
 /* Text of the last error raised on the calling thread by the functions above
  * (no counterpart in the reference, which prints to stderr in debug builds). */
 const char *dnnl_graph_compiler_last_error(void);

@@ -1,0 +1,130 @@
+"""CPU: the textual-MLIR front end (dnnl_graph_compiler_explain_mlir runs parse -> verify -> fuse ->
+plan without a GPU).  Modules follow what the reference's benchgc builds or holds: the MLP pattern
+(test/benchgc/src/benchgc/pattern/mlp.py), test/benchgc/cases/llama2.mlir (a decoder MLP block) and
+test/benchgc/cases/generic.mlir (a matmul spelled as linalg.generic)."""
+import importlib
+import os
+
+import pytest
+
+OK, UNIMPL, RUNTIME, INVALID_GRAPH = 0, 3, 5, 7
+REF_CASES = "/root/reference/test/benchgc/cases"
+
+
+@pytest.fixture(scope="module")
+def ga(gc):
+    return importlib.import_module("graph_compiler_amd.graph_api")
+
+
+@pytest.fixture(scope="module")
+def mm(gc):
+    return importlib.import_module("graph_compiler_amd.mlir_modules")
+
+
+def _steps(plan):
+    return [ln for ln in plan.splitlines() if not ln.startswith(("arena:", "target hints"))]
+
+
+def test_mlp_pattern_fuses_bias_and_activation_into_the_gemm(ga, mm):
+    st, plan = ga.explain_mlir(mm.mlp(128, [512, 256, 64], [True, False], "relu", "bf16"))
+    assert st == OK, plan
+    assert _steps(plan) == ["gemm_bf16: MatMul+bias+act", "gemm_bf16: MatMul+act"]
+    st, plan = ga.explain_mlir(mm.mlp(32, [64, 64], [True], "noop", "f32"))
+    assert st == OK and _steps(plan) == ["gemm_f32: MatMul+bias"]
+    # 1 / (1 + exp(-x)) written as four linalg ops is one sigmoid, which the GEMM epilogue takes
+    st, plan = ga.explain_mlir(mm.mlp(32, [64, 64], [True], "sigmoid", "f32"))
+    assert st == OK and _steps(plan) == ["gemm_f32: MatMul+bias+act"]
+
+
+def test_generic_contraction_is_a_matmul(ga, mm):
+    for tb in (False, True):
+        st, plan = ga.explain_mlir(mm.generic_matmul(16, 8, 4, "f32", transpose_b=tb))
+        assert st == OK, plan
+        assert _steps(plan)[-1] == "gemm_f32: MatMul"
+    # a body that is not multiply-accumulate is outside the subset
+    bad = mm.generic_matmul(16, 8, 4).replace("arith.mulf", "arith.subf")
+    assert ga.explain_mlir(bad)[0] == UNIMPL
+    # map results must be plain dims
+    bad = mm.generic_matmul(16, 8, 4).replace("-> (d0, d2)", "-> (d0 + d1, d2)")
+    assert ga.explain_mlir(bad)[0] == UNIMPL
+
+
+def test_decoder_block_plan(ga, mm):
+    st, plan = ga.explain_mlir(mm.decoder_mlp_block(32, 256, 512))
+    assert st == OK, plan
+    steps = _steps(plan)
+    assert sum(s.startswith("gemm_bf16") for s in steps) == 4
+    assert sum(s.startswith("reduce: ReduceSum") for s in steps) == 2
+    assert "eltwise: Sigmoid" in steps and not any("Exp" in s or "Neg" in s for s in steps)
+    # reshapes are views and broadcasts fold into the consumer's strides: neither is a launch
+    assert not any("Reshape" in s or "BroadcastTo" in s for s in steps)
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_CASES), reason="the reference tree is not on this machine")
+def test_reference_benchgc_cases_parse_and_plan(ga, mm):
+    st, plan = ga.explain_mlir(open(os.path.join(REF_CASES, "llama2.mlir")).read())
+    assert st == OK, plan
+    # same structure as the builder's block at the case's sizes
+    st2, plan2 = ga.explain_mlir(mm.decoder_mlp_block(32, 4096, 11008))
+    assert st2 == OK and _steps(plan) == _steps(plan2)
+    st, plan = ga.explain_mlir(open(os.path.join(REF_CASES, "generic.mlir")).read())
+    assert st == OK and _steps(plan) == ["gemm_f32: MatMul"]
+
+
+def test_target_spec_of_the_module_is_read(ga, mm):
+    """benchgc attaches the CPU's cache sizes and thread count (mlir/util.py:187-197)."""
+    spec = ('module attributes {\n dlti.target_system_spec = #dlti.target_system_spec<\n'
+            '  "CPU": #dlti.target_device_spec<\n'
+            '   #dlti.dl_entry<"L1_cache_size_in_bytes", 49152 : ui32>,\n'
+            '   #dlti.dl_entry<"L2_cache_size_in_bytes", 2097152 : ui64>,\n'
+            '   #dlti.dl_entry<"L3_cache_size_in_bytes", 110100480 : ui64>,\n'
+            '   #dlti.dl_entry<"num_threads", 56 : i32>,\n'
+            '   #dlti.dl_entry<"max_vector_width", 512 : i64>>\n >} {')
+    text = mm.mlp(32, [64, 64]).replace("module {", spec, 1)
+    st, plan = ga.explain_mlir(text)
+    assert st == OK, plan
+    line = [ln for ln in plan.splitlines() if ln.startswith("target hints")]
+    assert line and "num_threads=56" in line[0] and "L2_cache_size_in_bytes=2097152" in line[0]
+    assert _steps(plan) == ["gemm_f32: MatMul"]
+
+
+def _fn(body, args="%a: tensor<8x8xf32>, %b: tensor<8x8xf32>", res="tensor<8x8xf32>"):
+    return "func.func @f(%s) -> %s {\n%s\n}" % (args, res, body)
+
+
+def test_error_classes(ga):
+    ex = ga.explain_mlir
+    e = "%e = tensor.empty() : tensor<8x8xf32>\n"
+    ok = _fn(e + "%r = linalg.add ins(%a, %b : tensor<8x8xf32>, tensor<8x8xf32>) outs(%e : tensor<8x8xf32>) -> tensor<8x8xf32>\n"
+             "return %r : tensor<8x8xf32>")
+    st, plan = ex(ok)  # a bare function, no module around it
+    assert st == OK and _steps(plan) == ["eltwise: Add"]
+    # malformed text, undefined values -> invalid_graph
+    assert ex("module {")[0] == INVALID_GRAPH
+    assert ex(ok.replace("ins(%a, %b", "ins(%a, %nope"))[0] == INVALID_GRAPH
+    assert ex(ok.replace("return %r : tensor<8x8xf32>", ""))[0] == INVALID_GRAPH
+    assert ex(_fn("return"))[0] == INVALID_GRAPH  # nothing returned
+    # outside the subset -> unimplemented
+    assert ex(ok.replace("linalg.add", "linalg.conv_2d"))[0] == UNIMPL
+    assert ex(ok.replace("tensor<8x8xf32>", "tensor<?x8xf32>"))[0] == UNIMPL
+    assert ex(ok.replace("f32", "f8E4M3"))[0] == UNIMPL
+    assert ex(_fn("%r = scf.for %i = %a to %b : index {}\nreturn %r : tensor<8x8xf32>"))[0] == UNIMPL
+    st, msg = ex(ok.replace("linalg.add", "linalg.conv_2d"))
+    assert "linalg.conv_2d" in msg
+    # parses but does not verify (result shape) -> runtime_error, like a failed pipeline run
+    wrong = ok.replace("outs(%e : tensor<8x8xf32>) -> tensor<8x8xf32>", "outs(%e : tensor<8x8xf32>) -> tensor<8x4xf32>")
+    assert ex(wrong)[0] == RUNTIME
+    # accumulating matmul (init that is not zero) is not taken
+    acc = _fn("%r = linalg.matmul ins(%a, %b : tensor<8x8xf32>, tensor<8x8xf32>) outs(%a : tensor<8x8xf32>) -> tensor<8x8xf32>\n"
+              "return %r : tensor<8x8xf32>")
+    assert ex(acc)[0] == UNIMPL
+
+
+def test_returned_argument_constant_and_duplicate_are_copied(ga):
+    e = "%e = tensor.empty() : tensor<8x8xf32>\n"
+    body = (e + "%c = arith.constant dense<2.500000e+00> : tensor<8x8xf32>\n"
+            "%r = linalg.mul ins(%a, %c : tensor<8x8xf32>, tensor<8x8xf32>) outs(%e : tensor<8x8xf32>) -> tensor<8x8xf32>\n"
+            "return %r, %r, %a, %c : tensor<8x8xf32>, tensor<8x8xf32>, tensor<8x8xf32>, tensor<8x8xf32>")
+    st, plan = ga.explain_mlir(_fn(body, res="(tensor<8x8xf32>, tensor<8x8xf32>, tensor<8x8xf32>, tensor<8x8xf32>)"))
+    assert st == OK, plan
+    assert len(_steps(plan)) == 4  # the product, its copy, the copy of %a and the filled constant
