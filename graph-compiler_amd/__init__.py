@@ -20,7 +20,7 @@ ACT = {None: 0, "none": 0, "relu": 1, "gelu_erf": 2, "gelu_tanh": 3, "sigmoid": 
 
 # every symbol the public headers declare (checked by the CPU test-suite)
 EXPORTS = {
-    "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_int8", "gcmi_colsum_s8",
+    "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_bf16_nt", "gcmi_gemm_int8", "gcmi_colsum_s8",
                          "gcmi_gemm_f32", "gcmi_mha_fwd_bf16", "gcmi_mha_fwd_bf16_opt"],
     "gc_brgemm.h": ["dnnl_brgemm_dispatch", "dnnl_brgemm_tileconfig", "dnnl_brgemm_tilerelease",
                     "dnnl_brgemm_execute"],
@@ -49,6 +49,8 @@ def lib():
     L.gcmi_last_error.restype = C.c_char_p
     L.gcmi_gemm_bf16.restype = ci
     L.gcmi_gemm_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, ci, ci, ci, vp]
+    L.gcmi_gemm_bf16_nt.restype = ci
+    L.gcmi_gemm_bf16_nt.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, ci, ci, ci, vp]
     L.gcmi_gemm_int8.restype = ci
     L.gcmi_gemm_int8.argtypes = [vp, ci, vp, vp, i64, i64, i64, i64, i64, i64, vp, C.c_int32, vp, vp, ci, ci, vp]
     L.gcmi_colsum_s8.restype = ci
@@ -94,7 +96,7 @@ def gemm_bf16(A, B, bias=None, act=None, out_dtype=BF16, out=None):
     import torch
     M, K = A.shape
     K2, N = B.shape
-    assert K == K2 and A.stride(1) == 1 and B.stride(1) == 1
+    assert K == K2 and (A.stride(1) == 1 or K == 1) and (B.stride(1) == 1 or N == 1)
     if out is None:
         out = torch.empty((M, N), device=A.device, dtype=torch.bfloat16 if out_dtype == BF16 else torch.float32)
     bdt = BF16
@@ -103,6 +105,23 @@ def gemm_bf16(A, B, bias=None, act=None, out_dtype=BF16, out=None):
     check(lib().gcmi_gemm_bf16(_ptr(A), _ptr(B), _ptr(out), M, N, K, A.stride(0) if M > 1 else K,
                                B.stride(0) if K > 1 else N, out.stride(0) if M > 1 else N, _ptr(bias), bdt,
                                ACT[act], out_dtype, _stream()), "gcmi_gemm_bf16")
+    return out
+
+
+def gemm_bf16_nt(A, Bt, bias=None, act=None, out_dtype=BF16, out=None):
+    """A [M,K], Bt [N,K] (the weight as torch.nn.Linear stores it): A @ Bt.T without a transposed copy."""
+    import torch
+    M, K = A.shape
+    N, K2 = Bt.shape
+    assert K == K2 and (A.stride(1) == 1 or K == 1) and (Bt.stride(1) == 1 or K == 1)
+    if out is None:
+        out = torch.empty((M, N), device=A.device, dtype=torch.bfloat16 if out_dtype == BF16 else torch.float32)
+    bdt = BF16
+    if bias is not None:
+        bdt = BF16 if bias.dtype == torch.bfloat16 else F32
+    check(lib().gcmi_gemm_bf16_nt(_ptr(A), _ptr(Bt), _ptr(out), M, N, K, A.stride(0) if M > 1 else K,
+                                  Bt.stride(0) if N > 1 else K, out.stride(0) if M > 1 else N, _ptr(bias), bdt,
+                                  ACT[act], out_dtype, _stream()), "gcmi_gemm_bf16_nt")
     return out
 
 
@@ -141,7 +160,7 @@ def gemm_f32(A, B, bias=None, act=None, trans_a=False, trans_b=False, out=None):
         N, K2 = B.shape
     else:
         K2, N = B.shape
-    assert K == K2 and A.stride(1) == 1 and B.stride(1) == 1
+    assert K == K2 and (A.stride(1) == 1 or K == 1) and (B.stride(1) == 1 or N == 1)
     if out is None:
         out = torch.empty((M, N), device=A.device, dtype=torch.float32)
     check(lib().gcmi_gemm_f32(_ptr(A), _ptr(B), _ptr(out), M, N, K, A.stride(0), B.stride(0), out.stride(0),

@@ -531,8 +531,8 @@ void Executable::plan() {
       int64_t N = tB ? bs[Rb - 2] : bs[Rb - 1];
       int sa_slot = slot_for(mm.in[0]), sb_slot = slot_for(mm.in[1]);
       DT out_dt = T(mm.out[0]).dt;
-      if (A.dt == DT::bf16 && (tA || tB)) {
-        // the bf16 kernel reads row-major [M,K] and [K,N]: materialise the transposes
+      if (A.dt == DT::bf16 && tA) {
+        // the bf16 kernel reads A row-major [M,K] (B may be stored either way): materialise a transposed A
         // (once per executable when the operand is a constant: the analogue of the reference's weight
         // pre-packing of constant tensors, docs/CPU_pipeline_overview.md:58)
         auto transposed = [&](int slot, std::vector<int64_t> &shp, bool constant) {
@@ -550,10 +550,7 @@ void Executable::plan() {
           shp = d;
           return t;
         };
-        if (tA)
-          sa_slot = transposed(sa_slot, as, A.constant), tA = false;
-        if (tB)
-          sb_slot = transposed(sb_slot, bs, B.constant), tB = false;
+        sa_slot = transposed(sa_slot, as, A.constant), tA = false;
       }
       std::vector<int64_t> ba(as.begin(), as.end() - 2), bb(bs.begin(), bs.end() - 2), bo;
       broadcast_shape(ba, bb, bo);
@@ -760,9 +757,9 @@ void Executable::launch(const Step &s) {
              "MatMul f32");
     break;
   case Step::GemmBf16:
-    gc_check(gcmi_gemm_bf16(P(s.a) + s.a_off * 2, P(s.b) + s.b_off * 2, P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4),
-                            s.M, s.N, s.K, s.lda, s.ldb, s.ldc, P(s.bias), s.bias_dt ? s.bias_dt : GCMI_BF16, s.act,
-                            s.out_dt, stream_),
+    gc_check((s.tb ? gcmi_gemm_bf16_nt : gcmi_gemm_bf16)(
+                 P(s.a) + s.a_off * 2, P(s.b) + s.b_off * 2, P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4), s.M, s.N,
+                 s.K, s.lda, s.ldb, s.ldc, P(s.bias), s.bias_dt ? s.bias_dt : GCMI_BF16, s.act, s.out_dt, stream_),
              "MatMul bf16");
     break;
   case Step::ColSum:

@@ -63,16 +63,33 @@ extern "C" int gcmi_init(int device) {
   return ST_OK;
 }
 
+namespace {
+int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                  int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
+}
+
 extern "C" int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                               int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype,
                               void *stream) {
+  return gemm_bf16_any(false, A, B, C, M, N, K, lda, ldb, ldc, bias, bias_dtype, act, out_dtype, stream);
+}
+
+extern "C" int gcmi_gemm_bf16_nt(const void *A, const void *Bt, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                 int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype,
+                                 void *stream) {
+  return gemm_bf16_any(true, A, Bt, C, M, N, K, lda, ldb, ldc, bias, bias_dtype, act, out_dtype, stream);
+}
+
+namespace {
+int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                  int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream) {
   if (M < 0 || N < 0 || K < 0)
     return fail(ST_INVALID, "gemm_bf16: negative size");
   if (M == 0 || N == 0)
     return ST_OK;
   if (!A || !B || !C)
     return fail(ST_INVALID, "gemm_bf16: null operand");
-  if (lda < K || ldb < N || ldc < N)
+  if (lda < K || ldb < (trans_b ? K : N) || ldc < N)
     return fail(ST_INVALID, "gemm_bf16: leading dimension smaller than the row (lda %lld ldb %lld ldc %lld)",
                 (long long)lda, (long long)ldb, (long long)ldc);
   if (out_dtype != GCMI_BF16 && out_dtype != GCMI_F32)
@@ -84,8 +101,10 @@ extern "C" int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, 
   GemmParams p{};
   p.A = A, p.B = B, p.C = C, p.M = M, p.N = N, p.K = K, p.lda = lda, p.ldb = ldb, p.ldc = ldc;
   p.bias = bias, p.bias_dt = bias_dtype, p.act = act, p.out_dt = out_dtype;
+  p.trans_b = trans_b ? 1 : 0;
   return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
 }
+} // namespace
 
 extern "C" int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K,
                               int64_t lda, int64_t ldb, int64_t ldc, const int32_t *colsum, int32_t zp_a,

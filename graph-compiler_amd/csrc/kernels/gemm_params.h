@@ -24,6 +24,7 @@ struct GemmParams {
   // runs the epilogue
   int32_t splits;        // 0 or 1: off
   float *partial;
+  int32_t trans_b;       // bf16 only: B is stored [N,K] (k contiguous), ldb elements between its rows
 };
 
 struct F32GemmParams {

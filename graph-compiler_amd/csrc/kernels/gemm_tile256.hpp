@@ -284,7 +284,9 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, typename Mfma
   }
 }
 
-template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_kernel(GemmParams p) {
+// TB: B is stored [N,K] (k contiguous).  Its tile then has the geometry of the A tile (256 rows x 128 bytes of K),
+// takes the same swizzle, and its fragments are plain 16-byte reads like A's: no transposing LDS read is needed.
+template <int ES, bool EDGE, bool TB = false> __global__ __launch_bounds__(G_THREADS) void gemm_tile256_kernel(GemmParams p) {
   typedef MfmaOp<ES> Op;
   typedef typename Op::acc_t acc_t;
   constexpr int BK = G_KBYTES / ES;        // K elements per stage
@@ -320,7 +322,7 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
     int row = a_row0 + 64 * i;
     a_st[i] = row * 128 + ((a_c ^ ((row >> 1) & 7)) << 4);
     int krow = b_row0 + B_ROW_STEP * i;
-    b_st[i] = 32768 + krow * B_ROW_BYTES + ((b_c ^ ((krow % RG) * CW)) << 4);
+    b_st[i] = TB ? 32768 + a_st[i] : 32768 + krow * B_ROW_BYTES + ((b_c ^ ((krow % RG) * CW)) << 4);
   }
 
   // ---- LDS read offsets of this lane's MFMA fragments
@@ -340,6 +342,8 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
       int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
       int krow_lane = (ES == 2 ? 8 : 16) * (g >> 1) + kk;
       b_ld[j] = 32768 + krow_lane * B_ROW_BYTES + ((chunk ^ (kk * CW)) << 4) + sub;
+      if (TB) // row of the tile; + the k-step's chunk (swizzled like A's)
+        b_ld[j] = 32768 + (wn * 64 + j * 32 + l32) * 128;
     }
   }
 
@@ -363,8 +367,9 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
       ra[i] = load_chunk<EDGE>(Ab, m0 + a_row0 + 64 * i, p.M, kb + a_c * 16, k_bytes, lda_b);
 #pragma unroll
     for (int i = 0; i < 4; i++)
-      rb[i] = load_chunk<EDGE>(Bb, (int64_t)kt * BK + b_row0 + B_ROW_STEP * i, p.K, n0 * ES + b_c * 16,
-                               p.N * ES, ldb_b);
+      rb[i] = TB ? load_chunk<EDGE>(Bb, n0 + a_row0 + 64 * i, p.N, kb + a_c * 16, k_bytes, ldb_b)
+                 : load_chunk<EDGE>(Bb, (int64_t)kt * BK + b_row0 + B_ROW_STEP * i, p.K, n0 * ES + b_c * 16,
+                                    p.N * ES, ldb_b);
   };
   auto lstore = [&](int stage) {
     char *s = smem + stage * G_STAGE_BYTES;
@@ -402,9 +407,13 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
         af[i] = *reinterpret_cast<const uint4 *>(s + a_ld[ks] + i * 4096);
 #pragma unroll
       for (int j = 0; j < 2; j++) {
-        uint2 lo = Op::tr_read(s + b_ld[j] + ks * 8192);
-        uint2 hi = Op::tr_read(s + b_ld[j] + ks * 8192 + 2048);
-        bf[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        if (TB) {
+          bf[j] = *reinterpret_cast<const uint4 *>(s + b_ld[j] + (((2 * ks + lh) ^ sw) << 4));
+        } else {
+          uint2 lo = Op::tr_read(s + b_ld[j] + ks * 8192);
+          uint2 hi = Op::tr_read(s + b_ld[j] + ks * 8192 + 2048);
+          bf[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        }
       }
 #pragma unroll
       for (int j = 0; j < 2; j++)
@@ -441,7 +450,8 @@ template <int ES, bool EDGE> __global__ __launch_bounds__(G_THREADS) void gemm_t
 
 // SPLIT (split-K on a short A): only the first `mi` 32-row tiles of a wave hold rows of A; the others are
 // neither read from LDS nor multiplied.
-template <int ES, int KS, int WJ = 2, bool SPLIT = false> struct FastGemm {
+// TB (B stored [N,K]): the B tile is staged and read exactly like the A tile.
+template <int ES, int KS, int WJ = 2, bool SPLIT = false, bool TB = false> struct FastGemm {
   static constexpr int NWAVES = 16 / WJ; // 8 or 4
   int mi = 4;
   typedef MfmaOp<ES> Op;
@@ -463,7 +473,7 @@ template <int ES, int KS, int WJ = 2, bool SPLIT = false> struct FastGemm {
   static __device__ __forceinline__ int a_swz(int row) { return KS == 4 ? ((row >> 1) & 7) : ((row >> 2) & 3); }
 
   uint32_t a_src[NDMA], b_src[NDMA]; // per-lane byte offsets of this wave's DMA instructions
-  uint32_t a_ld[KS], b_ld[WJ];       // fragment read offsets
+  uint32_t a_ld[KS], b_ld[TB ? KS : WJ]; // fragment read offsets
   uint32_t a_xor;
   int wave_u; // wave id, wave-uniform
 
@@ -492,9 +502,13 @@ template <int ES, int KS, int WJ = 2, bool SPLIT = false> struct FastGemm {
     }
 #pragma unroll
     for (int j = 0; j < WJ; j++) {
-      uint2 lo = Op::tr_read(s + b_ld[j] + ks * 8192);
-      uint2 hi = Op::tr_read(s + b_ld[j] + ks * 8192 + 2048);
-      bf[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      if (TB) {
+        bf[j] = *reinterpret_cast<const uint4 *>(s + A_BYTES + b_ld[ks] + j * 32 * KB);
+      } else {
+        uint2 lo = Op::tr_read(s + b_ld[j] + ks * 8192);
+        uint2 hi = Op::tr_read(s + b_ld[j] + ks * 8192 + 2048);
+        bf[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
     }
   }
 
@@ -558,9 +572,9 @@ template <int ES, int KS, int WJ = 2, bool SPLIT = false> struct FastGemm {
   }
 };
 
-template <int ES, int KS, int WJ, bool SPLIT = false>
+template <int ES, int KS, int WJ, bool SPLIT = false, bool TB = false>
 __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmParams p) {
-  typedef FastGemm<ES, KS, WJ, SPLIT> FG;
+  typedef FastGemm<ES, KS, WJ, SPLIT, TB> FG;
   typedef typename FG::acc_t acc_t;
   constexpr int NST = FG::NST;
   // ring of NST stages (128 KiB); the epilogue reuses the whole array as 8 x 18 KiB staging regions
@@ -602,7 +616,7 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
     // B: B_ROWS_PER_DMA k-rows; lane -> (krow, physical chunk)
     int krow = (wave * FG::NDMA + i) * FG::B_ROWS_PER_DMA + lane / FG::B_CPR;
     int cb = (lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW);
-    g.b_src[i] = (uint32_t)(krow * ldb_b + cb * 16);
+    g.b_src[i] = TB ? (uint32_t)(row * ldb_b + c * 16) : (uint32_t)(krow * ldb_b + cb * 16);
   }
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) {
@@ -613,13 +627,21 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
     const int gq = lane >> 4, i16 = lane & 15;
     const int kk = ES == 2 ? (i16 >> 2) : (i16 >> 1);
     const int cc = ES == 2 ? (i16 & 3) : (i16 & 1);
+    if constexpr (TB) {
 #pragma unroll
-    for (int j = 0; j < WJ; j++) {
-      const int nb = wn * WJ + j; // 32-column block of the tile
-      int chunk = ES == 2 ? (nb * 4 + 2 * (gq & 1) + (cc >> 1)) : (nb * 2 + (gq & 1));
-      int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
-      int krow_lane = (ES == 2 ? 8 : 16) * (gq >> 1) + kk;
-      g.b_ld[j] = FG::A_BYTES + krow_lane * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + sub;
+      for (int ks = 0; ks < KS; ks++) {
+        int row = wn * 32 * WJ + l32; // + j*32
+        g.b_ld[ks] = row * FG::KB + (((2 * ks + lh) ^ FG::a_swz(row)) << 4);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < WJ; j++) {
+        const int nb = wn * WJ + j; // 32-column block of the tile
+        int chunk = ES == 2 ? (nb * 4 + 2 * (gq & 1) + (cc >> 1)) : (nb * 2 + (gq & 1));
+        int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
+        int krow_lane = (ES == 2 ? 8 : 16) * (gq >> 1) + kk;
+        g.b_ld[j] = FG::A_BYTES + krow_lane * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + sub;
+      }
     }
   }
 
@@ -632,13 +654,13 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
       for (int r = 0; r < 16; r++)
         acc[j][i][r] = 0;
 
-  const int64_t b_step = (int64_t)FG::BK * ldb_b;
+  const int64_t b_step = TB ? (int64_t)FG::KB : (int64_t)FG::BK * ldb_b; // bytes from one k-block of B to the next
   // K slice of this workgroup in ring groups (NST stages each): slices differ by at most one group
   const int groups = (int)(p.K / FG::BK) / NST, nsl = SPLIT ? p.splits : 1;
   const int g0 = (int)((int64_t)slice * groups / nsl), g1 = (int)((int64_t)(slice + 1) * groups / nsl);
   const int KT = (g1 - g0) * NST;
   const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b + (int64_t)g0 * NST * FG::KB; // first k-block; KB bytes each
-  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * ES + (int64_t)g0 * NST * b_step;   // BK rows per k-block
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + (TB ? n0 * ldb_b : n0 * ES) + (int64_t)g0 * NST * b_step;
 
   uint4 a0[4], b0[WJ], a1[4], b1[WJ];
   // prologue: request k-blocks 0 .. NST-2 (KT is a positive multiple of NST), wait for block 0
@@ -778,7 +800,9 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   const int KGROUP = 256 / ES; // K elements of one trip round the LDS ring
   const bool fast_but_m = p.N % G_BN == 0 && p.K % KGROUP == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
                           (p.lda * ES) % 16 == 0 && (p.ldb * ES) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
-                          p.lda * ES * G_BM < (int64_t)1 << 31 && p.ldb * ES * BK < (int64_t)1 << 31;
+                          p.lda * ES * G_BM < (int64_t)1 << 31 && p.ldb * ES * (p.trans_b ? G_BN : BK) < (int64_t)1 << 31;
+  if (p.trans_b && ES != 2)
+    return 3;
   bool fast = fast_but_m && p.M % G_BM == 0;
   p.splits = 0;
   p.partial = nullptr;
@@ -798,8 +822,14 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
         return 5;
       p.splits = splits;
       p.partial = ws;
-      hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true>), dim3((unsigned)(tiles_n * splits)),
-                         dim3(1024 / G_FAST_WJ), 0, stream, p);
+      if constexpr (ES == 2) {
+        if (p.trans_b)
+          hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true, true>),
+                             dim3((unsigned)(tiles_n * splits)), dim3(1024 / G_FAST_WJ), 0, stream, p);
+        else
+          hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true>), dim3((unsigned)(tiles_n * splits)),
+                             dim3(1024 / G_FAST_WJ), 0, stream, p);
+      }
       const unsigned rblocks = (unsigned)((p.M * (p.N / 4) + 255) / 256);
       switch (p.act) {
       case ACT_RELU:
@@ -824,6 +854,16 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   if (p.group_m <= 0)
     p.group_m = 4;
   dim3 grid((unsigned)nblk), block(G_THREADS);
+  if constexpr (ES == 2) {
+    if (p.trans_b) {
+      if (fast)
+        hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, false, true>), grid, dim3(1024 / G_FAST_WJ), 0,
+                           stream, p);
+      else
+        hipLaunchKernelGGL((gemm_tile256_kernel<ES, true, true>), grid, block, 0, stream, p);
+      return hipGetLastError() == hipSuccess ? 0 : 5;
+    }
+  }
   if (fast)
     hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ>), grid, dim3(1024 / G_FAST_WJ), 0, stream, p);
   else

@@ -56,6 +56,17 @@ int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, 
                    int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
 
 /*
+ * The same with B stored transposed: Bt [N,K] row-major (k contiguous, ldb
+ * elements between its rows), C = epilogue(A . Bt^T).  Takes over
+ * linalg.matmul_transpose_b / onednn_graph.matmul{transpose_b} on bf16
+ * (lib/gc/Transforms/OneDNNGraphToLinalg.cpp:421-499; the weights of
+ * test/benchgc/cases/llama2.mlir are stored this way).  No transposed copy is
+ * made: the tile of Bt is staged and read like the tile of A.
+ */
+int gcmi_gemm_bf16_nt(const void *A, const void *Bt, void *C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                      int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
+
+/*
  * 8-bit matmul with s32 accumulation and fused dequantise epilogue.
  * Takes over: the u8/s8 brgemm (lib/gc/ExecutionEngine/CPURuntime/Microkernel/
  * BrgemmNaive.cpp:102-140) under the deep-tile nest, the asymmetric-activation

@@ -200,23 +200,23 @@ def test_attention_partition(ga, orc, wl, dev, D, with_mask, scale_op):
 
 
 def test_constant_transposed_weight_is_prepared_once(ga, orc, wl, dev):
-    """x[32,512] . W^T with W stored [N,K] (transpose_b, as the reference's llama2 case stores its weights).
-    With property_type "constant" the row-major copy of W is made in the first execute only: a second execute
-    that is handed a different buffer under the same id still multiplies by the first contents.  Without the
-    property the copy is redone every time."""
-    M, K, N = 32, 512, 768
+    """W^T . x with W stored [K,M] (transpose_a): the bf16 kernel reads its first operand row-major, so a
+    transposed copy of W is made.  With property_type "constant" that happens in the first execute only: a second
+    execute that is handed a different buffer under the same id still multiplies by the first contents.  Without
+    the property the copy is redone every time."""
+    M, K, N = 768, 512, 32
     torch.manual_seed(21)
-    x = (torch.randn(M, K) * 0.5).to(torch.bfloat16)
-    W = (torch.randn(N, K) * 0.05).to(torch.bfloat16)
-    W2 = (torch.randn(N, K) * 0.05).to(torch.bfloat16)
+    x = (torch.randn(K, N) * 0.5).to(torch.bfloat16)
+    W = (torch.randn(K, M) * 0.05).to(torch.bfloat16)
+    W2 = (torch.randn(K, M) * 0.05).to(torch.bfloat16)
 
     def graph(prop):
-        return ga._graph([{"kind": "MatMul", "attrs": {"transpose_b": {"type": "bool", "value": 1}},
-                           "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [N, K], property_type=prop)],
+        return ga._graph([{"kind": "MatMul", "attrs": {"transpose_a": {"type": "bool", "value": 1}},
+                           "inputs": [ga._t(0, "bf16", [K, M], property_type=prop), ga._t(1, "bf16", [K, N])],
                            "outputs": [ga._t(2, "bf16", [M, N])]}], [0, 1], [2])
 
-    ref1 = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(x), wl.bf16_bits(W.t().contiguous())))
-    ref2 = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(x), wl.bf16_bits(W2.t().contiguous())))
+    ref1 = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(W.t().contiguous()), wl.bf16_bits(x)))
+    ref2 = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(W2.t().contiguous()), wl.bf16_bits(x)))
     for prop, second in (("constant", ref1), ("variable", ref2)):
         comp = ga.Compiler()
         st, exe = comp.compile(graph(prop))
@@ -226,11 +226,29 @@ def test_constant_transposed_weight_is_prepared_once(ga, orc, wl, dev):
         out = torch.zeros(M, N, dtype=torch.bfloat16)
         for Wt, ref in ((W, ref1), (W2, second)):
             for pass_device in (False, True):
-                xs, ws = (x.to(dev), Wt.to(dev)) if pass_device else (x, Wt)
-                assert exe.execute([(0, xs), (1, ws)], [(2, out)]) == 0
-                assert_close(ref, out.float().numpy(), 1e-2, "transpose_b %s" % prop)
+                ws, xs = (Wt.to(dev), x.to(dev)) if pass_device else (Wt, x)
+                assert exe.execute([(0, ws), (1, xs)], [(2, out)]) == 0
+                assert_close(ref, out.float().numpy(), 1e-2, "transpose_a %s" % prop)
         exe.close()
         comp.close()
+
+
+def test_transposed_b_weight_needs_no_copy(ga, orc, wl, dev):
+    """x[32,512] . W^T with W stored [N,K] (transpose_b, as the reference's llama2 case stores its weights):
+    one GEMM launch that reads W as it lies."""
+    M, K, N = 32, 512, 768
+    torch.manual_seed(22)
+    x = (torch.randn(M, K) * 0.5).to(torch.bfloat16)
+    W = (torch.randn(N, K) * 0.05).to(torch.bfloat16)
+    g = ga._graph([{"kind": "MatMul", "attrs": {"transpose_b": {"type": "bool", "value": 1}},
+                    "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [N, K])],
+                    "outputs": [ga._t(2, "bf16", [M, N])]}], [0, 1], [2])
+    st, plan = ga.explain(g)
+    assert st == 0 and [ln for ln in plan.splitlines() if not ln.startswith("arena")] == ["gemm_bf16: MatMul"]
+    out = torch.zeros(M, N, dtype=torch.bfloat16)
+    _run(ga, g, [(0, x), (1, W)], [(2, out)])
+    ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(x), wl.bf16_bits(W.t().contiguous())))
+    assert_close(ref, out.float().numpy(), 1e-2, "transpose_b")
 
 
 def test_chain_of_four_matmuls_with_shared_temporaries(ga, orc, wl, dev):

@@ -215,3 +215,42 @@ def test_short_a_takes_split_k(gc, orc, wl, dev, M, N, K, act, with_bias, out_f3
                          out_dtype=gc.F32 if out_f32 else gc.BF16)
     torch.cuda.synchronize()
     assert torch.equal(out, again)  # fixed summation order: reruns agree bit for bit
+
+
+NT_SHAPES = [(256, 256, 128), (512, 768, 256), (300, 200, 100), (257, 511, 129), (1, 7, 5), (33, 1, 64), (128, 256, 8),
+             (32, 4096, 4096), (1, 1024, 2048), (32, 11008, 4096)]
+
+
+@pytest.mark.parametrize("M,N,K", NT_SHAPES)
+def test_bf16_gemm_transposed_b(gc, orc, wl, dev, M, N, K):
+    """B stored [N,K] (linalg.matmul_transpose_b): against the oracle on A . Bt^T, and bit for bit against the
+    [K,N] kernel on a transposed copy -- both read the same products in the same order.  Covers whole-tile, ragged
+    and split-K (short A) shapes."""
+    torch.manual_seed(4)
+    A = (torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev)
+    Bt = (torch.randn(N, K) * 0.5).to(torch.bfloat16).to(dev)
+    bias = torch.randn(N).to(torch.bfloat16).to(dev)
+    B = Bt.t().contiguous()
+    for b, act, odt in [(None, None, gc.BF16), (bias, "relu", gc.BF16), (bias, "gelu_erf", gc.F32)]:
+        nt = gc.gemm_bf16_nt(A, Bt, b, act, odt)
+        nn = gc.gemm_bf16(A, B, b, act, odt)
+        torch.cuda.synchronize()
+        assert torch.equal(nt, nn), "NT differs from NN on the transposed copy (%s, %s)" % (act, odt)
+    if M * N * K <= 1 << 24:
+        ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A.cpu()), wl.bf16_bits(B.cpu())))
+        out = gc.gemm_bf16_nt(A, Bt)
+        torch.cuda.synchronize()
+        assert_close(ref, out.float().cpu().numpy(), 1e-2, "bf16 NT %dx%dx%d" % (M, N, K))
+
+
+def test_bf16_gemm_transposed_b_strided_rows(gc, dev):
+    """Rows of Bt further apart than K (a weight that is a slice of a wider one)."""
+    torch.manual_seed(6)
+    M, N, K = 256, 512, 256
+    A = torch.randn(M, K, device=dev).bfloat16()
+    wide = torch.randn(N, K + 64, device=dev).bfloat16()
+    Bt = wide[:, 8:8 + K]  # row stride K+64, start offset 16 bytes
+    out = gc.gemm_bf16_nt(A, Bt)
+    ref = gc.gemm_bf16(A, Bt.t().contiguous())
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
