@@ -97,7 +97,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32,decode,api")
+    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32,decode,api,block")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the 4096^3 GEMM the CPU baseline computes")
     ap.add_argument("--mha-mode", default="both", choices=["both", "skip", "every"],
                     help="attention: time the default entry point (masked key blocks skipped), the every-block mode, or both")
@@ -320,6 +320,61 @@ def main():
                                              "unit": "TFLOP/s", "note": "pageable host buffers: 64 MiB in, 32 MiB out per call"}}
         log("api execute: %.4f ms with device pointers, %.2f ms with host pointers" % (t_dev, t_host))
         del Ad, Bd, Cd
+
+    # ---------------- the llama-2 decoder MLP block of the reference's benchgc case, as textual MLIR through the API
+    if want("block"):
+        ga = importlib.import_module("graph_compiler_amd.graph_api")
+        mlm = importlib.import_module("graph_compiler_amd.mlir_modules")
+        T, H, Fd = 32, 4096, 11008
+        comp = ga.Compiler()
+        st, exe = comp.compile_mlir(mlm.decoder_mlp_block(T, H, Fd))
+        if st:
+            log("bench.py: compile_mlir of the decoder block failed with status %d: %s" %
+                (st, ga.api().dnnl_graph_compiler_last_error().decode()))
+            sys.exit(4)
+        bf = torch.bfloat16
+        torch.manual_seed(7)
+        rn = lambda *sh: torch.randn(*sh, device=dev)  # noqa: E731
+        nsets = 3  # 3 x 304 MB of weights: beyond the 256 MB Infinity Cache in rotation
+        sets = []
+        for _ in range(nsets):
+            sets.append([rn(1, T, H).to(bf), (rn(H, H) / H ** 0.5).to(bf), rn(1, T, H).to(bf),
+                         torch.full((1,), 1e-5, device=dev), (1 + 0.1 * rn(H)).to(bf), (rn(Fd, H) / H ** 0.5).to(bf),
+                         (rn(Fd, H) / H ** 0.5).to(bf), (rn(H, Fd) / Fd ** 0.5).to(bf), torch.full((1,), 1e-5, device=dev),
+                         (1 + 0.1 * rn(H)).to(bf)])
+        o1 = torch.empty(1, T, H, device=dev, dtype=bf)
+        o2 = torch.empty(1, T, H, device=dev, dtype=bf)
+        st_plan, plan = ga.explain_mlir(mlm.decoder_mlp_block(T, H, Fd))
+        n_launch = len([ln for ln in plan.splitlines() if not ln.startswith(("arena", "target"))])
+
+        def run_block(i):
+            rc = exe.execute(list(enumerate(sets[i % nsets])), [(10, o1), (11, o2)])
+            if rc:
+                raise RuntimeError("execute -> %d" % rc)
+
+        for i in range(3):
+            run_block(i)
+        torch.cuda.synchronize()
+        n = max(12, K // 2)
+        t0 = time.perf_counter()
+        for i in range(n):
+            run_block(i)
+        torch.cuda.synchronize()
+        t_blk = (time.perf_counter() - t0) * 1e3 / n
+        exe.close()
+        comp.close()
+        byts = 2.0 * (H * H + 3 * H * Fd) + 2.0 * 4 * T * H
+        gbs = byts / (t_blk * 1e-3) / 1e9
+        others["mlir_llama2_mlp_block"] = {
+            "workload": "test/benchgc/cases/llama2.mlir shape (32 tokens, hidden 4096, ffn 11008): o-proj + residual, RMSNorm, "
+                        "gated FFN, residual, RMSNorm; textual MLIR through compile_mlir/execute with device pointers; wall "
+                        "clock per execute (returns after completion); algorithmic bytes = the four weights + activations once",
+            "launches_per_execute": n_launch, "ms_per_execute": round(t_blk, 4),
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
+        log("mlir llama2 block: %.4f ms per execute, %d launches, %.0f GB/s of weights" % (t_blk, n_launch, gbs))
+        del sets
+        torch.cuda.empty_cache()
 
     if args.copy_calibration:
         src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <set>
@@ -14,6 +15,7 @@
 extern "C" {
 int gcmi_launch_eltwise(const gcmi::EltParams *p, hipStream_t stream);
 int gcmi_launch_reduce(const gcmi::ReduceParams *p, hipStream_t stream);
+int gcmi_launch_fused(const gcmi::FusedParams *p, hipStream_t stream);
 int gcmi_launch_softmax(const gcmi::SoftmaxParams *p, hipStream_t stream);
 }
 
@@ -184,6 +186,8 @@ void Executable::layout_arena() {
   for (int i = 0; i < (int)steps_.size(); i++) {
     const Step &s = steps_[i];
     for (int slot : {s.a, s.b, s.c, s.out, s.bias, s.mask, s.aux, s.scale_slot, s.scales_slot, s.zps_slot})
+      touch(slot, i);
+    for (int slot : s.f_in)
       touch(slot, i);
     if (s.once || (s.kind == Step::ColSum && s.op == 1))
       if (s.out >= 0)
@@ -617,6 +621,11 @@ void Executable::plan() {
     emit_at[last] = v;
   }
 
+  // GCMI_NO_POINTWISE_FUSION=1: one launch per op, for comparing the two ways of running a graph
+  // (sums still go to the row-sum kernel, alone)
+  const char *no_fuse = getenv("GCMI_NO_POINTWISE_FUSION");
+  plan_fusion(skip, claimed, emit_at, !(no_fuse && no_fuse[0] == '1'));
+
   // ---- emission pass, in op order
   for (size_t i = 0; i < n; i++) {
     if (skip[i])
@@ -628,6 +637,371 @@ void Executable::plan() {
       continue;
     }
     plan_generic(g_.ops[i]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Point-wise fusion: chains and DAGs of element-wise ops of one shape become one launch (a small register program,
+// gcmi::FusedParams), and such a group in front of a ReduceSum/ReduceMean is evaluated inside the reduction.  This
+// is the part of the reference's producer/consumer fusion (lib/gc/Transforms/IterativeTilingAndFusion.cpp:585-611,
+// 652-741) that is not already a GEMM epilogue.  A value leaves the chip only when something other than a
+// same-shaped point-wise op or a reduction reads it (a MatMul, a reshape, the caller); values with several
+// point-wise readers are recomputed in each group rather than stored.
+namespace {
+int pointwise_code(const Op &op) {
+  const std::string &k = op.kind;
+  if (k == "Add")
+    return gcmi::ELT_ADD;
+  if (k == "Subtract")
+    return gcmi::ELT_SUB;
+  if (k == "Multiply")
+    return gcmi::ELT_MUL;
+  if (k == "Divide")
+    return gcmi::ELT_DIV;
+  if (k == "Maximum")
+    return gcmi::ELT_MAX;
+  if (k == "ReLU")
+    return gcmi::ELT_RELU;
+  if (k == "Sigmoid")
+    return gcmi::ELT_SIGMOID;
+  if (k == "GELU")
+    return act_of(op) == GCMI_ACT_GELU_TANH ? gcmi::ELT_GELU_TANH : gcmi::ELT_GELU_ERF;
+  if (k == "Pow")
+    return gcmi::ELT_POW;
+  if (k == "Typecast" || k == "TypeCast")
+    return gcmi::ELT_COPY;
+  if (k == "Exp")
+    return gcmi::ELT_EXP;
+  if (k == "Neg")
+    return gcmi::ELT_NEG;
+  return -1;
+}
+bool storage_float(DT d) { return d == DT::f32 || d == DT::bf16 || d == DT::f16; }
+} // namespace
+
+std::vector<int64_t> squeezed(const std::vector<int64_t> &shape) {
+  std::vector<int64_t> r;
+  for (auto d : shape)
+    if (d != 1)
+      r.push_back(d);
+  return r;
+}
+
+void Executable::plan_fusion(std::vector<bool> &skip, const std::vector<bool> &claimed,
+                             std::map<size_t, std::vector<Step>> &emit_at, bool groups) {
+  const size_t n = g_.ops.size();
+  auto T = [&](size_t id) -> const LTensor & { return g_.tensors.at(id); };
+  // a reshape is a view of its source: readers of the view are readers of the source, and shapes are compared
+  // without their unit dims ([1,32,4096] and [32,4096] walk memory alike)
+  auto base = [&](size_t t) {
+    while (T(t).alias_of >= 0)
+      t = (size_t)T(t).alias_of;
+    return t;
+  };
+  auto view_op = [&](size_t i) { return g_.ops[i].kind == "Reshape"; };
+  std::map<size_t, std::vector<size_t>> consumers;
+  std::map<size_t, size_t> producer;
+  for (size_t i = 0; i < n; i++) {
+    if (view_op(i))
+      continue;
+    for (auto id : g_.ops[i].in)
+      consumers[base(id)].push_back(i);
+    for (auto id : g_.ops[i].out)
+      producer[id] = i;
+  }
+  std::set<size_t> outs;
+  for (auto id : g_.output_ids)
+    outs.insert(base(id));
+
+  // ops no GEMM or attention group has taken (as the matching pass left them: this pass must not see its own marks)
+  std::vector<bool> is_free(n);
+  for (size_t i = 0; i < n; i++)
+    is_free[i] = !skip[i] && !claimed[i] && !emit_at.count(i);
+  auto fusable = [&](size_t i) {
+    const Op &o = g_.ops[i];
+    if (!groups || !is_free[i] || pointwise_code(o) < 0 || o.out.size() != 1)
+      return false;
+    const LTensor &ot = T(o.out[0]);
+    if (!storage_float(ot.dt) || ot.shape.size() > (size_t)gcmi::ELT_MAX_RANK || !is_dense(ot))
+      return false;
+    for (auto id : o.in)
+      if (!storage_float(T(id).dt) || !is_dense(T(id)))
+        return false;
+    return true;
+  };
+  auto reduction = [&](size_t i) {
+    const Op &o = g_.ops[i];
+    if (!is_free[i] || !(o.kind == "ReduceSum" || o.kind == "ReduceMean"))
+      return false;
+    const LTensor &it = T(o.in[0]);
+    return storage_float(it.dt) && storage_float(T(o.out[0]).dt) && it.shape.size() <= (size_t)gcmi::ELT_MAX_RANK &&
+           is_dense(it);
+  };
+  std::set<size_t> forced; // tensors a group could not take in (size limits): they are stored after all
+  // does anything read this tensor from memory?
+  auto stored = [&](size_t t) {
+    if (outs.count(t) || forced.count(t))
+      return true;
+    auto it = consumers.find(t);
+    if (it == consumers.end() || it->second.empty())
+      return true;
+    for (size_t c : it->second) {
+      if (fusable(c) && squeezed(T(g_.ops[c].out[0]).shape) == squeezed(T(t).shape))
+        continue;
+      if (reduction(c))
+        continue;
+      return true;
+    }
+    return false;
+  };
+
+  std::set<size_t> taken_reductions;
+  for (size_t i = n; i-- > 0;) {
+    const Op &root = g_.ops[i];
+    const bool red_root = reduction(i);
+    if (red_root && taken_reductions.count(i))
+      continue;
+    if (!red_root && !(fusable(i) && stored(base(root.out[0]))))
+      continue;
+    // the group: point-wise ops on the row shape (`post`; without a sum this is the whole group), optionally a
+    // sum, and point-wise ops on the full shape in front of the sum (`pre`)
+    std::set<size_t> post, pre;
+    long red = red_root ? (long)i : -1;
+    std::vector<int64_t> row_dims = squeezed(T(root.out[0]).shape), full_dims;
+    if (red_root)
+      full_dims = squeezed(T(root.in[0]).shape);
+    // tensors (canonical) currently read from memory, per phase
+    std::vector<std::pair<size_t, int>> inputs; // phase 0 = pre, 1 = post
+    auto add_input = [&](std::vector<std::pair<size_t, int>> &v, size_t t, int phase) {
+      std::pair<size_t, int> e(base(t), phase);
+      if (std::find(v.begin(), v.end(), e) == v.end())
+        v.push_back(e);
+    };
+    if (red_root) {
+      add_input(inputs, root.in[0], 0);
+    } else {
+      post.insert(i);
+      for (auto id : root.in)
+        add_input(inputs, id, 1);
+    }
+    auto inside = [&](size_t t, int phase) {
+      auto pit = producer.find(t);
+      if (pit == producer.end())
+        return false;
+      if (phase == 1 && red >= 0 && (long)pit->second == red)
+        return true;
+      return (phase == 1 ? post : pre).count(pit->second) > 0;
+    };
+    std::set<std::pair<size_t, int>> declined;
+    for (bool grew = true; grew;) {
+      grew = false;
+      for (size_t k = 0; k < inputs.size(); k++) {
+        const size_t t = inputs[k].first;
+        const int phase = inputs[k].second;
+        auto pit = producer.find(t);
+        if (declined.count(inputs[k]) || pit == producer.end() || T(t).has_splat || stored(t))
+          continue;
+        const size_t po = pit->second;
+        const bool take_sum = phase == 1 && red < 0 && reduction(po) && consumers[t].size() == 1 &&
+                              squeezed(T(t).shape) == row_dims;
+        const bool take_op = fusable(po) && squeezed(T(t).shape) == (phase == 1 ? row_dims : full_dims);
+        if (!take_sum && !take_op)
+          continue;
+        std::vector<std::pair<size_t, int>> next;
+        for (auto &x : inputs)
+          if (x != inputs[k])
+            next.push_back(x);
+        const int in_phase = take_sum ? 0 : phase;
+        for (auto x : g_.ops[po].in)
+          if (!inside(base(x), in_phase))
+            add_input(next, x, in_phase);
+        const size_t count = post.size() + pre.size() + (red >= 0 || take_sum ? 1 : 0) + (take_sum ? 0 : 1);
+        // two inputs of slack: one tensor read through different broadcasts counts once here and twice below
+        if (count > (size_t)gcmi::FUSED_MAX_INS || next.size() + 2 > (size_t)gcmi::FUSED_MAX_IN) {
+          declined.insert(inputs[k]);
+          forced.insert(t);
+          continue;
+        }
+        if (take_sum) {
+          red = (long)po;
+          full_dims = squeezed(T(g_.ops[po].in[0]).shape);
+        } else {
+          (phase == 1 ? post : pre).insert(po);
+        }
+        inputs = next;
+        grew = true;
+        break;
+      }
+    }
+    if (red < 0 && post.size() == 1)
+      continue; // a lone op: the plain element-wise kernel
+
+    // ---- iteration space: [kept dims..., reduced dims...] of the sum's input, or the point-wise shape
+    Step s;
+    s.kind = Step::Fused;
+    std::vector<int> place; // position among the non-unit dims of the full shape -> iteration dim
+    size_t n_kept = row_dims.size();
+    if (red >= 0) {
+      const Op &ro = g_.ops[(size_t)red];
+      const std::vector<int64_t> &fs = T(ro.in[0]).shape;
+      std::vector<int64_t> axes;
+      if (ro.attrs.count("axes"))
+        axes = ro.attrs.at("axes").ia;
+      auto ca = canonical_axes(axes, (int64_t)fs.size());
+      std::vector<int64_t> kept, reduced;
+      std::vector<bool> is_red;
+      for (size_t d = 0; d < fs.size(); d++) {
+        if (fs[d] == 1)
+          continue;
+        bool r = std::find(ca.begin(), ca.end(), (int64_t)d) != ca.end();
+        (r ? reduced : kept).push_back(fs[d]);
+        is_red.push_back(r);
+      }
+      n_kept = kept.size();
+      place.resize(is_red.size());
+      int nk = 0, nr = 0;
+      for (size_t q = 0; q < is_red.size(); q++)
+        place[q] = is_red[q] ? (int)n_kept + nr++ : nk++;
+      s.dims = kept;
+      s.dims.insert(s.dims.end(), reduced.begin(), reduced.end());
+      s.n_red = 1;
+      for (auto d : reduced)
+        s.n_red *= d;
+      s.mean = ro.kind == "ReduceMean";
+      if (kept != squeezed(T(ro.out[0]).shape))
+        throw std::logic_error("reduction whose result shape does not match its kept dims");
+    } else {
+      s.dims = row_dims;
+    }
+    if (s.dims.size() > (size_t)gcmi::ELT_MAX_RANK)
+      throw std::logic_error("tensor rank above 6 is not supported");
+
+    // strides of operand x, as the member whose result has shape `ms` reads it, over the iteration dims
+    auto strides_of = [&](size_t x, const std::vector<int64_t> &ms, int phase) {
+      const LTensor &t = T(x);
+      std::vector<int64_t> st = dense_strides(t.shape), full(ms.size(), 0), it(s.dims.size(), 0);
+      if (!t.has_splat)
+        for (size_t d = 0; d < t.shape.size(); d++)
+          full[ms.size() - t.shape.size() + d] = t.shape[d] == 1 ? 0 : st[d];
+      size_t q = 0;
+      for (size_t d = 0; d < ms.size(); d++) {
+        if (ms[d] == 1)
+          continue;
+        const size_t pos = (phase == 0 && red >= 0) ? (size_t)place[q] : q; // post-phase dims are the leading (kept) ones
+        it[pos] = full[d];
+        q++;
+      }
+      return it;
+    };
+    struct In {
+      size_t tensor; // as named by the reader (a view keeps its own shape)
+      int phase;
+      std::vector<int64_t> str;
+    };
+    std::vector<In> ins_pre, ins_post;
+    std::map<size_t, int> reg_of_op;   // member op (or the sum) -> register, filled as instructions are numbered
+    std::vector<size_t> order_pre(pre.begin(), pre.end()), order_post(post.begin(), post.end());
+    // pass 1: collect inputs
+    auto operand_input = [&](size_t x, const std::vector<int64_t> &ms, int phase) -> int {
+      std::vector<In> &v = phase == 0 ? ins_pre : ins_post;
+      std::vector<int64_t> st = strides_of(x, ms, phase);
+      for (size_t k = 0; k < v.size(); k++)
+        if (base(v[k].tensor) == base(x) && v[k].str == st)
+          return (int)k;
+      v.push_back({x, phase, st});
+      return (int)v.size() - 1;
+    };
+    struct Use {
+      bool is_input;
+      int index;    // input index within its phase, or producing op
+      size_t op;
+    };
+    auto classify = [&](size_t x, const std::vector<int64_t> &ms, int phase) {
+      Use u{};
+      const size_t b = base(x);
+      if (inside(b, phase)) {
+        u.is_input = false;
+        u.op = producer.at(b);
+      } else {
+        u.is_input = true;
+        u.index = operand_input(x, ms, phase);
+      }
+      return u;
+    };
+    std::vector<std::vector<Use>> uses_pre, uses_post;
+    for (size_t m : order_pre) {
+      std::vector<Use> u;
+      for (auto x : g_.ops[m].in)
+        u.push_back(classify(x, T(g_.ops[m].out[0]).shape, 0));
+      uses_pre.push_back(u);
+    }
+    Use sum_use{};
+    if (red >= 0)
+      sum_use = classify(g_.ops[(size_t)red].in[0], T(g_.ops[(size_t)red].in[0]).shape, 0);
+    for (size_t m : order_post) {
+      std::vector<Use> u;
+      for (auto x : g_.ops[m].in)
+        u.push_back(classify(x, T(g_.ops[m].out[0]).shape, 1));
+      uses_post.push_back(u);
+    }
+    const int n_in_pre = (int)ins_pre.size(), n_in = n_in_pre + (int)ins_post.size();
+    if (n_in > gcmi::FUSED_MAX_IN || n_in < 1)
+      throw std::logic_error("point-wise fusion: input count out of range");
+    for (auto &v : {ins_pre, ins_post})
+      for (auto &e : v) {
+        s.f_in.push_back(slot_for(e.tensor));
+        s.f_in_dt.push_back(dt_dnnl(T(e.tensor).dt));
+        s.f_str.push_back(e.str);
+      }
+    auto reg_of = [&](const Use &u, int phase) {
+      return u.is_input ? (phase == 0 ? u.index : n_in_pre + u.index) : reg_of_op.at(u.op);
+    };
+    std::string names_pre, names_post;
+    auto emit_member = [&](size_t m, const std::vector<Use> &u, int phase, std::string &names) {
+      const Op &o = g_.ops[m];
+      Step::FIns f;
+      f.op = pointwise_code(o);
+      f.a = reg_of(u[0], phase);
+      f.b = u.size() > 1 ? reg_of(u[1], phase) : f.a;
+      f.dt = dt_dnnl(T(o.out[0]).dt);
+      f.imm = o.kind == "Pow" ? o.attr_f32("beta", 1.0f) : 0.0f;
+      reg_of_op[m] = n_in + (int)s.f_ins.size();
+      s.f_ins.push_back(f);
+      names += (names.empty() ? "" : "+") + o.kind;
+    };
+    for (size_t q = 0; q < order_pre.size(); q++)
+      emit_member(order_pre[q], uses_pre[q], 0, names_pre);
+    s.sum_ins = -1;
+    if (red >= 0) {
+      Step::FIns f;
+      f.op = gcmi::ELT_ROWSUM;
+      f.a = f.b = reg_of(sum_use, 0);
+      f.dt = dt_dnnl(T(g_.ops[(size_t)red].out[0]).dt);
+      f.imm = 0.0f;
+      s.sum_ins = (int)s.f_ins.size();
+      reg_of_op[(size_t)red] = n_in + s.sum_ins;
+      s.f_ins.push_back(f);
+    }
+    for (size_t q = 0; q < order_post.size(); q++)
+      emit_member(order_post[q], uses_post[q], 1, names_post);
+    s.n_in_pre = n_in_pre;
+    s.out = slot_for(root.out[0]);
+    s.out_dt = dt_dnnl(T(root.out[0]).dt);
+    s.red_reg = reg_of_op.at(i);
+    if (red >= 0) {
+      const std::string rk = g_.ops[(size_t)red].kind;
+      s.note = (names_post.empty() ? "" : names_post + " of ") + rk + (names_pre.empty() ? "" : " of " + names_pre);
+      taken_reductions.insert((size_t)red);
+      skip[(size_t)red] = true;
+    } else {
+      s.note = names_post;
+    }
+    for (size_t m : pre)
+      skip[m] = true;
+    for (size_t m : post)
+      skip[m] = true;
+    skip[i] = false;
+    emit_at[i] = {s};
   }
 }
 
@@ -824,6 +1198,40 @@ void Executable::launch(const Step &s) {
     gc_check(gcmi_launch_reduce(&p, stream_) ? 5 : 0, s.note.c_str());
     break;
   }
+  case Step::Fused: {
+    gcmi::FusedParams p{};
+    p.n_in = (int)s.f_in.size(), p.n_in_pre = s.n_in_pre, p.n_ins = (int)s.f_ins.size(), p.sum_ins = s.sum_ins;
+    const size_t r = s.dims.size(), pad = gcmi::ELT_MAX_RANK - r;
+    p.n = 1;
+    for (int d = 0; d < gcmi::ELT_MAX_RANK; d++)
+      p.dims[d] = 1;
+    for (size_t d = 0; d < r; d++)
+      p.dims[pad + d] = s.dims[d], p.n *= s.dims[d];
+    for (int k = 0; k < p.n_in; k++) {
+      p.in[k] = P(s.f_in[(size_t)k]), p.in_dt[k] = s.f_in_dt[(size_t)k];
+      for (size_t d = 0; d < r; d++)
+        p.in_str[k][pad + d] = s.f_str[(size_t)k][d];
+    }
+    for (int j = 0; j < p.n_ins; j++) {
+      const Step::FIns &f = s.f_ins[(size_t)j];
+      p.ins[j].op = f.op, p.ins[j].a = f.a, p.ins[j].b = f.b, p.ins[j].dt = f.dt, p.ins[j].imm = f.imm;
+    }
+    p.out = P(s.out), p.out_dt = s.out_dt, p.out_reg = s.red_reg;
+    p.n_red = s.sum_ins >= 0 ? s.n_red : 1, p.mean = s.mean;
+    // the furthest element any input index can reach lies inside its buffer, and the output fits
+    auto esz = [](int dt) { return dt == GCMI_F32 ? 4 : 2; };
+    for (int k = 0; k < p.n_in; k++) {
+      int64_t far = 0;
+      for (size_t d = 0; d < r; d++)
+        far += (s.dims[d] - 1) * s.f_str[(size_t)k][d];
+      if ((size_t)(far + 1) * (size_t)esz(p.in_dt[k]) > slots_[(size_t)s.f_in[(size_t)k]].bytes)
+        throw std::runtime_error("fused group: an input index runs past its buffer (" + s.note + ")");
+    }
+    if ((size_t)(p.n / p.n_red) * (size_t)esz(p.out_dt) > slots_[(size_t)s.out].bytes)
+      throw std::runtime_error("fused group: the result does not fit its buffer (" + s.note + ")");
+    gc_check(gcmi_launch_fused(&p, stream_) ? 5 : 0, s.note.c_str());
+    break;
+  }
   case Step::Softmax: {
     gcmi::SoftmaxParams p{};
     p.in = P(s.a), p.out = P(s.out), p.outer = s.outer, p.len = s.len, p.inner = s.inner, p.in_dt = s.a_dt, p.out_dt = s.out_dt;
@@ -907,7 +1315,7 @@ std::string Executable::describe() const {
   static const char *names[] = {"gemm_f32", "gemm_bf16", "gemm_int8", "colsum", "attention", "eltwise", "reduce", "softmax"};
   std::ostringstream os;
   for (auto &s : steps_)
-    os << names[(int)s.kind] << ": " << s.note << "\n";
+    os << (s.kind == Step::Fused ? (s.sum_ins >= 0 ? "reduce" : "fused") : names[(int)s.kind]) << ": " << s.note << "\n";
   if (!g_.target_hints.empty()) {
     os << "target hints (CPU, not used):";
     for (auto &h : g_.target_hints)

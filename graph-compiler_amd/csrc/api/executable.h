@@ -16,6 +16,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdint>
+#include <map>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -26,7 +27,7 @@
 namespace gcapi {
 
 struct Step {
-  enum Kind { GemmF32, GemmBf16, GemmInt8, ColSum, Mha, Elt, Reduce, Softmax } kind;
+  enum Kind { GemmF32, GemmBf16, GemmInt8, ColSum, Mha, Elt, Reduce, Softmax, Fused } kind;
   std::string note; // what was fused, for introspection
   bool once = false; // depends on constant tensors only: runs in the first execute, its result is kept
   // operands are arena slot indices (-1 = none)
@@ -52,6 +53,18 @@ struct Step {
   bool mean = false;
   // softmax
   int64_t outer = 0, len = 0, inner = 0;
+  // fused point-wise group (gcmi::FusedParams): inputs with their strides over `dims`, the program, and for a
+  // group that feeds a sum the row length and the register that is summed
+  struct FIns {
+    int op, a, b, dt;
+    float imm;
+  };
+  std::vector<int> f_in, f_in_dt;
+  std::vector<std::vector<int64_t>> f_str;
+  std::vector<FIns> f_ins;
+  int64_t n_red = 0;
+  int red_reg = 0; // the register that is stored
+  int n_in_pre = 0, sum_ins = -1;
 };
 
 struct Slot {
@@ -99,6 +112,8 @@ private:
   void plan();
   void layout_arena();
   void plan_generic(const Op &op);
+  void plan_fusion(std::vector<bool> &skip, const std::vector<bool> &claimed, std::map<size_t, std::vector<Step>> &emit_at,
+                   bool groups);
   void plan_matmul(size_t op_index, std::vector<bool> &done);
   bool try_int8(size_t op_index, std::vector<bool> &done);
   bool try_mha(size_t op_index, std::vector<bool> &done);

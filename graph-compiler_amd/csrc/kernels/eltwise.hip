@@ -118,6 +118,135 @@ __global__ void reduce_kernel(ReduceParams p) {
   store_from_f32(p.out, idx, p.dt, s);
 }
 
+// ---------------------------------------------------------------------------
+// Fused point-wise groups (FusedParams).  The register file lives in LDS, one column per thread
+// (regs[r][tid]: conflict free, and a register number that is only known at run time costs nothing extra).
+__device__ __forceinline__ float round_to_storage(float v, int dt) {
+  switch (dt) {
+  case DT_BF16: return bf16_bits_to_f32(f32_to_bf16_bits(v));
+  case DT_F16: return (float)(_Float16)v;
+  default: return v;
+  }
+}
+
+__device__ __forceinline__ float fused_op(int op, float x, float y, float imm) {
+  switch (op) {
+  case ELT_ADD: return x + y;
+  case ELT_SUB: return x - y;
+  case ELT_MUL: return x * y;
+  case ELT_DIV: return x / y;
+  case ELT_MAX: return (x != x || y != y) ? x + y : fmaxf(x, y);
+  case ELT_EXP: return expf(x);
+  case ELT_NEG: return -x;
+  case ELT_RELU: return apply_act(x, ACT_RELU);
+  case ELT_SIGMOID: return apply_act(x, ACT_SIGMOID);
+  case ELT_GELU_ERF: return apply_act(x, ACT_GELU_ERF);
+  case ELT_GELU_TANH: return apply_act(x, ACT_GELU_TANH);
+  case ELT_POW: return imm == 2.0f ? x * x : (imm == 1.0f ? x : (imm == 0.5f ? sqrtf(x) : powf(x, imm)));
+  default: return x; // ELT_COPY
+  }
+}
+
+static constexpr int FUSED_THREADS = 256;
+static constexpr int FUSED_REGS = FUSED_MAX_IN + FUSED_MAX_INS;
+
+// inputs k0 .. k1-1 of element idx into their registers
+template <typename IDX>
+__device__ __forceinline__ void fused_load(const FusedParams &p, float (*regs)[FUSED_THREADS], int tid, IDX idx, int k0,
+                                           int k1) {
+  IDX off[FUSED_MAX_IN];
+#pragma unroll
+  for (int k = 0; k < FUSED_MAX_IN; k++)
+    off[k] = 0;
+  IDX rem = idx;
+  for (int d = ELT_MAX_RANK - 1; d >= ELT_MAX_RANK - p.rank; d--) {
+    const IDX dim = (IDX)p.dims[d];
+    const IDX c = rem % dim;
+    rem /= dim;
+#pragma unroll
+    for (int k = 0; k < FUSED_MAX_IN; k++)
+      if (k >= k0 && k < k1)
+        off[k] += c * (IDX)p.in_str[k][d];
+  }
+#pragma unroll
+  for (int k = 0; k < FUSED_MAX_IN; k++)
+    if (k >= k0 && k < k1)
+      regs[k][tid] = load_as_f32(p.in[k], (int64_t)off[k], p.in_dt[k]);
+}
+
+// instructions j0 .. j1-1
+__device__ __forceinline__ void fused_run(const FusedParams &p, float (*regs)[FUSED_THREADS], int tid, int j0, int j1) {
+  for (int j = j0; j < j1; j++) {
+    const FusedIns in = p.ins[j];
+    const float x = regs[in.a][tid], y = regs[in.b][tid];
+    regs[p.n_in + j][tid] = round_to_storage(fused_op(in.op, x, y, in.imm), in.dt);
+  }
+}
+
+__global__ __launch_bounds__(FUSED_THREADS) void fused_pointwise_kernel(FusedParams p) {
+  __shared__ float regs[FUSED_REGS][FUSED_THREADS];
+  const int tid = threadIdx.x;
+  const bool small = p.n < ((int64_t)1 << 31); // 32-bit index arithmetic when the whole space fits
+  for (int64_t idx = (int64_t)blockIdx.x * FUSED_THREADS + tid; idx < p.n; idx += (int64_t)gridDim.x * FUSED_THREADS) {
+    if (small)
+      fused_load<uint32_t>(p, regs, tid, (uint32_t)idx, 0, p.n_in);
+    else
+      fused_load<int64_t>(p, regs, tid, idx, 0, p.n_in);
+    fused_run(p, regs, tid, 0, p.n_ins);
+    store_from_f32(p.out, idx, p.out_dt, regs[p.out_reg][tid]);
+  }
+}
+
+// ROWS rows per workgroup, FUSED_THREADS / ROWS threads per row (a multiple of 64: whole waves per row).
+// Partial sums are combined in a fixed tree, so results do not vary from run to run.
+template <int ROWS> __global__ __launch_bounds__(FUSED_THREADS) void fused_rowsum_kernel(FusedParams p) {
+  __shared__ float regs[FUSED_REGS][FUSED_THREADS];
+  __shared__ float wave_sum[FUSED_THREADS / 64];
+  constexpr int TPR = FUSED_THREADS / ROWS;
+  const int tid = threadIdx.x, sub = tid % TPR;
+  const int64_t rows = p.n / p.n_red;
+  const int64_t row = (int64_t)blockIdx.x * ROWS + tid / TPR;
+  const bool small = p.n < ((int64_t)1 << 31);
+  const FusedIns sum = p.ins[p.sum_ins];
+  float acc = 0.0f;
+  if (row < rows) {
+    for (int64_t r = sub; r < p.n_red; r += TPR) {
+      const int64_t idx = row * p.n_red + r;
+      if (small)
+        fused_load<uint32_t>(p, regs, tid, (uint32_t)idx, 0, p.n_in_pre);
+      else
+        fused_load<int64_t>(p, regs, tid, idx, 0, p.n_in_pre);
+      fused_run(p, regs, tid, 0, p.sum_ins);
+      acc += regs[sum.a][tid];
+    }
+  }
+#pragma unroll
+  for (int s = 32; s > 0; s >>= 1)
+    acc += __shfl_xor(acc, s);
+  if constexpr (TPR > 64) {
+    if ((tid & 63) == 0)
+      wave_sum[tid >> 6] = acc;
+    __syncthreads();
+    if (sub == 0) {
+      acc = 0.0f;
+      for (int w = 0; w < TPR / 64; w++)
+        acc += wave_sum[(tid >> 6) + w];
+    }
+  }
+  if (sub == 0 && row < rows) {
+    if (p.mean)
+      acc = acc / (float)p.n_red;
+    regs[p.n_in + p.sum_ins][tid] = round_to_storage(acc, sum.dt);
+    const int64_t idx = row * p.n_red; // the per-row inputs have stride 0 along the row
+    if (small)
+      fused_load<uint32_t>(p, regs, tid, (uint32_t)idx, p.n_in_pre, p.n_in);
+    else
+      fused_load<int64_t>(p, regs, tid, idx, p.n_in_pre, p.n_in);
+    fused_run(p, regs, tid, p.sum_ins + 1, p.n_ins);
+    store_from_f32(p.out, row, p.out_dt, regs[p.out_reg][tid]);
+  }
+}
+
 // softmax along an axis of length `len` and element stride `stride`; one wave
 // per row, rows enumerated as outer*inner
 __global__ __launch_bounds__(256) void softmax_kernel(SoftmaxParams p) {
@@ -155,6 +284,82 @@ extern "C" int gcmi_launch_eltwise(const EltParams *pp, hipStream_t stream) {
   if (blocks > 65536)
     blocks = 65536;
   hipLaunchKernelGGL(eltwise_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : 5;
+}
+extern "C" int gcmi_launch_fused(const FusedParams *pp, hipStream_t stream) {
+  FusedParams p = *pp;
+  if (p.n <= 0)
+    return 0;
+  const bool has_sum = p.sum_ins >= 0;
+  if (p.n_in < 1 || p.n_in > FUSED_MAX_IN || p.n_ins < 0 || p.n_ins > FUSED_MAX_INS || p.sum_ins >= p.n_ins)
+    return 2;
+  if (!has_sum)
+    p.n_in_pre = p.n_in, p.n_red = 1;
+  if (p.n_in_pre < 0 || p.n_in_pre > p.n_in || p.n_red < 1 || p.n % p.n_red != 0)
+    return 2;
+  for (int j = 0; j < p.n_ins; j++) {
+    // an instruction reads registers that are already written; before the sum, only per-element inputs
+    const FusedIns &f = p.ins[j];
+    const bool unary_sum = f.op == ELT_ROWSUM;
+    if ((f.op == ELT_ROWSUM) != (j == p.sum_ins))
+      return 2;
+    for (int r : {f.a, unary_sum ? f.a : f.b}) {
+      if (r < 0 || r >= p.n_in + j)
+        return 2;
+      if (has_sum && j <= p.sum_ins && r >= p.n_in_pre && r < p.n_in)
+        return 2;
+      if (has_sum && j > p.sum_ins && (r < p.n_in_pre || (r >= p.n_in && r < p.n_in + p.sum_ins)))
+        return 2; // per-element values do not exist after the sum
+    }
+  }
+  if (p.out_reg < 0 || p.out_reg >= p.n_in + p.n_ins || (has_sum && p.out_reg < p.n_in + p.sum_ins))
+    return 2;
+  // merge neighbouring iteration dims that every input walks contiguously (or not at all): fewer divisions per
+  // element.  The boundary between rows and the inside of a row is never merged across.
+  int64_t dims[ELT_MAX_RANK], str[FUSED_MAX_IN][ELT_MAX_RANK];
+  int nd = 0;
+  int64_t inner = 1; // elements of the dims to the right of d
+  for (int d = ELT_MAX_RANK - 1; d >= 0; d--) {
+    if (p.dims[d] == 1)
+      continue;
+    bool merge = nd > 0 && !(has_sum && inner == p.n_red);
+    for (int k = 0; k < p.n_in && merge; k++)
+      merge = p.in_str[k][d] == str[k][nd - 1] * dims[nd - 1];
+    if (merge) {
+      dims[nd - 1] *= p.dims[d];
+    } else {
+      dims[nd] = p.dims[d];
+      for (int k = 0; k < p.n_in; k++)
+        str[k][nd] = p.in_str[k][d];
+      nd++;
+    }
+    inner *= p.dims[d];
+  }
+  for (int d = 0; d < ELT_MAX_RANK; d++) {
+    const int src = ELT_MAX_RANK - 1 - d; // dims[] was filled innermost first
+    p.dims[d] = src < nd ? dims[src] : 1;
+    for (int k = 0; k < p.n_in; k++)
+      p.in_str[k][d] = src < nd ? str[k][src] : 0;
+  }
+  p.rank = nd;
+  if (has_sum) {
+    const int64_t rows = p.n / p.n_red;
+    if (p.n_red >= 1024 || rows < 64) {
+      if (rows > 0x7fffffff)
+        return 2;
+      hipLaunchKernelGGL(fused_rowsum_kernel<1>, dim3((unsigned)rows), dim3(FUSED_THREADS), 0, stream, p);
+    } else {
+      const int64_t blocks = (rows + 3) / 4;
+      if (blocks > 0x7fffffff)
+        return 2;
+      hipLaunchKernelGGL(fused_rowsum_kernel<4>, dim3((unsigned)blocks), dim3(FUSED_THREADS), 0, stream, p);
+    }
+  } else {
+    int64_t blocks = (p.n + FUSED_THREADS - 1) / FUSED_THREADS;
+    if (blocks > 16384)
+      blocks = 16384;
+    hipLaunchKernelGGL(fused_pointwise_kernel, dim3((unsigned)blocks), dim3(FUSED_THREADS), 0, stream, p);
+  }
   return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 extern "C" int gcmi_launch_reduce(const ReduceParams *pp, hipStream_t stream) {

@@ -147,3 +147,84 @@ def test_results_that_are_arguments_or_constants(ga, dev):
     outs = [np.zeros((8, 8), np.float32) for _ in range(4)]
     _run(ga, text, [(0, a)], [(1 + j, o) for j, o in enumerate(outs)])
     assert (outs[0] == a * 2.5).all() and (outs[1] == a * 2.5).all() and (outs[2] == a).all() and (outs[3] == 2.5).all()
+
+
+def _block_outputs(ga, mm, dev, T, H, F, seed):
+    torch.manual_seed(seed)
+    bf = torch.bfloat16
+    r = lambda *s: torch.randn(*s, device=dev)  # noqa: E731
+    args = [r(1, T, H).to(bf), (r(H, H) / H ** 0.5).to(bf), r(1, T, H).to(bf), torch.full((1,), 1e-5, device=dev),
+            (1 + 0.1 * r(H)).to(bf), (r(F, H) / H ** 0.5).to(bf), (r(F, H) / H ** 0.5).to(bf), (r(H, F) / F ** 0.5).to(bf),
+            torch.full((1,), 1e-6, device=dev), (1 + 0.1 * r(H)).to(bf)]
+    out, n2 = torch.zeros(1, T, H, device=dev, dtype=bf), torch.zeros(1, T, H, device=dev, dtype=bf)
+    _run(ga, mm.decoder_mlp_block(T, H, F), list(enumerate(args)), [(10, out), (11, n2)])
+    return out, n2
+
+
+def test_fused_groups_compute_what_the_single_ops_compute(ga, mm, dev, monkeypatch):
+    """Every instruction of a fused group rounds to its op's storage type, so fusing changes no bit: the decoder
+    block with the fusion pass on (10 launches) and off (one launch per op)."""
+    fused = _block_outputs(ga, mm, dev, 32, 512, 768, seed=3)
+    monkeypatch.setenv("GCMI_NO_POINTWISE_FUSION", "1")
+    single = _block_outputs(ga, mm, dev, 32, 512, 768, seed=3)
+    assert torch.equal(fused[0], single[0]) and torch.equal(fused[1], single[1])
+
+
+def test_fused_broadcasts_views_and_reductions(ga, dev):
+    """Row and column broadcasts, a middle-axis sum with a point-wise producer and consumer, a mean over two axes,
+    and views between the ops, against numpy in f32."""
+    text = """func.func @f(%x: tensor<6x40x24xf32>, %row: tensor<24xf32>, %col: tensor<6x40xf32>)
+        -> (tensor<6x24xf32>, tensor<6x40x24xf32>, tensor<40xf32>) {
+      %e3 = tensor.empty() : tensor<6x40x24xf32>
+      %e2 = tensor.empty() : tensor<6x24xf32>
+      %rb = linalg.broadcast ins(%row : tensor<24xf32>) outs(%e3 : tensor<6x40x24xf32>) dimensions = [0, 1]
+      %cb = linalg.broadcast ins(%col : tensor<6x40xf32>) outs(%e3 : tensor<6x40x24xf32>) dimensions = [2]
+      %0 = linalg.mul ins(%x, %rb : tensor<6x40x24xf32>, tensor<6x40x24xf32>) outs(%e3 : tensor<6x40x24xf32>) -> tensor<6x40x24xf32>
+      %1 = linalg.add ins(%0, %cb : tensor<6x40x24xf32>, tensor<6x40x24xf32>) outs(%e3 : tensor<6x40x24xf32>) -> tensor<6x40x24xf32>
+      %c0 = arith.constant 0.0 : f32
+      %z = linalg.fill ins(%c0 : f32) outs(%e2 : tensor<6x24xf32>) -> tensor<6x24xf32>
+      %s = linalg.reduce { arith.addf } ins(%1 : tensor<6x40x24xf32>) outs(%z : tensor<6x24xf32>) dimensions = [1]
+      %half = arith.constant dense<5.000000e-01> : tensor<6x24xf32>
+      %s2 = linalg.mul ins(%s, %half : tensor<6x24xf32>, tensor<6x24xf32>) outs(%e2 : tensor<6x24xf32>) -> tensor<6x24xf32>
+      %v = tensor.expand_shape %s2 [[0], [1, 2]] output_shape [6, 1, 24] : tensor<6x24xf32> into tensor<6x1x24xf32>
+      %vc = tensor.collapse_shape %v [[0], [1, 2]] : tensor<6x1x24xf32> into tensor<6x24xf32>
+      %sb = linalg.broadcast ins(%vc : tensor<6x24xf32>) outs(%e3 : tensor<6x40x24xf32>) dimensions = [1]
+      %2 = linalg.sub ins(%1, %sb : tensor<6x40x24xf32>, tensor<6x40x24xf32>) outs(%e3 : tensor<6x40x24xf32>) -> tensor<6x40x24xf32>
+      %3 = linalg.exp ins(%2 : tensor<6x40x24xf32>) outs(%e3 : tensor<6x40x24xf32>) -> tensor<6x40x24xf32>
+      %e1 = tensor.empty() : tensor<40xf32>
+      %z1 = linalg.fill ins(%c0 : f32) outs(%e1 : tensor<40xf32>) -> tensor<40xf32>
+      %m = linalg.reduce { arith.addf } ins(%0 : tensor<6x40x24xf32>) outs(%z1 : tensor<40xf32>) dimensions = [0, 2]
+      return %s2, %3, %m : tensor<6x24xf32>, tensor<6x40x24xf32>, tensor<40xf32>
+    }"""
+    st, plan = ga.explain_mlir(text)
+    assert st == 0, plan
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((6, 40, 24)).astype(np.float32) * 0.2
+    row = rng.standard_normal(24).astype(np.float32)
+    col = rng.standard_normal((6, 40)).astype(np.float32) * 0.1
+    o1, o2, o3 = np.zeros((6, 24), np.float32), np.zeros((6, 40, 24), np.float32), np.zeros(40, np.float32)
+    _run(ga, text, [(0, x), (1, row), (2, col)], [(3, o1), (4, o2), (5, o3)])
+    t0 = x * row
+    t1 = t0 + col[:, :, None]
+    s2 = t1.sum(1, dtype=np.float64) * 0.5
+    assert_close(s2, o1, 1e-5, "sum over the middle axis")
+    assert_close(np.exp(t1 - s2[:, None, :]), o2, 1e-4, "exp(x - row statistic)")
+    assert_close(t0.sum((0, 2), dtype=np.float64), o3, 1e-5, "sum over two axes")
+
+
+def test_reduce_json_fixtures_use_the_row_kernel(ga, dev):
+    """reduce_sum.json / reduce_mean.json style graphs at a size where one thread per output would crawl."""
+    x = torch.randn(48, 8192, device=dev)
+    for kind, ref in (("ReduceSum", x.double().sum(1)), ("ReduceMean", x.double().mean(1))):
+        g = ga._graph([{"kind": kind, "attrs": {"axes": {"type": "s64[]", "value": [1]},
+                                                 "keep_dims": {"type": "bool", "value": 0}},
+                        "inputs": [ga._t(0, "f32", [48, 8192])], "outputs": [ga._t(1, "f32", [48])]}], [0], [1])
+        out = torch.zeros(48, device=dev)
+        comp = ga.Compiler()
+        st, exe = comp.compile(g)
+        assert st == 0, ga.api().dnnl_graph_compiler_last_error().decode()
+        assert exe.execute([(0, x)], [(1, out)]) == 0
+        torch.cuda.synchronize()
+        exe.close()
+        comp.close()
+        assert_close(ref.cpu().numpy(), out.double().cpu().numpy(), 1e-5, kind)

@@ -50,14 +50,50 @@ def test_generic_contraction_is_a_matmul(ga, mm):
 
 
 def test_decoder_block_plan(ga, mm):
+    """31 linalg/tensor ops become 10 launches: four GEMMs, and per RMSNorm one launch for the row statistic
+    (x^2 summed, / H, + eps, ^-0.5 in one kernel) and one for the scaling."""
     st, plan = ga.explain_mlir(mm.decoder_mlp_block(32, 256, 512))
     assert st == OK, plan
-    steps = _steps(plan)
-    assert sum(s.startswith("gemm_bf16") for s in steps) == 4
-    assert sum(s.startswith("reduce: ReduceSum") for s in steps) == 2
-    assert "eltwise: Sigmoid" in steps and not any("Exp" in s or "Neg" in s for s in steps)
-    # reshapes are views and broadcasts fold into the consumer's strides: neither is a launch
-    assert not any("Reshape" in s or "BroadcastTo" in s for s in steps)
+    assert _steps(plan) == [
+        "gemm_bf16: MatMul",
+        "reduce: Divide+Add+Pow of ReduceSum of Add+TypeCast+Pow",
+        "fused: Add+TypeCast+Multiply+TypeCast+Multiply",
+        "gemm_bf16: MatMul",
+        "gemm_bf16: MatMul",
+        "fused: Sigmoid+Multiply+Multiply",  # 1/(1+exp(-x)) was recognised as one sigmoid first
+        "gemm_bf16: MatMul",
+        "fused: Add+Add",                    # the first residual sum is recomputed rather than stored
+        "reduce: Divide+Add+Pow of ReduceSum of TypeCast+Pow",
+        "fused: TypeCast+Multiply+TypeCast+Multiply"]
+
+
+def test_pointwise_fusion_rules(ga, monkeypatch):
+    t = "tensor<8x16xf32>"
+    e = "%e = tensor.empty() : " + t + "\n"
+
+    def fn(body, res=t, args="%a: " + t + ", %b: " + t):
+        return "func.func @f(%s) -> %s {\n%s%s\n}" % (args, res, e, body)
+
+    def bin(res, op, x, y):
+        return "%s = linalg.%s ins(%s, %s : %s, %s) outs(%%e : %s) -> %s\n" % (res, op, x, y, t, t, t, t)
+
+    # a chain is one launch; a value with two point-wise readers is not stored either
+    chain = fn(bin("%0", "add", "%a", "%b") + bin("%1", "mul", "%0", "%0") + bin("%2", "sub", "%1", "%0") + "return %2 : " + t)
+    assert _steps(ga.explain_mlir(chain)[1]) == ["fused: Add+Multiply+Subtract"]
+    # a value that is also returned is stored: it ends its own group, and its readers load it
+    two = fn(bin("%0", "add", "%a", "%b") + bin("%1", "mul", "%0", "%b") + bin("%2", "sub", "%1", "%a") +
+             "return %0, %2 : " + t + ", " + t, res="(" + t + ", " + t + ")")
+    assert _steps(ga.explain_mlir(two)[1]) == ["eltwise: Add", "fused: Multiply+Subtract"]
+    # a matmul operand is stored
+    mmul = fn(bin("%0", "add", "%a", "%b") + bin("%1", "mul", "%0", "%b") +
+              "%c0 = arith.constant 0.0 : f32\n%z = linalg.fill ins(%c0 : f32) outs(%e : " + t + ") -> " + t + "\n"
+              "%2 = linalg.matmul_transpose_b ins(%1, %a : " + t + ", " + t + ") outs(%ez : tensor<8x8xf32>) -> tensor<8x8xf32>\n"
+              "return %2 : tensor<8x8xf32>", res="tensor<8x8xf32>").replace(
+                  "%c0 = arith", "%ez = tensor.empty() : tensor<8x8xf32>\n%c0 = arith")
+    assert _steps(ga.explain_mlir(mmul)[1]) == ["fused: Add+Multiply", "gemm_f32: MatMul"]
+    # the switch that turns the pass off: one launch per op
+    monkeypatch.setenv("GCMI_NO_POINTWISE_FUSION", "1")
+    assert _steps(ga.explain_mlir(chain)[1]) == ["eltwise: Add", "eltwise: Multiply", "eltwise: Subtract"]
 
 
 @pytest.mark.skipif(not os.path.isdir(REF_CASES), reason="the reference tree is not on this machine")
