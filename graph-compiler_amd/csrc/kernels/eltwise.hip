@@ -148,18 +148,29 @@ __device__ __forceinline__ float fused_op(int op, float x, float y, float imm) {
 }
 
 static constexpr int FUSED_THREADS = 256;
-static constexpr int FUSED_REGS = FUSED_MAX_IN + FUSED_MAX_INS;
 
-// inputs k0 .. k1-1 of element idx into their registers
+// The register file: register r of thread tid is regs[r * blockDim.x + tid] in dynamic LDS, sized by the launcher
+// to the registers the program uses.
+struct FusedRegs {
+  float *base;
+  int threads, tid;
+  __device__ __forceinline__ float &operator[](int r) const { return base[r * threads + tid]; }
+};
+
+// adds to off[k] (inputs k0 .. k1-1) the contribution of the coordinates of `idx` over iteration dims d_lo .. d_hi-1
+// (innermost first); a single dim needs no division
 template <typename IDX>
-__device__ __forceinline__ void fused_load(const FusedParams &p, float (*regs)[FUSED_THREADS], int tid, IDX idx, int k0,
-                                           int k1) {
-  IDX off[FUSED_MAX_IN];
+__device__ __forceinline__ void fused_offsets(const FusedParams &p, IDX idx, int d_lo, int d_hi, int k0, int k1,
+                                              IDX (&off)[FUSED_MAX_IN]) {
+  if (d_hi - d_lo == 1) {
 #pragma unroll
-  for (int k = 0; k < FUSED_MAX_IN; k++)
-    off[k] = 0;
+    for (int k = 0; k < FUSED_MAX_IN; k++)
+      if (k >= k0 && k < k1)
+        off[k] += idx * (IDX)p.in_str[k][d_lo];
+    return;
+  }
   IDX rem = idx;
-  for (int d = ELT_MAX_RANK - 1; d >= ELT_MAX_RANK - p.rank; d--) {
+  for (int d = d_hi - 1; d >= d_lo; d--) {
     const IDX dim = (IDX)p.dims[d];
     const IDX c = rem % dim;
     rem /= dim;
@@ -168,56 +179,102 @@ __device__ __forceinline__ void fused_load(const FusedParams &p, float (*regs)[F
       if (k >= k0 && k < k1)
         off[k] += c * (IDX)p.in_str[k][d];
   }
-#pragma unroll
-  for (int k = 0; k < FUSED_MAX_IN; k++)
-    if (k >= k0 && k < k1)
-      regs[k][tid] = load_as_f32(p.in[k], (int64_t)off[k], p.in_dt[k]);
 }
 
 // instructions j0 .. j1-1
-__device__ __forceinline__ void fused_run(const FusedParams &p, float (*regs)[FUSED_THREADS], int tid, int j0, int j1) {
+__device__ __forceinline__ void fused_run(const FusedParams &p, const FusedRegs &regs, int j0, int j1) {
   for (int j = j0; j < j1; j++) {
     const FusedIns in = p.ins[j];
-    const float x = regs[in.a][tid], y = regs[in.b][tid];
-    regs[p.n_in + j][tid] = round_to_storage(fused_op(in.op, x, y, in.imm), in.dt);
+    const float x = regs[in.a], y = regs[in.b];
+    regs[p.n_in + j] = round_to_storage(fused_op(in.op, x, y, in.imm), in.dt);
   }
 }
 
-__global__ __launch_bounds__(FUSED_THREADS) void fused_pointwise_kernel(FusedParams p) {
-  __shared__ float regs[FUSED_REGS][FUSED_THREADS];
-  const int tid = threadIdx.x;
-  const bool small = p.n < ((int64_t)1 << 31); // 32-bit index arithmetic when the whole space fits
-  for (int64_t idx = (int64_t)blockIdx.x * FUSED_THREADS + tid; idx < p.n; idx += (int64_t)gridDim.x * FUSED_THREADS) {
-    if (small)
-      fused_load<uint32_t>(p, regs, tid, (uint32_t)idx, 0, p.n_in);
-    else
-      fused_load<int64_t>(p, regs, tid, idx, 0, p.n_in);
-    fused_run(p, regs, tid, 0, p.n_ins);
-    store_from_f32(p.out, idx, p.out_dt, regs[p.out_reg][tid]);
+// The parameter block is read many times (once per instruction per element) and the kernel-argument segment is
+// slow to reach on a first touch: all threads copy it into LDS together, one word each, so its cache lines are
+// fetched side by side instead of one after the other.
+__device__ __forceinline__ void fused_params_to_lds(FusedParams *dst) {
+  const uint32_t *src = (const uint32_t *)__builtin_amdgcn_kernarg_segment_ptr();
+  uint32_t *d = reinterpret_cast<uint32_t *>(dst);
+  for (unsigned w = threadIdx.x; w < sizeof(FusedParams) / 4; w += blockDim.x)
+    d[w] = src[w];
+  __syncthreads();
+}
+
+template <typename IDX> __device__ __forceinline__ void fused_pointwise_body(const FusedParams &p, const FusedRegs &regs) {
+  const int d0 = ELT_MAX_RANK - p.rank;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < p.n; idx += (int64_t)gridDim.x * blockDim.x) {
+    IDX off[FUSED_MAX_IN];
+#pragma unroll
+    for (int k = 0; k < FUSED_MAX_IN; k++)
+      off[k] = 0;
+    fused_offsets<IDX>(p, (IDX)idx, d0, ELT_MAX_RANK, 0, p.n_in, off);
+#pragma unroll
+    for (int k = 0; k < FUSED_MAX_IN; k++)
+      if (k < p.n_in)
+        regs[k] = load_as_f32(p.in[k], (int64_t)off[k], p.in_dt[k]);
+    fused_run(p, regs, 0, p.n_ins);
+    store_from_f32(p.out, idx, p.out_dt, regs[p.out_reg]);
   }
 }
 
-// ROWS rows per workgroup, FUSED_THREADS / ROWS threads per row (a multiple of 64: whole waves per row).
-// Partial sums are combined in a fixed tree, so results do not vary from run to run.
-template <int ROWS> __global__ __launch_bounds__(FUSED_THREADS) void fused_rowsum_kernel(FusedParams p) {
-  __shared__ float regs[FUSED_REGS][FUSED_THREADS];
-  __shared__ float wave_sum[FUSED_THREADS / 64];
-  constexpr int TPR = FUSED_THREADS / ROWS;
+__global__ __launch_bounds__(FUSED_THREADS) void fused_pointwise_kernel(FusedParams) {
+  extern __shared__ float fused_lds[];
+  __shared__ FusedParams p;
+  fused_params_to_lds(&p);
+  const FusedRegs regs{fused_lds, (int)blockDim.x, (int)threadIdx.x};
+  if (p.n < ((int64_t)1 << 31)) // 32-bit index arithmetic when the whole space fits
+    fused_pointwise_body<uint32_t>(p, regs);
+  else
+    fused_pointwise_body<int64_t>(p, regs);
+}
+
+// TPR threads work on one row (a multiple of 64: whole waves), THREADS / TPR rows per workgroup.  The loads of
+// several elements per thread are in flight together; partial sums are combined in a fixed tree, so results do not
+// vary from run to run.
+template <typename IDX, int THREADS, int TPR>
+__device__ __forceinline__ void fused_rowsum_body(const FusedParams &p, const FusedRegs &regs, float *wave_sum) {
+  constexpr int U = TPR >= 1024 ? 2 : 4; // 1024 threads leave 128 registers per lane
   const int tid = threadIdx.x, sub = tid % TPR;
   const int64_t rows = p.n / p.n_red;
-  const int64_t row = (int64_t)blockIdx.x * ROWS + tid / TPR;
-  const bool small = p.n < ((int64_t)1 << 31);
+  const int64_t row = (int64_t)blockIdx.x * (THREADS / TPR) + tid / TPR;
+  const int d0 = ELT_MAX_RANK - p.rank, d_row = ELT_MAX_RANK - p.rank_red;
   const FusedIns sum = p.ins[p.sum_ins];
   float acc = 0.0f;
+  IDX base[FUSED_MAX_IN];
+#pragma unroll
+  for (int k = 0; k < FUSED_MAX_IN; k++)
+    base[k] = 0;
   if (row < rows) {
-    for (int64_t r = sub; r < p.n_red; r += TPR) {
-      const int64_t idx = row * p.n_red + r;
-      if (small)
-        fused_load<uint32_t>(p, regs, tid, (uint32_t)idx, 0, p.n_in_pre);
-      else
-        fused_load<int64_t>(p, regs, tid, idx, 0, p.n_in_pre);
-      fused_run(p, regs, tid, 0, p.sum_ins);
-      acc += regs[sum.a][tid];
+    fused_offsets<IDX>(p, (IDX)row, d0, d_row, 0, p.n_in, base);
+    for (int64_t r0 = sub; r0 < p.n_red; r0 += (int64_t)TPR * U) {
+      float v[U][FUSED_MAX_IN];
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const int64_t r = r0 + (int64_t)u * TPR;
+        if (r < p.n_red) {
+          IDX off[FUSED_MAX_IN];
+#pragma unroll
+          for (int k = 0; k < FUSED_MAX_IN; k++)
+            off[k] = base[k];
+          fused_offsets<IDX>(p, (IDX)r, d_row, ELT_MAX_RANK, 0, p.n_in_pre, off);
+#pragma unroll
+          for (int k = 0; k < FUSED_MAX_IN; k++)
+            if (k < p.n_in_pre)
+              v[u][k] = load_as_f32(p.in[k], (int64_t)off[k], p.in_dt[k]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        if (r0 + (int64_t)u * TPR < p.n_red) {
+#pragma unroll
+          for (int k = 0; k < FUSED_MAX_IN; k++)
+            if (k < p.n_in_pre)
+              regs[k] = v[u][k];
+          fused_run(p, regs, 0, p.sum_ins);
+          acc += regs[sum.a];
+        }
+      }
     }
   }
 #pragma unroll
@@ -236,15 +293,26 @@ template <int ROWS> __global__ __launch_bounds__(FUSED_THREADS) void fused_rowsu
   if (sub == 0 && row < rows) {
     if (p.mean)
       acc = acc / (float)p.n_red;
-    regs[p.n_in + p.sum_ins][tid] = round_to_storage(acc, sum.dt);
-    const int64_t idx = row * p.n_red; // the per-row inputs have stride 0 along the row
-    if (small)
-      fused_load<uint32_t>(p, regs, tid, (uint32_t)idx, p.n_in_pre, p.n_in);
-    else
-      fused_load<int64_t>(p, regs, tid, idx, p.n_in_pre, p.n_in);
-    fused_run(p, regs, tid, p.sum_ins + 1, p.n_ins);
-    store_from_f32(p.out, row, p.out_dt, regs[p.out_reg][tid]);
+    regs[p.n_in + p.sum_ins] = round_to_storage(acc, sum.dt);
+#pragma unroll
+    for (int k = 0; k < FUSED_MAX_IN; k++) // the per-row inputs have stride 0 along the row
+      if (k >= p.n_in_pre && k < p.n_in)
+        regs[k] = load_as_f32(p.in[k], (int64_t)base[k], p.in_dt[k]);
+    fused_run(p, regs, p.sum_ins + 1, p.n_ins);
+    store_from_f32(p.out, row, p.out_dt, regs[p.out_reg]);
   }
+}
+
+template <int THREADS, int TPR> __global__ __launch_bounds__(THREADS) void fused_rowsum_kernel(FusedParams) {
+  extern __shared__ float fused_lds[];
+  __shared__ float wave_sum[THREADS / 64];
+  __shared__ FusedParams p;
+  fused_params_to_lds(&p);
+  const FusedRegs regs{fused_lds, THREADS, (int)threadIdx.x};
+  if (p.n < ((int64_t)1 << 31))
+    fused_rowsum_body<uint32_t, THREADS, TPR>(p, regs, wave_sum);
+  else
+    fused_rowsum_body<int64_t, THREADS, TPR>(p, regs, wave_sum);
 }
 
 // softmax along an axis of length `len` and element stride `stride`; one wave
@@ -342,23 +410,30 @@ extern "C" int gcmi_launch_fused(const FusedParams *pp, hipStream_t stream) {
       p.in_str[k][d] = src < nd ? str[k][src] : 0;
   }
   p.rank = nd;
+  // collapsed dims that lie inside a row
+  p.rank_red = 0;
+  for (int64_t in_row = 1; has_sum && in_row < p.n_red && p.rank_red < nd; p.rank_red++)
+    in_row *= dims[p.rank_red];
+  const size_t n_regs = (size_t)(p.n_in + p.n_ins);
   if (has_sum) {
     const int64_t rows = p.n / p.n_red;
-    if (p.n_red >= 1024 || rows < 64) {
-      if (rows > 0x7fffffff)
-        return 2;
-      hipLaunchKernelGGL(fused_rowsum_kernel<1>, dim3((unsigned)rows), dim3(FUSED_THREADS), 0, stream, p);
+    if (rows > 0x7fffffff)
+      return 2;
+    // few long rows: 1024 threads per row when their registers fit the 64 KiB a launch may ask for
+    if (p.n_red >= 2048 && rows < 1024 && n_regs * 1024 * 4 + sizeof(FusedParams) + 256 <= 65536) {
+      hipLaunchKernelGGL((fused_rowsum_kernel<1024, 1024>), dim3((unsigned)rows), dim3(1024), n_regs * 1024 * 4, stream, p);
+    } else if (p.n_red >= 512 || rows < 64) {
+      hipLaunchKernelGGL((fused_rowsum_kernel<256, 256>), dim3((unsigned)rows), dim3(256), n_regs * 256 * 4, stream, p);
     } else {
-      const int64_t blocks = (rows + 3) / 4;
-      if (blocks > 0x7fffffff)
-        return 2;
-      hipLaunchKernelGGL(fused_rowsum_kernel<4>, dim3((unsigned)blocks), dim3(FUSED_THREADS), 0, stream, p);
+      hipLaunchKernelGGL((fused_rowsum_kernel<256, 64>), dim3((unsigned)((rows + 3) / 4)), dim3(256), n_regs * 256 * 4, stream,
+                         p);
     }
   } else {
     int64_t blocks = (p.n + FUSED_THREADS - 1) / FUSED_THREADS;
     if (blocks > 16384)
       blocks = 16384;
-    hipLaunchKernelGGL(fused_pointwise_kernel, dim3((unsigned)blocks), dim3(FUSED_THREADS), 0, stream, p);
+    hipLaunchKernelGGL(fused_pointwise_kernel, dim3((unsigned)blocks), dim3(FUSED_THREADS), n_regs * FUSED_THREADS * 4, stream,
+                       p);
   }
   return hipGetLastError() == hipSuccess ? 0 : 5;
 }

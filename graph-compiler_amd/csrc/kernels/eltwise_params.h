@@ -64,7 +64,7 @@ struct FusedParams {
   int32_t in_dt[FUSED_MAX_IN];
   int32_t out_dt, out_reg;
   int32_t n_in, n_in_pre, n_ins, sum_ins; // sum_ins: -1 without a sum
-  int32_t rank;                           // trailing dims that are not 1 (set by the launcher)
+  int32_t rank, rank_red;                 // dims after merging, and how many of them lie inside a row (set by the launcher)
   int32_t mean;
   FusedIns ins[FUSED_MAX_INS];
 };
