@@ -235,18 +235,28 @@ def main():
                 sets.append(((torch.randn(Md, Kdd) * 0.1).to(torch.bfloat16).to(dev),
                              (torch.randn(Kdd, Nd) * 0.02).to(torch.bfloat16).to(dev),
                              torch.empty(Md, Nd, device=dev, dtype=torch.bfloat16)))
-            t = time_launches(torch, lambda i: gc.gemm_bf16(sets[i][0], sets[i][1], out=sets[i][2]), nsets, K, W)
             byts = 2.0 * (Md * Kdd + Kdd * Nd + Md * Nd)
-            gbs = byts / (t["kernel_ms_mean"] * 1e-3) / 1e9
-            dec["%dx%dx%d" % (Md, Nd, Kdd)] = {
-                "ms_per_step": round(t["ms_per_step"], 5), "kernel_ms_mean": round(t["kernel_ms_mean"], 5),
-                "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                             "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
-            log("bf16 decode gemm %dx%dx%d: %.4f ms  %.0f GB/s of operands" % (Md, Nd, Kdd, t["kernel_ms_mean"], gbs))
+            entry = {}
+            for layout in ("kn", "nk"):
+                if layout == "nk":  # the same weights stored [N,K], as torch.nn.Linear and the reference's llama2 case do
+                    sets = [(a, b.t().contiguous(), c) for (a, b, c) in sets]
+                    fn = lambda i: gc.gemm_bf16_nt(sets[i][0], sets[i][1], out=sets[i][2])  # noqa: E731
+                else:
+                    fn = lambda i: gc.gemm_bf16(sets[i][0], sets[i][1], out=sets[i][2])  # noqa: E731
+                t = time_launches(torch, fn, nsets, K, W)
+                gbs = byts / (t["kernel_ms_mean"] * 1e-3) / 1e9
+                entry["weights_" + layout] = {
+                    "ms_per_step": round(t["ms_per_step"], 5), "kernel_ms_mean": round(t["kernel_ms_mean"], 5),
+                    "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
+                log("bf16 decode gemm %dx%dx%d weights [%s]: %.4f ms  %.0f GB/s of operands" %
+                    (Md, Nd, Kdd, layout, t["kernel_ms_mean"], gbs))
+            dec["%dx%dx%d" % (Md, Nd, Kdd)] = entry
             del sets
             torch.cuda.empty_cache()
-        others["bf16_decode_gemm"] = {"workload": "A[32 x K] . W[K x N] bf16, two launches (K slices, then reduction + epilogue); "
-                                                  "algorithmic bytes = A + W + C once", "shapes": dec}
+        others["bf16_decode_gemm"] = {"workload": "A[32 x K] . W bf16 with W stored [K,N] (tile kernel over K slices) and [N,K] "
+                                                  "(weight-streaming kernel); two launches each (partial sums, then reduction + "
+                                                  "epilogue); algorithmic bytes = A + W + C once", "shapes": dec}
 
     # ---------------- f32 plumbing case (configs[0])
     if want("f32"):

@@ -218,14 +218,21 @@ def test_short_a_takes_split_k(gc, orc, wl, dev, M, N, K, act, with_bias, out_f3
 
 
 NT_SHAPES = [(256, 256, 128), (512, 768, 256), (300, 200, 100), (257, 511, 129), (1, 7, 5), (33, 1, 64), (128, 256, 8),
-             (32, 4096, 4096), (1, 1024, 2048), (32, 11008, 4096)]
+             (32, 4096, 4096), (1, 1024, 2048), (32, 11008, 4096), (64, 512, 2048), (33, 1024, 1024), (17, 2048, 512),
+             (32, 4096, 11008), (65, 1024, 1024), (32, 1056, 1088)]
+
+
+def _streams_weights(M, N, K):
+    """Shapes the [N,K] entry point gives to the weight-streaming kernel (short A, enough weights)."""
+    return M <= 64 and N % 32 == 0 and K % 64 == 0 and K >= 256 and N * K >= 1 << 20
 
 
 @pytest.mark.parametrize("M,N,K", NT_SHAPES)
 def test_bf16_gemm_transposed_b(gc, orc, wl, dev, M, N, K):
-    """B stored [N,K] (linalg.matmul_transpose_b): against the oracle on A . Bt^T, and bit for bit against the
-    [K,N] kernel on a transposed copy -- both read the same products in the same order.  Covers whole-tile, ragged
-    and split-K (short A) shapes."""
+    """B stored [N,K] (linalg.matmul_transpose_b): against the oracle on A . Bt^T, and against the [K,N] kernel on
+    a transposed copy -- bit for bit where both run the tile kernels (same products, same order), to rounding
+    where the short-A shapes take the weight-streaming kernel (another summation order).  Covers whole-tile,
+    ragged, split-K and streaming shapes, one and two row tiles."""
     torch.manual_seed(4)
     A = (torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev)
     Bt = (torch.randn(N, K) * 0.5).to(torch.bfloat16).to(dev)
@@ -234,13 +241,32 @@ def test_bf16_gemm_transposed_b(gc, orc, wl, dev, M, N, K):
     for b, act, odt in [(None, None, gc.BF16), (bias, "relu", gc.BF16), (bias, "gelu_erf", gc.F32)]:
         nt = gc.gemm_bf16_nt(A, Bt, b, act, odt)
         nn = gc.gemm_bf16(A, B, b, act, odt)
+        again = gc.gemm_bf16_nt(A, Bt, b, act, odt)
         torch.cuda.synchronize()
-        assert torch.equal(nt, nn), "NT differs from NN on the transposed copy (%s, %s)" % (act, odt)
+        assert torch.equal(nt, again), "two runs differ"
+        if _streams_weights(M, N, K):
+            pre = (A.float() @ Bt.float().t()).cpu().numpy()  # magnitude of the value that was rounded before the bias
+            assert_close(nn.float().cpu().numpy(), nt.float().cpu().numpy(), 1e-2 if odt == gc.BF16 else 1e-4,
+                         "NT against NN (%s)" % act, mag=pre)
+        else:
+            assert torch.equal(nt, nn), "NT differs from NN on the transposed copy (%s, %s)" % (act, odt)
     if M * N * K <= 1 << 24:
         ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A.cpu()), wl.bf16_bits(B.cpu())))
         out = gc.gemm_bf16_nt(A, Bt)
         torch.cuda.synchronize()
         assert_close(ref, out.float().cpu().numpy(), 1e-2, "bf16 NT %dx%dx%d" % (M, N, K))
+
+
+def test_bf16_gemm_streaming_kernel_exact_on_integers(gc, dev):
+    """Small integers: every product and partial sum is exact in f32, so any summation order gives the same bits.
+    32 and 64 rows, K slices of unequal length (K/64 = 43 steps over 16 waves)."""
+    torch.manual_seed(8)
+    for M, N, K in [(32, 1024, 2752), (64, 1024, 2752), (5, 4096, 256)]:
+        A = torch.randint(-3, 4, (M, K), device=dev).to(torch.bfloat16)
+        Bt = torch.randint(-3, 4, (N, K), device=dev).to(torch.bfloat16)
+        out = gc.gemm_bf16_nt(A, Bt, out_dtype=gc.F32)
+        torch.cuda.synchronize()
+        assert torch.equal(out, A.float() @ Bt.float().t())
 
 
 def test_bf16_gemm_transposed_b_strided_rows(gc, dev):
