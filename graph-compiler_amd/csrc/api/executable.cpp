@@ -674,7 +674,12 @@ int pointwise_code(const Op &op) {
     return gcmi::ELT_EXP;
   if (k == "Neg")
     return gcmi::ELT_NEG;
-  return -1;
+  static const std::map<std::string, int> more = {
+      {"Minimum", gcmi::ELT_MIN}, {"Abs", gcmi::ELT_ABS},     {"Ceil", gcmi::ELT_CEIL},     {"Floor", gcmi::ELT_FLOOR},
+      {"Erf", gcmi::ELT_ERF},     {"Log", gcmi::ELT_LOG},     {"Round", gcmi::ELT_ROUND},   {"Rsqrt", gcmi::ELT_RSQRT},
+      {"Sqrt", gcmi::ELT_SQRT},   {"Square", gcmi::ELT_SQUARE}, {"Tanh", gcmi::ELT_TANH},   {"Reciprocal", gcmi::ELT_RECIP}};
+  auto it = more.find(k);
+  return it == more.end() ? -1 : it->second;
 }
 bool storage_float(DT d) { return d == DT::f32 || d == DT::bf16 || d == DT::f16; }
 } // namespace
@@ -1051,21 +1056,13 @@ void Executable::plan_generic(const Op &op) {
     steps_.push_back(std::move(s));
     return;
   }
-  if (k == "Add" || k == "Subtract" || k == "Multiply" || k == "Divide" || k == "Maximum") {
-    s.op = k == "Add" ? gcmi::ELT_ADD : k == "Subtract" ? gcmi::ELT_SUB : k == "Multiply" ? gcmi::ELT_MUL
-           : k == "Divide" ? gcmi::ELT_DIV : gcmi::ELT_MAX;
+  if (pointwise_code(op) >= 0 && op.in.size() == 2) {
+    s.op = pointwise_code(op);
     s.a = slot_for(op.in[0]), s.b = slot_for(op.in[1]), s.out = slot_for(op.out[0]);
     s.a_dt = dt_dnnl(T(op.in[0]).dt), s.b_dt = dt_dnnl(T(op.in[1]).dt), s.out_dt = dt_dnnl(out.dt);
     s.dims = out.shape, s.sa = bstrides(T(op.in[0])), s.sb = bstrides(T(op.in[1]));
-  } else if (k == "ReLU" || k == "Sigmoid" || k == "GELU" || k == "Pow" || k == "Typecast" || k == "TypeCast" ||
-             k == "Exp" || k == "Neg") {
-    s.op = k == "ReLU" ? gcmi::ELT_RELU
-           : k == "Exp" ? gcmi::ELT_EXP
-           : k == "Neg" ? gcmi::ELT_NEG
-           : k == "Sigmoid" ? gcmi::ELT_SIGMOID
-           : k == "GELU" ? (act_of(op) == GCMI_ACT_GELU_TANH ? gcmi::ELT_GELU_TANH : gcmi::ELT_GELU_ERF)
-           : k == "Pow" ? gcmi::ELT_POW
-                        : gcmi::ELT_COPY;
+  } else if (pointwise_code(op) >= 0 && op.in.size() == 1) {
+    s.op = pointwise_code(op);
     s.alpha = k == "Pow" ? op.attr_f32("beta", 1.0f) : 0.0f;
     s.a = slot_for(op.in[0]), s.out = slot_for(op.out[0]);
     s.a_dt = dt_dnnl(T(op.in[0]).dt), s.out_dt = dt_dnnl(out.dt);

@@ -85,7 +85,8 @@ static const std::set<std::string> &extension_ops() {
 bool is_known_op(const std::string &k) { return reference_ops().count(k) || extension_ops().count(k); }
 bool is_extension_op(const std::string &k) { return extension_ops().count(k) != 0; }
 bool is_internal_op(const std::string &k) {
-  static const std::set<std::string> s = {"Maximum", "Exp", "Neg", "Reshape", "Transpose", "BroadcastTo"};
+  static const std::set<std::string> s = {"Maximum", "Minimum", "Exp",  "Neg",    "Abs",  "Ceil",       "Floor",   "Erf",       "Log",
+                                          "Round",   "Rsqrt",   "Sqrt", "Square", "Tanh", "Reciprocal", "Reshape", "Transpose", "BroadcastTo"};
   return s.count(k) != 0;
 }
 
@@ -388,7 +389,7 @@ void verify_graph(const Graph &g) {
       if (T(id).unranked)
         vfail(op, "unranked result");
     const std::string &k = op.kind;
-    if (k == "Add" || k == "Subtract" || k == "Multiply" || k == "Divide" || k == "Maximum") {
+    if (k == "Add" || k == "Subtract" || k == "Multiply" || k == "Divide" || k == "Maximum" || k == "Minimum") {
       if (op.in.size() != 2 || op.out.size() != 1)
         vfail(op, "expects 2 operands and 1 result");
       std::vector<int64_t> o;
@@ -398,7 +399,9 @@ void verify_graph(const Graph &g) {
         vfail(op, "operand shapes do not broadcast to the result shape");
       if (!op.attr_bool("auto_broadcast", true) && T(op.in[0]).shape != T(op.in[1]).shape)
         vfail(op, "auto_broadcast is none but shapes differ");
-    } else if (k == "ReLU" || k == "Sigmoid" || k == "Pow" || k == "GELU" || k == "Exp" || k == "Neg") {
+    } else if (k == "ReLU" || k == "Sigmoid" || k == "Pow" || k == "GELU" || k == "Exp" || k == "Neg" || k == "Abs" ||
+               k == "Ceil" || k == "Floor" || k == "Erf" || k == "Log" || k == "Round" || k == "Rsqrt" || k == "Sqrt" ||
+               k == "Square" || k == "Tanh" || k == "Reciprocal") {
       if (op.in.size() != 1 || op.out.size() != 1)
         vfail(op, "expects 1 operand and 1 result");
       if (T(op.in[0]).shape != T(op.out[0]).shape || T(op.in[0]).dt != T(op.out[0]).dt || !is_float(T(op.in[0]).dt))

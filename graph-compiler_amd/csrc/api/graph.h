@@ -76,7 +76,8 @@ bool is_extension_op(const std::string &kind);
 
 Graph parse_graph(const char *json);
 
-// ops only the MLIR front end produces (mlir_text.h): Maximum, Exp, Neg (element-wise), Reshape (a view),
+// ops only the MLIR front end produces (mlir_text.h): Maximum, Minimum, Exp, Neg, Abs, Ceil, Floor, Erf, Log, Round,
+// Rsqrt, Sqrt, Square, Tanh, Reciprocal (element-wise), Reshape (a view),
 // Transpose {perm}, BroadcastTo {dims: the result dimensions that are added}
 bool is_internal_op(const std::string &kind);
 

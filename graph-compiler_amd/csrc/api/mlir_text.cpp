@@ -508,14 +508,19 @@ void parse_op(Cursor &c, Builder &b, const std::string &res, const std::string &
       static const std::map<std::string, std::string> point = {
           {"arith.addf", "Add"},      {"arith.subf", "Subtract"}, {"arith.mulf", "Multiply"}, {"arith.divf", "Divide"},
           {"arith.maximumf", "Maximum"}, {"arith.maxnumf", "Maximum"}, {"arith.negf", "Neg"},  {"math.exp", "Exp"},
-          {"arith.extf", "TypeCast"}, {"arith.truncf", "TypeCast"}};
+          {"arith.extf", "TypeCast"}, {"arith.truncf", "TypeCast"}, {"arith.minimumf", "Minimum"}, {"arith.minnumf", "Minimum"},
+          {"math.absf", "Abs"},       {"math.ceil", "Ceil"},     {"math.floor", "Floor"},    {"math.erf", "Erf"},
+          {"math.log", "Log"},        {"math.round", "Round"},   {"math.rsqrt", "Rsqrt"},    {"math.sqrt", "Sqrt"},
+          {"math.tanh", "Tanh"}};
       for (auto &m : maps)
         if (!identity(m))
           unimpl("point-wise linalg.generic with maps that are not the identity");
       if (body.size() != 1 || !point.count(body[0]))
-        unimpl("linalg.generic body (one of addf, subf, mulf, divf, maximumf, negf, exp, extf, truncf is taken)");
+        unimpl("linalg.generic body (a single arith/math op: addf, subf, mulf, divf, maximumf, minimumf, negf, extf, truncf, "
+               "exp, absf, ceil, floor, erf, log, round, rsqrt, sqrt, tanh)");
       const std::string kind = point.at(body[0]);
-      const bool unary = kind == "Neg" || kind == "Exp" || kind == "TypeCast";
+      static const std::set<std::string> two = {"Add", "Subtract", "Multiply", "Divide", "Maximum", "Minimum"};
+      const bool unary = !two.count(kind);
       if (in_names.size() != (unary ? 1u : 2u))
         bad("linalg.generic: operand count does not fit its body");
       std::vector<size_t> in;
@@ -586,8 +591,8 @@ void parse_op(Cursor &c, Builder &b, const std::string &res, const std::string &
     b.g.ops.back().out = {id};
     return;
   }
-  static const std::map<std::string, std::string> binary = {{"add", "Add"},      {"sub", "Subtract"}, {"mul", "Multiply"},
-                                                            {"div", "Divide"},   {"max", "Maximum"}};
+  static const std::map<std::string, std::string> binary = {{"add", "Add"},    {"sub", "Subtract"}, {"mul", "Multiply"},
+                                                            {"div", "Divide"}, {"max", "Maximum"},  {"min", "Minimum"}};
   auto splat_of = [&](const std::string &n, double &x) {
     const Value &v = b.val(n);
     if (v.kind != Value::Tensor)
@@ -623,11 +628,73 @@ void parse_op(Cursor &c, Builder &b, const std::string &res, const std::string &
     b.g.ops.back().out = {result(rt)};
     return;
   }
-  if (op == "negf" || op == "exp" || op == "copy") {
+  // the named unary ops of benchgc's linalg driver (test/benchgc/src/benchgc/linalg/eltwise.py)
+  static const std::map<std::string, std::string> unary = {
+      {"negf", "Neg"},   {"exp", "Exp"},     {"copy", "TypeCast"}, {"abs", "Abs"},       {"ceil", "Ceil"},
+      {"floor", "Floor"}, {"erf", "Erf"},    {"log", "Log"},       {"round", "Round"},   {"rsqrt", "Rsqrt"},
+      {"sqrt", "Sqrt"},  {"square", "Square"}, {"tanh", "Tanh"},   {"reciprocal", "Reciprocal"}};
+  if (unary.count(op)) {
     if (in_names.size() != 1)
       bad("linalg." + op + " takes one input");
-    b.add_op(op == "negf" ? "Neg" : op == "exp" ? "Exp" : "TypeCast", {b.operand(in_names[0])}, 0);
+    b.add_op(unary.at(op), {b.operand(in_names[0])}, 0);
     b.g.ops.back().out = {result(rt)};
+    return;
+  }
+  // vector forms of the contraction (test/benchgc/src/benchgc/linalg/matmul.py): a vector operand is viewed as a
+  // one-row or one-column matrix and the unit dim is dropped from the result again
+  if (op == "matvec" || op == "vecmat" || op == "dot" || op == "batch_matvec" || op == "batch_vecmat" ||
+      op == "batch_reduce_matmul") {
+    if (in_names.size() != 2)
+      bad("linalg." + op + " takes two inputs");
+    if (!b.is_zero_init(out_names[0]))
+      unimpl("linalg." + op + " accumulating into a non-zero tensor");
+    auto view = [&](size_t src, std::vector<int64_t> shape) {
+      Type t;
+      t.tensor = true, t.dt = b.g.tensors.at(src).dt, t.shape = std::move(shape);
+      size_t v = b.new_tensor(t);
+      b.g.tensors[v].alias_of = (long)src;
+      b.add_op("Reshape", {src}, v);
+      return v;
+    };
+    size_t a = b.operand(in_names[0]), w = b.operand(in_names[1]);
+    const std::vector<int64_t> as = in_types[0].shape, ws = in_types[1].shape;
+    std::vector<int64_t> mm_shape; // result of the matrix product before the unit dim goes
+    if (op == "matvec" || op == "vecmat" || op == "dot") {
+      const size_t want_a = op == "matvec" ? 2 : 1, want_w = op == "vecmat" ? 2 : 1;
+      if (as.size() != want_a || ws.size() != want_w)
+        bad("linalg." + op + ": operand ranks");
+      // numpy matmul rules cover these as they are: [M,K]x[K] -> [M], [K]x[K,N] -> [N], [K]x[K] -> [1]
+      mm_shape = op == "dot" ? std::vector<int64_t>{1} : rt.shape;
+    } else if (op == "batch_matvec") {
+      if (as.size() != 3 || ws.size() != 2)
+        bad("linalg.batch_matvec: operand ranks");
+      w = view(w, {ws[0], ws[1], 1});
+      mm_shape = {as[0], as[1], 1};
+    } else if (op == "batch_vecmat") {
+      if (as.size() != 2 || ws.size() != 3)
+        bad("linalg.batch_vecmat: operand ranks");
+      a = view(a, {as[0], 1, as[1]});
+      mm_shape = {ws[0], 1, ws[2]};
+    } else { // batch_reduce_matmul: sum over the batch of [M,K] x [K,N]
+      if (as.size() != 3 || ws.size() != 3)
+        bad("linalg.batch_reduce_matmul: operand ranks");
+      mm_shape = {as[0], as[1], ws[2]};
+    }
+    Type mt = rt;
+    mt.shape = mm_shape;
+    size_t prod = b.new_tensor(mt);
+    b.add_op("MatMul", {a, w}, prod);
+    if (op == "batch_reduce_matmul") {
+      Op &o = b.add_op("ReduceSum", {prod}, 0);
+      o.attrs["axes"] = attr_ints({0});
+      o.attrs["keep_dims"] = attr_bool(false);
+      b.g.ops.back().out = {result(rt)};
+    } else if (mm_shape != rt.shape) {
+      size_t v = view(prod, rt.shape);
+      b.def(res, v, rt);
+    } else {
+      b.def(res, prod, rt);
+    }
     return;
   }
   if (op == "broadcast") {

@@ -4,7 +4,10 @@
 //   tensor.empty, arith.constant (scalar or dense splat), linalg.fill,
 //   linalg.matmul / matmul_transpose_a / matmul_transpose_b / batch_matmul /
 //   batch_matmul_transpose_b,
-//   linalg.add / sub / mul / div / max / powf, linalg.negf / exp / copy,
+//   linalg.matvec / vecmat / dot / batch_matvec / batch_vecmat / batch_reduce_matmul,
+//   linalg.generic that is a contraction (multiply-accumulate over one reduction dim) or one point-wise op,
+//   linalg.add / sub / mul / div / max / min / powf,
+//   linalg.negf / exp / copy / abs / ceil / floor / erf / log / round / rsqrt / sqrt / square / tanh / reciprocal,
 //   linalg.broadcast, linalg.transpose, linalg.softmax, linalg.reduce (sum),
 //   tensor.collapse_shape / tensor.expand_shape, return.
 // The module becomes the same graph IR the JSON front end produces (graph.h), so

@@ -42,6 +42,45 @@ __device__ __forceinline__ void store_from_f32(void *p, int64_t i, int dt, float
   }
 }
 
+// one point-wise op in f32 (shared by the single-op kernel and the fused programs)
+__device__ __forceinline__ float round_to_storage(float v, int dt) {
+  switch (dt) {
+  case DT_BF16: return bf16_bits_to_f32(f32_to_bf16_bits(v));
+  case DT_F16: return (float)(_Float16)v;
+  default: return v;
+  }
+}
+
+__device__ __forceinline__ float fused_op(int op, float x, float y, float imm) {
+  switch (op) {
+  case ELT_ADD: return x + y;
+  case ELT_SUB: return x - y;
+  case ELT_MUL: return x * y;
+  case ELT_DIV: return x / y;
+  case ELT_MAX: return (x != x || y != y) ? x + y : fmaxf(x, y);
+  case ELT_EXP: return expf(x);
+  case ELT_NEG: return -x;
+  case ELT_RELU: return apply_act(x, ACT_RELU);
+  case ELT_SIGMOID: return apply_act(x, ACT_SIGMOID);
+  case ELT_GELU_ERF: return apply_act(x, ACT_GELU_ERF);
+  case ELT_GELU_TANH: return apply_act(x, ACT_GELU_TANH);
+  case ELT_POW: return imm == 2.0f ? x * x : (imm == 1.0f ? x : (imm == 0.5f ? sqrtf(x) : powf(x, imm)));
+  case ELT_MIN: return (x != x || y != y) ? x + y : fminf(x, y); // arith.minimumf: NaN propagates
+  case ELT_ABS: return fabsf(x);
+  case ELT_CEIL: return ceilf(x);
+  case ELT_FLOOR: return floorf(x);
+  case ELT_ERF: return erff(x);
+  case ELT_LOG: return logf(x);
+  case ELT_ROUND: return roundf(x); // math.round: halves away from zero
+  case ELT_RSQRT: return 1.0f / sqrtf(x);
+  case ELT_SQRT: return sqrtf(x);
+  case ELT_SQUARE: return x * x;
+  case ELT_TANH: return tanhf(x);
+  case ELT_RECIP: return 1.0f / x;
+  default: return x; // ELT_COPY
+  }
+}
+
 // out[idx] = op(a[idx . sa], b[idx . sb]); out is dense row-major over dims
 __global__ void eltwise_kernel(EltParams p) {
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < p.n; idx += (int64_t)gridDim.x * blockDim.x) {
@@ -59,18 +98,6 @@ __global__ void eltwise_kernel(EltParams p) {
     if (p.b)
       y = load_as_f32(p.b, ib, p.b_dt);
     switch (p.op) {
-    case ELT_ADD: r = x + y; break;
-    case ELT_SUB: r = x - y; break;
-    case ELT_MUL: r = x * y; break;
-    case ELT_DIV: r = x / y; break;
-    case ELT_MAX: r = (x != x || y != y) ? x + y : fmaxf(x, y); break; // arith.maximumf: NaN propagates
-    case ELT_EXP: r = expf(x); break;
-    case ELT_NEG: r = -x; break;
-    case ELT_RELU: r = apply_act(x, ACT_RELU); break;
-    case ELT_SIGMOID: r = apply_act(x, ACT_SIGMOID); break;
-    case ELT_GELU_ERF: r = apply_act(x, ACT_GELU_ERF); break;
-    case ELT_GELU_TANH: r = apply_act(x, ACT_GELU_TANH); break;
-    case ELT_POW: r = p.alpha == 2.0f ? x * x : (p.alpha == 1.0f ? x : (p.alpha == 0.5f ? sqrtf(x) : powf(x, p.alpha))); break;
     case ELT_DEQUANT: {
       float sc = p.scales ? p.scales[p.n_scales > 1 ? ch : 0] : 1.0f;
       float zp = p.zps ? (float)p.zps[p.n_scales > 1 ? ch : 0] : 0.0f;
@@ -83,7 +110,7 @@ __global__ void eltwise_kernel(EltParams p) {
       r = rintf(x / sc) + zp;
       break;
     }
-    default: r = x; break; // ELT_COPY: typecast / strided gather
+    default: r = fused_op(p.op, x, y, p.alpha); break; // ELT_COPY (typecast / strided gather) and the arithmetic ops
     }
     store_from_f32(p.out, idx, p.out_dt, r);
   }
@@ -121,32 +148,6 @@ __global__ void reduce_kernel(ReduceParams p) {
 // ---------------------------------------------------------------------------
 // Fused point-wise groups (FusedParams).  The register file lives in LDS, one column per thread
 // (regs[r][tid]: conflict free, and a register number that is only known at run time costs nothing extra).
-__device__ __forceinline__ float round_to_storage(float v, int dt) {
-  switch (dt) {
-  case DT_BF16: return bf16_bits_to_f32(f32_to_bf16_bits(v));
-  case DT_F16: return (float)(_Float16)v;
-  default: return v;
-  }
-}
-
-__device__ __forceinline__ float fused_op(int op, float x, float y, float imm) {
-  switch (op) {
-  case ELT_ADD: return x + y;
-  case ELT_SUB: return x - y;
-  case ELT_MUL: return x * y;
-  case ELT_DIV: return x / y;
-  case ELT_MAX: return (x != x || y != y) ? x + y : fmaxf(x, y);
-  case ELT_EXP: return expf(x);
-  case ELT_NEG: return -x;
-  case ELT_RELU: return apply_act(x, ACT_RELU);
-  case ELT_SIGMOID: return apply_act(x, ACT_SIGMOID);
-  case ELT_GELU_ERF: return apply_act(x, ACT_GELU_ERF);
-  case ELT_GELU_TANH: return apply_act(x, ACT_GELU_TANH);
-  case ELT_POW: return imm == 2.0f ? x * x : (imm == 1.0f ? x : (imm == 0.5f ? sqrtf(x) : powf(x, imm)));
-  default: return x; // ELT_COPY
-  }
-}
-
 static constexpr int FUSED_THREADS = 256;
 
 // The register file: register r of thread tid is regs[r * blockDim.x + tid] in dynamic LDS, sized by the launcher

@@ -9,7 +9,8 @@ static constexpr int ELT_MAX_RANK = 6;
 enum EltOp : int {
   ELT_COPY = 0, ELT_ADD, ELT_SUB, ELT_MUL, ELT_DIV, ELT_RELU, ELT_SIGMOID, ELT_GELU_ERF, ELT_GELU_TANH, ELT_POW,
   ELT_DEQUANT, ELT_QUANT, ELT_MAX, ELT_EXP, ELT_NEG,
-  ELT_ROWSUM // only inside a FusedParams program: the row sum of a register
+  ELT_ROWSUM, // only inside a FusedParams program: the row sum of a register
+  ELT_MIN, ELT_ABS, ELT_CEIL, ELT_FLOOR, ELT_ERF, ELT_LOG, ELT_ROUND, ELT_RSQRT, ELT_SQRT, ELT_SQUARE, ELT_TANH, ELT_RECIP
 };
 
 struct EltParams {

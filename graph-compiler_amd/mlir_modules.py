@@ -201,3 +201,15 @@ def attention(batch, seq, head_dim, scale, dtype="bf16"):
     p = f.emit("linalg.softmax dimension(2) ins(%s : %s) outs(%s : %s) -> %s" % (sc, t, e, t, t))
     o = _matmul(f, "batch_matmul", p, [B, S, S], "%arg2", [B, S, D], [B, S, D], dtype)
     return _module([ttype([B, S, D], dtype)] * 3, [ttype([B, S, D], dtype)], f, [o])
+
+
+def linalg_op(op, in_shapes, out_shape, dtype="f32"):
+    """One named linalg op over the function's arguments, outs zero-filled: what benchgc's linalg driver builds
+    (test/benchgc/src/benchgc/linalg/{eltwise,binary,matmul}.py)."""
+    f = _Fn()
+    z = _zeros(f, out_shape, dtype)
+    ins = ["%%arg%d" % i for i in range(len(in_shapes))]
+    types = [ttype(s, dtype) for s in in_shapes]
+    to = ttype(out_shape, dtype)
+    r = f.emit("linalg.%s ins(%s : %s) outs(%s : %s) -> %s" % (op, ", ".join(ins), ", ".join(types), z, to, to))
+    return _module(types, [to], f, [r])

@@ -111,11 +111,15 @@ dnnl_status_t dnnl_graph_compiler_explain(const char *graph_json, char *buf, siz
 
 /* compile / explain for a module in MLIR's textual form: one func.func over
  * ranked tensors made of tensor.empty, arith.constant, linalg.{fill, matmul,
- * matmul_transpose_a/b, batch_matmul, batch_matmul_transpose_b, add, sub, mul,
- * div, max, powf, negf, exp, copy, broadcast, transpose, softmax, reduce(addf)}
- * and tensor.{collapse,expand}_shape -- the subset of the reference's benchgc
- * cases (test/benchgc/cases/llama2.mlir) and MLP/matmul patterns
- * (test/benchgc/src/benchgc/pattern/mlp.py).  Takes over what gc-cpu-runner /
+ * matmul_transpose_a/b, batch_matmul, batch_matmul_transpose_a/b, matvec,
+ * vecmat, dot, batch_matvec, batch_vecmat, batch_reduce_matmul, add, sub, mul,
+ * div, max, min, powf, negf, exp, copy, abs, ceil, floor, erf, log, round,
+ * rsqrt, sqrt, square, tanh, reciprocal, broadcast, transpose, softmax,
+ * reduce(addf), generic (a contraction or a single point-wise op)} and
+ * tensor.{collapse,expand}_shape -- the subset of the reference's benchgc
+ * cases (test/benchgc/cases/{llama2,generic}.mlir), its MLP pattern
+ * (test/benchgc/src/benchgc/pattern/mlp.py) and the element-wise, binary and
+ * matmul cases of its linalg driver (test/benchgc/src/benchgc/linalg/).  Takes over what gc-cpu-runner /
  * benchgc `--driver mlir` do with such a module on the CPU
  * (src/gc-cpu-runner/gc-cpu-runner.cpp, test/benchgc/src/benchgc/runner.py).
  * Tensor ids for execute: function argument i has id i, result j has id

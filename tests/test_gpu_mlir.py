@@ -228,3 +228,58 @@ def test_reduce_json_fixtures_use_the_row_kernel(ga, dev):
         exe.close()
         comp.close()
         assert_close(ref.cpu().numpy(), out.double().cpu().numpy(), 1e-5, kind)
+
+
+UNARY = {"abs": torch.abs, "ceil": torch.ceil, "floor": torch.floor, "erf": torch.erf, "log": torch.log,
+         "negf": torch.neg, "exp": torch.exp, "rsqrt": torch.rsqrt, "sqrt": torch.sqrt, "square": torch.square,
+         "tanh": torch.tanh, "reciprocal": torch.reciprocal,
+         "round": lambda x: torch.sign(x) * torch.floor(torch.abs(x) + 0.5)}  # math.round: halves away from zero
+BINARY = {"add": torch.add, "sub": torch.sub, "mul": torch.mul, "div": torch.div, "max": torch.maximum,
+          "min": torch.minimum}
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_linalg_driver_elementwise_ops(ga, mm, dev, dtype):
+    """Every named unary and binary op of benchgc's linalg driver (test/benchgc/src/benchgc/linalg/{eltwise,binary}.py
+    hold the torch references used here), f32 to 1e-4 (libm-grade device functions) and bf16 to one rounding."""
+    td = torch.float32 if dtype == "f32" else torch.bfloat16
+    torch.manual_seed(12)
+    shape = [3, 50, 40]
+    pos = (torch.rand(shape, device=dev) * 4 + 0.25).to(td)            # log, sqrt, rsqrt, reciprocal
+    any_ = ((torch.rand(shape, device=dev) - 0.5) * 6.3).to(td)
+    any_[0, 0, :6] = torch.tensor([0.5, -0.5, 1.5, -1.5, 2.5, -2.5]).to(td)  # ties of round
+    other = ((torch.rand(shape, device=dev) - 0.5) * 4 + 0.01).to(td)
+    for op, fn in UNARY.items():
+        x = pos if op in ("log", "sqrt", "rsqrt", "reciprocal") else any_
+        out = torch.zeros(shape, device=dev, dtype=td)
+        _run(ga, mm.linalg_op(op, [shape], shape, dtype), [(0, x)], [(1, out)])
+        ref = fn(x.double()).to(td)
+        assert_close(ref.double().cpu().numpy(), out.double().cpu().numpy(), 1e-4 if dtype == "f32" else 1e-2, op)
+    for op, fn in BINARY.items():
+        out = torch.zeros(shape, device=dev, dtype=td)
+        _run(ga, mm.linalg_op(op, [shape, shape], shape, dtype), [(0, any_), (1, other)], [(2, out)])
+        ref = fn(any_.double(), other.double()).to(td)
+        assert_close(ref.double().cpu().numpy(), out.double().cpu().numpy(), 1e-6 if dtype == "f32" else 1e-2, op)
+
+
+def test_linalg_driver_contractions(ga, mm, dev):
+    """matmul.py of the same driver: every 2-D, batched and vector form, on small integers (exact in f32)."""
+    rng = np.random.default_rng(4)
+    r = lambda *s: rng.integers(-3, 4, s).astype(np.float32)  # noqa: E731
+    B, M, K, N = 3, 24, 40, 16
+    cases = [("matmul", [r(M, K), r(K, N)], lambda a, b: a @ b),
+             ("matmul_transpose_a", [r(K, M), r(K, N)], lambda a, b: a.T @ b),
+             ("matmul_transpose_b", [r(M, K), r(N, K)], lambda a, b: a @ b.T),
+             ("batch_matmul", [r(B, M, K), r(B, K, N)], lambda a, b: a @ b),
+             ("batch_matmul_transpose_a", [r(B, K, M), r(B, K, N)], lambda a, b: a.transpose(0, 2, 1) @ b),
+             ("batch_matmul_transpose_b", [r(B, M, K), r(B, N, K)], lambda a, b: a @ b.transpose(0, 2, 1)),
+             ("matvec", [r(M, K), r(K)], lambda a, b: a @ b), ("vecmat", [r(K), r(K, N)], lambda a, b: a @ b),
+             ("dot", [r(K), r(K)], lambda a, b: np.array(a @ b, np.float32)),
+             ("batch_matvec", [r(B, M, K), r(B, K)], lambda a, b: np.einsum("bmk,bk->bm", a, b)),
+             ("batch_vecmat", [r(B, K), r(B, K, N)], lambda a, b: np.einsum("bk,bkn->bn", a, b)),
+             ("batch_reduce_matmul", [r(B, M, K), r(B, K, N)], lambda a, b: np.einsum("bmk,bkn->mn", a, b))]
+    for op, ins, fn in cases:
+        ref = fn(*ins)
+        out = np.full(ref.shape, -7.0, np.float32)
+        _run(ga, mm.linalg_op(op, [list(a.shape) for a in ins], list(ref.shape)), list(enumerate(ins)), [(2, out)])
+        assert (out == ref).all(), op

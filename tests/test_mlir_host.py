@@ -164,3 +164,26 @@ def test_returned_argument_constant_and_duplicate_are_copied(ga):
     st, plan = ga.explain_mlir(_fn(body, res="(tensor<8x8xf32>, tensor<8x8xf32>, tensor<8x8xf32>, tensor<8x8xf32>)"))
     assert st == OK, plan
     assert len(_steps(plan)) == 4  # the product, its copy, the copy of %a and the filled constant
+
+
+def test_linalg_driver_single_ops_plan(ga, mm):
+    """The element-wise, binary and matmul cases of benchgc's linalg driver, one op per module."""
+    for op in ("abs", "ceil", "floor", "erf", "log", "negf", "exp", "round", "rsqrt", "sqrt", "square", "tanh", "reciprocal"):
+        st, plan = ga.explain_mlir(mm.linalg_op(op, [[4, 8]], [4, 8]))
+        assert st == OK and len(_steps(plan)) == 1 and _steps(plan)[0].startswith("eltwise:"), (op, plan)
+    for op in ("add", "sub", "mul", "div", "max", "min"):
+        st, plan = ga.explain_mlir(mm.linalg_op(op, [[4, 8], [4, 8]], [4, 8]))
+        assert st == OK and len(_steps(plan)) == 1, (op, plan)
+    cases = [("matmul", [[8, 16], [16, 4]], [8, 4]), ("matmul_transpose_a", [[16, 8], [16, 4]], [8, 4]),
+             ("matmul_transpose_b", [[8, 16], [4, 16]], [8, 4]), ("batch_matmul", [[3, 8, 16], [3, 16, 4]], [3, 8, 4]),
+             ("batch_matmul_transpose_a", [[3, 16, 8], [3, 16, 4]], [3, 8, 4]),
+             ("batch_matmul_transpose_b", [[3, 8, 16], [3, 4, 16]], [3, 8, 4]),
+             ("matvec", [[8, 16], [16]], [8]), ("vecmat", [[16], [16, 4]], [4]), ("dot", [[16], [16]], []),
+             ("batch_matvec", [[3, 8, 16], [3, 16]], [3, 8]), ("batch_vecmat", [[3, 16], [3, 16, 4]], [3, 4]),
+             ("batch_reduce_matmul", [[3, 8, 16], [3, 16, 4]], [8, 4])]
+    for op, ins, out in cases:
+        st, plan = ga.explain_mlir(mm.linalg_op(op, ins, out))
+        assert st == OK, (op, plan)
+        assert any(s.startswith("gemm_f32") for s in _steps(plan)), (op, plan)
+    # packed layouts and convolutions are outside the subset
+    assert ga.explain_mlir(mm.linalg_op("mmt4d", [[2, 2, 4, 4], [2, 2, 4, 4]], [2, 2, 4, 4]))[0] == UNIMPL
