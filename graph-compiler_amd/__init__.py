@@ -20,7 +20,8 @@ ACT = {None: 0, "none": 0, "relu": 1, "gelu_erf": 2, "gelu_tanh": 3, "sigmoid": 
 
 # every symbol the public headers declare (checked by the CPU test-suite)
 EXPORTS = {
-    "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_bf16_nt", "gcmi_gemm_int8", "gcmi_colsum_s8",
+    "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_bf16_nt", "gcmi_gemm_bf16_batched", "gcmi_gemm_f32_batched",
+                         "gcmi_gemm_int8", "gcmi_colsum_s8",
                          "gcmi_gemm_f32", "gcmi_mha_fwd_bf16", "gcmi_mha_fwd_bf16_opt"],
     "gc_brgemm.h": ["dnnl_brgemm_dispatch", "dnnl_brgemm_tileconfig", "dnnl_brgemm_tilerelease",
                     "dnnl_brgemm_execute"],
@@ -50,6 +51,10 @@ def lib():
     L.gcmi_gemm_bf16.restype = ci
     L.gcmi_gemm_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, ci, ci, ci, vp]
     L.gcmi_gemm_bf16_nt.restype = ci
+    L.gcmi_gemm_bf16_batched.restype = ci
+    L.gcmi_gemm_bf16_batched.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, vp, ci, ci, ci, vp]
+    L.gcmi_gemm_f32_batched.restype = ci
+    L.gcmi_gemm_f32_batched.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, ci, vp, ci, vp]
     L.gcmi_gemm_bf16_nt.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, ci, ci, ci, vp]
     L.gcmi_gemm_int8.restype = ci
     L.gcmi_gemm_int8.argtypes = [vp, ci, vp, vp, i64, i64, i64, i64, i64, i64, vp, C.c_int32, vp, vp, ci, ci, vp]
@@ -122,6 +127,27 @@ def gemm_bf16_nt(A, Bt, bias=None, act=None, out_dtype=BF16, out=None):
     check(lib().gcmi_gemm_bf16_nt(_ptr(A), _ptr(Bt), _ptr(out), M, N, K, A.stride(0) if M > 1 else K,
                                   Bt.stride(0) if N > 1 else K, out.stride(0) if M > 1 else N, _ptr(bias), bdt,
                                   ACT[act], out_dtype, _stream()), "gcmi_gemm_bf16_nt")
+    return out
+
+
+def gemm_batched(A, B, trans_b=False, bias=None, act=None, out=None):
+    """A [batch, M, K]; B [batch, K, N] ([batch, N, K] with trans_b) or 2-D (shared by all batches); bf16 or f32."""
+    import torch
+    nb, M, K = A.shape
+    Bm = B if B.dim() == 3 else B.unsqueeze(0)
+    N = Bm.shape[1] if trans_b else Bm.shape[2]
+    assert A.is_contiguous() and B.is_contiguous() and (Bm.shape[2] if trans_b else Bm.shape[1]) == K
+    if out is None:
+        out = torch.empty((nb, M, N), device=A.device, dtype=A.dtype)
+    sb = 0 if B.dim() == 2 else Bm.shape[1] * Bm.shape[2]
+    if A.dtype == torch.float32:
+        check(lib().gcmi_gemm_f32_batched(_ptr(A), _ptr(B), _ptr(out), nb, M, N, K, K, Bm.shape[2], N, M * K, sb, M * N,
+                                          0, int(trans_b), _ptr(bias), ACT[act], _stream()), "gcmi_gemm_f32_batched")
+    else:
+        bdt = BF16 if bias is None or bias.dtype == torch.bfloat16 else F32
+        check(lib().gcmi_gemm_bf16_batched(_ptr(A), _ptr(B), _ptr(out), nb, M, N, K, K, Bm.shape[2], N, M * K, sb, M * N,
+                                           int(trans_b), _ptr(bias), bdt, ACT[act], BF16, _stream()),
+              "gcmi_gemm_bf16_batched")
     return out
 
 

@@ -577,16 +577,24 @@ void Executable::plan() {
         return off;
       };
       int out_slot = slot_for(chain.empty() ? mm.out[0] : cur);
-      int64_t reps = flatten ? 1 : nb;
+      // batches that advance every operand by a fixed stride (or share it) are one launch; other broadcast
+      // patterns fall back to one launch per batch
+      auto uniform = [&](const std::vector<int64_t> &bd) { return bd == bo || prod(bd, 0, bd.size()) == 1; };
+      const bool strided = !flatten && nb > 1 && nb <= 65535 && uniform(ba) && uniform(bb);
+      int64_t reps = flatten || strided ? 1 : nb;
       for (int64_t bi = 0; bi < reps; bi++) {
         Step s;
         s.kind = A.dt == DT::f32 ? Step::GemmF32 : Step::GemmBf16;
-        s.note = std::string("MatMul") + fused + (reps > 1 ? " (batched)" : "");
+        s.note = std::string("MatMul") + fused + (strided ? " (" + std::to_string(nb) + " batches)" : reps > 1 ? " (batched)" : "");
+        if (strided) {
+          s.batch = nb;
+          s.a_bs = ba == bo ? a_mat : 0, s.b_bs = bb == bo ? b_mat : 0, s.c_bs = M * N;
+        }
         s.a = sa_slot, s.b = sb_slot, s.out = out_slot;
         s.M = flatten ? M * nb : M, s.N = N, s.K = K;
         s.lda = as[Ra - 1], s.ldb = bs[Rb - 1], s.ldc = N;
         s.ta = tA, s.tb = tB;
-        if (!flatten) {
+        if (!flatten && !strided) {
           s.a_off = batch_off(ba, bi) * a_mat, s.b_off = batch_off(bb, bi) * b_mat, s.out_off = bi * M * N;
         }
         s.bias = bias_t >= 0 ? slot_for((size_t)bias_t) : -1;
@@ -1123,14 +1131,16 @@ void Executable::launch(const Step &s) {
   auto P = [&](int slot) -> char * { return slot < 0 ? nullptr : (char *)ptr_[(size_t)slot]; };
   switch (s.kind) {
   case Step::GemmF32:
-    gc_check(gcmi_gemm_f32((const float *)P(s.a) + s.a_off, (const float *)P(s.b) + s.b_off, (float *)P(s.out) + s.out_off,
-                           s.M, s.N, s.K, s.lda, s.ldb, s.ldc, s.ta, s.tb, (const float *)P(s.bias), s.act, stream_),
+    gc_check(gcmi_gemm_f32_batched((const float *)P(s.a) + s.a_off, (const float *)P(s.b) + s.b_off,
+                                   (float *)P(s.out) + s.out_off, s.batch, s.M, s.N, s.K, s.lda, s.ldb, s.ldc, s.a_bs, s.b_bs,
+                                   s.c_bs, s.ta, s.tb, (const float *)P(s.bias), s.act, stream_),
              "MatMul f32");
     break;
   case Step::GemmBf16:
-    gc_check((s.tb ? gcmi_gemm_bf16_nt : gcmi_gemm_bf16)(
-                 P(s.a) + s.a_off * 2, P(s.b) + s.b_off * 2, P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4), s.M, s.N,
-                 s.K, s.lda, s.ldb, s.ldc, P(s.bias), s.bias_dt ? s.bias_dt : GCMI_BF16, s.act, s.out_dt, stream_),
+    gc_check(gcmi_gemm_bf16_batched(P(s.a) + s.a_off * 2, P(s.b) + s.b_off * 2,
+                                    P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4), s.batch, s.M, s.N, s.K, s.lda,
+                                    s.ldb, s.ldc, s.a_bs, s.b_bs, s.c_bs, s.tb ? 1 : 0, P(s.bias),
+                                    s.bias_dt ? s.bias_dt : GCMI_BF16, s.act, s.out_dt, stream_),
              "MatMul bf16");
     break;
   case Step::ColSum:

@@ -34,6 +34,7 @@ struct Step {
   int a = -1, b = -1, c = -1, out = -1, bias = -1, mask = -1, aux = -1;
   int64_t M = 0, N = 0, K = 0, lda = 0, ldb = 0, ldc = 0;
   int64_t a_off = 0, b_off = 0, out_off = 0; // element offsets (batched fallbacks)
+  int64_t batch = 1, a_bs = 0, b_bs = 0, c_bs = 0; // strided batch in one launch (0 stride: shared operand)
   bool ta = false, tb = false;
   int act = 0, out_dt = 0, bias_dt = 0, a_dt = 0;
   int32_t zp = 0;

@@ -65,7 +65,8 @@ extern "C" int gcmi_init(int device) {
 
 namespace {
 int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
-                  int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
+                  int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream,
+                  int64_t batch = 1, int64_t a_bs = 0, int64_t b_bs = 0, int64_t c_bs = 0);
 }
 
 extern "C" int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -80,9 +81,26 @@ extern "C" int gcmi_gemm_bf16_nt(const void *A, const void *Bt, void *C, int64_t
   return gemm_bf16_any(true, A, Bt, C, M, N, K, lda, ldb, ldc, bias, bias_dtype, act, out_dtype, stream);
 }
 
+extern "C" int gcmi_gemm_bf16_batched(const void *A, const void *B, void *C, int64_t batch, int64_t M, int64_t N,
+                                      int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a,
+                                      int64_t stride_b, int64_t stride_c, int trans_b, const void *bias,
+                                      int bias_dtype, int act, int out_dtype, void *stream) {
+  if (batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0)
+    return fail(ST_INVALID, "gemm_bf16_batched: negative batch count or stride");
+  if (batch == 0)
+    return ST_OK;
+  if (batch > 65535)
+    return fail(ST_UNIMPL, "gemm_bf16_batched: more than 65535 batches in one call");
+  if (batch > 1 && stride_c < (M - 1) * ldc + N)
+    return fail(ST_INVALID, "gemm_bf16_batched: results of different batches would overlap");
+  return gemm_bf16_any(trans_b != 0, A, B, C, M, N, K, lda, ldb, ldc, bias, bias_dtype, act, out_dtype, stream, batch,
+                       stride_a, stride_b, stride_c);
+}
+
 namespace {
 int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
-                  int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream) {
+                  int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream,
+                  int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs) {
   if (M < 0 || N < 0 || K < 0)
     return fail(ST_INVALID, "gemm_bf16: negative size");
   if (M == 0 || N == 0)
@@ -102,6 +120,7 @@ int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M
   p.A = A, p.B = B, p.C = C, p.M = M, p.N = N, p.K = K, p.lda = lda, p.ldb = ldb, p.ldc = ldc;
   p.bias = bias, p.bias_dt = bias_dtype, p.act = act, p.out_dt = out_dtype;
   p.trans_b = trans_b ? 1 : 0;
+  p.batch = batch, p.a_bs = a_bs, p.b_bs = b_bs, p.c_bs = c_bs;
   return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
 }
 } // namespace
@@ -152,6 +171,21 @@ extern "C" int gcmi_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, 
 extern "C" int gcmi_gemm_f32(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                              int64_t ldb, int64_t ldc, int trans_a, int trans_b, const float *bias, int act,
                              void *stream) {
+  return gcmi_gemm_f32_batched(A, B, C, 1, M, N, K, lda, ldb, ldc, 0, 0, 0, trans_a, trans_b, bias, act, stream);
+}
+
+extern "C" int gcmi_gemm_f32_batched(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N,
+                                     int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a,
+                                     int64_t stride_b, int64_t stride_c, int trans_a, int trans_b, const float *bias,
+                                     int act, void *stream) {
+  if (batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0)
+    return fail(ST_INVALID, "gemm_f32: negative batch count or stride");
+  if (batch == 0)
+    return ST_OK;
+  if (batch > 65535)
+    return fail(ST_UNIMPL, "gemm_f32: more than 65535 batches in one call");
+  if (batch > 1 && stride_c < (M - 1) * ldc + N)
+    return fail(ST_INVALID, "gemm_f32: results of different batches would overlap");
   if (M < 0 || N < 0 || K < 0)
     return fail(ST_INVALID, "gemm_f32: negative size");
   if (M == 0 || N == 0)
@@ -167,6 +201,7 @@ extern "C" int gcmi_gemm_f32(const float *A, const float *B, float *C, int64_t M
   p.a_rs = trans_a ? 1 : lda, p.a_cs = trans_a ? lda : 1;
   p.b_rs = trans_b ? 1 : ldb, p.b_cs = trans_b ? ldb : 1;
   p.ldc = ldc, p.bias = bias, p.act = act, p.beta = 0.0f;
+  p.batch = batch, p.a_bs = stride_a, p.b_bs = stride_b, p.c_bs = stride_c;
   return launched(gcmi_launch_gemm_f32(&p, (hipStream_t)stream), "gemm_f32");
 }
 

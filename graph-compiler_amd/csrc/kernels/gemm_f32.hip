@@ -29,6 +29,7 @@ template <int BT> __global__ __launch_bounds__(256) void gemm_f32_kernel(F32Gemm
   __shared__ float Bs[BK][BT + 4];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
   const int64_t m0 = (int64_t)blockIdx.y * BT, n0 = (int64_t)blockIdx.x * BT;
+  p.A += (int64_t)blockIdx.z * p.a_bs, p.B += (int64_t)blockIdx.z * p.b_bs, p.C += (int64_t)blockIdx.z * p.c_bs;
   // slice element e of this thread: (row/col within the tile, k within the slice);
   // the contiguous direction of each operand runs along consecutive threads
   int am[PER], ak[PER], bn[PER], bk[PER];
@@ -162,9 +163,12 @@ extern "C" int gcmi_launch_gemm_f32(const F32GemmParams *pp, hipStream_t stream)
   if (p.M <= 0 || p.N <= 0)
     return 0;
   // the largest tile that still gives every compute unit a workgroup
-  auto tiles = [&](int bt) { return ((p.N + bt - 1) / bt) * ((p.M + bt - 1) / bt); };
+  const int64_t nbatch = p.batch > 1 ? p.batch : 1;
+  if (nbatch > 65535)
+    return 2;
+  auto tiles = [&](int bt) { return ((p.N + bt - 1) / bt) * ((p.M + bt - 1) / bt) * nbatch; };
   const int bt = tiles(64) >= 256 ? 64 : tiles(32) >= 256 ? 32 : 16;
-  dim3 grid((unsigned)((p.N + bt - 1) / bt), (unsigned)((p.M + bt - 1) / bt)), block(256);
+  dim3 grid((unsigned)((p.N + bt - 1) / bt), (unsigned)((p.M + bt - 1) / bt), (unsigned)nbatch), block(256);
   if (grid.y > 65535)
     return 2;
   if (bt == 64)

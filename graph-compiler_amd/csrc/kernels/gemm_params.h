@@ -25,6 +25,9 @@ struct GemmParams {
   int32_t splits;        // 0 or 1: off
   float *partial;
   int32_t trans_b;       // bf16 only: B is stored [N,K] (k contiguous), ldb elements between its rows
+  // strided batch (bf16 tile kernels): blockIdx.y is the batch index, operands advance by these element strides
+  // (0 = the operand is shared by all batches).  batch <= 1: a single GEMM.
+  int64_t batch, a_bs, b_bs, c_bs;
 };
 
 struct F32GemmParams {
@@ -37,6 +40,7 @@ struct F32GemmParams {
   const float *bias;
   int32_t act;
   float beta; // 0: overwrite, 1: accumulate into C before the epilogue
+  int64_t batch, a_bs, b_bs, c_bs; // strided batch in blockIdx.z (0 stride = shared operand); batch <= 1: single GEMM
 };
 
 struct MhaParams {

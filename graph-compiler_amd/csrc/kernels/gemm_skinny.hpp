@@ -125,7 +125,7 @@ static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream) {
   GemmParams p = *pp;
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
-  if (!p.trans_b || p.M < 1 || p.M > 64 || p.N % 32 != 0 || p.K % 64 != 0 || p.K < 256 || !al16(p.A) || !al16(p.B) ||
+  if (!p.trans_b || p.batch > 1 || p.M < 1 || p.M > 64 || p.N % 32 != 0 || p.K % 64 != 0 || p.K < 256 || !al16(p.A) || !al16(p.B) ||
       !al16(p.C) || (p.lda * 2) % 16 != 0 || (p.ldb * 2) % 16 != 0 || (p.ldc * out_es) % 16 != 0 || p.out_dt == DT_S32 ||
       p.N / 32 > 0x3fffff)
     return -1;

@@ -309,8 +309,10 @@ template <int ES, bool EDGE, bool TB = false> __global__ __launch_bounds__(G_THR
   const int64_t m0 = (int64_t)tm * G_BM, n0 = (int64_t)tn * G_BN;
 
   const int64_t lda_b = p.lda * ES, ldb_b = p.ldb * ES;
-  const char *Ab = reinterpret_cast<const char *>(p.A);
-  const char *Bb = reinterpret_cast<const char *>(p.B);
+  const int64_t bz = blockIdx.y; // batch
+  const char *Ab = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * ES;
+  const char *Bb = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * ES;
+  p.C = reinterpret_cast<char *>(p.C) + bz * p.c_bs * (p.out_dt == DT_BF16 ? 2 : 4);
 
   // ---- global -> register staging assignment: 4 A chunks + 4 B chunks per thread
   const int a_row0 = tid >> 3, a_c = tid & 7;             // rows a_row0 + 64*i
@@ -597,6 +599,12 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
   }
   const int64_t m0 = (int64_t)tm * G_BM, n0 = (int64_t)tn * G_BN;
   const int64_t lda_b = p.lda * ES, ldb_b = p.ldb * ES;
+  if (!SPLIT) { // strided batch in blockIdx.y
+    const int64_t bz = blockIdx.y;
+    p.A = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * ES;
+    p.B = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * ES;
+    p.C = reinterpret_cast<char *>(p.C) + bz * p.c_bs * (p.out_dt == DT_BF16 ? 2 : 4);
+  }
 
   FG g;
   g.wave_u = wave;
@@ -809,7 +817,14 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   // One tile row and too few column tiles to fill the GPU (decode-style shapes such as 32 x 4096 x 4096): the
   // weights have to stream from HBM through all compute units, so K is cut into slices, one workgroup per
   // (column tile, slice); partial sums go through the workspace and a small second kernel.
-  if (ES == 2 && fast_but_m && tiles_m == 1 && p.out_dt != DT_S32) {
+  const int64_t nbatch = p.batch > 1 ? p.batch : 1;
+  if (nbatch > 65535)
+    return 2;
+  if (nbatch == 1)
+    p.a_bs = p.b_bs = p.c_bs = 0;
+  else if (!((p.a_bs * ES) % 16 == 0 && (p.b_bs * ES) % 16 == 0 && (p.c_bs * out_es) % 16 == 0))
+    fast = false; // every batch's operands must keep the alignment the fast path loads with
+  if (ES == 2 && fast_but_m && tiles_m == 1 && p.out_dt != DT_S32 && nbatch == 1) {
     const int n_cu = gcmi_num_cus();
     const int groups = (int)(p.K / KGROUP);
     int splits = (n_cu + tiles_n - 1) / tiles_n;
@@ -853,7 +868,7 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   }
   if (p.group_m <= 0)
     p.group_m = 4;
-  dim3 grid((unsigned)nblk), block(G_THREADS);
+  dim3 grid((unsigned)nblk, (unsigned)nbatch), block(G_THREADS);
   if constexpr (ES == 2) {
     if (p.trans_b) {
       if (fast)

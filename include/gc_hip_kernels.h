@@ -67,6 +67,19 @@ int gcmi_gemm_bf16_nt(const void *A, const void *Bt, void *C, int64_t M, int64_t
                       int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
 
 /*
+ * Strided batches of the same GEMM in one launch: batch b reads A + b*stride_a,
+ * B + b*stride_b and writes C + b*stride_c (element strides; 0 shares the
+ * operand between batches; at most 65535 batches).  trans_b as in
+ * gcmi_gemm_bf16_nt.  Takes over linalg.batch_matmul{,_transpose_b} and the
+ * batch dims of onednn_graph.matmul (lib/gc/Dialect/OneDNNGraph/
+ * OneDNNGraphOps.cpp:204-310; the reference tiles the batch as the outermost
+ * parallel loop, lib/gc/Transforms/DeepTileContractionOp.cpp:570-575).
+ */
+int gcmi_gemm_bf16_batched(const void *A, const void *B, void *C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                           int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                           int trans_b, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
+
+/*
  * 8-bit matmul with s32 accumulation and fused dequantise epilogue.
  * Takes over: the u8/s8 brgemm (lib/gc/ExecutionEngine/CPURuntime/Microkernel/
  * BrgemmNaive.cpp:102-140) under the deep-tile nest, the asymmetric-activation
@@ -98,6 +111,11 @@ int gcmi_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, int32_t *co
  */
 int gcmi_gemm_f32(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                   int64_t ldc, int trans_a, int trans_b, const float *bias, int act, void *stream);
+
+/* The f32 GEMM over strided batches (see gcmi_gemm_bf16_batched). */
+int gcmi_gemm_f32_batched(const float *A, const float *B, float *C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                          int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                          int trans_a, int trans_b, const float *bias, int act, void *stream);
 
 /*
  * Fused multi-head attention forward, bf16, head_dim 128:

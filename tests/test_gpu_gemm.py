@@ -280,3 +280,30 @@ def test_bf16_gemm_transposed_b_strided_rows(gc, dev):
     ref = gc.gemm_bf16(A, Bt.t().contiguous())
     torch.cuda.synchronize()
     assert torch.equal(out, ref)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("nb,M,N,K", [(6, 256, 256, 128), (3, 100, 72, 50), (16, 128, 64, 64), (2, 512, 768, 256)])
+def test_batched_gemm_one_launch(gc, dev, dtype, nb, M, N, K):
+    """Strided batches in one launch against the same GEMMs one at a time (bit for bit: the same kernel runs on
+    each batch), with B per batch, B stored [N,K], and one B shared by all batches; and against torch."""
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    torch.manual_seed(31)
+    A = (torch.randn(nb, M, K, device=dev) * 0.5).to(td)
+    B = (torch.randn(nb, K, N, device=dev) * 0.5).to(td)
+    bias = torch.randn(N, device=dev).to(td)
+    one = gc.gemm_bf16 if dtype == "bf16" else gc.gemm_f32
+    out = gc.gemm_batched(A, B, bias=bias, act="relu")
+    ref = torch.stack([one(A[b], B[b], bias, "relu") for b in range(nb)])
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+    exact = torch.relu(A.double() @ B.double() + bias.double())
+    assert_close(exact.cpu().numpy(), out.double().cpu().numpy(), 2e-2 if dtype == "bf16" else 1e-4, "batched %s" % dtype,
+                 mag=(A.double() @ B.double()).cpu().numpy())
+    Bt = B.transpose(1, 2).contiguous()
+    out_t = gc.gemm_batched(A, Bt, trans_b=True, bias=bias, act="relu")
+    shared = gc.gemm_batched(A, B[0].contiguous())
+    ref_s = torch.stack([one(A[b], B[0].contiguous()) for b in range(nb)])
+    torch.cuda.synchronize()
+    assert torch.equal(out_t, ref) if dtype == "bf16" else torch.allclose(out_t, ref, rtol=1e-5, atol=1e-5)
+    assert torch.equal(shared, ref_s)
