@@ -692,6 +692,8 @@ int pointwise_code(const Op &op) {
 bool storage_float(DT d) { return d == DT::f32 || d == DT::bf16 || d == DT::f16; }
 } // namespace
 
+static int fused_registers(const Step &s);
+
 std::vector<int64_t> squeezed(const std::vector<int64_t> &shape) {
   std::vector<int64_t> r;
   for (auto d : shape)
@@ -769,6 +771,7 @@ void Executable::plan_fusion(std::vector<bool> &skip, const std::vector<bool> &c
   };
 
   std::set<size_t> taken_reductions;
+  std::vector<size_t> fused_roots;
   for (size_t i = n; i-- > 0;) {
     const Op &root = g_.ops[i];
     const bool red_root = reduction(i);
@@ -965,6 +968,7 @@ void Executable::plan_fusion(std::vector<bool> &skip, const std::vector<bool> &c
         s.f_in.push_back(slot_for(e.tensor));
         s.f_in_dt.push_back(dt_dnnl(T(e.tensor).dt));
         s.f_str.push_back(e.str);
+        s.f_in_tensor.push_back(base(e.tensor));
       }
     auto reg_of = [&](const Use &u, int phase) {
       return u.is_input ? (phase == 0 ? u.index : n_in_pre + u.index) : reg_of_op.at(u.op);
@@ -1010,11 +1014,129 @@ void Executable::plan_fusion(std::vector<bool> &skip, const std::vector<bool> &c
       s.note = names_post;
     }
     for (size_t m : pre)
-      skip[m] = true;
+      skip[m] = true, s.f_members.push_back(m);
     for (size_t m : post)
-      skip[m] = true;
+      skip[m] = true, s.f_members.push_back(m);
+    if (red >= 0)
+      s.f_members.push_back((size_t)red);
+    s.f_out_tensor = base(root.out[0]);
+    s.f_place = place;
+    if (fused_registers(s) > gcmi::FUSED_MAX_PHYS)
+      throw std::logic_error("point-wise group with more than " + std::to_string(gcmi::FUSED_MAX_PHYS) +
+                             " values alive at once (" + s.note + ")");
     skip[i] = false;
     emit_at[i] = {s};
+    fused_roots.push_back(i);
+  }
+
+  // ---- a row statistic and the point-wise group that scales by it become one launch (a normalisation): the
+  // second group runs as a second pass over the row inside the row kernel
+  std::sort(fused_roots.begin(), fused_roots.end());
+  for (size_t i2 : fused_roots) {
+    auto it2 = emit_at.find(i2);
+    if (it2 == emit_at.end() || it2->second.size() != 1)
+      continue;
+    Step &s2 = it2->second[0];
+    if (s2.kind != Step::Fused || s2.sum_ins >= 0)
+      continue;
+    for (size_t k = 0; k < s2.f_in_tensor.size(); k++) {
+      const size_t r = s2.f_in_tensor[k];
+      auto pit = producer.find(r);
+      if (pit == producer.end() || outs.count(r))
+        continue;
+      // the group that writes r: emitted at its last op
+      size_t i1 = n;
+      for (size_t cand : fused_roots)
+        if (cand < i2 && emit_at.count(cand) && emit_at[cand].size() == 1 && emit_at[cand][0].kind == Step::Fused &&
+            emit_at[cand][0].sum_ins >= 0 && emit_at[cand][0].row_end < 0 && emit_at[cand][0].f_out_tensor == r)
+          i1 = cand;
+      if (i1 == n)
+        continue;
+      const Step &s1 = emit_at[i1][0];
+      // nothing but this group reads r
+      bool only_here = true;
+      for (size_t c : consumers[r])
+        only_here = only_here && std::find(s2.f_members.begin(), s2.f_members.end(), c) != s2.f_members.end();
+      // the same non-unit dims, and r broadcast exactly along the summed ones
+      const size_t nd = s1.dims.size();
+      if (!only_here || s1.f_place.size() != nd || s2.dims.size() != nd)
+        continue;
+      bool same = true;
+      for (size_t q = 0; q < nd; q++)
+        same = same && s2.dims[q] == s1.dims[(size_t)s1.f_place[q]];
+      const size_t n_kept = nd - [&] {
+        size_t c = 0;
+        int64_t in_row = 1;
+        for (size_t d = nd; d-- > 0 && in_row < s1.n_red;)
+          in_row *= s1.dims[d], c++;
+        return c;
+      }();
+      std::vector<int64_t> kept(s1.dims.begin(), s1.dims.begin() + (long)n_kept), kst = dense_strides(kept);
+      for (size_t q = 0; q < nd && same; q++) {
+        const size_t pos = (size_t)s1.f_place[q];
+        same = s2.f_str[k][q] == (pos < n_kept ? kst[pos] : 0);
+      }
+      const size_t n_in_new = s1.f_in.size() + s2.f_in.size() - 1, n_ins_new = s1.f_ins.size() + s2.f_ins.size();
+      if (!same || n_in_new > (size_t)gcmi::FUSED_MAX_IN || n_ins_new > (size_t)gcmi::FUSED_MAX_INS)
+        continue;
+      // one workgroup walks a row twice: worth it when there are rows enough to fill the GPU; a few long rows
+      // (32 tokens x 4096) are quicker as a row kernel and a point-wise kernel spread over all compute units
+      int64_t rows = 1;
+      for (size_t d = 0; d < n_kept; d++)
+        rows *= s1.dims[d];
+      const char *min_rows = getenv("GCMI_ROW_MERGE_MIN_ROWS"); // tuning knob; default 512
+      if (rows < (min_rows ? atoll(min_rows) : 512))
+        continue;
+      Step m = s1;
+      m.note = s2.note + " after " + s1.note;
+      m.n_in_row = (int)s1.f_in.size();
+      m.row_end = (int)s1.f_ins.size();
+      const int shift1 = (int)n_in_new - (int)s1.f_in.size(); // results of the first group move up by this much
+      for (auto &f : m.f_ins) {
+        if (f.a >= (int)s1.f_in.size())
+          f.a += shift1;
+        if (f.b >= (int)s1.f_in.size())
+          f.b += shift1;
+      }
+      const int r_reg = s1.red_reg + shift1;
+      auto permute = [&](const std::vector<int64_t> &by_dim) {
+        std::vector<int64_t> it(nd, 0);
+        for (size_t q = 0; q < nd; q++)
+          it[(size_t)s1.f_place[q]] = by_dim[q];
+        return it;
+      };
+      std::vector<int> in_map(s2.f_in.size(), -1);
+      for (size_t x = 0; x < s2.f_in.size(); x++) {
+        if (x == k)
+          continue;
+        in_map[x] = (int)m.f_in.size();
+        m.f_in.push_back(s2.f_in[x]);
+        m.f_in_dt.push_back(s2.f_in_dt[x]);
+        m.f_str.push_back(permute(s2.f_str[x]));
+        m.f_in_tensor.push_back(s2.f_in_tensor[x]);
+      }
+      auto map2 = [&](int reg) {
+        if (reg == (int)k)
+          return r_reg;
+        if (reg < (int)s2.f_in.size())
+          return in_map[(size_t)reg];
+        return (int)n_in_new + (int)s1.f_ins.size() + (reg - (int)s2.f_in.size());
+      };
+      for (auto f : s2.f_ins) {
+        f.a = map2(f.a), f.b = map2(f.b);
+        m.f_ins.push_back(f);
+      }
+      m.out = s2.out, m.out_dt = s2.out_dt, m.red_reg = map2(s2.red_reg);
+      m.out_str = permute(dense_strides(s2.dims));
+      m.f_members.insert(m.f_members.end(), s2.f_members.begin(), s2.f_members.end());
+      m.f_out_tensor = s2.f_out_tensor;
+      if (fused_registers(m) > gcmi::FUSED_MAX_PHYS)
+        continue;
+      skip[i1] = true;
+      emit_at.erase(i1);
+      it2->second[0] = m;
+      break;
+    }
   }
 }
 
@@ -1126,6 +1248,39 @@ void Executable::plan_generic(const Op &op) {
   steps_.push_back(std::move(s));
 }
 
+// the parameter block of a fused step, without the operand addresses
+static void fill_fused_params(const Step &s, gcmi::FusedParams &p) {
+  p.n_in = (int)s.f_in.size(), p.n_in_pre = s.n_in_pre, p.n_ins = (int)s.f_ins.size(), p.sum_ins = s.sum_ins;
+  const size_t r = s.dims.size(), pad = gcmi::ELT_MAX_RANK - r;
+  p.n = 1;
+  for (int d = 0; d < gcmi::ELT_MAX_RANK; d++)
+    p.dims[d] = 1;
+  for (size_t d = 0; d < r; d++)
+    p.dims[pad + d] = s.dims[d], p.n *= s.dims[d];
+  for (int k = 0; k < p.n_in; k++) {
+    p.in_dt[k] = s.f_in_dt[(size_t)k];
+    for (size_t d = 0; d < r; d++)
+      p.in_str[k][pad + d] = s.f_str[(size_t)k][d];
+  }
+  for (int j = 0; j < p.n_ins; j++) {
+    const Step::FIns &f = s.f_ins[(size_t)j];
+    p.ins[j].op = f.op, p.ins[j].a = f.a, p.ins[j].b = f.b, p.ins[j].dt = f.dt, p.ins[j].imm = f.imm;
+  }
+  p.out_dt = s.out_dt, p.out_reg = s.red_reg;
+  p.n_red = s.sum_ins >= 0 ? s.n_red : 1, p.mean = s.mean;
+  const bool second_pass = s.row_end >= 0;
+  p.n_in_row = second_pass ? s.n_in_row : p.n_in, p.row_end = second_pass ? s.row_end : p.n_ins;
+  for (size_t d = 0; d < r && second_pass; d++)
+    p.out_str[pad + d] = s.out_str[d];
+}
+
+// physical registers the step's program needs (the kernels hold gcmi::FUSED_MAX_PHYS)
+static int fused_registers(const Step &s) {
+  gcmi::FusedParams p{};
+  fill_fused_params(s, p);
+  return gcmi::fused_allocate(p);
+}
+
 // ---------------------------------------------------------------------------
 void Executable::launch(const Step &s) {
   auto P = [&](int slot) -> char * { return slot < 0 ? nullptr : (char *)ptr_[(size_t)slot]; };
@@ -1207,24 +1362,12 @@ void Executable::launch(const Step &s) {
   }
   case Step::Fused: {
     gcmi::FusedParams p{};
-    p.n_in = (int)s.f_in.size(), p.n_in_pre = s.n_in_pre, p.n_ins = (int)s.f_ins.size(), p.sum_ins = s.sum_ins;
-    const size_t r = s.dims.size(), pad = gcmi::ELT_MAX_RANK - r;
-    p.n = 1;
-    for (int d = 0; d < gcmi::ELT_MAX_RANK; d++)
-      p.dims[d] = 1;
-    for (size_t d = 0; d < r; d++)
-      p.dims[pad + d] = s.dims[d], p.n *= s.dims[d];
-    for (int k = 0; k < p.n_in; k++) {
-      p.in[k] = P(s.f_in[(size_t)k]), p.in_dt[k] = s.f_in_dt[(size_t)k];
-      for (size_t d = 0; d < r; d++)
-        p.in_str[k][pad + d] = s.f_str[(size_t)k][d];
-    }
-    for (int j = 0; j < p.n_ins; j++) {
-      const Step::FIns &f = s.f_ins[(size_t)j];
-      p.ins[j].op = f.op, p.ins[j].a = f.a, p.ins[j].b = f.b, p.ins[j].dt = f.dt, p.ins[j].imm = f.imm;
-    }
-    p.out = P(s.out), p.out_dt = s.out_dt, p.out_reg = s.red_reg;
-    p.n_red = s.sum_ins >= 0 ? s.n_red : 1, p.mean = s.mean;
+    fill_fused_params(s, p);
+    const size_t r = s.dims.size();
+    const bool second_pass = s.row_end >= 0;
+    for (int k = 0; k < p.n_in; k++)
+      p.in[k] = P(s.f_in[(size_t)k]);
+    p.out = P(s.out);
     // the furthest element any input index can reach lies inside its buffer, and the output fits
     auto esz = [](int dt) { return dt == GCMI_F32 ? 4 : 2; };
     for (int k = 0; k < p.n_in; k++) {
@@ -1234,7 +1377,7 @@ void Executable::launch(const Step &s) {
       if ((size_t)(far + 1) * (size_t)esz(p.in_dt[k]) > slots_[(size_t)s.f_in[(size_t)k]].bytes)
         throw std::runtime_error("fused group: an input index runs past its buffer (" + s.note + ")");
     }
-    if ((size_t)(p.n / p.n_red) * (size_t)esz(p.out_dt) > slots_[(size_t)s.out].bytes)
+    if ((size_t)(second_pass ? p.n : p.n / p.n_red) * (size_t)esz(p.out_dt) > slots_[(size_t)s.out].bytes)
       throw std::runtime_error("fused group: the result does not fit its buffer (" + s.note + ")");
     gc_check(gcmi_launch_fused(&p, stream_) ? 5 : 0, s.note.c_str());
     break;

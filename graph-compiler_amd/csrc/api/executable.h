@@ -66,6 +66,13 @@ struct Step {
   int64_t n_red = 0;
   int red_reg = 0; // the register that is stored
   int n_in_pre = 0, sum_ins = -1;
+  int n_in_row = -1, row_end = -1;   // second pass of a row kernel (-1: none)
+  std::vector<int64_t> out_str;      // its output strides over `dims`
+  // planning only: what the group holds (ops, the tensor behind each input, the tensor it writes) and, for a
+  // group with a sum, where each non-unit dim of the full shape sits in `dims`
+  std::vector<size_t> f_members, f_in_tensor;
+  size_t f_out_tensor = 0;
+  std::vector<int> f_place;
 };
 
 struct Slot {

@@ -149,17 +149,81 @@ __global__ void reduce_kernel(ReduceParams p) {
 // Fused point-wise groups (FusedParams).  The register file lives in LDS, one column per thread
 // (regs[r][tid]: conflict free, and a register number that is only known at run time costs nothing extra).
 static constexpr int FUSED_THREADS = 256;
+static constexpr int FU = 4; // elements a thread carries through the program together
 
-// The register file: register r of thread tid is regs[r * blockDim.x + tid] in dynamic LDS, sized by the launcher
-// to the registers the program uses.
+// fused groups hold float storage types only: one 4-byte or one 2-byte load
+__device__ __forceinline__ float fused_load_f32(const void *p, int64_t i, int dt) {
+  if (dt == DT_F32)
+    return reinterpret_cast<const float *>(p)[i];
+  const uint16_t h = reinterpret_cast<const uint16_t *>(p)[i];
+  return dt == DT_BF16 ? bf16_bits_to_f32(h) : (float)__builtin_bit_cast(_Float16, h);
+}
+__device__ __forceinline__ void fused_store_f32(void *p, int64_t i, int dt, float v) {
+  if (dt == DT_F32)
+    reinterpret_cast<float *>(p)[i] = v;
+  else
+    reinterpret_cast<uint16_t *>(p)[i] = dt == DT_BF16 ? f32_to_bf16_bits(v) : __builtin_bit_cast(uint16_t, (_Float16)v);
+}
+
+// The register file: register r of thread t is the 16-byte slot (r * threads + t) of dynamic LDS, holding the FU
+// elements the thread carries (one ds_read_b128 / ds_write_b128 per access, conflict free).  Register numbers are
+// only known at run time, which costs nothing extra this way.
+typedef float fused_vec __attribute__((ext_vector_type(FU)));
 struct FusedRegs {
-  float *base;
+  fused_vec *base;
   int threads, tid;
-  __device__ __forceinline__ float &operator[](int r) const { return base[r * threads + tid]; }
+  __device__ __forceinline__ fused_vec get(int r) const { return base[r * threads + tid]; }
+  __device__ __forceinline__ void set(int r, fused_vec v) const { base[r * threads + tid] = v; }
 };
 
-// adds to off[k] (inputs k0 .. k1-1) the contribution of the coordinates of `idx` over iteration dims d_lo .. d_hi-1
-// (innermost first); a single dim needs no division
+// The parameter block is read many times (once per instruction per step) and the kernel-argument segment is slow to
+// reach on a first touch: all threads copy it into LDS together, one word each, so its cache lines are fetched side
+// by side instead of one after the other.
+__device__ __forceinline__ void fused_params_to_lds(FusedParams *dst) {
+  const uint32_t *src = (const uint32_t *)__builtin_amdgcn_kernarg_segment_ptr();
+  uint32_t *d = reinterpret_cast<uint32_t *>(dst);
+  for (unsigned w = threadIdx.x; w < sizeof(FusedParams) / 4; w += blockDim.x)
+    d[w] = src[w];
+  __syncthreads();
+}
+
+// instructions j0 .. j1-1 on the FU elements a thread holds
+__device__ __forceinline__ void fused_run(const FusedParams &p, const FusedRegs &f, int j0, int j1) {
+  for (int j = j0; j < j1; j++) {
+    const FusedIns in = p.ins[j];
+    const int op = __builtin_amdgcn_readfirstlane(in.op), dt = __builtin_amdgcn_readfirstlane(in.dt);
+    const float imm = in.imm;
+    const fused_vec x = f.get(in.a), y = f.get(in.b);
+    fused_vec v;
+    switch (op) {
+#define EACH(expr)                                                                                                        \
+  _Pragma("unroll") for (int u = 0; u < FU; u++) v[u] = (expr);                                                           \
+  break;
+    case ELT_ADD: v = x + y; break;
+    case ELT_SUB: v = x - y; break;
+    case ELT_MUL: v = x * y; break;
+    case ELT_DIV: EACH(x[u] / y[u])
+    case ELT_NEG: v = -x; break;
+    case ELT_SQUARE: v = x * x; break;
+    case ELT_COPY: v = x; break;
+    default: EACH(fused_op(op, x[u], y[u], imm))
+#undef EACH
+    }
+    if (dt == DT_BF16) {
+#pragma unroll
+      for (int u = 0; u < FU; u++)
+        v[u] = bf16_bits_to_f32(f32_to_bf16_bits(v[u]));
+    } else if (dt == DT_F16) {
+#pragma unroll
+      for (int u = 0; u < FU; u++)
+        v[u] = (float)(_Float16)v[u];
+    }
+    f.set(in.d, v);
+  }
+}
+
+// offsets of inputs k0 .. k1-1 for element idx, coordinates taken over iteration dims d_lo .. d_hi-1 (innermost
+// first), added to off[]; a single dim needs no division
 template <typename IDX>
 __device__ __forceinline__ void fused_offsets(const FusedParams &p, IDX idx, int d_lo, int d_hi, int k0, int k1,
                                               IDX (&off)[FUSED_MAX_IN]) {
@@ -182,101 +246,174 @@ __device__ __forceinline__ void fused_offsets(const FusedParams &p, IDX idx, int
   }
 }
 
-// instructions j0 .. j1-1
-__device__ __forceinline__ void fused_run(const FusedParams &p, const FusedRegs &regs, int j0, int j1) {
-  for (int j = j0; j < j1; j++) {
-    const FusedIns in = p.ins[j];
-    const float x = regs[in.a], y = regs[in.b];
-    regs[p.n_in + j] = round_to_storage(fused_op(in.op, x, y, in.imm), in.dt);
+// Four consecutive elements of one input: one 16- or 8-byte load when the input is contiguous there (vec), else
+// four loads `step` elements apart (step 0: a broadcast along the innermost dim)
+__device__ __forceinline__ fused_vec fused_load_quad(const void *p, int64_t i, int dt, bool vec, int64_t step) {
+  fused_vec v;
+  if (vec) {
+    if (dt == DT_F32) {
+      const f32x4_t q = *reinterpret_cast<const f32x4_t *>(reinterpret_cast<const float *>(p) + i);
+      v[0] = q[0], v[1] = q[1], v[2] = q[2], v[3] = q[3];
+    } else {
+      const uint2 q = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p) + i);
+      const uint16_t h[4] = {(uint16_t)q.x, (uint16_t)(q.x >> 16), (uint16_t)q.y, (uint16_t)(q.y >> 16)};
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        v[u] = dt == DT_BF16 ? bf16_bits_to_f32(h[u]) : (float)__builtin_bit_cast(_Float16, h[u]);
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      v[u] = fused_load_f32(p, i + u * step, dt);
+  }
+  return v;
+}
+__device__ __forceinline__ void fused_store_quad(void *p, int64_t i, int dt, bool vec, int64_t step, fused_vec v) {
+  if (vec) {
+    if (dt == DT_F32) {
+      *reinterpret_cast<f32x4_t *>(reinterpret_cast<float *>(p) + i) = f32x4_t{v[0], v[1], v[2], v[3]};
+    } else {
+      uint16_t h[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        h[u] = dt == DT_BF16 ? f32_to_bf16_bits(v[u]) : __builtin_bit_cast(uint16_t, (_Float16)v[u]);
+      *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p) + i) =
+          make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      fused_store_f32(p, i + u * step, dt, v[u]);
   }
 }
+static_assert(FU == 4, "the quad loads and stores move four elements");
 
-// The parameter block is read many times (once per instruction per element) and the kernel-argument segment is
-// slow to reach on a first touch: all threads copy it into LDS together, one word each, so its cache lines are
-// fetched side by side instead of one after the other.
-__device__ __forceinline__ void fused_params_to_lds(FusedParams *dst) {
-  const uint32_t *src = (const uint32_t *)__builtin_amdgcn_kernarg_segment_ptr();
-  uint32_t *d = reinterpret_cast<uint32_t *>(dst);
-  for (unsigned w = threadIdx.x; w < sizeof(FusedParams) / 4; w += blockDim.x)
-    d[w] = src[w];
-  __syncthreads();
-}
-
-template <typename IDX> __device__ __forceinline__ void fused_pointwise_body(const FusedParams &p, const FusedRegs &regs) {
-  const int d0 = ELT_MAX_RANK - p.rank;
-  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < p.n; idx += (int64_t)gridDim.x * blockDim.x) {
+// Inputs k0 .. k1-1 of the four elements a thread holds into their registers.  quad: the elements are e0 .. e0+3
+// of one innermost row (the launcher sets it when the innermost dim is a multiple of 4), so one set of offsets
+// serves all four; otherwise they are the separate elements e[u] (ok[u] false: skipped).
+template <typename IDX>
+__device__ __forceinline__ void fused_load(const FusedParams &p, const FusedRegs &f, const IDX (&e)[FU], const bool (&ok)[FU],
+                                           const IDX (&base)[FUSED_MAX_IN], int d_lo, int d_hi, int k0, int k1) {
+  if (p.quad) {
+    if (!ok[0])
+      return;
     IDX off[FUSED_MAX_IN];
 #pragma unroll
     for (int k = 0; k < FUSED_MAX_IN; k++)
-      off[k] = 0;
-    fused_offsets<IDX>(p, (IDX)idx, d0, ELT_MAX_RANK, 0, p.n_in, off);
+      off[k] = base[k];
+    fused_offsets<IDX>(p, e[0], d_lo, d_hi, k0, k1, off);
+    fused_vec v[FUSED_MAX_IN];
+#pragma unroll
+    for (int k = 0; k < FUSED_MAX_IN; k++) // all loads are issued before the first LDS write waits for one
+      if (k >= k0 && k < k1)
+        v[k] = fused_load_quad(p.in[k], (int64_t)off[k], p.in_dt[k], (p.vec_mask >> k) & 1,
+                               p.in_str[k][ELT_MAX_RANK - 1]);
 #pragma unroll
     for (int k = 0; k < FUSED_MAX_IN; k++)
-      if (k < p.n_in)
-        regs[k] = load_as_f32(p.in[k], (int64_t)off[k], p.in_dt[k]);
-    fused_run(p, regs, 0, p.n_ins);
-    store_from_f32(p.out, idx, p.out_dt, regs[p.out_reg]);
+      if (k >= k0 && k < k1)
+        f.set(p.in_reg[k], v[k]);
+    return;
+  }
+  fused_vec v[FUSED_MAX_IN];
+#pragma unroll
+  for (int u = 0; u < FU; u++) {
+    IDX off[FUSED_MAX_IN];
+#pragma unroll
+    for (int k = 0; k < FUSED_MAX_IN; k++)
+      off[k] = base[k];
+    if (ok[u])
+      fused_offsets<IDX>(p, e[u], d_lo, d_hi, k0, k1, off);
+#pragma unroll
+    for (int k = 0; k < FUSED_MAX_IN; k++)
+      if (k >= k0 && k < k1)
+        v[k][u] = ok[u] ? fused_load_f32(p.in[k], (int64_t)off[k], p.in_dt[k]) : 0.0f;
+  }
+#pragma unroll
+  for (int k = 0; k < FUSED_MAX_IN; k++)
+    if (k >= k0 && k < k1)
+      f.set(p.in_reg[k], v[k]);
+}
+
+// the four elements of thread `t` in the step that starts at element c0, `threads` threads taking part
+template <typename IDX>
+__device__ __forceinline__ void fused_elements(const FusedParams &p, int64_t c0, int64_t limit, int t, int threads,
+                                               IDX (&e)[FU], bool (&ok)[FU]) {
+#pragma unroll
+  for (int u = 0; u < FU; u++) {
+    // quad: four consecutive elements per thread; otherwise consecutive threads take consecutive elements
+    const int64_t idx = p.quad ? c0 + (int64_t)FU * t + u : c0 + (int64_t)u * threads + t;
+    ok[u] = idx < limit;
+    e[u] = (IDX)idx;
   }
 }
 
-__global__ __launch_bounds__(FUSED_THREADS) void fused_pointwise_kernel(FusedParams) {
-  extern __shared__ float fused_lds[];
+// IDX: 32-bit index arithmetic when the whole iteration space fits (the launcher picks), 64-bit otherwise.
+// A workgroup takes FU * FUSED_THREADS consecutive elements per step.
+template <typename IDX> __global__ __launch_bounds__(FUSED_THREADS) void fused_pointwise_kernel(FusedParams) {
+  extern __shared__ fused_vec fused_lds[];
   __shared__ FusedParams p;
   fused_params_to_lds(&p);
-  const FusedRegs regs{fused_lds, (int)blockDim.x, (int)threadIdx.x};
-  if (p.n < ((int64_t)1 << 31)) // 32-bit index arithmetic when the whole space fits
-    fused_pointwise_body<uint32_t>(p, regs);
-  else
-    fused_pointwise_body<int64_t>(p, regs);
+  const FusedRegs f{fused_lds, FUSED_THREADS, (int)threadIdx.x};
+  const int d0 = ELT_MAX_RANK - p.rank;
+  IDX zero[FUSED_MAX_IN];
+#pragma unroll
+  for (int k = 0; k < FUSED_MAX_IN; k++)
+    zero[k] = 0;
+  const int64_t chunk = (int64_t)FU * FUSED_THREADS;
+  for (int64_t c0 = (int64_t)blockIdx.x * chunk; c0 < p.n; c0 += (int64_t)gridDim.x * chunk) {
+    IDX e[FU];
+    bool ok[FU];
+    fused_elements<IDX>(p, c0, p.n, threadIdx.x, FUSED_THREADS, e, ok);
+    fused_load<IDX>(p, f, e, ok, zero, d0, ELT_MAX_RANK, 0, p.n_in);
+    fused_run(p, f, 0, p.n_ins);
+    const fused_vec v = f.get(p.out_reg);
+    if (p.quad) { // the output is dense: four consecutive elements are contiguous
+      if (ok[0])
+        fused_store_quad(p.out, (int64_t)e[0], p.out_dt, p.out_vec, 1, v);
+    } else {
+#pragma unroll
+      for (int u = 0; u < FU; u++)
+        if (ok[u])
+          fused_store_f32(p.out, (int64_t)e[u], p.out_dt, v[u]);
+    }
+  }
 }
 
-// TPR threads work on one row (a multiple of 64: whole waves), THREADS / TPR rows per workgroup.  The loads of
-// several elements per thread are in flight together; partial sums are combined in a fixed tree, so results do not
-// vary from run to run.
+// TPR threads work on one row (a multiple of 64: whole waves), THREADS / TPR rows per workgroup.  Every thread of a
+// row ends up with the row's sum (partial sums are combined in a fixed tree: results do not vary from run to run)
+// and runs the per-row instructions itself, so the second pass needs no exchange.
 template <typename IDX, int THREADS, int TPR>
-__device__ __forceinline__ void fused_rowsum_body(const FusedParams &p, const FusedRegs &regs, float *wave_sum) {
-  constexpr int U = TPR >= 1024 ? 2 : 4; // 1024 threads leave 128 registers per lane
+__global__ __launch_bounds__(THREADS) void fused_rowsum_kernel(FusedParams) {
+  extern __shared__ fused_vec fused_lds[];
+  __shared__ float wave_sum[THREADS / 64];
+  __shared__ FusedParams p;
+  fused_params_to_lds(&p);
+  const FusedRegs f{fused_lds, THREADS, (int)threadIdx.x};
   const int tid = threadIdx.x, sub = tid % TPR;
   const int64_t rows = p.n / p.n_red;
-  const int64_t row = (int64_t)blockIdx.x * (THREADS / TPR) + tid / TPR;
+  const int64_t row_raw = (int64_t)blockIdx.x * (THREADS / TPR) + tid / TPR;
+  const bool live = row_raw < rows;
+  const int64_t row = live ? row_raw : rows - 1; // threads past the last row shadow it and store nothing
   const int d0 = ELT_MAX_RANK - p.rank, d_row = ELT_MAX_RANK - p.rank_red;
-  const FusedIns sum = p.ins[p.sum_ins];
-  float acc = 0.0f;
+  const int sum_a = p.ins[p.sum_ins].a, sum_d = p.ins[p.sum_ins].d, sum_dt = p.ins[p.sum_ins].dt;
   IDX base[FUSED_MAX_IN];
 #pragma unroll
   for (int k = 0; k < FUSED_MAX_IN; k++)
     base[k] = 0;
-  if (row < rows) {
-    fused_offsets<IDX>(p, (IDX)row, d0, d_row, 0, p.n_in, base);
-    for (int64_t r0 = sub; r0 < p.n_red; r0 += (int64_t)TPR * U) {
-      float v[U][FUSED_MAX_IN];
+  fused_offsets<IDX>(p, (IDX)row, d0, d_row, 0, p.n_in, base);
+
+  float acc = 0.0f;
+  for (int64_t r0 = 0; r0 < p.n_red; r0 += (int64_t)TPR * FU) {
+    IDX e[FU];
+    bool ok[FU];
+    fused_elements<IDX>(p, r0, p.n_red, sub, TPR, e, ok);
+    fused_load<IDX>(p, f, e, ok, base, d_row, ELT_MAX_RANK, 0, p.n_in_pre);
+    fused_run(p, f, 0, p.sum_ins);
+    const fused_vec v = f.get(sum_a);
 #pragma unroll
-      for (int u = 0; u < U; u++) {
-        const int64_t r = r0 + (int64_t)u * TPR;
-        if (r < p.n_red) {
-          IDX off[FUSED_MAX_IN];
-#pragma unroll
-          for (int k = 0; k < FUSED_MAX_IN; k++)
-            off[k] = base[k];
-          fused_offsets<IDX>(p, (IDX)r, d_row, ELT_MAX_RANK, 0, p.n_in_pre, off);
-#pragma unroll
-          for (int k = 0; k < FUSED_MAX_IN; k++)
-            if (k < p.n_in_pre)
-              v[u][k] = load_as_f32(p.in[k], (int64_t)off[k], p.in_dt[k]);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < U; u++) {
-        if (r0 + (int64_t)u * TPR < p.n_red) {
-#pragma unroll
-          for (int k = 0; k < FUSED_MAX_IN; k++)
-            if (k < p.n_in_pre)
-              regs[k] = v[u][k];
-          fused_run(p, regs, 0, p.sum_ins);
-          acc += regs[sum.a];
-        }
-      }
-    }
+    for (int u = 0; u < FU; u++)
+      if (p.quad ? ok[0] : ok[u])
+        acc += v[u];
   }
 #pragma unroll
   for (int s = 32; s > 0; s >>= 1)
@@ -285,35 +422,58 @@ __device__ __forceinline__ void fused_rowsum_body(const FusedParams &p, const Fu
     if ((tid & 63) == 0)
       wave_sum[tid >> 6] = acc;
     __syncthreads();
-    if (sub == 0) {
-      acc = 0.0f;
-      for (int w = 0; w < TPR / 64; w++)
-        acc += wave_sum[(tid >> 6) + w];
+    acc = 0.0f;
+    const int w0 = (tid / TPR) * (TPR / 64);
+    for (int w = 0; w < TPR / 64; w++)
+      acc += wave_sum[w0 + w];
+  }
+  if (p.mean)
+    acc = acc / (float)p.n_red;
+  acc = sum_dt == DT_BF16 ? bf16_bits_to_f32(f32_to_bf16_bits(acc)) : sum_dt == DT_F16 ? (float)(_Float16)acc : acc;
+  f.set(sum_d, fused_vec(acc));
+  // per-row inputs (stride 0 along the row): the same value in every element slot
+#pragma unroll
+  for (int k = 0; k < FUSED_MAX_IN; k++)
+    if (k >= p.n_in_pre && k < p.n_in_row)
+      f.set(p.in_reg[k], fused_vec(fused_load_f32(p.in[k], (int64_t)base[k], p.in_dt[k])));
+  fused_run(p, f, p.sum_ins + 1, p.row_end);
+  if (p.row_end >= p.n_ins) { // no second pass: one value per row
+    const fused_vec v = f.get(p.out_reg);
+    if (sub == 0 && live)
+      fused_store_f32(p.out, row, p.out_dt, v[0]);
+    return;
+  }
+  // second pass: the output is walked through its own strides
+  auto out_offset = [&](IDX idx, int d_lo, int d_hi) {
+    IDX o = 0, rem = idx;
+    for (int d = d_hi - 1; d >= d_lo; d--) {
+      const IDX dim = (IDX)p.dims[d];
+      o += (rem % dim) * (IDX)p.out_str[d];
+      rem /= dim;
+    }
+    return o;
+  };
+  const IDX obase = out_offset((IDX)row, d0, d_row);
+  for (int64_t r0 = 0; r0 < p.n_red; r0 += (int64_t)TPR * FU) {
+    IDX e[FU];
+    bool ok[FU];
+    fused_elements<IDX>(p, r0, p.n_red, sub, TPR, e, ok);
+    fused_load<IDX>(p, f, e, ok, base, d_row, ELT_MAX_RANK, p.n_in_row, p.n_in);
+    fused_run(p, f, p.row_end, p.n_ins);
+    const fused_vec v = f.get(p.out_reg);
+    if (!live)
+      continue;
+    if (p.quad) {
+      if (ok[0])
+        fused_store_quad(p.out, (int64_t)(obase + out_offset(e[0], d_row, ELT_MAX_RANK)), p.out_dt, p.out_vec,
+                         p.out_str[ELT_MAX_RANK - 1], v);
+    } else {
+#pragma unroll
+      for (int u = 0; u < FU; u++)
+        if (ok[u])
+          fused_store_f32(p.out, (int64_t)(obase + out_offset(e[u], d_row, ELT_MAX_RANK)), p.out_dt, v[u]);
     }
   }
-  if (sub == 0 && row < rows) {
-    if (p.mean)
-      acc = acc / (float)p.n_red;
-    regs[p.n_in + p.sum_ins] = round_to_storage(acc, sum.dt);
-#pragma unroll
-    for (int k = 0; k < FUSED_MAX_IN; k++) // the per-row inputs have stride 0 along the row
-      if (k >= p.n_in_pre && k < p.n_in)
-        regs[k] = load_as_f32(p.in[k], (int64_t)base[k], p.in_dt[k]);
-    fused_run(p, regs, p.sum_ins + 1, p.n_ins);
-    store_from_f32(p.out, row, p.out_dt, regs[p.out_reg]);
-  }
-}
-
-template <int THREADS, int TPR> __global__ __launch_bounds__(THREADS) void fused_rowsum_kernel(FusedParams) {
-  extern __shared__ float fused_lds[];
-  __shared__ float wave_sum[THREADS / 64];
-  __shared__ FusedParams p;
-  fused_params_to_lds(&p);
-  const FusedRegs regs{fused_lds, THREADS, (int)threadIdx.x};
-  if (p.n < ((int64_t)1 << 31))
-    fused_rowsum_body<uint32_t, THREADS, TPR>(p, regs, wave_sum);
-  else
-    fused_rowsum_body<int64_t, THREADS, TPR>(p, regs, wave_sum);
 }
 
 // softmax along an axis of length `len` and element stride `stride`; one wave
@@ -363,29 +523,46 @@ extern "C" int gcmi_launch_fused(const FusedParams *pp, hipStream_t stream) {
   if (p.n_in < 1 || p.n_in > FUSED_MAX_IN || p.n_ins < 0 || p.n_ins > FUSED_MAX_INS || p.sum_ins >= p.n_ins)
     return 2;
   if (!has_sum)
-    p.n_in_pre = p.n_in, p.n_red = 1;
-  if (p.n_in_pre < 0 || p.n_in_pre > p.n_in || p.n_red < 1 || p.n % p.n_red != 0)
+    p.n_in_pre = p.n_in_row = p.n_in, p.row_end = p.n_ins, p.n_red = 1;
+  if (p.n_in_pre < 0 || p.n_in_pre > p.n_in_row || p.n_in_row > p.n_in || p.n_red < 1 || p.n % p.n_red != 0 ||
+      (has_sum && (p.row_end <= p.sum_ins || p.row_end > p.n_ins)))
     return 2;
+  auto is_float = [](int dt) { return dt == DT_F32 || dt == DT_BF16 || dt == DT_F16; };
+  for (int k = 0; k < p.n_in; k++)
+    if (!is_float(p.in_dt[k]) || !p.in[k])
+      return 2;
+  if (!is_float(p.out_dt) || !p.out)
+    return 2;
+  const bool second_pass = has_sum && p.row_end < p.n_ins;
+  if (!second_pass && p.n_in_row != p.n_in)
+    return 2;
+  // every instruction reads registers that are already written and that exist in its phase: before the sum the
+  // per-element inputs and results; per row the sum, the per-row inputs and results; in the second pass the
+  // per-row values, its own inputs and results
+  auto phase_of_ins = [&](int j) { return !has_sum ? 0 : j < p.sum_ins ? 0 : j < p.row_end ? 1 : 2; };
+  auto readable = [&](int r, int j) {
+    if (r < 0 || r >= p.n_in + j)
+      return false;
+    if (!has_sum)
+      return true;
+    const int ph = j <= p.sum_ins ? 0 : phase_of_ins(j); // the sum itself reads a per-element value
+    const int src = r < p.n_in ? (r < p.n_in_pre ? 0 : r < p.n_in_row ? 1 : 2) : phase_of_ins(r - p.n_in);
+    return ph == 0 ? src == 0 : ph == 1 ? src == 1 : src >= 1;
+  };
   for (int j = 0; j < p.n_ins; j++) {
-    // an instruction reads registers that are already written; before the sum, only per-element inputs
     const FusedIns &f = p.ins[j];
-    const bool unary_sum = f.op == ELT_ROWSUM;
     if ((f.op == ELT_ROWSUM) != (j == p.sum_ins))
       return 2;
-    for (int r : {f.a, unary_sum ? f.a : f.b}) {
-      if (r < 0 || r >= p.n_in + j)
-        return 2;
-      if (has_sum && j <= p.sum_ins && r >= p.n_in_pre && r < p.n_in)
-        return 2;
-      if (has_sum && j > p.sum_ins && (r < p.n_in_pre || (r >= p.n_in && r < p.n_in + p.sum_ins)))
-        return 2; // per-element values do not exist after the sum
-    }
+    if (!readable(f.a, j) || !readable(f.op == ELT_ROWSUM ? f.a : f.b, j))
+      return 2;
   }
-  if (p.out_reg < 0 || p.out_reg >= p.n_in + p.n_ins || (has_sum && p.out_reg < p.n_in + p.sum_ins))
+  if (p.out_reg < 0 || p.out_reg >= p.n_in + p.n_ins)
+    return 2;
+  if (has_sum && phase_of_ins(p.out_reg - p.n_in) != (second_pass ? 2 : 1))
     return 2;
   // merge neighbouring iteration dims that every input walks contiguously (or not at all): fewer divisions per
   // element.  The boundary between rows and the inside of a row is never merged across.
-  int64_t dims[ELT_MAX_RANK], str[FUSED_MAX_IN][ELT_MAX_RANK];
+  int64_t dims[ELT_MAX_RANK], str[FUSED_MAX_IN][ELT_MAX_RANK], ostr[ELT_MAX_RANK];
   int nd = 0;
   int64_t inner = 1; // elements of the dims to the right of d
   for (int d = ELT_MAX_RANK - 1; d >= 0; d--) {
@@ -394,12 +571,15 @@ extern "C" int gcmi_launch_fused(const FusedParams *pp, hipStream_t stream) {
     bool merge = nd > 0 && !(has_sum && inner == p.n_red);
     for (int k = 0; k < p.n_in && merge; k++)
       merge = p.in_str[k][d] == str[k][nd - 1] * dims[nd - 1];
+    if (merge && second_pass)
+      merge = p.out_str[d] == ostr[nd - 1] * dims[nd - 1];
     if (merge) {
       dims[nd - 1] *= p.dims[d];
     } else {
       dims[nd] = p.dims[d];
       for (int k = 0; k < p.n_in; k++)
         str[k][nd] = p.in_str[k][d];
+      ostr[nd] = p.out_str[d];
       nd++;
     }
     inner *= p.dims[d];
@@ -409,32 +589,76 @@ extern "C" int gcmi_launch_fused(const FusedParams *pp, hipStream_t stream) {
     p.dims[d] = src < nd ? dims[src] : 1;
     for (int k = 0; k < p.n_in; k++)
       p.in_str[k][d] = src < nd ? str[k][src] : 0;
+    p.out_str[d] = src < nd ? ostr[src] : 0;
   }
   p.rank = nd;
+  // quad mode: the innermost dim holds whole groups of four, so a thread's four elements share every outer
+  // coordinate; an operand contiguous there and aligned (base address and outer strides) moves as one vector
+  // (dims are never merged across the boundary of a row, so with a sum the innermost dim lies inside the row
+  // whenever the row has more than one element)
+  p.quad = nd > 0 && dims[0] % 4 == 0 && (!has_sum || p.n_red > 1) ? 1 : 0;
+  p.vec_mask = 0, p.out_vec = 0;
+  if (p.quad) {
+    auto aligned = [&](const void *ptr, int dt, const int64_t *st_of_dim) {
+      const uintptr_t need = dt == DT_F32 ? 16 : 8;
+      if (reinterpret_cast<uintptr_t>(ptr) % need != 0)
+        return false;
+      for (int d = 1; d < nd; d++)
+        if (st_of_dim[d] % 4 != 0)
+          return false;
+      return st_of_dim[0] == 1;
+    };
+    for (int k = 0; k < p.n_in; k++)
+      if (aligned(p.in[k], p.in_dt[k], str[k]))
+        p.vec_mask |= 1 << k;
+    if (second_pass) {
+      p.out_vec = aligned(p.out, p.out_dt, ostr) ? 1 : 0;
+    } else {
+      const uintptr_t need = p.out_dt == DT_F32 ? 16 : 8;
+      p.out_vec = !has_sum && reinterpret_cast<uintptr_t>(p.out) % need == 0 ? 1 : 0;
+    }
+  }
   // collapsed dims that lie inside a row
   p.rank_red = 0;
   for (int64_t in_row = 1; has_sum && in_row < p.n_red && p.rank_red < nd; p.rank_red++)
     in_row *= dims[p.rank_red];
-  const size_t n_regs = (size_t)(p.n_in + p.n_ins);
+  if (fused_allocate(p) > FUSED_MAX_PHYS)
+    return 3;
+  const size_t lds = (size_t)p.n_phys * 256 * sizeof(float) * FU; // the kernels with 256 threads
+  const bool small = p.n < ((int64_t)1 << 31);
   if (has_sum) {
     const int64_t rows = p.n / p.n_red;
     if (rows > 0x7fffffff)
       return 2;
-    // few long rows: 1024 threads per row when their registers fit the 64 KiB a launch may ask for
-    if (p.n_red >= 2048 && rows < 1024 && n_regs * 1024 * 4 + sizeof(FusedParams) + 256 <= 65536) {
-      hipLaunchKernelGGL((fused_rowsum_kernel<1024, 1024>), dim3((unsigned)rows), dim3(1024), n_regs * 1024 * 4, stream, p);
-    } else if (p.n_red >= 512 || rows < 64) {
-      hipLaunchKernelGGL((fused_rowsum_kernel<256, 256>), dim3((unsigned)rows), dim3(256), n_regs * 256 * 4, stream, p);
-    } else {
-      hipLaunchKernelGGL((fused_rowsum_kernel<256, 64>), dim3((unsigned)((rows + 3) / 4)), dim3(256), n_regs * 256 * 4, stream,
-                         p);
+    // few long rows: as many threads per row as the registers leave room for in 64 KiB of LDS
+    const size_t per_thread = (size_t)p.n_phys * sizeof(float) * FU, room = 65536 - sizeof(FusedParams) - 512;
+    if (rows < 512 && p.n_red >= 2048 && per_thread * 512 <= room) { // (1024 threads leave 128 registers: spills)
+      const dim3 grid((unsigned)rows), block(512);
+      if (small)
+        hipLaunchKernelGGL((fused_rowsum_kernel<uint32_t, 512, 512>), grid, block, per_thread * 512, stream, p);
+      else
+        hipLaunchKernelGGL((fused_rowsum_kernel<int64_t, 512, 512>), grid, block, per_thread * 512, stream, p);
+    } else if (p.n_red >= 512 || rows < 64) { // a workgroup of 256 per row
+      const dim3 grid((unsigned)rows), block(256);
+      if (small)
+        hipLaunchKernelGGL((fused_rowsum_kernel<uint32_t, 256, 256>), grid, block, lds, stream, p);
+      else
+        hipLaunchKernelGGL((fused_rowsum_kernel<int64_t, 256, 256>), grid, block, lds, stream, p);
+    } else { // a wave per row
+      const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+      if (small)
+        hipLaunchKernelGGL((fused_rowsum_kernel<uint32_t, 256, 64>), grid, block, lds, stream, p);
+      else
+        hipLaunchKernelGGL((fused_rowsum_kernel<int64_t, 256, 64>), grid, block, lds, stream, p);
     }
   } else {
-    int64_t blocks = (p.n + FUSED_THREADS - 1) / FUSED_THREADS;
+    int64_t blocks = (p.n + FU * FUSED_THREADS - 1) / (FU * FUSED_THREADS);
     if (blocks > 16384)
       blocks = 16384;
-    hipLaunchKernelGGL(fused_pointwise_kernel, dim3((unsigned)blocks), dim3(FUSED_THREADS), n_regs * FUSED_THREADS * 4, stream,
-                       p);
+    if (small)
+      hipLaunchKernelGGL(fused_pointwise_kernel<uint32_t>, dim3((unsigned)blocks), dim3(FUSED_THREADS), lds, stream, p);
+    else
+      hipLaunchKernelGGL(fused_pointwise_kernel<int64_t>, dim3((unsigned)blocks), dim3(FUSED_THREADS), lds, stream, p);
   }
   return hipGetLastError() == hipSuccess ? 0 : 5;
 }

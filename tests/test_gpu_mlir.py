@@ -165,9 +165,12 @@ def test_fused_groups_compute_what_the_single_ops_compute(ga, mm, dev, monkeypat
     """Every instruction of a fused group rounds to its op's storage type, so fusing changes no bit: the decoder
     block with the fusion pass on (10 launches) and off (one launch per op)."""
     fused = _block_outputs(ga, mm, dev, 32, 512, 768, seed=3)
+    fused_rows = _block_outputs(ga, mm, dev, 640, 256, 512, seed=4)  # rows enough for the one-launch normalisation
     monkeypatch.setenv("GCMI_NO_POINTWISE_FUSION", "1")
     single = _block_outputs(ga, mm, dev, 32, 512, 768, seed=3)
+    single_rows = _block_outputs(ga, mm, dev, 640, 256, 512, seed=4)
     assert torch.equal(fused[0], single[0]) and torch.equal(fused[1], single[1])
+    assert torch.equal(fused_rows[0], single_rows[0]) and torch.equal(fused_rows[1], single_rows[1])
 
 
 def test_fused_broadcasts_views_and_reductions(ga, dev):
@@ -283,3 +286,31 @@ def test_linalg_driver_contractions(ga, mm, dev):
         out = np.full(ref.shape, -7.0, np.float32)
         _run(ga, mm.linalg_op(op, [list(a.shape) for a in ins], list(ref.shape)), list(enumerate(ins)), [(2, out)])
         assert (out == ref).all(), op
+
+
+def test_row_statistic_and_scaling_in_one_launch(ga, dev):
+    """y = x / sum over the MIDDLE axis of x^2 (a normalisation whose rows are strided in memory): the statistic and
+    the scaling are one kernel, the second pass writes through the output's own strides."""
+    text = """func.func @f(%x: tensor<36x40x24xf32>, %g: tensor<24xf32>) -> tensor<36x40x24xf32> {
+      %e3 = tensor.empty() : tensor<36x40x24xf32>
+      %e2 = tensor.empty() : tensor<36x24xf32>
+      %c0 = arith.constant 0.0 : f32
+      %z = linalg.fill ins(%c0 : f32) outs(%e2 : tensor<36x24xf32>) -> tensor<36x24xf32>
+      %sq = linalg.square ins(%x : tensor<36x40x24xf32>) outs(%e3 : tensor<36x40x24xf32>) -> tensor<36x40x24xf32>
+      %s = linalg.reduce { arith.addf } ins(%sq : tensor<36x40x24xf32>) outs(%z : tensor<36x24xf32>) dimensions = [1]
+      %rs = linalg.rsqrt ins(%s : tensor<36x24xf32>) outs(%e2 : tensor<36x24xf32>) -> tensor<36x24xf32>
+      %sb = linalg.broadcast ins(%rs : tensor<36x24xf32>) outs(%e3 : tensor<36x40x24xf32>) dimensions = [1]
+      %gb = linalg.broadcast ins(%g : tensor<24xf32>) outs(%e3 : tensor<36x40x24xf32>) dimensions = [0, 1]
+      %n = linalg.mul ins(%x, %sb : tensor<36x40x24xf32>, tensor<36x40x24xf32>) outs(%e3 : tensor<36x40x24xf32>) -> tensor<36x40x24xf32>
+      %y = linalg.mul ins(%n, %gb : tensor<36x40x24xf32>, tensor<36x40x24xf32>) outs(%e3 : tensor<36x40x24xf32>) -> tensor<36x40x24xf32>
+      return %y : tensor<36x40x24xf32>
+    }"""
+    st, plan = ga.explain_mlir(text)
+    assert st == 0 and plan.startswith("reduce: Multiply+Multiply after Rsqrt of ReduceSum of Square\narena"), plan
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((36, 40, 24)).astype(np.float32)
+    g = rng.standard_normal(24).astype(np.float32)
+    out = np.zeros((36, 40, 24), np.float32)
+    _run(ga, text, [(0, x), (1, g)], [(2, out)])
+    ref = x / np.sqrt((x.astype(np.float64) ** 2).sum(1, keepdims=True)) * g
+    assert_close(ref, out, 1e-5, "normalisation over the middle axis")

@@ -50,8 +50,9 @@ def test_generic_contraction_is_a_matmul(ga, mm):
 
 
 def test_decoder_block_plan(ga, mm):
-    """31 linalg/tensor ops become 10 launches: four GEMMs, and per RMSNorm one launch for the row statistic
-    (x^2 summed, / H, + eps, ^-0.5 in one kernel) and one for the scaling."""
+    """31 linalg/tensor ops become 10 launches at 32 tokens: four GEMMs, per RMSNorm one launch for the row statistic
+    (x^2 summed, / H, + eps, ^-0.5 in one kernel) and one for the scaling, the gate, the residual.  With rows enough
+    to fill the GPU (1024 tokens) the scaling runs as a second pass inside the row kernel: 8 launches."""
     st, plan = ga.explain_mlir(mm.decoder_mlp_block(32, 256, 512))
     assert st == OK, plan
     assert _steps(plan) == [
@@ -65,6 +66,17 @@ def test_decoder_block_plan(ga, mm):
         "fused: Add+Add",                    # the first residual sum is recomputed rather than stored
         "reduce: Divide+Add+Pow of ReduceSum of TypeCast+Pow",
         "fused: TypeCast+Multiply+TypeCast+Multiply"]
+    st, plan = ga.explain_mlir(mm.decoder_mlp_block(1024, 256, 512))
+    assert st == OK, plan
+    assert _steps(plan) == [
+        "gemm_bf16: MatMul",
+        "reduce: Add+TypeCast+Multiply+TypeCast+Multiply after Divide+Add+Pow of ReduceSum of Add+TypeCast+Pow",
+        "gemm_bf16: MatMul",
+        "gemm_bf16: MatMul",
+        "fused: Sigmoid+Multiply+Multiply",
+        "gemm_bf16: MatMul",
+        "fused: Add+Add",
+        "reduce: TypeCast+Multiply+TypeCast+Multiply after Divide+Add+Pow of ReduceSum of TypeCast+Pow"]
 
 
 def test_pointwise_fusion_rules(ga, monkeypatch):
