@@ -1,12 +1,16 @@
-// Generic element-wise, reduction, softmax and (de)quantise kernels for the ops
-// of a partition that are not fused into a GEMM or attention kernel.  Every op
+// Element-wise, reduction, softmax and (de)quantise kernels for the ops of a
+// partition that are not fused into a GEMM or attention kernel: single-op
+// kernels, and the kernels that run a whole group of point-wise ops (with an
+// optional row sum inside) as one launch.  Every op
 // reads its operands in their storage type (f32 / bf16 / f16 / s8 / u8 / s32),
 // computes in f32 and rounds once to the result type, which is what the
 // reference's bf16->f32 emulation does to each op
 // (lib/gc/Transforms/Pipeline.cpp:79-95).  Semantics per op:
 //   Add/Subtract/Multiply/Divide  numpy broadcasting
 //                                 (lib/gc/Transforms/OneDNNGraphToLinalg.cpp:64-118)
-//   Maximum / Exp / Neg           linalg.max, linalg.exp, linalg.negf of the MLIR front end
+//   Maximum / Minimum / Exp / Neg / Abs / Ceil / Floor / Erf / Log / Round / Rsqrt / Sqrt / Square / Tanh /
+//   Reciprocal                    the named linalg ops of the MLIR front end (arith / math semantics; Round is
+//                                 math.round, halves away from zero)
 //   ReLU max(x,0), Sigmoid 1/(1+exp(-x)), Pow x^beta, Typecast = copy with rounding
 //                                 (OneDNNGraphToLinalg.cpp:331-358)
 //   ReduceSum / ReduceMean        sum over axes, mean divides by the count (:505-559)
