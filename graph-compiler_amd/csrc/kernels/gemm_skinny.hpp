@@ -115,8 +115,41 @@ template <int MT> __global__ __launch_bounds__(SK_WAVES * 64, 2) void gemm_skinn
       v[c] = sum;
     }
     const int64_t m = mt * 32 + l32, n = n0 + 8 * q + 4 * lh;
-    if (m < p.M)
+    if (m >= p.M)
+      continue;
+    if (p.splits > 1) {
       *reinterpret_cast<f32x4_t *>(part + m * p.N + n) = v;
+      continue;
+    }
+    // one slice: this workgroup holds the whole sum, the epilogue runs here (same rounding points as the second pass)
+    float o32[4];
+    uint16_t o16[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      float b = 0.0f;
+      if (p.bias)
+        b = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n + c])
+                                 : reinterpret_cast<const float *>(p.bias)[n + c];
+      float x = v[c];
+      if (p.out_dt == DT_BF16) {
+        x = round_bf16(x);
+        if (p.bias)
+          x = round_bf16(x + b);
+        if (p.act != ACT_NONE)
+          x = round_bf16(apply_act(x, p.act));
+      } else {
+        if (p.bias)
+          x = x + b;
+        x = apply_act(x, p.act);
+      }
+      o32[c] = x;
+      o16[c] = f32_to_bf16_bits(x);
+    }
+    if (p.out_dt == DT_BF16)
+      *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.C) + m * p.ldc + n) =
+          make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
+    else
+      *reinterpret_cast<f32x4_t *>(reinterpret_cast<float *>(p.C) + m * p.ldc + n) = f32x4_t{o32[0], o32[1], o32[2], o32[3]};
   }
 }
 
@@ -134,14 +167,16 @@ static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream) {
     return -1;
   const int mt = p.M <= 32 ? 1 : 2;
   const int n_cu = gcmi_num_cus(), nblocks = (int)(p.N / 32), steps = (int)(p.K / 64);
-  // workgroup slices: fill whole rounds of two workgroups per compute unit, keep every wave at two or more steps,
-  // and keep the partial-sum traffic (S x M x N f32, written and read) small against the weights
+  // workgroup slices: whole rounds of one workgroup per compute unit (measured: 32 x 4096 x 4096 takes 20 us with
+  // 128 workgroups, 15 us with 256, 17 us with 512; a compute unit pulls about 17 GB/s whatever it has in flight, so
+  // all of them must pull, evenly), every wave at two or more steps, and little partial-sum traffic (S x M x N f32,
+  // written and read) against the weights.  One slice needs no second kernel: the epilogue runs in place.
   int best = 1;
   double best_score = -1.0;
   for (int s = 1; s <= 16; s++) {
     if (steps / (s * SK_WAVES) < 2 || (int64_t)s * p.M * p.N > G_SPLITK_WS_FLOATS)
       break;
-    const double rounds = (double)nblocks * s / (2.0 * n_cu);
+    const double rounds = (double)nblocks * s / (double)n_cu;
     const double fill = rounds / (double)(int64_t)(rounds + 0.999999);
     const double extra = (double)s * (32.0 * mt) * 8.0 / ((double)p.K * 2.0);
     const double score = fill / (1.0 + extra);
@@ -160,6 +195,8 @@ static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream) {
     hipLaunchKernelGGL(gemm_skinny_nt_kernel<1>, grid, block, 0, stream, p);
   else
     hipLaunchKernelGGL(gemm_skinny_nt_kernel<2>, grid, block, 0, stream, p);
+  if (best == 1) // the epilogue ran in the kernel
+    return hipGetLastError() == hipSuccess ? 0 : 5;
   const unsigned rblocks = (unsigned)((p.M * (p.N / 4) + 255) / 256);
   switch (p.act) {
   case ACT_RELU:

@@ -219,7 +219,7 @@ def test_short_a_takes_split_k(gc, orc, wl, dev, M, N, K, act, with_bias, out_f3
 
 NT_SHAPES = [(256, 256, 128), (512, 768, 256), (300, 200, 100), (257, 511, 129), (1, 7, 5), (33, 1, 64), (128, 256, 8),
              (32, 4096, 4096), (1, 1024, 2048), (32, 11008, 4096), (64, 512, 2048), (33, 1024, 1024), (17, 2048, 512),
-             (32, 4096, 11008), (65, 1024, 1024), (32, 1056, 1088)]
+             (32, 4096, 11008), (65, 1024, 1024), (32, 1056, 1088), (32, 8192, 1024), (64, 8192, 512)]
 
 
 def _streams_weights(M, N, K):
@@ -259,9 +259,10 @@ def test_bf16_gemm_transposed_b(gc, orc, wl, dev, M, N, K):
 
 def test_bf16_gemm_streaming_kernel_exact_on_integers(gc, dev):
     """Small integers: every product and partial sum is exact in f32, so any summation order gives the same bits.
-    32 and 64 rows, K slices of unequal length (K/64 = 43 steps over 16 waves)."""
+    32 and 64 rows, K slices of unequal length (K/64 = 43 steps over 16 waves), and wide N where one slice per
+    workgroup is enough and the epilogue runs inside the streaming kernel."""
     torch.manual_seed(8)
-    for M, N, K in [(32, 1024, 2752), (64, 1024, 2752), (5, 4096, 256)]:
+    for M, N, K in [(32, 1024, 2752), (64, 1024, 2752), (5, 4096, 256), (32, 8192, 1024), (40, 16384, 512)]:
         A = torch.randint(-3, 4, (M, K), device=dev).to(torch.bfloat16)
         Bt = torch.randint(-3, 4, (N, K), device=dev).to(torch.bfloat16)
         out = gc.gemm_bf16_nt(A, Bt, out_dtype=gc.F32)
