@@ -1053,7 +1053,9 @@ void Executable::plan_fusion(std::vector<bool> &skip, const std::vector<bool> &c
       if (i1 == n)
         continue;
       const Step &s1 = emit_at[i1][0];
-      // nothing but this group reads r
+      // nothing but this group reads r, and it reads it one way (one input)
+      if (std::count(s2.f_in_tensor.begin(), s2.f_in_tensor.end(), r) != 1)
+        continue;
       bool only_here = true;
       for (size_t c : consumers[r])
         only_here = only_here && std::find(s2.f_members.begin(), s2.f_members.end(), c) != s2.f_members.end();

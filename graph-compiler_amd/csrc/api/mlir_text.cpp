@@ -793,7 +793,7 @@ void fuse_sigmoid(Graph &g, const std::set<size_t> &outputs) {
 // consumer does the same.  The operand is used as it is when it maps to the trailing result dimensions,
 // otherwise through a view with 1s at the added dimensions.
 void fold_broadcasts(Graph &g, const std::set<size_t> &outputs, size_t &next_id) {
-  static const std::set<std::string> binary = {"Add", "Subtract", "Multiply", "Divide", "Maximum"};
+  static const std::set<std::string> binary = {"Add", "Subtract", "Multiply", "Divide", "Maximum", "Minimum"};
   auto users = users_of(g);
   for (size_t i = 0; i < g.ops.size(); i++) {
     Op &o = g.ops[i];
@@ -838,6 +838,35 @@ void fold_broadcasts(Graph &g, const std::set<size_t> &outputs, size_t &next_id)
     if (o.kind != "Dead")
       keep.push_back(o);
   g.ops.swap(keep);
+}
+
+// x . transpose(w) written as linalg.transpose + linalg.matmul (what exporters emit for a Linear layer) is the
+// matmul with the transpose flag: the kernels read either layout in place
+void fold_transposes(Graph &g) {
+  std::map<size_t, size_t> producer;
+  for (size_t i = 0; i < g.ops.size(); i++)
+    producer[g.ops[i].out[0]] = i;
+  for (auto &mm : g.ops) {
+    if (mm.kind != "MatMul")
+      continue;
+    for (size_t side = 0; side < 2 && side < mm.in.size(); side++) {
+      auto it = producer.find(mm.in[side]);
+      if (it == producer.end() || g.ops[it->second].kind != "Transpose")
+        continue;
+      const Op &t = g.ops[it->second];
+      const std::vector<int64_t> &perm = t.attrs.at("perm").ia;
+      const size_t r = perm.size();
+      bool last_two = r >= 2 && perm[r - 1] == (int64_t)r - 2 && perm[r - 2] == (int64_t)r - 1;
+      for (size_t d = 0; d + 2 < r; d++)
+        last_two = last_two && perm[d] == (int64_t)d;
+      if (!last_two)
+        continue;
+      const char *flag = side == 0 ? "transpose_a" : "transpose_b";
+      const bool was = mm.attrs.count(flag) && mm.attrs.at(flag).b;
+      mm.attrs[flag] = attr_bool(!was);
+      mm.in[side] = t.in[0];
+    }
+  }
 }
 
 void drop_dead_ops(Graph &g, const std::set<size_t> &outputs) {
@@ -1022,6 +1051,7 @@ Graph parse_mlir(const char *text) {
   std::set<size_t> outs(g.output_ids.begin(), g.output_ids.end());
   fuse_sigmoid(g, outs);
   fold_broadcasts(g, outs, b.next_id);
+  fold_transposes(g);
   drop_dead_ops(g, outs);
   if (g.output_ids.empty())
     bad("the function returns nothing");

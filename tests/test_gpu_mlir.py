@@ -314,3 +314,42 @@ def test_row_statistic_and_scaling_in_one_launch(ga, dev):
     _run(ga, text, [(0, x), (1, g)], [(2, out)])
     ref = x / np.sqrt((x.astype(np.float64) ** 2).sum(1, keepdims=True)) * g
     assert_close(ref, out, 1e-5, "normalisation over the middle axis")
+
+
+def test_transpose_and_unfolded_broadcast(ga, dev):
+    """linalg.transpose is a strided copy; a linalg.broadcast whose result is returned (nothing to fold it into) is a
+    stride-0 copy."""
+    text = """func.func @f(%x: tensor<8x16x4xf32>, %v: tensor<16xf32>) -> (tensor<4x8x16xf32>, tensor<8x16xf32>) {
+      %e = tensor.empty() : tensor<4x8x16xf32>
+      %t = linalg.transpose ins(%x : tensor<8x16x4xf32>) outs(%e : tensor<4x8x16xf32>) permutation = [2, 0, 1]
+      %c = arith.constant dense<1.500000e+00> : tensor<4x8x16xf32>
+      %y = linalg.mul ins(%t, %c : tensor<4x8x16xf32>, tensor<4x8x16xf32>) outs(%e : tensor<4x8x16xf32>) -> tensor<4x8x16xf32>
+      %e2 = tensor.empty() : tensor<8x16xf32>
+      %b = linalg.broadcast ins(%v : tensor<16xf32>) outs(%e2 : tensor<8x16xf32>) dimensions = [0]
+      return %y, %b : tensor<4x8x16xf32>, tensor<8x16xf32>
+    }"""
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal((8, 16, 4)).astype(np.float32)
+    v = rng.standard_normal(16).astype(np.float32)
+    y, b = np.zeros((4, 8, 16), np.float32), np.zeros((8, 16), np.float32)
+    _run(ga, text, [(0, x), (1, v)], [(2, y), (3, b)])
+    assert (y == x.transpose(2, 0, 1) * np.float32(1.5)).all()
+    assert (b == np.broadcast_to(v, (8, 16))).all()
+
+
+def test_linear_layer_spelled_with_a_transpose(ga, dev):
+    text = """func.func @f(%x: tensor<64x256xbf16>, %w: tensor<512x256xbf16>) -> tensor<64x512xbf16> {
+      %et = tensor.empty() : tensor<256x512xbf16>
+      %wt = linalg.transpose ins(%w : tensor<512x256xbf16>) outs(%et : tensor<256x512xbf16>) permutation = [1, 0]
+      %c0 = arith.constant 0.0 : bf16
+      %e = tensor.empty() : tensor<64x512xbf16>
+      %z = linalg.fill ins(%c0 : bf16) outs(%e : tensor<64x512xbf16>) -> tensor<64x512xbf16>
+      %y = linalg.matmul ins(%x, %wt : tensor<64x256xbf16>, tensor<256x512xbf16>) outs(%z : tensor<64x512xbf16>) -> tensor<64x512xbf16>
+      return %y : tensor<64x512xbf16>
+    }"""
+    torch.manual_seed(17)
+    x = torch.randn(64, 256, device=dev).bfloat16()
+    w = (torch.randn(512, 256, device=dev) * 0.1).bfloat16()
+    y = torch.zeros(64, 512, device=dev, dtype=torch.bfloat16)
+    _run(ga, text, [(0, x), (1, w)], [(2, y)])
+    assert_close((x.double() @ w.double().t()).cpu().numpy(), y.double().cpu().numpy(), 1e-2, "linear with transpose")

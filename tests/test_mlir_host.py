@@ -199,3 +199,22 @@ def test_linalg_driver_single_ops_plan(ga, mm):
         assert any(s.startswith("gemm_f32") for s in _steps(plan)), (op, plan)
     # packed layouts and convolutions are outside the subset
     assert ga.explain_mlir(mm.linalg_op("mmt4d", [[2, 2, 4, 4], [2, 2, 4, 4]], [2, 2, 4, 4]))[0] == UNIMPL
+
+
+def test_transpose_in_front_of_a_matmul_becomes_its_flag(ga):
+    """x . transpose(w), as exporters write a Linear layer: one GEMM that reads w as it lies."""
+    text = """func.func @f(%x: tensor<64x256xbf16>, %w: tensor<512x256xbf16>) -> tensor<64x512xbf16> {
+      %et = tensor.empty() : tensor<256x512xbf16>
+      %wt = linalg.transpose ins(%w : tensor<512x256xbf16>) outs(%et : tensor<256x512xbf16>) permutation = [1, 0]
+      %c0 = arith.constant 0.0 : bf16
+      %e = tensor.empty() : tensor<64x512xbf16>
+      %z = linalg.fill ins(%c0 : bf16) outs(%e : tensor<64x512xbf16>) -> tensor<64x512xbf16>
+      %y = linalg.matmul ins(%x, %wt : tensor<64x256xbf16>, tensor<256x512xbf16>) outs(%z : tensor<64x512xbf16>) -> tensor<64x512xbf16>
+      return %y : tensor<64x512xbf16>
+    }"""
+    st, plan = ga.explain_mlir(text)
+    assert st == OK and _steps(plan) == ["gemm_bf16: MatMul"], plan
+    # a transpose that is not of the last two dims stays a copy
+    other = text.replace("permutation = [1, 0]", "permutation = [0, 1]").replace("tensor<256x512xbf16>", "tensor<512x256xbf16>")
+    st, plan = ga.explain_mlir(other)
+    assert st != OK or "Transpose" in plan
