@@ -5,9 +5,12 @@
 
 A step is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM.  The headline workload is the bf16 4096^3 GEMM; the
-int8 MLP layer, the bf16 MLP chain, fused attention and the f32 plumbing case
-are measured in the same run and reported under "others".  One JSON line goes
-to stdout; progress goes to stderr.
+int8 MLP layer, the bf16 MLP chain, fused attention, decode-shaped GEMMs (32
+rows against Llama FFN weights, HBM bound), the f32 plumbing case, the vendor
+libraries on the same shapes, the headline GEMM through the partition API and
+the llama-2 MLP block through the textual-MLIR entry point are measured in the
+same run and reported under "others" (--only picks some of them).  One JSON
+line goes to stdout; progress goes to stderr.
 
 Kernel durations come from HIP events recorded on the stream the kernels are
 launched on (torch's current stream), one pair per launch.  Inputs rotate over
