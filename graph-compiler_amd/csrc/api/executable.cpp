@@ -748,6 +748,8 @@ void Executable::plan_fusion(std::vector<bool> &skip, const std::vector<bool> &c
     const Op &o = g_.ops[i];
     if (!is_free[i] || !(o.kind == "ReduceSum" || o.kind == "ReduceMean"))
       return false;
+    if (!o.attrs.count("axes") || o.attrs.at("axes").ia.empty())
+      return false; // nothing is reduced: a copy (plan_generic)
     const LTensor &it = T(o.in[0]);
     return storage_float(it.dt) && storage_float(T(o.out[0]).dt) && it.shape.size() <= (size_t)gcmi::ELT_MAX_RANK &&
            is_dense(it);
@@ -1219,6 +1221,13 @@ void Executable::plan_generic(const Op &op) {
     if (ax < 0)
       ax += (int64_t)out.shape.size();
     s.ch_axis = (int)ax;
+  } else if ((k == "ReduceSum" || k == "ReduceMean") && (!op.attrs.count("axes") || op.attrs.at("axes").ia.empty())) {
+    // no axes: the op returns its operand
+    s.note = k + " without axes (copy)";
+    s.op = gcmi::ELT_COPY;
+    s.a = slot_for(op.in[0]), s.out = slot_for(op.out[0]);
+    s.a_dt = dt_dnnl(T(op.in[0]).dt), s.out_dt = dt_dnnl(out.dt);
+    s.dims = {out.numel()}, s.sa = {1};
   } else if (k == "ReduceSum" || k == "ReduceMean") {
     const LTensor &in = T(op.in[0]);
     std::vector<int64_t> axes;

@@ -361,12 +361,9 @@ bool broadcast_shape(const std::vector<int64_t> &a, const std::vector<int64_t> &
 }
 
 std::vector<int64_t> canonical_axes(const std::vector<int64_t> &axes, int64_t rank) {
+  // no axes: nothing is reduced, the op returns its operand
+  // (lib/gc/Dialect/OneDNNGraph/OneDNNGraphOps.cpp:116-120, lib/gc/Transforms/OneDNNGraphToLinalg.cpp:320-324)
   std::vector<int64_t> o;
-  if (axes.empty()) {
-    for (int64_t i = 0; i < rank; i++)
-      o.push_back(i);
-    return o;
-  }
   for (auto a : axes)
     o.push_back(a < 0 ? a + rank : a);
   std::sort(o.begin(), o.end());

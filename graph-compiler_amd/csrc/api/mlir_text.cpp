@@ -420,6 +420,77 @@ void parse_op(Cursor &c, Builder &b, const std::string &res, const std::string &
     (void)from;
     return;
   }
+  if (name.rfind("onednn_graph.", 0) == 0) {
+    // the reference's front-end dialect (test/mlir/test/gc/Dialect/OneDNNGraph/*.mlir): the ops of the JSON schema
+    // in MLIR's generic form   %r = onednn_graph.op %a, %b {attrs} : (types) -> type
+    need_res();
+    static const std::map<std::string, std::string> kinds = {
+        {"add", "Add"},         {"mul", "Multiply"},    {"sub", "Subtract"},        {"div", "Divide"},
+        {"matmul", "MatMul"},   {"relu", "ReLU"},       {"sigmoid", "Sigmoid"},     {"pow", "Pow"},
+        {"type_cast", "TypeCast"}, {"reduce_sum", "ReduceSum"}, {"reduce_mean", "ReduceMean"}};
+    const std::string op = name.substr(13);
+    if (!kinds.count(op))
+      unimpl("operation " + name);
+    std::vector<size_t> in;
+    do
+      in.push_back(b.operand(c.ssa()));
+    while (c.accept(","));
+    std::string attrs;
+    if (c.peek("{"))
+      attrs = c.group_text('{', '}');
+    c.expect(":");
+    c.expect("(");
+    size_t n_types = 0;
+    if (!c.accept(")")) {
+      do {
+        c.type();
+        n_types++;
+      } while (c.accept(","));
+      c.expect(")");
+    }
+    c.expect("->");
+    Type rt = c.type();
+    if (n_types != in.size())
+      bad(name + ": operand and type counts differ");
+    Op &o = b.add_op(kinds.at(op), in, 0);
+    auto flag = [&](const char *key) {
+      size_t k = attrs.find(key);
+      if (k == std::string::npos)
+        return false;
+      size_t e = attrs.find('=', k);
+      return e != std::string::npos && attrs.compare(attrs.find_first_not_of(" \t\n", e + 1), 4, "true") == 0;
+    };
+    if (op == "matmul") {
+      if (flag("transpose_a"))
+        o.attrs["transpose_a"] = attr_bool(true);
+      if (flag("transpose_b"))
+        o.attrs["transpose_b"] = attr_bool(true);
+    } else if (op == "pow") {
+      size_t k = attrs.find("beta");
+      if (k == std::string::npos)
+        bad("onednn_graph.pow without beta");
+      Cursor a(attrs.c_str() + attrs.find('=', k) + 1);
+      o.attrs["beta"] = attr_f32((float)a.number());
+    } else if (op == "reduce_sum" || op == "reduce_mean") {
+      std::vector<int64_t> axes;
+      size_t k = attrs.find("axes");
+      if (k != std::string::npos) {
+        size_t colon = attrs.find(':', attrs.find("array<", k));
+        if (colon == std::string::npos)
+          bad(name + ": axes must be array<i64: ...>");
+        Cursor a(attrs.c_str() + colon + 1);
+        do
+          axes.push_back((int64_t)a.number());
+        while (a.accept(","));
+      }
+      o.attrs["axes"] = attr_ints(axes);
+      o.attrs["keep_dims"] = attr_bool(flag("keep_dims"));
+    }
+    size_t id = b.new_tensor(rt);
+    b.def(res, id, rt);
+    b.g.ops.back().out = {id};
+    return;
+  }
   if (name.rfind("linalg.", 0) != 0)
     unimpl("operation " + name);
   need_res();

@@ -9,7 +9,10 @@
 //   linalg.add / sub / mul / div / max / min / powf,
 //   linalg.negf / exp / copy / abs / ceil / floor / erf / log / round / rsqrt / sqrt / square / tanh / reciprocal,
 //   linalg.broadcast, linalg.transpose, linalg.softmax, linalg.reduce (sum),
-//   tensor.collapse_shape / tensor.expand_shape, return.
+//   tensor.collapse_shape / tensor.expand_shape, return,
+//   and the reference's front-end dialect onednn_graph.{matmul, add, mul, sub, div, relu, sigmoid, pow, type_cast,
+//   reduce_sum, reduce_mean} (test/mlir/test/gc/Dialect/OneDNNGraph/*.mlir).
+// The first function of the text is compiled; anything after it is not looked at.
 // The module becomes the same graph IR the JSON front end produces (graph.h), so
 // verification, fusion and execution are shared.  Tensor ids: function argument
 // i has id i; result j of the function has id (number of arguments) + j.

@@ -119,7 +119,11 @@ dnnl_status_t dnnl_graph_compiler_explain(const char *graph_json, char *buf, siz
  * tensor.{collapse,expand}_shape -- the subset of the reference's benchgc
  * cases (test/benchgc/cases/{llama2,generic}.mlir), its MLP pattern
  * (test/benchgc/src/benchgc/pattern/mlp.py) and the element-wise, binary and
- * matmul cases of its linalg driver (test/benchgc/src/benchgc/linalg/).  Takes over what gc-cpu-runner /
+ * matmul cases of its linalg driver (test/benchgc/src/benchgc/linalg/); and
+ * the ops of the reference's front-end dialect, onednn_graph.{matmul, add, mul,
+ * sub, div, relu, sigmoid, pow, type_cast, reduce_sum, reduce_mean}
+ * (test/mlir/test/gc/Dialect/OneDNNGraph/).  The first function of the text is
+ * compiled.  Takes over what gc-cpu-runner /
  * benchgc `--driver mlir` do with such a module on the CPU
  * (src/gc-cpu-runner/gc-cpu-runner.cpp, test/benchgc/src/benchgc/runner.py).
  * Tensor ids for execute: function argument i has id i, result j has id

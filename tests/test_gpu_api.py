@@ -269,3 +269,13 @@ def test_chain_of_four_matmuls_with_shared_temporaries(ga, orc, wl, dev):
     for W in Ws:
         cur = orc.matmul_bf16(cur, wl.bf16_bits(W))
     assert_close(orc.bf16_to_f32(cur), out.float().numpy(), 4e-2, "four chained matmuls (four rounding points)")
+
+
+def test_reduce_without_axes_returns_its_operand(ga, dev):
+    """lib/gc/Dialect/OneDNNGraph/OneDNNGraphOps.cpp:116-120: no reduce axes, no reduction."""
+    x = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    out = np.zeros_like(x)
+    g = ga._graph([{"kind": "ReduceSum", "inputs": [ga._t(0, "f32", [2, 3, 4])], "outputs": [ga._t(1, "f32", [2, 3, 4])]}],
+                  [0], [1])
+    _run(ga, g, [(0, x)], [(1, out)])
+    assert (out == x).all()

@@ -353,3 +353,24 @@ def test_linear_layer_spelled_with_a_transpose(ga, dev):
     y = torch.zeros(64, 512, device=dev, dtype=torch.bfloat16)
     _run(ga, text, [(0, x), (1, w)], [(2, y)])
     assert_close((x.double() @ w.double().t()).cpu().numpy(), y.double().cpu().numpy(), 1e-2, "linear with transpose")
+
+
+def test_onednn_graph_dialect_module(ga, dev):
+    """The reference's front-end dialect: matmul (+bias, transposed weight) -> sigmoid -> f32 -> square -> row mean."""
+    text = """func.func @f(%x: tensor<64x128xbf16>, %w: tensor<256x128xbf16>, %b: tensor<256xbf16>) -> tensor<64x1xf32> {
+      %0 = onednn_graph.matmul %x, %w, %b {transpose_b = true}
+           : (tensor<64x128xbf16>, tensor<256x128xbf16>, tensor<256xbf16>) -> tensor<64x256xbf16>
+      %1 = onednn_graph.sigmoid %0 : (tensor<64x256xbf16>) -> tensor<64x256xbf16>
+      %2 = onednn_graph.type_cast %1 : (tensor<64x256xbf16>) -> tensor<64x256xf32>
+      %3 = onednn_graph.pow %2 {beta = 2.0 : f32} : (tensor<64x256xf32>) -> tensor<64x256xf32>
+      %4 = onednn_graph.reduce_mean %3 {axes = array<i64: -1>, keep_dims = true} : (tensor<64x256xf32>) -> tensor<64x1xf32>
+      return %4 : tensor<64x1xf32>
+    }"""
+    torch.manual_seed(23)
+    x = torch.randn(64, 128, device=dev).bfloat16()
+    w = (torch.randn(256, 128, device=dev) * 0.1).bfloat16()
+    b = torch.randn(256, device=dev).bfloat16()
+    out = torch.zeros(64, 1, device=dev)
+    _run(ga, text, [(0, x), (1, w), (2, b)], [(3, out)])
+    h = torch.sigmoid(((x.float() @ w.float().t()).bfloat16() + b).float()).bfloat16().float()
+    assert_close((h * h).mean(1, keepdim=True).cpu().numpy(), out.cpu().numpy(), 1e-2, "dialect module")

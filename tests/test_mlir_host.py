@@ -218,3 +218,43 @@ def test_transpose_in_front_of_a_matmul_becomes_its_flag(ga):
     other = text.replace("permutation = [1, 0]", "permutation = [0, 1]").replace("tensor<256x512xbf16>", "tensor<512x256xbf16>")
     st, plan = ga.explain_mlir(other)
     assert st != OK or "Transpose" in plan
+
+
+REF_DIALECT = "/root/reference/test/mlir/test/gc/Dialect/OneDNNGraph"
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_DIALECT), reason="the reference tree is not on this machine")
+def test_reference_onednn_graph_dialect_files(ga):
+    """Every function of the reference's own front-end dialect tests parses and plans (one function per text)."""
+    import re
+    n = 0
+    for name in ("onednn-graph-llama2.mlir", "onednn-graph-mlp.mlir", "onednn-graph-ops.mlir", "onednn-graph-to-linalg.mlir"):
+        text = open(os.path.join(REF_DIALECT, name)).read()
+        text = "\n".join(ln for ln in text.splitlines() if not ln.lstrip().startswith("//"))
+        for fn in re.split(r"(?=func\.func)", text):
+            if not fn.startswith("func.func") or "onednn_graph." not in fn:
+                continue  # the @main drivers of the runnable tests call the function above them
+            st, plan = ga.explain_mlir(fn)
+            assert st == OK, (name, fn[:80], plan)
+            n += 1
+    assert n >= 20
+    st, plan = ga.explain_mlir(open(os.path.join(REF_DIALECT, "onednn-graph-mlp.mlir")).read())
+    assert _steps(plan) == ["gemm_bf16: MatMul+bias+act", "gemm_bf16: MatMul+bias+act"]
+
+
+def test_onednn_graph_dialect_ops(ga):
+    t = "tensor<64x128xbf16>"
+    text = """func.func @f(%x: tensor<64x128xbf16>, %w: tensor<256x128xbf16>, %b: tensor<256xbf16>) -> tensor<64x1xf32> {
+      %0 = onednn_graph.matmul %x, %w, %b {transpose_b = true}
+           : (tensor<64x128xbf16>, tensor<256x128xbf16>, tensor<256xbf16>) -> tensor<64x256xbf16>
+      %1 = onednn_graph.sigmoid %0 : (tensor<64x256xbf16>) -> tensor<64x256xbf16>
+      %2 = onednn_graph.type_cast %1 : (tensor<64x256xbf16>) -> tensor<64x256xf32>
+      %3 = onednn_graph.pow %2 {beta = 2.0 : f32} : (tensor<64x256xf32>) -> tensor<64x256xf32>
+      %4 = onednn_graph.reduce_mean %3 {axes = array<i64: -1>, keep_dims = true} : (tensor<64x256xf32>) -> tensor<64x1xf32>
+      return %4 : tensor<64x1xf32>
+    }"""
+    st, plan = ga.explain_mlir(text)
+    assert st == OK, plan
+    assert _steps(plan) == ["gemm_bf16: MatMul+bias+act", "reduce: ReduceMean of TypeCast+Pow"]
+    assert ga.explain_mlir(text.replace("onednn_graph.sigmoid", "onednn_graph.softplus"))[0] == UNIMPL
+    assert ga.explain_mlir(text.replace("{beta = 2.0 : f32} ", ""))[0] == INVALID_GRAPH
