@@ -197,24 +197,7 @@ static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream) {
     hipLaunchKernelGGL(gemm_skinny_nt_kernel<2>, grid, block, 0, stream, p);
   if (best == 1) // the epilogue ran in the kernel
     return hipGetLastError() == hipSuccess ? 0 : 5;
-  const unsigned rblocks = (unsigned)((p.M * (p.N / 4) + 255) / 256);
-  switch (p.act) {
-  case ACT_RELU:
-    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_RELU>, dim3(rblocks), dim3(256), 0, stream, p);
-    break;
-  case ACT_GELU_ERF:
-    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_GELU_ERF>, dim3(rblocks), dim3(256), 0, stream, p);
-    break;
-  case ACT_GELU_TANH:
-    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_GELU_TANH>, dim3(rblocks), dim3(256), 0, stream, p);
-    break;
-  case ACT_SIGMOID:
-    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_SIGMOID>, dim3(rblocks), dim3(256), 0, stream, p);
-    break;
-  default:
-    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_NONE>, dim3(rblocks), dim3(256), 0, stream, p);
-    break;
-  }
+  launch_splitk_reduce(p, stream);
   return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 

@@ -794,6 +794,28 @@ template <int ACT> __global__ __launch_bounds__(256) void gemm_splitk_reduce_ker
 static constexpr int64_t G_SPLITK_WS_FLOATS = (int64_t)8 << 20; // 32 MiB
 static __device__ __align__(256) float gemm_splitk_ws[G_SPLITK_WS_FLOATS];
 
+// second pass of every K-sliced GEMM: one thread per four outputs, the activation as a template argument
+static void launch_splitk_reduce(const GemmParams &p, hipStream_t stream) {
+  const dim3 grid((unsigned)((p.M * (p.N / 4) + 255) / 256)), block(256);
+  switch (p.act) {
+  case ACT_RELU:
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_RELU>, grid, block, 0, stream, p);
+    break;
+  case ACT_GELU_ERF:
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_GELU_ERF>, grid, block, 0, stream, p);
+    break;
+  case ACT_GELU_TANH:
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_GELU_TANH>, grid, block, 0, stream, p);
+    break;
+  case ACT_SIGMOID:
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_SIGMOID>, grid, block, 0, stream, p);
+    break;
+  default:
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_NONE>, grid, block, 0, stream, p);
+    break;
+  }
+}
+
 // Host-side launch of the 256x256 tile kernels for one element size.
 template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t stream) {
   GemmParams p = *pp;
@@ -845,24 +867,7 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
           hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true>), dim3((unsigned)(tiles_n * splits)),
                              dim3(1024 / G_FAST_WJ), 0, stream, p);
       }
-      const unsigned rblocks = (unsigned)((p.M * (p.N / 4) + 255) / 256);
-      switch (p.act) {
-      case ACT_RELU:
-        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_RELU>, dim3(rblocks), dim3(256), 0, stream, p);
-        break;
-      case ACT_GELU_ERF:
-        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_GELU_ERF>, dim3(rblocks), dim3(256), 0, stream, p);
-        break;
-      case ACT_GELU_TANH:
-        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_GELU_TANH>, dim3(rblocks), dim3(256), 0, stream, p);
-        break;
-      case ACT_SIGMOID:
-        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_SIGMOID>, dim3(rblocks), dim3(256), 0, stream, p);
-        break;
-      default:
-        hipLaunchKernelGGL(gemm_splitk_reduce_kernel<ACT_NONE>, dim3(rblocks), dim3(256), 0, stream, p);
-        break;
-      }
+      launch_splitk_reduce(p, stream);
       return hipGetLastError() == hipSuccess ? 0 : 5;
     }
   }
