@@ -35,6 +35,31 @@ void gc_check(int rc, const char *what) {
     throw std::runtime_error(std::string(what) + ": " + gcmi_last_error());
 }
 
+// IEEE binary16 bits of x, round to nearest even (the host compiler has no half type)
+static uint16_t f32_to_f16_bits(float x) {
+  uint32_t u;
+  memcpy(&u, &x, 4);
+  const uint32_t sign = (u >> 16) & 0x8000u;
+  u &= 0x7fffffffu;
+  if (u >= 0x7f800000u) // inf / nan
+    return (uint16_t)(sign | 0x7c00u | (u > 0x7f800000u ? 0x200u : 0));
+  if (u >= 0x477ff000u) // rounds to 65520 or more: inf
+    return (uint16_t)(sign | 0x7c00u);
+  if (u < 0x38800000u) { // below the smallest normal half: fixed point with 24 fraction bits
+    if (u < 0x33000000u)
+      return (uint16_t)sign; // under half of the smallest subnormal
+    const int shift = 126 - (int)(u >> 23); // 14 .. 24
+    const uint32_t mant = (u & 0x7fffffu) | 0x800000u;
+    const uint32_t q = mant >> shift, rem = mant & ((1u << shift) - 1), half = 1u << (shift - 1);
+    return (uint16_t)(sign | (q + (rem > half || (rem == half && (q & 1)))));
+  }
+  const uint32_t e = (u >> 23) - 112, m = u & 0x7fffffu;
+  uint32_t h = (e << 10) | (m >> 13);
+  const uint32_t rem = m & 0x1fffu;
+  h += rem > 0x1000u || (rem == 0x1000u && (h & 1));
+  return (uint16_t)(sign | h);
+}
+
 std::vector<int64_t> dense_strides(const std::vector<int64_t> &shape) {
   std::vector<int64_t> s(shape.size(), 1);
   for (int i = (int)shape.size() - 2; i >= 0; i--)
@@ -118,6 +143,8 @@ int Executable::slot_for(size_t tid) {
       uint32_t u;
       memcpy(&u, &f, 4);
       bits = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+    } else if (t.dt == DT::f16) {
+      bits = f32_to_f16_bits(f);
     } else
       throw std::logic_error(std::string("Constant of this dtype is not supported: ") + dt_name(t.dt));
     int s = const_slot(&bits, (size_t)es);

@@ -374,3 +374,44 @@ def test_onednn_graph_dialect_module(ga, dev):
     _run(ga, text, [(0, x), (1, w), (2, b)], [(3, out)])
     h = torch.sigmoid(((x.float() @ w.float().t()).bfloat16() + b).float()).bfloat16().float()
     assert_close((h * h).mean(1, keepdim=True).cpu().numpy(), out.cpu().numpy(), 1e-2, "dialect module")
+
+
+@pytest.mark.parametrize("shape,axis", [((5, 7, 3), 2), ((5, 7, 3), 0), ((9, 130), 1), ((3, 1030), 1), ((257, 6), 1),
+                                        ((2, 3, 5, 7), 1)])
+def test_fused_kernels_on_odd_shapes_f16(ga, dev, shape, axis):
+    """Shapes whose innermost dim is not a multiple of four (one element at a time instead of quads), row counts that
+    leave part of the last workgroup idle, one to many elements per thread, f16 storage: a point-wise chain, a sum
+    over `axis` with a producer and an op on the row result, and the normalisation that uses it."""
+    def t(s, dt="f16"):
+        return "tensor<%s%s>" % ("".join("%dx" % d for d in s), dt)
+    kept = [d for i, d in enumerate(shape) if i != axis]
+    full, row = t(shape), t(kept)
+    rowdims = ", ".join(str(i) for i in range(len(shape)) if i == axis)
+    text = f"""func.func @f(%x: {full}, %y: {full}) -> ({full}, {row}, {full}) {{
+      %e = tensor.empty() : {full}
+      %er = tensor.empty() : {row}
+      %two = arith.constant dense<2.000000e+00> : {full}
+      %a = linalg.mul ins(%x, %two : {full}, {full}) outs(%e : {full}) -> {full}
+      %b = linalg.add ins(%a, %y : {full}, {full}) outs(%e : {full}) -> {full}
+      %zero = arith.constant dense<0.000000e+00> : {full}
+      %c = linalg.max ins(%b, %zero : {full}, {full}) outs(%e : {full}) -> {full}
+      %c0 = arith.constant 0.0 : f16
+      %z = linalg.fill ins(%c0 : f16) outs(%er : {row}) -> {row}
+      %s = linalg.reduce {{ arith.addf }} ins(%c : {full}) outs(%z : {row}) dimensions = [{rowdims}]
+      %one = arith.constant dense<1.000000e+00> : {row}
+      %s1 = linalg.add ins(%s, %one : {row}, {row}) outs(%er : {row}) -> {row}
+      %sb = linalg.broadcast ins(%s1 : {row}) outs(%e : {full}) dimensions = [{rowdims}]
+      %n = linalg.div ins(%c, %sb : {full}, {full}) outs(%e : {full}) -> {full}
+      return %c, %s1, %n : {full}, {row}, {full}
+    }}"""
+    torch.manual_seed(3)
+    x = (torch.rand(shape, device=dev) - 0.3).half()
+    y = (torch.rand(shape, device=dev) - 0.5).half()
+    c, s1, nrm = torch.zeros(shape, device=dev).half(), torch.zeros(kept, device=dev).half(), torch.zeros(shape, device=dev).half()
+    _run(ga, text, [(0, x), (1, y)], [(2, c), (3, s1), (4, nrm)])
+    rc = torch.relu(((x.float() * 2).half().float() + y.float()).half().float()).half()
+    assert torch.equal(c, rc)
+    rs = (rc.float().sum(axis).half().float() + 1).half()
+    assert_close(rs.float().cpu().numpy(), s1.float().cpu().numpy(), 2e-3, "row sums f16")  # f16: 2^-11 per rounding
+    rn = (rc.float() / s1.float().unsqueeze(axis)).half()
+    assert_close(rn.float().cpu().numpy(), nrm.float().cpu().numpy(), 2e-3, "normalised f16")
