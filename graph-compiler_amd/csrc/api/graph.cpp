@@ -79,7 +79,9 @@ static const std::set<std::string> &reference_ops() {
 static const std::set<std::string> &extension_ops() {
   // spelled as in the oneDNN Graph specification; semantics from the reference's
   // legacy core (GELU, Dequantize, Quantize, SoftMax) -- see the README
-  static const std::set<std::string> s = {"GELU", "Dequantize", "Quantize", "SoftMax", "TypeCast"};
+  // and the element-wise ops of that specification the point-wise kernels have anyway
+  static const std::set<std::string> s = {"GELU", "Dequantize", "Quantize", "SoftMax",    "TypeCast", "Abs",    "Exp", "Log",
+                                          "Maximum", "Minimum", "Reciprocal", "Sqrt", "Square", "Tanh"};
   return s;
 }
 bool is_known_op(const std::string &k) { return reference_ops().count(k) || extension_ops().count(k); }

@@ -279,3 +279,28 @@ def test_reduce_without_axes_returns_its_operand(ga, dev):
                   [0], [1])
     _run(ga, g, [(0, x)], [(1, out)])
     assert (out == x).all()
+
+
+def test_json_elementwise_extension_ops(ga, dev):
+    """Element-wise ops of the oneDNN Graph specification beyond the reference's eleven, as JSON: a chain that the
+    planner runs as one fused launch."""
+    shape = [6, 50]
+    ops, src = [], 0
+    chain = ["Abs", "Sqrt", "Tanh", "Exp", "Log", "Square", "Reciprocal"]
+    for i, kind in enumerate(chain):
+        ops.append({"kind": kind, "inputs": [ga._t(src, "f32", shape)], "outputs": [ga._t(10 + i, "f32", shape)]})
+        src = 10 + i
+    ops.append({"kind": "Maximum", "inputs": [ga._t(src, "f32", shape), ga._t(1, "f32", shape)], "outputs": [ga._t(30, "f32", shape)]})
+    ops.append({"kind": "Minimum", "inputs": [ga._t(30, "f32", shape), ga._t(2, "f32", [50])], "outputs": [ga._t(31, "f32", shape)]})
+    g = ga._graph(ops, [0, 1, 2], [31])
+    st, plan = ga.explain(g)
+    assert st == 0 and plan.startswith("fused: Abs+Sqrt+Tanh+Exp+Log+Square+Reciprocal+Maximum+Minimum"), plan
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(shape) * 2).astype(np.float32)
+    y = rng.standard_normal(shape).astype(np.float32) + 1
+    z = rng.standard_normal(50).astype(np.float32) + 1.5
+    out = np.zeros(shape, np.float32)
+    _run(ga, g, [(0, x), (1, y), (2, z)], [(31, out)])
+    t = np.tanh(np.sqrt(np.abs(x.astype(np.float64))))
+    ref = np.minimum(np.maximum(1.0 / np.square(np.log(np.exp(t))), y), z)
+    assert_close(ref, out, 1e-4, "element-wise extension ops")
