@@ -20,7 +20,7 @@ ACT = {None: 0, "none": 0, "relu": 1, "gelu_erf": 2, "gelu_tanh": 3, "sigmoid": 
 
 # every symbol the public headers declare (checked by the CPU test-suite)
 EXPORTS = {
-    "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_bf16_nt", "gcmi_gemm_bf16_batched", "gcmi_gemm_f32_batched",
+    "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_bf16_nt", "gcmi_gemm_bf16_batched", "gcmi_gemm_bf16_residual", "gcmi_gemm_f32_batched",
                          "gcmi_gemm_int8", "gcmi_colsum_s8",
                          "gcmi_gemm_f32", "gcmi_mha_fwd_bf16", "gcmi_mha_fwd_bf16_opt"],
     "gc_brgemm.h": ["dnnl_brgemm_dispatch", "dnnl_brgemm_tileconfig", "dnnl_brgemm_tilerelease",
@@ -53,6 +53,8 @@ def lib():
     L.gcmi_gemm_bf16_nt.restype = ci
     L.gcmi_gemm_bf16_batched.restype = ci
     L.gcmi_gemm_bf16_batched.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, vp, ci, ci, ci, vp]
+    L.gcmi_gemm_bf16_residual.restype = ci
+    L.gcmi_gemm_bf16_residual.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, vp, ci, ci, vp, i64, ci, ci, vp]
     L.gcmi_gemm_f32_batched.restype = ci
     L.gcmi_gemm_f32_batched.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, ci, vp, ci, vp]
     L.gcmi_gemm_bf16_nt.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, ci, ci, ci, vp]
@@ -127,6 +129,27 @@ def gemm_bf16_nt(A, Bt, bias=None, act=None, out_dtype=BF16, out=None):
     check(lib().gcmi_gemm_bf16_nt(_ptr(A), _ptr(Bt), _ptr(out), M, N, K, A.stride(0) if M > 1 else K,
                                   Bt.stride(0) if N > 1 else K, out.stride(0) if M > 1 else N, _ptr(bias), bdt,
                                   ACT[act], out_dtype, _stream()), "gcmi_gemm_bf16_nt")
+    return out
+
+
+def gemm_bf16_residual(A, B, residual, trans_b=False, bias=None, act=None, out_dtype=BF16, out=None):
+    """act(A @ B + bias) + residual in one launch; B is [K,N], or [N,K] with trans_b.  residual: [M,N] bf16 or f32."""
+    import torch
+    M, K = A.shape
+    N = B.shape[0] if trans_b else B.shape[1]
+    assert B.shape[1 if trans_b else 0] == K and (A.stride(1) == 1 or K == 1) and (B.stride(1) == 1 or B.shape[1] == 1)
+    assert tuple(residual.shape) == (M, N) and (residual.stride(1) == 1 or N == 1)
+    if out is None:
+        out = torch.empty((M, N), device=A.device, dtype=torch.bfloat16 if out_dtype == BF16 else torch.float32)
+    bdt = BF16
+    if bias is not None:
+        bdt = BF16 if bias.dtype == torch.bfloat16 else F32
+    rdt = BF16 if residual.dtype == torch.bfloat16 else F32
+    check(lib().gcmi_gemm_bf16_residual(_ptr(A), _ptr(B), _ptr(out), 1, M, N, K, A.stride(0) if M > 1 else K,
+                                        B.stride(0) if B.shape[0] > 1 else B.shape[1], out.stride(0) if M > 1 else N,
+                                        0, 0, 0, int(trans_b), _ptr(bias), bdt, ACT[act],
+                                        _ptr(residual), residual.stride(0) if M > 1 else N, rdt, out_dtype, _stream()),
+          "gcmi_gemm_bf16_residual")
     return out
 
 

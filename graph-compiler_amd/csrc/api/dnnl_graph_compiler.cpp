@@ -209,6 +209,45 @@ extern "C" dnnl_status_t dnnl_graph_compiler_explain_mlir(const char *module_tex
   }
 }
 
+extern "C" dnnl_status_t dnnl_graph_compiler_generated_source_mlir(const char *module_text, const char *check_arch, char *buf,
+                                                                   size_t len) {
+  try {
+    gcapi::Executable e(gcapi::parse_mlir(module_text), true);
+    const std::vector<gcjit::FusedKernelSource> ks = e.generated_kernels();
+    std::string d;
+    for (const auto &k : ks)
+      d += k.source + "\n";
+    if (buf && len) {
+      size_t n = d.size() < len - 1 ? d.size() : len - 1;
+      memcpy(buf, d.data(), n);
+      buf[n] = 0;
+    }
+    if (check_arch && !ks.empty()) {
+      const std::string log = gcjit::compile_only(ks, check_arch);
+      if (!log.empty()) {
+        remember(log.c_str());
+        return dnnl_runtime_error;
+      }
+    }
+    return dnnl_success;
+  } catch (const std::invalid_argument &e) {
+    remember(e.what());
+    return dnnl_invalid_graph;
+  } catch (const std::logic_error &e) {
+    remember(e.what());
+    return dnnl_unimplemented;
+  } catch (const std::bad_alloc &) {
+    return dnnl_out_of_memory;
+  } catch (const std::exception &e) {
+    remember(e.what());
+    return dnnl_runtime_error;
+  } catch (...) {
+    return dnnl_runtime_error;
+  }
+}
+
+extern "C" long dnnl_graph_compiler_generated_kernel_launches(void) { return gcapi::Executable::generated_launches(); }
+
 // gc-c shims
 extern "C" MlirDialectHandle mlirGetDialectHandle__onednn_graph__(void) { return MlirDialectHandle{nullptr}; }
 extern "C" MlirDialectHandle mlirGetDialectHandle__cpuruntime__(void) { return MlirDialectHandle{nullptr}; }

@@ -1,6 +1,7 @@
 #include "executable.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -192,6 +193,7 @@ void Executable::init(bool dry) {
     if (!s.init.empty())
       hip_check(hipMemcpy(arena_ + s.offset, s.init.data(), s.init.size(), hipMemcpyHostToDevice), "upload constants");
   ptr_.resize(slots_.size());
+  build_generated_kernels();
 }
 
 // One allocation per executable, temporaries with disjoint lifetimes share memory: the tick-based merge
@@ -476,22 +478,32 @@ void Executable::plan() {
     if (bias_t >= 0 && !(flat && is_row_vector(T((size_t)bias_t), Nn)))
       bias_t = -1; // handled as a separate Add below
     int act = 0;
+    long res_t = -1; // a tensor of the result's shape that is added last (a residual connection): bf16 GEMMs
     size_t cur = mm.out[0], last = i;
     std::vector<size_t> chain;
     DT gemm_dt = int8 ? DT::f32 : A.dt;
     if (flat && (gemm_dt == DT::f32 || gemm_dt == DT::bf16) && (bias_in_matmul ? bias_t >= 0 : true)) {
-      while (single_use(cur)) {
+      while (single_use(cur) && res_t < 0) {
         size_t ci = consumers[cur][0];
         const Op &c = g_.ops[ci];
         if (claimed[ci])
           break;
-        if (c.kind == "Add" && bias_t < 0 && act == 0) {
+        if (c.kind == "Add") {
           size_t other = c.in[0] == cur ? c.in[1] : c.in[0];
           const LTensor &bt = T(other);
           bool dt_ok = bt.dt == T(cur).dt;
-          if (!is_row_vector(bt, Nn) || !dt_ok || T(c.out[0]).shape != T(cur).shape)
+          if (!dt_ok || T(c.out[0]).shape != T(cur).shape)
             break;
-          bias_t = (long)other;
+          if (bias_t < 0 && act == 0 && is_row_vector(bt, Nn))
+            bias_t = (long)other;
+          else if (!int8 && gemm_dt == DT::bf16 && bt.shape == T(cur).shape && !bt.has_splat)
+            res_t = (long)other;
+          else
+            break;
+        } else if (c.kind == "Reshape" && T(c.out[0]).alias_of >= 0 && !T(c.out[0]).shape.empty() &&
+                   T(c.out[0]).shape.back() == Nn) {
+          // a view of the result that keeps its rows (tensor.expand_shape to [1, M, N] and the like): the ops
+          // behind it fuse as they would without it
         } else if (act_of(c) > 0 && act == 0) {
           act = act_of(c);
         } else if (int8 && (c.kind == "Typecast" || c.kind == "TypeCast") && T(c.out[0]).dt == DT::bf16) {
@@ -514,6 +526,8 @@ void Executable::plan() {
       fused += "+bias";
     if (act)
       fused += "+act";
+    if (res_t >= 0)
+      fused += "+residual";
     if (int8 && flat) {
       const Op &da = g_.ops[dq_a], &dw = g_.ops[dq_w];
       const LTensor &qa = T(da.in[0]), &qw = T(dw.in[0]);
@@ -626,6 +640,8 @@ void Executable::plan() {
         }
         s.bias = bias_t >= 0 ? slot_for((size_t)bias_t) : -1;
         s.bias_dt = bias_t >= 0 ? dt_dnnl(T((size_t)bias_t).dt) : 0;
+        s.c = res_t >= 0 ? slot_for((size_t)res_t) : -1;
+        s.b_dt = res_t >= 0 ? dt_dnnl(T((size_t)res_t).dt) : 0;
         s.act = act;
         s.out_dt = dt_dnnl(chain.empty() ? out_dt : T(cur).dt);
         v.push_back(s);
@@ -1319,6 +1335,59 @@ static int fused_registers(const Step &s) {
   return gcmi::fused_allocate(p);
 }
 
+// Kernels specialised for the fused groups of this plan (jit/fused_jit.h).  GCMI_NO_GENERATED_KERNELS=1 keeps the
+// library's interpreter kernels, which compute the same bits (tests compare the two).  A group the generator does not
+// cover, or a compiler that is missing or fails, also leaves the interpreter in place.
+std::vector<gcjit::FusedKernelSource> Executable::generated_kernels() const {
+  std::vector<gcjit::FusedKernelSource> ks;
+  for (size_t i = 0; i < steps_.size(); i++) {
+    const Step &s = steps_[i];
+    if (s.kind != Step::Fused)
+      continue;
+    gcmi::FusedParams p{};
+    fill_fused_params(s, p);
+    int same_as[gcmi::FUSED_MAX_IN];
+    for (int k = 0; k < p.n_in; k++) {
+      same_as[k] = -1;
+      for (int j = 0; j < k && same_as[k] < 0; j++)
+        if (s.f_in[(size_t)j] == s.f_in[(size_t)k] && s.f_str[(size_t)j] == s.f_str[(size_t)k] && p.in_dt[j] == p.in_dt[k])
+          same_as[k] = j;
+    }
+    gcjit::FusedKernelSource k;
+    if (gcjit::generate_fused(p, same_as, "gcmi_fused_step" + std::to_string(i), k)) {
+      k.source = "// " + s.note + "\n" + k.source;
+      ks.push_back(std::move(k));
+    }
+  }
+  return ks;
+}
+
+static std::atomic<long> g_generated_launches{0};
+long Executable::generated_launches() { return g_generated_launches.load(); }
+
+void Executable::build_generated_kernels() {
+  const char *off = getenv("GCMI_NO_GENERATED_KERNELS");
+  if (off && off[0] == '1')
+    return;
+  const std::vector<gcjit::FusedKernelSource> ks = generated_kernels();
+  if (ks.empty())
+    return;
+  std::string error;
+  jit_module_ = gcjit::Module::build(ks, error);
+  if (!jit_module_) {
+    const char *strict = getenv("GCMI_GENERATED_KERNELS_REQUIRED");
+    if (strict && strict[0] == '1')
+      throw std::runtime_error("generated kernels: " + error);
+    return;
+  }
+  for (const gcjit::FusedKernelSource &k : ks) {
+    const size_t i = (size_t)std::stoul(k.name.substr(strlen("gcmi_fused_step")));
+    Step &s = steps_[i];
+    s.jit_fn = jit_module_->function(k.name);
+    s.jit_grid = k.grid, s.jit_block = k.block, s.jit_vectors = k.quad;
+  }
+}
+
 // ---------------------------------------------------------------------------
 void Executable::launch(const Step &s) {
   auto P = [&](int slot) -> char * { return slot < 0 ? nullptr : (char *)ptr_[(size_t)slot]; };
@@ -1330,10 +1399,12 @@ void Executable::launch(const Step &s) {
              "MatMul f32");
     break;
   case Step::GemmBf16:
-    gc_check(gcmi_gemm_bf16_batched(P(s.a) + s.a_off * 2, P(s.b) + s.b_off * 2,
-                                    P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4), s.batch, s.M, s.N, s.K, s.lda,
-                                    s.ldb, s.ldc, s.a_bs, s.b_bs, s.c_bs, s.tb ? 1 : 0, P(s.bias),
-                                    s.bias_dt ? s.bias_dt : GCMI_BF16, s.act, s.out_dt, stream_),
+    // s.c: the residual tensor (same shape as the result), s.b_dt its type
+    gc_check(gcmi_gemm_bf16_residual(P(s.a) + s.a_off * 2, P(s.b) + s.b_off * 2,
+                                     P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4), s.batch, s.M, s.N, s.K, s.lda,
+                                     s.ldb, s.ldc, s.a_bs, s.b_bs, s.c_bs, s.tb ? 1 : 0, P(s.bias),
+                                     s.bias_dt ? s.bias_dt : GCMI_BF16, s.act, P(s.c), s.N, s.b_dt ? s.b_dt : GCMI_BF16,
+                                     s.out_dt, stream_),
              "MatMul bf16");
     break;
   case Step::ColSum:
@@ -1417,6 +1488,20 @@ void Executable::launch(const Step &s) {
     }
     if ((size_t)(second_pass ? p.n : p.n / p.n_red) * (size_t)esz(p.out_dt) > slots_[(size_t)s.out].bytes)
       throw std::runtime_error("fused group: the result does not fit its buffer (" + s.note + ")");
+    if (s.jit_fn) {
+      bool aligned = (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
+      for (int k = 0; k < p.n_in; k++)
+        aligned = aligned && (reinterpret_cast<uintptr_t>(p.in[k]) & 15) == 0;
+      if (aligned || !s.jit_vectors) {
+        void *args[gcmi::FUSED_MAX_IN + 1];
+        for (int k = 0; k < p.n_in; k++)
+          args[k] = (void *)&p.in[k];
+        args[p.n_in] = (void *)&p.out;
+        hip_check(hipModuleLaunchKernel(s.jit_fn, s.jit_grid, 1, 1, s.jit_block, 1, 1, 0, stream_, args, nullptr), s.note.c_str());
+        g_generated_launches++;
+        break;
+      }
+    }
     gc_check(gcmi_launch_fused(&p, stream_) ? 5 : 0, s.note.c_str());
     break;
   }

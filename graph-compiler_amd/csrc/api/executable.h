@@ -23,6 +23,7 @@
 
 #include "dnnl_graph_compiler.h"
 #include "graph.h"
+#include "jit/fused_jit.h"
 
 namespace gcapi {
 
@@ -73,6 +74,10 @@ struct Step {
   std::vector<size_t> f_members, f_in_tensor;
   size_t f_out_tensor = 0;
   std::vector<int> f_place;
+  // the kernel generated for this group when the partition was compiled (null: the library's interpreter runs it)
+  hipFunction_t jit_fn = nullptr;
+  unsigned jit_grid = 0, jit_block = 0;
+  bool jit_vectors = false; // it moves 16-byte vectors: the operands must be aligned
 };
 
 struct Slot {
@@ -98,6 +103,10 @@ public:
   const Graph &graph() const { return g_; }
   const std::vector<Step> &steps() const { return steps_; }
   std::string describe() const; // one line per step
+  // HIP source of the kernels that are generated for the fused groups of this plan (dry plans included)
+  std::vector<gcjit::FusedKernelSource> generated_kernels() const;
+  // launches of generated kernels by all executables of the process (tests check that the generated path ran)
+  static long generated_launches();
 
 private:
   Graph g_;
@@ -112,6 +121,7 @@ private:
   std::unordered_map<int, bool> colsum_valid_; // ColSum results of constant weights are computed once
   std::vector<char> step_done_;                // per step: a `once` step has run
   std::vector<char> const_staged_;             // per slot: a constant host input has been copied to the device
+  std::shared_ptr<gcjit::Module> jit_module_;  // the generated kernels of the fused groups
 
   int new_slot(size_t bytes, long tensor_id = -1);
   int slot_for(size_t tensor_id);
@@ -128,6 +138,7 @@ private:
   void add_copy(int src_slot, DT src_dt, const std::vector<int64_t> &dims, const std::vector<int64_t> &strides,
                 int dst_slot, DT dst_dt);
   void launch(const Step &s);
+  void build_generated_kernels();
 };
 
 } // namespace gcapi

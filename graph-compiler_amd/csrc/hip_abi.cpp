@@ -66,7 +66,8 @@ extern "C" int gcmi_init(int device) {
 namespace {
 int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream,
-                  int64_t batch = 1, int64_t a_bs = 0, int64_t b_bs = 0, int64_t c_bs = 0);
+                  int64_t batch = 1, int64_t a_bs = 0, int64_t b_bs = 0, int64_t c_bs = 0, const void *residual = nullptr,
+                  int64_t ldr = 0, int residual_dtype = 0);
 }
 
 extern "C" int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -97,10 +98,34 @@ extern "C" int gcmi_gemm_bf16_batched(const void *A, const void *B, void *C, int
                        stride_a, stride_b, stride_c);
 }
 
+extern "C" int gcmi_gemm_bf16_residual(const void *A, const void *B, void *C, int64_t batch, int64_t M, int64_t N,
+                                       int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a,
+                                       int64_t stride_b, int64_t stride_c, int trans_b, const void *bias,
+                                       int bias_dtype, int act, const void *residual, int64_t ldr, int residual_dtype,
+                                       int out_dtype, void *stream) {
+  if (batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0)
+    return fail(ST_INVALID, "gemm_bf16_residual: negative batch count or stride");
+  if (batch == 0)
+    return ST_OK;
+  if (batch > 65535)
+    return fail(ST_UNIMPL, "gemm_bf16_residual: more than 65535 batches in one call");
+  if (batch > 1 && stride_c < (M - 1) * ldc + N)
+    return fail(ST_INVALID, "gemm_bf16_residual: results of different batches would overlap");
+  if (residual) {
+    if (residual_dtype != GCMI_BF16 && residual_dtype != GCMI_F32)
+      return fail(ST_UNIMPL, "gemm_bf16_residual: residual_dtype %d", residual_dtype);
+    if (ldr < N || (batch > 1 && stride_c < (M - 1) * ldr + N))
+      return fail(ST_INVALID, "gemm_bf16_residual: residual rows or batches overlap (ldr %lld)", (long long)ldr);
+  }
+  return gemm_bf16_any(trans_b != 0, A, B, C, M, N, K, lda, ldb, ldc, bias, bias_dtype, act, out_dtype, stream, batch,
+                       stride_a, stride_b, stride_c, residual, ldr, residual_dtype);
+}
+
 namespace {
 int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream,
-                  int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs) {
+                  int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs, const void *residual, int64_t ldr,
+                  int residual_dtype) {
   if (M < 0 || N < 0 || K < 0)
     return fail(ST_INVALID, "gemm_bf16: negative size");
   if (M == 0 || N == 0)
@@ -121,6 +146,7 @@ int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M
   p.bias = bias, p.bias_dt = bias_dtype, p.act = act, p.out_dt = out_dtype;
   p.trans_b = trans_b ? 1 : 0;
   p.batch = batch, p.a_bs = a_bs, p.b_bs = b_bs, p.c_bs = c_bs;
+  p.residual = residual, p.ldr = ldr, p.residual_dt = residual_dtype;
   return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
 }
 } // namespace

@@ -1,0 +1,111 @@
+// Device-side arithmetic shared by every kernel: bf16 rounding, the activations of the GEMM epilogues and the table
+// of point-wise ops.  No includes (the including file supplies the HIP runtime, the fixed-width integer types and
+// op_codes.h): this text is also handed to the run-time compiler, so that generated kernels and the kernels built
+// with the library compute the same bits.
+#ifndef GCMI_DEVICE_MATH_HPP
+#define GCMI_DEVICE_MATH_HPP
+
+namespace gcmi {
+
+// f32 -> bf16, round to nearest even, NaN -> 0x7FC0: the reference's bf16_t
+// constructor (include/gc/ExecutionEngine/CPURuntime/Microkernel/
+// BrgemmInterface.h:83-92).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) {
+  uint32_t bits = __float_as_uint(v);
+  uint32_t r = (bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16;
+  return (v != v) ? (uint16_t)0x7FC0u : (uint16_t)r;
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+__device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+// erf(x) as an odd rational P(x^2)*x / Q(x^2) on |x| <= 3.95 (beyond that erf
+// rounds to +-1 in f32); absolute error below 5e-7.  The reference evaluates erf
+// with approximations of the same class (a table of degree-5 polynomials, or
+// Abramowitz-Stegun 7.1.26 with absolute error 1.5e-7:
+// legacy/core/src/compiler/ir/transform/cpu/target_specific_lower.cpp:1012-1130),
+// so nothing finer than that is pinned by it.  About 20 VALU operations, no branches.
+__device__ __forceinline__ float erf_rational(float x) {
+  const float xc = __builtin_amdgcn_fmed3f(x, -3.95f, 3.95f);
+  const float x2 = xc * xc;
+  float p = -2.72614225801306e-10f;
+  p = fmaf(p, x2, 2.77068142495902e-08f);
+  p = fmaf(p, x2, -2.10102402082508e-06f);
+  p = fmaf(p, x2, -5.69250639462346e-05f);
+  p = fmaf(p, x2, -7.34990630326855e-04f);
+  p = fmaf(p, x2, -2.95459980854025e-03f);
+  p = fmaf(p, x2, -1.60960333262415e-02f);
+  float q = -1.45660718464996e-05f;
+  q = fmaf(q, x2, -2.13374055278905e-04f);
+  q = fmaf(q, x2, -1.68282697438203e-03f);
+  q = fmaf(q, x2, -7.37332916720468e-03f);
+  q = fmaf(q, x2, -1.42647390514189e-02f);
+  const float r = __builtin_amdgcn_fmed3f((p * xc) * __builtin_amdgcn_rcpf(q), -1.0f, 1.0f);
+  return fabsf(x) >= 3.95f ? copysignf(1.0f, x) : r;
+}
+
+// Activation in f32.  Operation order follows the reference graphs:
+// ReLU   = max(x, 0), NaN propagates (lib/gc/Transforms/OneDNNGraphToLinalg.cpp:355-358)
+// GELU   = ((erf(x*c)+1)*x)*0.5, c = 0x3f3504f3 (legacy/core/src/ops/gelu.cpp:110-131)
+// tanh   = (x*(tanh((((x*x)*0.044715+1)*x)*0.79788458)+1))*0.5 (gelu.cpp:78-108)
+// sigmoid= 1/(1+exp(-x)) (lib/gc/Dialect/Linalgx/LinalgxOps.cpp:42-61)
+__device__ __forceinline__ float apply_act(float x, int act) {
+  switch (act) {
+  case ACT_RELU:
+    return (x != x) ? x : fmaxf(x, 0.0f);
+  case ACT_GELU_ERF: {
+    const float c = __uint_as_float(0x3f3504f3u);
+    return ((erf_rational(x * c) + 1.0f) * x) * 0.5f;
+  }
+  case ACT_GELU_TANH: {
+    float t = (((x * x) * 0.044715f + 1.0f) * x) * 0.79788458f;
+    return (x * (tanhf(t) + 1.0f)) * 0.5f;
+  }
+  case ACT_SIGMOID:
+    return 1.0f / (1.0f + expf(-x));
+  default:
+    return x;
+  }
+}
+
+// one point-wise op in f32 (shared by the single-op kernel and the fused programs)
+__device__ __forceinline__ float round_to_storage(float v, int dt) {
+  switch (dt) {
+  case DT_BF16: return bf16_bits_to_f32(f32_to_bf16_bits(v));
+  case DT_F16: return (float)(_Float16)v;
+  default: return v;
+  }
+}
+
+__device__ __forceinline__ float fused_op(int op, float x, float y, float imm) {
+  switch (op) {
+  case ELT_ADD: return x + y;
+  case ELT_SUB: return x - y;
+  case ELT_MUL: return x * y;
+  case ELT_DIV: return x / y;
+  case ELT_MAX: return (x != x || y != y) ? x + y : fmaxf(x, y);
+  case ELT_EXP: return expf(x);
+  case ELT_NEG: return -x;
+  case ELT_RELU: return apply_act(x, ACT_RELU);
+  case ELT_SIGMOID: return apply_act(x, ACT_SIGMOID);
+  case ELT_GELU_ERF: return apply_act(x, ACT_GELU_ERF);
+  case ELT_GELU_TANH: return apply_act(x, ACT_GELU_TANH);
+  case ELT_POW: return imm == 2.0f ? x * x : (imm == 1.0f ? x : (imm == 0.5f ? sqrtf(x) : powf(x, imm)));
+  case ELT_MIN: return (x != x || y != y) ? x + y : fminf(x, y); // arith.minimumf: NaN propagates
+  case ELT_ABS: return fabsf(x);
+  case ELT_CEIL: return ceilf(x);
+  case ELT_FLOOR: return floorf(x);
+  case ELT_ERF: return erff(x);
+  case ELT_LOG: return logf(x);
+  case ELT_ROUND: return roundf(x); // math.round: halves away from zero
+  case ELT_RSQRT: return 1.0f / sqrtf(x);
+  case ELT_SQRT: return sqrtf(x);
+  case ELT_SQUARE: return x * x;
+  case ELT_TANH: return tanhf(x);
+  case ELT_RECIP: return 1.0f / x;
+  default: return x; // ELT_COPY
+  }
+}
+
+} // namespace gcmi
+
+#endif

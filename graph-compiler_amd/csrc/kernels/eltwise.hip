@@ -46,45 +46,6 @@ __device__ __forceinline__ void store_from_f32(void *p, int64_t i, int dt, float
   }
 }
 
-// one point-wise op in f32 (shared by the single-op kernel and the fused programs)
-__device__ __forceinline__ float round_to_storage(float v, int dt) {
-  switch (dt) {
-  case DT_BF16: return bf16_bits_to_f32(f32_to_bf16_bits(v));
-  case DT_F16: return (float)(_Float16)v;
-  default: return v;
-  }
-}
-
-__device__ __forceinline__ float fused_op(int op, float x, float y, float imm) {
-  switch (op) {
-  case ELT_ADD: return x + y;
-  case ELT_SUB: return x - y;
-  case ELT_MUL: return x * y;
-  case ELT_DIV: return x / y;
-  case ELT_MAX: return (x != x || y != y) ? x + y : fmaxf(x, y);
-  case ELT_EXP: return expf(x);
-  case ELT_NEG: return -x;
-  case ELT_RELU: return apply_act(x, ACT_RELU);
-  case ELT_SIGMOID: return apply_act(x, ACT_SIGMOID);
-  case ELT_GELU_ERF: return apply_act(x, ACT_GELU_ERF);
-  case ELT_GELU_TANH: return apply_act(x, ACT_GELU_TANH);
-  case ELT_POW: return imm == 2.0f ? x * x : (imm == 1.0f ? x : (imm == 0.5f ? sqrtf(x) : powf(x, imm)));
-  case ELT_MIN: return (x != x || y != y) ? x + y : fminf(x, y); // arith.minimumf: NaN propagates
-  case ELT_ABS: return fabsf(x);
-  case ELT_CEIL: return ceilf(x);
-  case ELT_FLOOR: return floorf(x);
-  case ELT_ERF: return erff(x);
-  case ELT_LOG: return logf(x);
-  case ELT_ROUND: return roundf(x); // math.round: halves away from zero
-  case ELT_RSQRT: return 1.0f / sqrtf(x);
-  case ELT_SQRT: return sqrtf(x);
-  case ELT_SQUARE: return x * x;
-  case ELT_TANH: return tanhf(x);
-  case ELT_RECIP: return 1.0f / x;
-  default: return x; // ELT_COPY
-  }
-}
-
 // out[idx] = op(a[idx . sa], b[idx . sb]); out is dense row-major over dims
 __global__ void eltwise_kernel(EltParams p) {
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < p.n; idx += (int64_t)gridDim.x * blockDim.x) {
@@ -525,109 +486,10 @@ extern "C" int gcmi_launch_fused(const FusedParams *pp, hipStream_t stream) {
   FusedParams p = *pp;
   if (p.n <= 0)
     return 0;
+  const int bad = fused_prepare(p, false);
+  if (bad)
+    return bad;
   const bool has_sum = p.sum_ins >= 0;
-  if (p.n_in < 1 || p.n_in > FUSED_MAX_IN || p.n_ins < 0 || p.n_ins > FUSED_MAX_INS || p.sum_ins >= p.n_ins)
-    return 2;
-  if (!has_sum)
-    p.n_in_pre = p.n_in_row = p.n_in, p.row_end = p.n_ins, p.n_red = 1;
-  if (p.n_in_pre < 0 || p.n_in_pre > p.n_in_row || p.n_in_row > p.n_in || p.n_red < 1 || p.n % p.n_red != 0 ||
-      (has_sum && (p.row_end <= p.sum_ins || p.row_end > p.n_ins)))
-    return 2;
-  auto is_float = [](int dt) { return dt == DT_F32 || dt == DT_BF16 || dt == DT_F16; };
-  for (int k = 0; k < p.n_in; k++)
-    if (!is_float(p.in_dt[k]) || !p.in[k])
-      return 2;
-  if (!is_float(p.out_dt) || !p.out)
-    return 2;
-  const bool second_pass = has_sum && p.row_end < p.n_ins;
-  if (!second_pass && p.n_in_row != p.n_in)
-    return 2;
-  // every instruction reads registers that are already written and that exist in its phase: before the sum the
-  // per-element inputs and results; per row the sum, the per-row inputs and results; in the second pass the
-  // per-row values, its own inputs and results
-  auto phase_of_ins = [&](int j) { return !has_sum ? 0 : j < p.sum_ins ? 0 : j < p.row_end ? 1 : 2; };
-  auto readable = [&](int r, int j) {
-    if (r < 0 || r >= p.n_in + j)
-      return false;
-    if (!has_sum)
-      return true;
-    const int ph = j <= p.sum_ins ? 0 : phase_of_ins(j); // the sum itself reads a per-element value
-    const int src = r < p.n_in ? (r < p.n_in_pre ? 0 : r < p.n_in_row ? 1 : 2) : phase_of_ins(r - p.n_in);
-    return ph == 0 ? src == 0 : ph == 1 ? src == 1 : src >= 1;
-  };
-  for (int j = 0; j < p.n_ins; j++) {
-    const FusedIns &f = p.ins[j];
-    if ((f.op == ELT_ROWSUM) != (j == p.sum_ins))
-      return 2;
-    if (!readable(f.a, j) || !readable(f.op == ELT_ROWSUM ? f.a : f.b, j))
-      return 2;
-  }
-  if (p.out_reg < 0 || p.out_reg >= p.n_in + p.n_ins)
-    return 2;
-  if (has_sum && phase_of_ins(p.out_reg - p.n_in) != (second_pass ? 2 : 1))
-    return 2;
-  // merge neighbouring iteration dims that every input walks contiguously (or not at all): fewer divisions per
-  // element.  The boundary between rows and the inside of a row is never merged across.
-  int64_t dims[ELT_MAX_RANK], str[FUSED_MAX_IN][ELT_MAX_RANK], ostr[ELT_MAX_RANK];
-  int nd = 0;
-  int64_t inner = 1; // elements of the dims to the right of d
-  for (int d = ELT_MAX_RANK - 1; d >= 0; d--) {
-    if (p.dims[d] == 1)
-      continue;
-    bool merge = nd > 0 && !(has_sum && inner == p.n_red);
-    for (int k = 0; k < p.n_in && merge; k++)
-      merge = p.in_str[k][d] == str[k][nd - 1] * dims[nd - 1];
-    if (merge && second_pass)
-      merge = p.out_str[d] == ostr[nd - 1] * dims[nd - 1];
-    if (merge) {
-      dims[nd - 1] *= p.dims[d];
-    } else {
-      dims[nd] = p.dims[d];
-      for (int k = 0; k < p.n_in; k++)
-        str[k][nd] = p.in_str[k][d];
-      ostr[nd] = p.out_str[d];
-      nd++;
-    }
-    inner *= p.dims[d];
-  }
-  for (int d = 0; d < ELT_MAX_RANK; d++) {
-    const int src = ELT_MAX_RANK - 1 - d; // dims[] was filled innermost first
-    p.dims[d] = src < nd ? dims[src] : 1;
-    for (int k = 0; k < p.n_in; k++)
-      p.in_str[k][d] = src < nd ? str[k][src] : 0;
-    p.out_str[d] = src < nd ? ostr[src] : 0;
-  }
-  p.rank = nd;
-  // quad mode: the innermost dim holds whole groups of four, so a thread's four elements share every outer
-  // coordinate; an operand contiguous there and aligned (base address and outer strides) moves as one vector
-  // (dims are never merged across the boundary of a row, so with a sum the innermost dim lies inside the row
-  // whenever the row has more than one element)
-  p.quad = nd > 0 && dims[0] % 4 == 0 && (!has_sum || p.n_red > 1) ? 1 : 0;
-  p.vec_mask = 0, p.out_vec = 0;
-  if (p.quad) {
-    auto aligned = [&](const void *ptr, int dt, const int64_t *st_of_dim) {
-      const uintptr_t need = dt == DT_F32 ? 16 : 8;
-      if (reinterpret_cast<uintptr_t>(ptr) % need != 0)
-        return false;
-      for (int d = 1; d < nd; d++)
-        if (st_of_dim[d] % 4 != 0)
-          return false;
-      return st_of_dim[0] == 1;
-    };
-    for (int k = 0; k < p.n_in; k++)
-      if (aligned(p.in[k], p.in_dt[k], str[k]))
-        p.vec_mask |= 1 << k;
-    if (second_pass) {
-      p.out_vec = aligned(p.out, p.out_dt, ostr) ? 1 : 0;
-    } else {
-      const uintptr_t need = p.out_dt == DT_F32 ? 16 : 8;
-      p.out_vec = !has_sum && reinterpret_cast<uintptr_t>(p.out) % need == 0 ? 1 : 0;
-    }
-  }
-  // collapsed dims that lie inside a row
-  p.rank_red = 0;
-  for (int64_t in_row = 1; has_sum && in_row < p.n_red && p.rank_red < nd; p.rank_red++)
-    in_row *= dims[p.rank_red];
   if (fused_allocate(p) > FUSED_MAX_PHYS)
     return 3;
   const size_t lds = (size_t)p.n_phys * 256 * sizeof(float) * FU; // the kernels with 256 threads

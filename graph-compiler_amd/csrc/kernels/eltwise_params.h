@@ -1,17 +1,11 @@
 // Argument blocks of the generic element-wise / reduce / softmax kernels.
 #pragma once
 #include <stdint.h>
+#include "op_codes.h"
 
 namespace gcmi {
 
 static constexpr int ELT_MAX_RANK = 6;
-
-enum EltOp : int {
-  ELT_COPY = 0, ELT_ADD, ELT_SUB, ELT_MUL, ELT_DIV, ELT_RELU, ELT_SIGMOID, ELT_GELU_ERF, ELT_GELU_TANH, ELT_POW,
-  ELT_DEQUANT, ELT_QUANT, ELT_MAX, ELT_EXP, ELT_NEG,
-  ELT_ROWSUM, // only inside a FusedParams program: the row sum of a register
-  ELT_MIN, ELT_ABS, ELT_CEIL, ELT_FLOOR, ELT_ERF, ELT_LOG, ELT_ROUND, ELT_RSQRT, ELT_SQRT, ELT_SQUARE, ELT_TANH, ELT_RECIP
-};
 
 struct EltParams {
   const void *a;
@@ -86,6 +80,118 @@ struct FusedParams {
   int32_t n_phys;                  // physical registers in use
   FusedIns ins[FUSED_MAX_INS];
 };
+
+// Validates a fused program and brings its iteration space into the form the kernels walk: neighbouring dims merged,
+// the four-element mode and the vector moves decided, the dims inside a row counted.  Returns 0, or 2 for a
+// program that is not well formed.  assume_aligned: decide the vector moves from the strides alone (for code that is
+// generated before the addresses are known and checks them when it is launched).
+inline int fused_prepare(FusedParams &p, bool assume_aligned) {
+  enum { PDT_F16 = 1, PDT_BF16 = 2, PDT_F32 = 3 }; // dnnl_data_type_t values, as everywhere in these parameter blocks
+  const bool has_sum = p.sum_ins >= 0;
+  if (p.n_in < 1 || p.n_in > FUSED_MAX_IN || p.n_ins < 0 || p.n_ins > FUSED_MAX_INS || p.sum_ins >= p.n_ins)
+    return 2;
+  if (!has_sum)
+    p.n_in_pre = p.n_in_row = p.n_in, p.row_end = p.n_ins, p.n_red = 1;
+  if (p.n_in_pre < 0 || p.n_in_pre > p.n_in_row || p.n_in_row > p.n_in || p.n_red < 1 || p.n % p.n_red != 0 ||
+      (has_sum && (p.row_end <= p.sum_ins || p.row_end > p.n_ins)))
+    return 2;
+  auto is_float = [](int dt) { return dt == PDT_F32 || dt == PDT_BF16 || dt == PDT_F16; };
+  for (int k = 0; k < p.n_in; k++)
+    if (!is_float(p.in_dt[k]) || (!p.in[k] && !assume_aligned))
+      return 2;
+  if (!is_float(p.out_dt) || (!p.out && !assume_aligned))
+    return 2;
+  const bool second_pass = has_sum && p.row_end < p.n_ins;
+  if (!second_pass && p.n_in_row != p.n_in)
+    return 2;
+  // every instruction reads registers that are already written and that exist in its phase: before the sum the
+  // per-element inputs and results; per row the sum, the per-row inputs and results; in the second pass the
+  // per-row values, its own inputs and results
+  auto phase_of_ins = [&](int j) { return !has_sum ? 0 : j < p.sum_ins ? 0 : j < p.row_end ? 1 : 2; };
+  auto readable = [&](int r, int j) {
+    if (r < 0 || r >= p.n_in + j)
+      return false;
+    if (!has_sum)
+      return true;
+    const int ph = j <= p.sum_ins ? 0 : phase_of_ins(j); // the sum itself reads a per-element value
+    const int src = r < p.n_in ? (r < p.n_in_pre ? 0 : r < p.n_in_row ? 1 : 2) : phase_of_ins(r - p.n_in);
+    return ph == 0 ? src == 0 : ph == 1 ? src == 1 : src >= 1;
+  };
+  for (int j = 0; j < p.n_ins; j++) {
+    const FusedIns &f = p.ins[j];
+    if ((f.op == ELT_ROWSUM) != (j == p.sum_ins))
+      return 2;
+    if (!readable(f.a, j) || !readable(f.op == ELT_ROWSUM ? f.a : f.b, j))
+      return 2;
+  }
+  if (p.out_reg < 0 || p.out_reg >= p.n_in + p.n_ins)
+    return 2;
+  if (has_sum && phase_of_ins(p.out_reg - p.n_in) != (second_pass ? 2 : 1))
+    return 2;
+  // merge neighbouring iteration dims that every input walks contiguously (or not at all): fewer divisions per
+  // element.  The boundary between rows and the inside of a row is never merged across.
+  int64_t dims[ELT_MAX_RANK], str[FUSED_MAX_IN][ELT_MAX_RANK], ostr[ELT_MAX_RANK];
+  int nd = 0;
+  int64_t inner = 1; // elements of the dims to the right of d
+  for (int d = ELT_MAX_RANK - 1; d >= 0; d--) {
+    if (p.dims[d] == 1)
+      continue;
+    bool merge = nd > 0 && !(has_sum && inner == p.n_red);
+    for (int k = 0; k < p.n_in && merge; k++)
+      merge = p.in_str[k][d] == str[k][nd - 1] * dims[nd - 1];
+    if (merge && second_pass)
+      merge = p.out_str[d] == ostr[nd - 1] * dims[nd - 1];
+    if (merge) {
+      dims[nd - 1] *= p.dims[d];
+    } else {
+      dims[nd] = p.dims[d];
+      for (int k = 0; k < p.n_in; k++)
+        str[k][nd] = p.in_str[k][d];
+      ostr[nd] = p.out_str[d];
+      nd++;
+    }
+    inner *= p.dims[d];
+  }
+  for (int d = 0; d < ELT_MAX_RANK; d++) {
+    const int src = ELT_MAX_RANK - 1 - d; // dims[] was filled innermost first
+    p.dims[d] = src < nd ? dims[src] : 1;
+    for (int k = 0; k < p.n_in; k++)
+      p.in_str[k][d] = src < nd ? str[k][src] : 0;
+    p.out_str[d] = src < nd ? ostr[src] : 0;
+  }
+  p.rank = nd;
+  // quad mode: the innermost dim holds whole groups of four, so a thread's four elements share every outer
+  // coordinate; an operand contiguous there and aligned (base address and outer strides) moves as one vector
+  // (dims are never merged across the boundary of a row, so with a sum the innermost dim lies inside the row
+  // whenever the row has more than one element)
+  p.quad = nd > 0 && dims[0] % 4 == 0 && (!has_sum || p.n_red > 1) ? 1 : 0;
+  p.vec_mask = 0, p.out_vec = 0;
+  if (p.quad) {
+    auto aligned = [&](const void *ptr, int dt, const int64_t *st_of_dim) {
+      const uintptr_t need = dt == PDT_F32 ? 16 : 8;
+      if (!assume_aligned && reinterpret_cast<uintptr_t>(ptr) % need != 0)
+        return false;
+      for (int d = 1; d < nd; d++)
+        if (st_of_dim[d] % 4 != 0)
+          return false;
+      return st_of_dim[0] == 1;
+    };
+    for (int k = 0; k < p.n_in; k++)
+      if (aligned(p.in[k], p.in_dt[k], str[k]))
+        p.vec_mask |= 1 << k;
+    if (second_pass) {
+      p.out_vec = aligned(p.out, p.out_dt, ostr) ? 1 : 0;
+    } else {
+      const uintptr_t need = p.out_dt == PDT_F32 ? 16 : 8;
+      p.out_vec = !has_sum && (assume_aligned || reinterpret_cast<uintptr_t>(p.out) % need == 0) ? 1 : 0;
+    }
+  }
+  // collapsed dims that lie inside a row
+  p.rank_red = 0;
+  for (int64_t in_row = 1; has_sum && in_row < p.n_red && p.rank_red < nd; p.rank_red++)
+    in_row *= dims[p.rank_red];
+  return 0;
+}
 
 // Register allocation by lifetimes, on a validated program in single-assignment form.  Program order: inputs of a
 // phase, then its instructions.  Phases 1 and 3 repeat per element, so a register may be reused inside a phase as

@@ -28,6 +28,11 @@ struct GemmParams {
   // strided batch (bf16 tile kernels): blockIdx.y is the batch index, operands advance by these element strides
   // (0 = the operand is shared by all batches).  batch <= 1: a single GEMM.
   int64_t batch, a_bs, b_bs, c_bs;
+  // bf16 GEMMs: a tensor of the shape of C that is added last, after bias and activation (a residual connection);
+  // with bf16 output the sum is rounded like every other op of a bf16 graph.  Batches advance it like C.
+  const void *residual; // null: none
+  int64_t ldr;          // elements between its rows
+  int32_t residual_dt;  // DT_BF16 or DT_F32
 };
 
 struct F32GemmParams {

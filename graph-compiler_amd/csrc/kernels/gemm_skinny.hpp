@@ -130,17 +130,26 @@ template <int MT> __global__ __launch_bounds__(SK_WAVES * 64, 2) void gemm_skinn
       if (p.bias)
         b = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n + c])
                                  : reinterpret_cast<const float *>(p.bias)[n + c];
-      float x = v[c];
+      float x = v[c], r = 0.0f;
+      if (p.residual)
+        r = p.residual_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.residual)[m * p.ldr + n + c])
+                                     : reinterpret_cast<const float *>(p.residual)[m * p.ldr + n + c];
       if (p.out_dt == DT_BF16) {
         x = round_bf16(x);
         if (p.bias)
           x = round_bf16(x + b);
         if (p.act != ACT_NONE)
           x = round_bf16(apply_act(x, p.act));
+        if (p.residual)
+          x = round_bf16(x + r);
       } else {
         if (p.bias)
           x = x + b;
         x = apply_act(x, p.act);
+        if (p.residual) { // kept apart from the activation's last multiply: the sum equals a separate add
+#pragma clang fp contract(off)
+          x = x + r;
+        }
       }
       o32[c] = x;
       o16[c] = f32_to_bf16_bits(x);

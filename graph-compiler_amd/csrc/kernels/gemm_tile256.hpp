@@ -181,6 +181,26 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
           return;
         uint32_t o32[4];
         uint16_t o16[4];
+        float res4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (ES == 2 && p.residual) {
+          const int64_t at = m * p.ldr + n;
+          if (!EDGE) { // the launcher sends unaligned residuals to the EDGE kernels
+            if (p.residual_dt == DT_BF16) {
+              const uint2 v = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.residual) + at);
+              res4[0] = __uint_as_float(v.x << 16), res4[1] = __uint_as_float(v.x & 0xffff0000u);
+              res4[2] = __uint_as_float(v.y << 16), res4[3] = __uint_as_float(v.y & 0xffff0000u);
+            } else {
+              const f32x4_t v = *reinterpret_cast<const f32x4_t *>(reinterpret_cast<const float *>(p.residual) + at);
+              res4[0] = v[0], res4[1] = v[1], res4[2] = v[2], res4[3] = v[3];
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              if (n + e < p.N)
+                res4[e] = p.residual_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.residual)[at + e])
+                                                   : reinterpret_cast<const float *>(p.residual)[at + e];
+          }
+        }
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           if (ES == 1) {
@@ -200,6 +220,7 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
             }
           } else {
             float x = (float)acc[j][i][4 * q + e];
+            const float r = res4[e];
             if (p.out_dt == DT_BF16) {
               // bf16 graph: round after the matmul and after every bf16 op
               // (lib/gc/Transforms/Pipeline.cpp:79-95)
@@ -208,12 +229,18 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
                 x = round_bf16(x + bias4[e]);
               if (ACT != ACT_NONE)
                 x = round_bf16(act_const<ACT>(x));
+              if (p.residual)
+                x = round_bf16(x + r);
               o16[e] = f32_to_bf16_bits(x);
               o32[e] = 0;
             } else {
               if (p.bias)
                 x = x + bias4[e];
               x = act_const<ACT>(x);
+              if (p.residual) { // kept apart from the activation's last multiply: the sum equals a separate add
+#pragma clang fp contract(off)
+                x = x + r;
+              }
               o32[e] = __float_as_uint(x);
               o16[e] = 0;
             }
@@ -313,6 +340,8 @@ template <int ES, bool EDGE, bool TB = false> __global__ __launch_bounds__(G_THR
   const char *Ab = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * ES;
   const char *Bb = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * ES;
   p.C = reinterpret_cast<char *>(p.C) + bz * p.c_bs * (p.out_dt == DT_BF16 ? 2 : 4);
+  if (p.residual)
+    p.residual = reinterpret_cast<const char *>(p.residual) + bz * p.c_bs * (p.residual_dt == DT_BF16 ? 2 : 4);
 
   // ---- global -> register staging assignment: 4 A chunks + 4 B chunks per thread
   const int a_row0 = tid >> 3, a_c = tid & 7;             // rows a_row0 + 64*i
@@ -604,6 +633,8 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
     p.A = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * ES;
     p.B = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * ES;
     p.C = reinterpret_cast<char *>(p.C) + bz * p.c_bs * (p.out_dt == DT_BF16 ? 2 : 4);
+  if (p.residual)
+    p.residual = reinterpret_cast<const char *>(p.residual) + bz * p.c_bs * (p.residual_dt == DT_BF16 ? 2 : 4);
   }
 
   FG g;
@@ -767,17 +798,26 @@ template <int ACT> __global__ __launch_bounds__(256) void gemm_splitk_reduce_ker
   float o32[4];
 #pragma unroll
   for (int e = 0; e < 4; e++) {
-    float x = a[e];
+    float x = a[e], r = 0.0f;
+    if (p.residual)
+      r = p.residual_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.residual)[m * p.ldr + n + e])
+                                   : reinterpret_cast<const float *>(p.residual)[m * p.ldr + n + e];
     if (p.out_dt == DT_BF16) { // bf16 graph: round after the matmul and after every bf16 op
       x = round_bf16(x);
       if (p.bias)
         x = round_bf16(x + bias4[e]);
       if (ACT != ACT_NONE)
         x = round_bf16(act_const<ACT>(x));
+      if (p.residual)
+        x = round_bf16(x + r);
     } else {
       if (p.bias)
         x = x + bias4[e];
       x = act_const<ACT>(x);
+      if (p.residual) { // kept apart from the activation's last multiply: the sum equals a separate add
+#pragma clang fp contract(off)
+        x = x + r;
+      }
     }
     o32[e] = x;
     o16[e] = f32_to_bf16_bits(x);
@@ -828,10 +868,15 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   const int BK = G_KBYTES / ES;
   // fast path: whole tiles, 16-byte aligned rows, and a tile's rows reachable with 32-bit byte offsets
   const int KGROUP = 256 / ES; // K elements of one trip round the LDS ring
-  const bool fast_but_m = p.N % G_BN == 0 && p.K % KGROUP == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) &&
+  const int res_es = p.residual_dt == DT_BF16 ? 2 : 4;
+  // the kernels for whole tiles read four residual elements with one load
+  const bool res_vec = !p.residual || (al16(p.residual) && (p.ldr * res_es) % 16 == 0);
+  const bool fast_but_m = p.N % G_BN == 0 && p.K % KGROUP == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) && res_vec &&
                           (p.lda * ES) % 16 == 0 && (p.ldb * ES) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
                           p.lda * ES * G_BM < (int64_t)1 << 31 && p.ldb * ES * (p.trans_b ? G_BN : BK) < (int64_t)1 << 31;
   if (p.trans_b && ES != 2)
+    return 3;
+  if (p.residual && (ES != 2 || (p.residual_dt != DT_BF16 && p.residual_dt != DT_F32) || p.out_dt == DT_S32))
     return 3;
   bool fast = fast_but_m && p.M % G_BM == 0;
   p.splits = 0;
@@ -844,7 +889,8 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
     return 2;
   if (nbatch == 1)
     p.a_bs = p.b_bs = p.c_bs = 0;
-  else if (!((p.a_bs * ES) % 16 == 0 && (p.b_bs * ES) % 16 == 0 && (p.c_bs * out_es) % 16 == 0))
+  else if (!((p.a_bs * ES) % 16 == 0 && (p.b_bs * ES) % 16 == 0 && (p.c_bs * out_es) % 16 == 0 &&
+             (!p.residual || (p.c_bs * res_es) % 16 == 0)))
     fast = false; // every batch's operands must keep the alignment the fast path loads with
   if (ES == 2 && fast_but_m && tiles_m == 1 && p.out_dt != DT_S32 && nbatch == 1) {
     const int n_cu = gcmi_num_cus();

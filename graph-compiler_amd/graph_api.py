@@ -15,7 +15,8 @@ EXPORTS["dnnl_graph_compiler.h"] = [
     "dnnl_graph_compiler_get_version", "dnnl_graph_compiler_create", "dnnl_graph_compiler_destroy",
     "dnnl_graph_compiler_compile", "dnnl_graph_compiler_destroy_executable", "dnnl_graph_compiler_execute",
     "dnnl_graph_compiler_explain", "dnnl_graph_compiler_last_error",
-    "dnnl_graph_compiler_compile_mlir", "dnnl_graph_compiler_explain_mlir"]
+    "dnnl_graph_compiler_compile_mlir", "dnnl_graph_compiler_explain_mlir", "dnnl_graph_compiler_generated_source_mlir",
+    "dnnl_graph_compiler_generated_kernel_launches"]
 
 SUCCESS, OUT_OF_MEMORY, INVALID_ARGUMENTS, UNIMPLEMENTED, RUNTIME_ERROR, INVALID_GRAPH = 0, 1, 2, 3, 5, 7
 
@@ -59,6 +60,10 @@ def api():
         L.dnnl_graph_compiler_compile_mlir.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
         L.dnnl_graph_compiler_explain_mlir.restype = C.c_int
         L.dnnl_graph_compiler_explain_mlir.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t]
+        L.dnnl_graph_compiler_generated_source_mlir.restype = C.c_int
+        L.dnnl_graph_compiler_generated_source_mlir.argtypes = [C.c_char_p, C.c_char_p, C.c_char_p, C.c_size_t]
+        L.dnnl_graph_compiler_generated_kernel_launches.restype = C.c_long
+        L.dnnl_graph_compiler_generated_kernel_launches.argtypes = []
         _bound = True
     return L
 
@@ -75,6 +80,19 @@ def explain_mlir(module_text):
     buf = C.create_string_buffer(1 << 16)
     st = api().dnnl_graph_compiler_explain_mlir(module_text.encode(), buf, len(buf))
     return st, (buf.value.decode() if st == 0 else api().dnnl_graph_compiler_last_error().decode())
+
+
+def generated_source_mlir(module_text, check_arch=None):
+    """HIP source of the kernels that compile_mlir generates for the fused groups of a module; with check_arch
+    ("gfx950") the source is also compiled (no GPU needed) and a failure is reported with the compiler's log."""
+    buf = C.create_string_buffer(1 << 20)
+    st = api().dnnl_graph_compiler_generated_source_mlir(module_text.encode(), check_arch.encode() if check_arch else None,
+                                                         buf, len(buf))
+    return st, (buf.value.decode() if st == 0 else api().dnnl_graph_compiler_last_error().decode())
+
+
+def generated_kernel_launches():
+    return api().dnnl_graph_compiler_generated_kernel_launches()
 
 
 def _tensor(tid, arr):

@@ -132,6 +132,25 @@ dnnl_status_t dnnl_graph_compiler_compile_mlir(const struct dnnl_graph_compiler 
                                                const struct dnnl_graph_compiler_executable **exe);
 dnnl_status_t dnnl_graph_compiler_explain_mlir(const char *module_text, char *buf, size_t len);
 
+/* Groups of point-wise ops (with an optional row sum inside) that the plan runs
+ * as one launch get a kernel of their own when the partition is compiled: HIP
+ * source written for the group's exact shapes, strides, types and ops, and
+ * compiled with hiprtc -- the counterpart of the reference lowering each fused
+ * group to its own loop nest and compiling it with LLVM
+ * (lib/gc/Transforms/Pipeline.cpp:152-194,
+ * lib/gc/ExecutionEngine/Driver/Driver.cpp:63-82).  The generated kernels give
+ * the same bits as the library's generic kernels for such groups, which stay
+ * in place when hiprtc is missing, when GCMI_NO_GENERATED_KERNELS=1 is set, or
+ * when an operand is not 16-byte aligned.
+ * ..._generated_source_mlir writes that source for a module (as accepted by
+ * compile_mlir) into buf without touching a GPU; with check_arch (for example
+ * "gfx950") it also compiles it and returns dnnl_runtime_error with the
+ * compiler's log as last error if that fails.
+ * ..._generated_kernel_launches counts the launches of generated kernels in
+ * this process so far. */
+dnnl_status_t dnnl_graph_compiler_generated_source_mlir(const char *module_text, const char *check_arch, char *buf, size_t len);
+long dnnl_graph_compiler_generated_kernel_launches(void);
+
 /* Text of the last error raised on the calling thread by the functions above
  * (no counterpart in the reference, which prints to stderr in debug builds). */
 const char *dnnl_graph_compiler_last_error(void);

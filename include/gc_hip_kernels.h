@@ -80,6 +80,25 @@ int gcmi_gemm_bf16_batched(const void *A, const void *B, void *C, int64_t batch,
                            int trans_b, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
 
 /*
+ * gcmi_gemm_bf16_batched with a residual connection in the epilogue:
+ * C = act(A.B + bias) + R, R a tensor of the shape of C (residual_dtype
+ * GCMI_BF16 or GCMI_F32, ldr elements between its rows, batch b at
+ * R + b*stride_c; NULL: none).  With out_dtype GCMI_BF16 the sum is rounded
+ * to bf16 like every other op of a bf16 graph, so the result equals a matmul
+ * followed by a separate add bit for bit.  Takes over the add that the
+ * reference fuses into the matmul's innermost loop nest as a consumer
+ * (tileAndFuseConsumerOfOpResult, lib/gc/Transforms/
+ * IterativeTilingAndFusion.cpp:505-560; the matmuls of
+ * test/benchgc/cases/llama2.mlir:10 and :75 end in one).
+ * R may be C itself (every element is read before it is written), but must not
+ * overlap it otherwise.
+ */
+int gcmi_gemm_bf16_residual(const void *A, const void *B, void *C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                            int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                            int trans_b, const void *bias, int bias_dtype, int act, const void *residual, int64_t ldr,
+                            int residual_dtype, int out_dtype, void *stream);
+
+/*
  * 8-bit matmul with s32 accumulation and fused dequantise epilogue.
  * Takes over: the u8/s8 brgemm (lib/gc/ExecutionEngine/CPURuntime/Microkernel/
  * BrgemmNaive.cpp:102-140) under the deep-tile nest, the asymmetric-activation

@@ -308,3 +308,71 @@ def test_batched_gemm_one_launch(gc, dev, dtype, nb, M, N, K):
     torch.cuda.synchronize()
     assert torch.equal(out_t, ref) if dtype == "bf16" else torch.allclose(out_t, ref, rtol=1e-5, atol=1e-5)
     assert torch.equal(shared, ref_s)
+
+
+# every kernel that can finish a bf16 GEMM: whole tiles (staged bf16 stores / direct f32 stores), partial tiles,
+# K sliced over workgroups with the second pass, weights stored [N,K] streamed by the short-A kernel with one
+# slice (epilogue in the kernel) and with several (second pass), and [N,K] weights through the tile kernel
+RESIDUAL_CASES = [(512, 512, 256, False), (256, 768, 512, True), (300, 200, 100, False), (257, 130, 96, True),
+                  (64, 512, 2048, False), (32, 4096, 4096, True), (32, 11008, 4096, True), (48, 8192, 512, True),
+                  (1, 7, 5, False)]
+
+
+@pytest.mark.parametrize("M,N,K,nt", RESIDUAL_CASES)
+@pytest.mark.parametrize("res_dtype,out_f32", [("bf16", False), ("f32", False), ("f32", True), ("bf16", True)])
+@pytest.mark.parametrize("epi", ["none", "bias_gelu"])
+def test_bf16_gemm_residual_equals_separate_add(gc, dev, M, N, K, nt, res_dtype, out_f32, epi):
+    """act(A.B + bias) + R in the epilogue is, bit for bit, the same GEMM without R followed by an add that rounds
+    once more when the result is bf16 (the rounding points of the reference's bf16 graphs)."""
+    torch.manual_seed(M * 7 + N)
+    A = (torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev)
+    B = (torch.randn((N, K) if nt else (K, N)) * 0.5).to(torch.bfloat16).to(dev)
+    R = torch.randn(M, N).to(torch.bfloat16 if res_dtype == "bf16" else torch.float32).to(dev)
+    bias = torch.randn(N).to(torch.bfloat16).to(dev) if epi != "none" else None
+    act = "gelu_erf" if epi != "none" else None
+    odt = gc.F32 if out_f32 else gc.BF16
+    plain = (gc.gemm_bf16_nt if nt else gc.gemm_bf16)(A, B, bias, act, out_dtype=odt)
+    fused = gc.gemm_bf16_residual(A, B, R, trans_b=nt, bias=bias, act=act, out_dtype=odt)
+    torch.cuda.synchronize()
+    want = plain.float() + R.float()  # one f32 add, as in the kernel
+    if not out_f32:
+        want = want.to(torch.bfloat16)
+    assert fused.dtype == want.dtype and torch.equal(fused, want), \
+        "max diff " + str((fused.float() - want.float()).abs().max().item())
+
+
+def test_bf16_gemm_residual_unaligned_and_strided(gc, dev):
+    """A residual whose rows are not 16-byte aligned goes through the kernels that load element by element; row
+    strides larger than the row are honoured."""
+    M, N, K = 256, 256, 128
+    torch.manual_seed(3)
+    A = (torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev)
+    B = (torch.randn(K, N) * 0.5).to(torch.bfloat16).to(dev)
+    big = torch.randn(M, N + 3).to(torch.bfloat16).to(dev)
+    plain = gc.gemm_bf16(A, B)
+    for R in (big[:, 1:N + 1], big[:, :N]):
+        fused = gc.gemm_bf16_residual(A, B, R)
+        torch.cuda.synchronize()
+        assert torch.equal(fused, (plain.float() + R.float()).to(torch.bfloat16))
+
+
+def test_bf16_gemm_residual_in_place_and_errors(gc, dev):
+    M, N, K = 512, 256, 192
+    torch.manual_seed(4)
+    A = (torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev)
+    B = (torch.randn(K, N) * 0.5).to(torch.bfloat16).to(dev)
+    R = torch.randn(M, N).to(torch.bfloat16).to(dev)
+    want = (gc.gemm_bf16(A, B).float() + R.float()).to(torch.bfloat16)
+    acc = R.clone()
+    gc.gemm_bf16_residual(A, B, acc, out=acc)  # x += A.B: every element is read before it is written
+    torch.cuda.synchronize()
+    assert torch.equal(acc, want)
+    L = gc.lib()
+    import ctypes as C
+    vp = lambda t: C.c_void_p(t.data_ptr())
+    st = L.gcmi_gemm_bf16_residual(vp(A), vp(B), vp(acc), 1, M, N, K, K, N, N, 0, 0, 0, 0, None, gc.BF16, 0, vp(R), N - 1,
+                                   gc.BF16, gc.BF16, None)
+    assert st != 0 and b"ldr" in L.gcmi_last_error()
+    st = L.gcmi_gemm_bf16_residual(vp(A), vp(B), vp(acc), 1, M, N, K, K, N, N, 0, 0, 0, 0, None, gc.BF16, 0, vp(R), N,
+                                   gc.S32, gc.BF16, None)
+    assert st != 0 and b"residual_dtype" in L.gcmi_last_error()

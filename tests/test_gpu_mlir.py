@@ -24,6 +24,18 @@ def mm(gc):
     return importlib.import_module("graph_compiler_amd.mlir_modules")
 
 
+@pytest.fixture(autouse=True, params=["generated", "library"])
+def fused_kernels(request, monkeypatch):
+    """Every test of this file runs twice: with the kernels that are generated for the fused groups when a module is
+    compiled (a failure to generate or compile them is an error here, not a quiet return to the library's kernels),
+    and with the library's generic kernels for such groups."""
+    if request.param == "library":
+        monkeypatch.setenv("GCMI_NO_GENERATED_KERNELS", "1")
+    else:
+        monkeypatch.setenv("GCMI_GENERATED_KERNELS_REQUIRED", "1")
+    return request.param
+
+
 def _run(ga, text, ins, outs):
     comp = ga.Compiler()
     try:
@@ -415,3 +427,54 @@ def test_fused_kernels_on_odd_shapes_f16(ga, dev, shape, axis):
     assert_close(rs.float().cpu().numpy(), s1.float().cpu().numpy(), 2e-3, "row sums f16")  # f16: 2^-11 per rounding
     rn = (rc.float() / s1.float().unsqueeze(axis)).half()
     assert_close(rn.float().cpu().numpy(), nrm.float().cpu().numpy(), 2e-3, "normalised f16")
+
+
+@pytest.mark.parametrize("M,K,N,nt", [(32, 4096, 4096, True), (300, 96, 200, False), (512, 256, 768, False)])
+def test_residual_connection_runs_in_the_matmul(ga, gc, dev, M, K, N, nt):
+    """x + relu(a.W + b), the result viewed as [1,M,N] in between: one launch, and bit for bit what the matmul with
+    bias and ReLU followed by a separate bf16 add gives."""
+    mt, at_ = "tensor<%dx%dxbf16>" % (M, N), "tensor<%dx%dxbf16>" % (M, K)
+    wt, t3, bt = "tensor<%dx%dxbf16>" % ((N, K) if nt else (K, N)), "tensor<1x%dx%dxbf16>" % (M, N), "tensor<%dxbf16>" % N
+    text = ("func.func @f(%a: " + at_ + ", %w: " + wt + ", %b: " + bt + ", %x: " + t3 + ") -> " + t3 + " {\n"
+            "  %z = arith.constant 0.0 : bf16\n"
+            "  %e = tensor.empty() : " + mt + "\n"
+            "  %f = linalg.fill ins(%z : bf16) outs(%e : " + mt + ") -> " + mt + "\n"
+            "  %m = linalg." + ("matmul_transpose_b" if nt else "matmul") + " ins(%a, %w : " + at_ + ", " + wt + ") outs(%f : " + mt + ") -> " + mt + "\n"
+            "  %bb = linalg.broadcast ins(%b : " + bt + ") outs(%e : " + mt + ") dimensions = [0]\n"
+            "  %s = linalg.add ins(%m, %bb : " + mt + ", " + mt + ") outs(%e : " + mt + ") -> " + mt + "\n"
+            "  %r = linalg.max ins(%s, %f : " + mt + ", " + mt + ") outs(%e : " + mt + ") -> " + mt + "\n"
+            "  %v = tensor.expand_shape %r [[0, 1], [2]] output_shape [1, " + str(M) + ", " + str(N) + "] : " + mt + " into " + t3 + "\n"
+            "  %e3 = tensor.empty() : " + t3 + "\n"
+            "  %o = linalg.add ins(%x, %v : " + t3 + ", " + t3 + ") outs(%e3 : " + t3 + ") -> " + t3 + "\n"
+            "  return %o : " + t3 + "\n}")
+    st, plan = ga.explain_mlir(text)
+    assert st == 0 and [l for l in plan.splitlines() if not l.startswith("arena")] == ["gemm_bf16: MatMul+bias+act+residual"], plan
+    torch.manual_seed(11)
+    a = (torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev)
+    w = (torch.randn((N, K) if nt else (K, N)) * 0.1).to(torch.bfloat16).to(dev)
+    b = torch.randn(N).to(torch.bfloat16).to(dev)
+    x = torch.randn(1, M, N).to(torch.bfloat16).to(dev)
+    o = torch.empty(1, M, N, dtype=torch.bfloat16, device=dev)
+    _run(ga, text, [(0, a), (1, w), (2, b), (3, x)], [(4, o)])
+    plain = (gc.gemm_bf16_nt if nt else gc.gemm_bf16)(a, w, b, "relu")
+    torch.cuda.synchronize()
+    assert torch.equal(o[0], (plain.float() + x[0].float()).to(torch.bfloat16))
+
+
+def test_generated_kernels_give_the_bits_of_the_library_kernels(ga, mm, dev, monkeypatch, fused_kernels):
+    """The kernels written out for a module's fused groups evaluate the library kernels' expressions in their order:
+    the decoder block (row statistics, scalings, the gate) at three shapes gives the same bits either way, and the
+    generated kernels are the ones that ran."""
+    if fused_kernels == "library":
+        pytest.skip("compares the two modes itself")
+    shapes = [(32, 512, 768, 3), (640, 256, 512, 4), (1024, 1024, 256, 5), (7, 36, 40, 6)]
+    before = ga.generated_kernel_launches()
+    gen = [_block_outputs(ga, mm, dev, T, H, F, seed) for T, H, F, seed in shapes]
+    ran = ga.generated_kernel_launches() - before
+    assert ran >= 3 * len(shapes), ran
+    monkeypatch.setenv("GCMI_NO_GENERATED_KERNELS", "1")
+    before = ga.generated_kernel_launches()
+    lib = [_block_outputs(ga, mm, dev, T, H, F, seed) for T, H, F, seed in shapes]
+    assert ga.generated_kernel_launches() == before
+    for (a0, a1), (b0, b1) in zip(gen, lib):
+        assert torch.equal(a0, b0) and torch.equal(a1, b1)
