@@ -894,8 +894,9 @@ void Executable::plan_fusion(std::vector<bool> &skip, const std::vector<bool> &c
         break;
       }
     }
-    if (red < 0 && post.size() == 1)
-      continue; // a lone op: the plain element-wise kernel
+    if (red < 0 && post.size() == 1 && !groups)
+      continue; // one launch per op was asked for: the plain element-wise kernel
+    // (otherwise a lone op is a group of one: four elements per thread, vector moves, a generated kernel)
 
     // ---- iteration space: [kept dims..., reduced dims...] of the sum's input, or the point-wise shape
     Step s;
@@ -1131,8 +1132,10 @@ void Executable::plan_fusion(std::vector<bool> &skip, const std::vector<bool> &c
       int64_t rows = 1;
       for (size_t d = 0; d < n_kept; d++)
         rows *= s1.dims[d];
-      const char *min_rows = getenv("GCMI_ROW_MERGE_MIN_ROWS"); // tuning knob; default 512
-      if (rows < (min_rows ? atoll(min_rows) : 512))
+      // (that holds for the library's generic row kernel, whose fixed cost per workgroup is high; a generated
+      // kernel is quicker as one launch at every row count)
+      const char *min_rows = getenv("GCMI_ROW_MERGE_MIN_ROWS"), *no_gen = getenv("GCMI_NO_GENERATED_KERNELS"); // tuning knob
+      if (rows < (min_rows ? atoll(min_rows) : no_gen && no_gen[0] == '1' ? 512 : 1))
         continue;
       Step m = s1;
       m.note = s2.note + " after " + s1.note;

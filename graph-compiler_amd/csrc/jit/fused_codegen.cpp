@@ -54,10 +54,13 @@ struct Gen {
     o << ind << "}\n";
   }
 
-  // inputs k0 .. k1-1 at offsets off<k> into registers r<k>[0..W)
-  void loads(int k0, int k1, const std::string &ind) {
+  // inputs k0 .. k1-1 at offsets off<k> into registers r<k>[0..W); `held` inputs are not loaded (see keep_from)
+  std::vector<int> keep_from; // second-pass input k -> the first-pass input whose values are still in registers, or -1
+  void loads(int k0, int k1, const std::string &ind, bool skip_held = false) {
     const int last = ELT_MAX_RANK - 1;
     for (int k = k0; k < k1; k++) {
+      if (skip_held && keep_from[(size_t)k] >= 0)
+        continue;
       const bool f32 = p.in_dt[k] == gcmi::DT_F32, vec = W == 4 && ((p.vec_mask >> k) & 1);
       const std::string src = "reinterpret_cast<const " + std::string(ctype(p.in_dt[k])) + " *>(in" + std::to_string(k) + ")";
       o << ind << "float r" << k << "[" << W << "];\n";
@@ -181,7 +184,6 @@ bool wide_indices(const FusedParams &p) {
 } // namespace
 
 bool generate_fused(const FusedParams &raw, const int *same_as, const std::string &name, FusedKernelSource &out) {
-  (void)same_as;
   FusedParams p = raw;
   if (p.n <= 0 || gcmi::fused_prepare(p, true) != 0)
     return false;
@@ -281,10 +283,22 @@ bool generate_fused(const FusedParams &raw, const int *same_as, const std::strin
     g.offsets("row", d0, d_row, t, "  ");
   }
   const int64_t step_elems = (int64_t)tpr * 4, trips = (p.n_red + step_elems - 1) / step_elems;
+  // A second-pass input that is a first-pass input again (the row that is normalised) is not read twice when a
+  // thread's share of the row is small enough to stay in registers.
+  g.keep_from.assign((size_t)p.n_in, -1);
+  std::vector<char> kept((size_t)p.n_in, 0);
+  if (second_pass && same_as && trips <= 8)
+    for (int k = p.n_in_row; k < p.n_in; k++)
+      if (same_as[k] >= 0 && same_as[k] < p.n_in_pre)
+        g.keep_from[(size_t)k] = same_as[k], kept[(size_t)same_as[k]] = 1;
+  for (int k = 0; k < p.n_in_pre; k++)
+    if (kept[(size_t)k])
+      o << "  float keep" << k << "[" << trips << "][" << g.W * (p.quad ? 1 : 4) << "] = {};\n";
   auto row_loop = [&](int k0, int k1, int j0, int j1, bool pass2) {
     if (trips <= 8)
       o << "#pragma unroll\n";
-    o << "  for (" << g.idx << " s0_ = 0; s0_ < (" << g.idx << ")" << Gen::num(p.n_red) << "; s0_ += " << step_elems << ") {\n";
+    o << "  for (int it_ = 0; it_ < " << trips << "; it_++) {\n    const " << g.idx << " s0_ = (" << g.idx << ")it_ * " << step_elems
+      << ";\n";
     auto body = [&](const std::string &e, const std::string &ind) {
       std::vector<std::pair<std::string, const int64_t *>> t;
       std::vector<std::string> names;
@@ -299,7 +313,19 @@ bool generate_fused(const FusedParams &raw, const int *same_as, const std::strin
         t.emplace_back("ooff", p.out_str);
       }
       g.offsets(e, d_row, ELT_MAX_RANK, t, ind);
-      g.loads(k0, k1, ind);
+      g.loads(k0, k1, ind, pass2);
+      // quad: a thread's four elements of the step; otherwise element u of the step (the loop variable around this body)
+      for (int k = k0; k < k1; k++) {
+        const std::string slot = p.quad ? "" : "u * 1 + ";
+        if (!pass2 && kept[(size_t)k])
+          for (int u = 0; u < g.W; u++)
+            o << ind << "keep" << k << "[it_][" << slot << u << "] = r" << k << "[" << u << "];\n";
+        if (pass2 && g.keep_from[(size_t)k] >= 0) {
+          o << ind << "float r" << k << "[" << g.W << "];\n";
+          for (int u = 0; u < g.W; u++)
+            o << ind << "r" << k << "[" << u << "] = keep" << g.keep_from[(size_t)k] << "[it_][" << slot << u << "];\n";
+        }
+      }
       g.ops(j0, j1, g.W, ind);
       if (!pass2) {
         for (int u = 0; u < g.W; u++)

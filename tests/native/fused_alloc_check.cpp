@@ -6,9 +6,6 @@
 #include <cstdlib>
 #include <cstring>
 #include <vector>
-namespace gcmi {
-enum { DT_F32 = 3 };
-}
 #include "kernels/eltwise_params.h"
 using namespace gcmi;
 

@@ -77,7 +77,7 @@ def test_intermediate_that_is_an_output_is_not_fused_away(ga):
     g = json.loads(ga.matmul_bias_relu_json(64, 64, 64))
     g["output_ports"] = [3, 4]  # the pre-activation tensor is wanted too
     st, plan = ga.explain(json.dumps(g))
-    assert st == OK and _steps(plan) == ["gemm_f32: MatMul+bias", "eltwise: ReLU"]
+    assert st == OK and _steps(plan) == ["gemm_f32: MatMul+bias", "fused: ReLU"]
 
 
 def _mutate(fn):
