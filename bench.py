@@ -7,9 +7,10 @@ A step is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM.  The headline workload is the bf16 4096^3 GEMM; the
 int8 MLP layer, the bf16 MLP chain, fused attention, decode-shaped GEMMs (32
 rows against Llama FFN weights, HBM bound), the f32 plumbing case, the vendor
-libraries on the same shapes, the headline GEMM through the partition API and
-the llama-2 MLP block through the textual-MLIR entry point are measured in the
-same run and reported under "others" (--only picks some of them).  One JSON
+libraries on the same shapes, the headline GEMM through the partition API, the
+llama-2 MLP block through the textual-MLIR entry point and its RMSNorm alone at
+prefill size (a fused group with a generated kernel, HBM bound) are measured in
+the same run and reported under "others" (--only picks some of them).  One JSON
 line goes to stdout; progress goes to stderr.
 
 Kernel durations come from HIP events recorded on the stream the kernels are
@@ -100,7 +101,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32,decode,api,block")
+    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32,decode,api,block,norm")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the 4096^3 GEMM the CPU baseline computes")
     ap.add_argument("--mha-mode", default="both", choices=["both", "skip", "every"],
                     help="attention: time the default entry point (masked key blocks skipped), the every-block mode, or both")
@@ -387,6 +388,56 @@ def main():
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
         log("mlir llama2 block: %.4f ms per execute, %d launches, %.0f GB/s of weights" % (t_blk, n_launch, gbs))
         del sets
+        torch.cuda.empty_cache()
+
+    # ---------------- a fused group alone: the RMSNorm of the same case at prefill size (HBM bound)
+    if want("norm"):
+        ga = importlib.import_module("graph_compiler_amd.graph_api")
+        mlm = importlib.import_module("graph_compiler_amd.mlir_modules")
+        T, H = 16384, 4096
+        comp = ga.Compiler()
+        st, exe = comp.compile_mlir(mlm.rmsnorm(T, H))
+        if st:
+            log("bench.py: compile_mlir of the RMSNorm failed with status %d: %s" %
+                (st, ga.api().dnnl_graph_compiler_last_error().decode()))
+            sys.exit(4)
+        torch.manual_seed(8)
+        nsets = 3  # 3 x 256 MiB of rows in rotation: beyond the Infinity Cache
+        xs = [torch.randn(1, T, H, device=dev).to(torch.bfloat16) for _ in range(nsets)]
+        outs = [torch.empty(1, T, H, device=dev, dtype=torch.bfloat16) for _ in range(nsets)]
+        eps = torch.full((1,), 1e-5, device=dev)
+        gamma = (1 + 0.1 * torch.randn(H, device=dev)).to(torch.bfloat16)
+        before = ga.generated_kernel_launches()
+
+        def run_norm(i):
+            rc = exe.execute([(0, xs[i % nsets]), (1, eps), (2, gamma)], [(3, outs[i % nsets])])
+            if rc:
+                raise RuntimeError("execute -> %d" % rc)
+
+        for i in range(3):
+            run_norm(i)
+        torch.cuda.synchronize()
+        n = max(12, K // 2)
+        t0 = time.perf_counter()
+        for i in range(n):
+            run_norm(i)
+        torch.cuda.synchronize()
+        t_norm = (time.perf_counter() - t0) * 1e3 / n
+        generated = ga.generated_kernel_launches() - before == n + 3
+        exe.close()
+        comp.close()
+        byts = 2.0 * 2 * T * H  # each row read once and written once
+        gbs = byts / (t_norm * 1e-3) / 1e9
+        others["mlir_rmsnorm_16384x4096"] = {
+            "workload": "RMSNorm of test/benchgc/cases/llama2.mlir on 16384 tokens x 4096 (bf16 in and out, f32 inside): 13 linalg/"
+                        "tensor ops, one launch; textual MLIR through compile_mlir/execute with device pointers; wall clock per "
+                        "execute (returns after completion); algorithmic bytes = the rows read once and written once",
+            "kernel": "generated at compile time (hiprtc)" if generated else "the library's generic row kernel",
+            "ms_per_execute": round(t_norm, 4),
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
+        log("mlir rmsnorm %dx%d: %.4f ms per execute, %.0f GB/s (%s kernel)" % (T, H, t_norm, gbs, "generated" if generated else "library"))
+        del xs, outs
         torch.cuda.empty_cache()
 
     if args.copy_calibration:

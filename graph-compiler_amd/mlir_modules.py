@@ -130,6 +130,15 @@ def _rmsnorm(f, x, tokens, hidden, eps_arg, gamma_arg):
     return _binary(f, "mul", g, nb, full, "bf16")
 
 
+def rmsnorm(tokens, hidden):
+    """The RMSNorm of test/benchgc/cases/llama2.mlir alone: (x [1,tokens,hidden] bf16, eps [1] f32, gamma [hidden]
+    bf16) -> [1,tokens,hidden] bf16.  Tensor ids: arguments 0..2, the result 3."""
+    f = _Fn()
+    n = _rmsnorm(f, "%arg0", tokens, hidden, "%arg1", "%arg2")
+    return _module([ttype([1, tokens, hidden], "bf16"), ttype([1], "f32"), ttype([hidden], "bf16")],
+                   [ttype([1, tokens, hidden], "bf16")], f, [n])
+
+
 def decoder_mlp_block(tokens=32, hidden=4096, ffn=11008):
     """The second half of a llama-2 decoder layer, as test/benchgc/cases/llama2.mlir spells it:
 
