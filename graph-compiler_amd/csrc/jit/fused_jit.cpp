@@ -57,7 +57,12 @@ bool compile(const std::string &src, const std::string &arch, std::vector<char> 
 }
 
 std::mutex g_mu;
-std::map<std::string, std::shared_ptr<Module>> g_cache; // "<device>|<source>" -> module
+// "<device>|<source>" -> module.  Never destroyed: its modules would be unloaded during static destruction, when the
+// HIP runtime may already be gone.
+std::map<std::string, std::shared_ptr<Module>> &cache() {
+  static auto *c = new std::map<std::string, std::shared_ptr<Module>>();
+  return *c;
+}
 
 } // namespace
 
@@ -87,8 +92,8 @@ std::shared_ptr<Module> Module::build(const std::vector<FusedKernelSource> &kern
   }
   const std::string src = full_source(kernels), key = std::to_string(dev) + "|" + src;
   std::lock_guard<std::mutex> lock(g_mu);
-  auto it = g_cache.find(key);
-  if (it != g_cache.end())
+  auto it = cache().find(key);
+  if (it != cache().end())
     return it->second;
   std::vector<char> code;
   if (!compile(src, prop.gcnArchName, code, error))
@@ -99,7 +104,7 @@ std::shared_ptr<Module> Module::build(const std::vector<FusedKernelSource> &kern
     error = "hipModuleLoadData failed";
     return nullptr;
   }
-  g_cache[key] = m;
+  cache()[key] = m;
   return m;
 }
 

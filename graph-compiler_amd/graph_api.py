@@ -148,6 +148,25 @@ class Executable:
 
         return api().dnnl_graph_compiler_execute(self.h, pack(inputs), pack(outputs))
 
+    def bind(self, inputs, outputs):
+        """The tensor arrays for execute(), built once: bind(...)() is then the C call alone, which is what a C or
+        C++ caller pays (building the ctypes structures for a dozen tensors costs more than a small module runs)."""
+        keep = []
+
+        def pack(items):
+            arr = (Tensor * max(len(items), 1))()
+            for i, (tid, a) in enumerate(items):
+                t, dims = _tensor(tid, a)
+                keep.append((dims, a))
+                arr[i] = t
+            return arr
+
+        ins, outs, fn, h = pack(inputs), pack(outputs), api().dnnl_graph_compiler_execute, self.h
+
+        def call(_keep=keep):
+            return fn(h, ins, outs)
+        return call
+
     def close(self):
         if self.h:
             api().dnnl_graph_compiler_destroy_executable(self.h)

@@ -304,3 +304,22 @@ def test_json_elementwise_extension_ops(ga, dev):
     t = np.tanh(np.sqrt(np.abs(x.astype(np.float64))))
     ref = np.minimum(np.maximum(1.0 / np.square(np.log(np.exp(t))), y), z)
     assert_close(ref, out, 1e-4, "element-wise extension ops")
+
+
+def test_bound_tensor_lists_execute_repeatedly(ga, dev):
+    """Executable.bind builds the tensor structs once; calling it is the C execute alone, any number of times, and
+    sees the buffers' current contents."""
+    gcomp = ga.Compiler()
+    st, exe = gcomp.compile(_res("add.json"))
+    assert st == 0
+    a = torch.arange(128, dtype=torch.float32, device=dev)
+    b = torch.ones(128, dtype=torch.float32, device=dev)
+    out = torch.zeros(128, dtype=torch.float32, device=dev)
+    call = exe.bind([(0, a), (1, b)], [(2, out)])
+    for k in range(3):
+        b.fill_(float(k))
+        torch.cuda.synchronize()
+        assert call() == 0
+        assert torch.equal(out, a + k)
+    exe.close()
+    gcomp.close()
