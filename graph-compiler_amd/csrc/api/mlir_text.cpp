@@ -880,6 +880,23 @@ void fold_broadcasts(Graph &g, const std::set<size_t> &outputs, size_t &next_id)
     bool leading = true;
     for (size_t k = 0; k < added.size(); k++)
       leading = leading && std::find(added.begin(), added.end(), (int64_t)k) != added.end();
+    // the operand that would stand in for the broadcast: the source itself, or a view of it with unit dims
+    std::vector<int64_t> repl_shape = in.shape;
+    if (!leading) {
+      repl_shape = out.shape;
+      for (auto d : added)
+        repl_shape[(size_t)d] = 1;
+    }
+    // every reader must still see its result shape in its operands (an op on two broadcasts of row vectors has no
+    // full-shape operand left once both are folded: that broadcast stays a copy)
+    for (size_t u : users[out.id]) {
+      const Op &r = g.ops[u];
+      std::vector<int64_t> sa = r.in[0] == out.id ? repl_shape : g.tensors.at(r.in[0]).shape,
+                           sb = r.in[1] == out.id ? repl_shape : g.tensors.at(r.in[1]).shape, so;
+      ok = ok && broadcast_shape(sa, sb, so) && so == g.tensors.at(r.out[0]).shape;
+    }
+    if (!ok)
+      continue;
     size_t repl;
     if (leading) {
       repl = o.in[0];

@@ -91,6 +91,9 @@ struct Gen {
       } else {
         o << ind << "r" << k << "[0] = " << conv(src + "[off" + std::to_string(k) + "]") << ";\n";
       }
+      if (!f32) // the widened value is opaque to the ops that read it (see ops())
+        for (int u = 0; u < W; u++)
+          o << ind << "asm volatile(\"\" : \"+v\"(r" << k << "[" << u << "]));\n";
     }
   }
 
@@ -118,12 +121,17 @@ struct Gen {
         case gcmi::ELT_COPY: e = x; break;
         default: e = "gcmi::fused_op(" + std::to_string(in.op) + ", " + x + ", " + y + ", " + fimm(in.imm) + ")"; break;
         }
+        // Every op stands alone, as in the library kernel where its operands come out of LDS: a barrier keeps the
+        // compiler from contracting a multiply into the next op's add, or from narrowing f16 -> sqrt -> f16 to a
+        // half-precision instruction with other rounding.
         o << ind << d << " = " << e << ";\n";
+        if (in.dt == gcmi::DT_BF16 || in.dt == gcmi::DT_F16)
+          o << ind << "asm volatile(\"\" : \"+v\"(" << d << "));\n";
         if (in.dt == gcmi::DT_BF16)
           o << ind << d << " = gcmi::bf16_bits_to_f32(gcmi::f32_to_bf16_bits(" << d << "));\n";
         else if (in.dt == gcmi::DT_F16)
           o << ind << d << " = (float)(_Float16)" << d << ";\n";
-        o << ind << "asm volatile(\"\" : \"+v\"(" << d << "));\n"; // nothing is contracted across ops
+        o << ind << "asm volatile(\"\" : \"+v\"(" << d << "));\n";
       }
     }
   }

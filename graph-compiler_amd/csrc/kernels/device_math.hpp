@@ -95,7 +95,7 @@ __device__ __forceinline__ float fused_op(int op, float x, float y, float imm) {
   case ELT_CEIL: return ceilf(x);
   case ELT_FLOOR: return floorf(x);
   case ELT_ERF: return erff(x);
-  case ELT_LOG: return logf(x);
+  case ELT_LOG: return __builtin_logf(x); // spelled as the builtin: the offline headers and the run-time compiler's resolve logf differently
   case ELT_ROUND: return roundf(x); // math.round: halves away from zero
   case ELT_RSQRT: return 1.0f / sqrtf(x);
   case ELT_SQRT: return sqrtf(x);

@@ -1,0 +1,126 @@
+"""GPU: the kernels generated for fused point-wise groups against the library's generic kernels for the same groups,
+on seeded random programs -- random chains of the named unary and binary linalg ops over full-shape, row-broadcast
+and column-broadcast operands, storage types f32 / bf16 / f16, shapes inside and outside the four-elements-per-thread
+mode, optionally with a sum over the last or the first axis and a normalisation behind it.  The bar is bit equality
+(NaNs and infinities included: results are compared as integers), since both run the same expressions in the same order."""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+UNARY = ["abs", "ceil", "floor", "negf", "exp", "tanh", "square", "erf", "sqrt", "rsqrt", "log", "reciprocal", "round"]
+BINARY = ["add", "sub", "mul", "div", "max", "min"]
+SHAPES = [(5, 7, 3), (8, 64), (33, 130), (4, 6, 10, 12), (300,), (2, 1028), (64, 2048), (3, 4100), (600, 8)]
+
+
+@pytest.fixture(scope="module")
+def ga(gc, dev):
+    return importlib.import_module("graph_compiler_amd.graph_api")
+
+
+def _t(shape, dt):
+    return "tensor<" + "".join("%dx" % d for d in shape) + dt + ">"
+
+
+def random_module(rng, shape, dt):
+    """-> (text, argument shapes, result shapes).  Arguments: x, y (full shape), r (last dim), c (all but the last dim)."""
+    full = _t(shape, dt)
+    args = [("%x", shape), ("%y", shape)]
+    lines = ["%e = tensor.empty() : " + full]
+    values = ["%x", "%y"]
+    if len(shape) > 1:
+        args += [("%r", shape[-1:]), ("%c", shape[:-1])]
+        lines.append("%rb = linalg.broadcast ins(%r : " + _t(shape[-1:], dt) + ") outs(%e : " + full + ") dimensions = [" +
+                     ", ".join(str(i) for i in range(len(shape) - 1)) + "]")
+        lines.append("%cb = linalg.broadcast ins(%c : " + _t(shape[:-1], dt) + ") outs(%e : " + full + ") dimensions = [" +
+                     str(len(shape) - 1) + "]")
+        values += ["%rb", "%cb"]
+    n = 0
+
+    def emit(op, operands, ty, outs):
+        nonlocal n
+        n += 1
+        name = "%v" + str(n)
+        lines.append(name + " = linalg." + op + " ins(" + ", ".join(operands) + " : " + ", ".join([ty] * len(operands)) + ") outs(" +
+                     outs + " : " + ty + ") -> " + ty)
+        return name
+
+    for _ in range(int(rng.integers(1, 8))):
+        if rng.random() < 0.45:
+            values.append(emit(UNARY[int(rng.integers(len(UNARY)))], [values[int(rng.integers(len(values)))]], full, "%e"))
+        else:
+            a, b = values[int(rng.integers(len(values)))], values[int(rng.integers(len(values)))]
+            values.append(emit(BINARY[int(rng.integers(len(BINARY)))], [a, b], full, "%e"))
+    results, res_types = [values[-1]], [full]
+    kind = rng.random()
+    if len(shape) > 1 and kind < 0.6:  # a sum over one axis, an op on the row values, and (sometimes) a normalisation
+        axis = len(shape) - 1 if kind < 0.45 else 0
+        kept = [d for i, d in enumerate(shape) if i != axis]
+        row = _t(kept, dt)
+        lines.append("%er = tensor.empty() : " + row)
+        lines.append("%c0 = arith.constant 0.0 : " + dt)
+        lines.append("%z = linalg.fill ins(%c0 : " + dt + ") outs(%er : " + row + ") -> " + row)
+        lines.append("%s = linalg.reduce { arith.addf } ins(" + values[-1] + " : " + full + ") outs(%z : " + row + ") dimensions = [" +
+                     str(axis) + "]")
+        lines.append("%one = arith.constant dense<1.000000e+00> : " + row)
+        s1 = emit("add", ["%s", "%one"], row, "%er")
+        results, res_types = [s1], [row]
+        if rng.random() < 0.7:
+            lines.append("%sb = linalg.broadcast ins(" + s1 + " : " + row + ") outs(%e : " + full + ") dimensions = [" + str(axis) + "]")
+            nrm = emit("div", [values[-1], "%sb"], full, "%e")
+            if rng.random() < 0.5 and len(shape) > 1:
+                nrm = emit("mul", [nrm, "%rb"], full, "%e")
+            results, res_types = [nrm], [full]
+            if rng.random() < 0.5:
+                results, res_types = [s1, nrm], [row, full]
+    sig = ", ".join(a + ": " + _t(s, dt) for a, s in args)
+    ret = ", ".join(results) + " : " + ", ".join(res_types)
+    text = ("func.func @f(" + sig + ") -> (" + ", ".join(res_types) + ") {\n  " + "\n  ".join(lines) + "\n  return " + ret + "\n}")
+    shapes_of = {full: list(shape)}
+    if len(shape) > 1:
+        shapes_of[_t([d for i, d in enumerate(shape) if i != len(shape) - 1], dt)] = list(shape[:-1])
+        shapes_of[_t(list(shape[1:]), dt)] = list(shape[1:])
+    return text, [s for _, s in args], [shapes_of[t] for t in res_types]
+
+
+def _run(ga, text, ins, outs):
+    comp = ga.Compiler()
+    try:
+        st, exe = comp.compile_mlir(text)
+        assert st == 0, "compile_mlir -> %d: %s\n%s" % (st, ga.api().dnnl_graph_compiler_last_error().decode(), text)
+        try:
+            assert exe.execute(ins, outs) == 0, ga.api().dnnl_graph_compiler_last_error().decode()
+            torch.cuda.synchronize()
+        finally:
+            exe.close()
+    finally:
+        comp.close()
+
+
+@pytest.mark.parametrize("seed", range(72))
+def test_random_groups_generated_equals_library(ga, dev, monkeypatch, seed):
+    rng = np.random.default_rng(1000 + seed)
+    shape = SHAPES[seed % len(SHAPES)]
+    dt = ["f32", "bf16", "f16"][(seed // len(SHAPES) + seed) % 3]
+    td = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[dt]
+    text, arg_shapes, res_shapes = random_module(rng, shape, dt)
+    torch.manual_seed(seed)
+    ins = [((torch.rand(s, device=dev) - 0.4) * 3).to(td) for s in arg_shapes]
+    runs = []
+    for mode in ("generated", "library"):
+        if mode == "library":
+            monkeypatch.setenv("GCMI_NO_GENERATED_KERNELS", "1")
+        else:
+            monkeypatch.setenv("GCMI_GENERATED_KERNELS_REQUIRED", "1")
+        before = ga.generated_kernel_launches()
+        outs = [torch.full(s, 7.0, device=dev, dtype=td) for s in res_shapes]
+        _run(ga, text, list(enumerate(ins)), [(len(ins) + j, o) for j, o in enumerate(outs)])
+        assert (ga.generated_kernel_launches() > before) == (mode == "generated"), text
+        runs.append(outs)
+    bits = torch.int32 if dt == "f32" else torch.int16
+    for a, b in zip(*runs):
+        same = torch.equal(a.view(bits), b.view(bits))
+        assert same, "%s\nfirst difference at %s" % (text, (a.view(bits) != b.view(bits)).nonzero()[:4].tolist())

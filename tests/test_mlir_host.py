@@ -335,3 +335,21 @@ def test_generated_source_of_the_decoder_block(ga, mm):
     assert "__shfl_xor" in src and "gcmi::fused_op(" in src
     st, msg = ga.generated_source_mlir("func.func @f(", "gfx950")
     assert st != OK
+
+
+def test_ops_whose_operands_are_all_broadcasts(ga):
+    """linalg.broadcast is folded into its readers' strides only where each reader keeps an operand arrangement that
+    still broadcasts to its result: add(row, row) over [8,64] would be a [64] result, so that broadcast stays a copy."""
+    t = "tensor<8x64xf32>"
+    text = ("func.func @f(%x: T, %r: tensor<64xf32>, %c: tensor<8xf32>) -> (T, T) {\n"
+            "  %e = tensor.empty() : T\n"
+            "  %rb = linalg.broadcast ins(%r : tensor<64xf32>) outs(%e : T) dimensions = [0]\n"
+            "  %cb = linalg.broadcast ins(%c : tensor<8xf32>) outs(%e : T) dimensions = [1]\n"
+            "  %v1 = linalg.sub ins(%x, %cb : T, T) outs(%e : T) -> T\n"
+            "  %v2 = linalg.add ins(%rb, %rb : T, T) outs(%e : T) -> T\n"
+            "  %v3 = linalg.mul ins(%v1, %v2 : T, T) outs(%e : T) -> T\n"
+            "  %v4 = linalg.max ins(%cb, %x : T, T) outs(%e : T) -> T\n"
+            "  return %v3, %v4 : T, T\n}").replace("T", t)
+    st, plan = ga.explain_mlir(text)
+    assert st == OK, plan
+    assert _steps(plan) == ["eltwise: BroadcastTo (stride-0 copy)", "fused: Subtract+Add+Multiply", "fused: Maximum"], plan
