@@ -175,7 +175,7 @@ def _block_outputs(ga, mm, dev, T, H, F, seed):
 
 def test_fused_groups_compute_what_the_single_ops_compute(ga, mm, dev, monkeypatch):
     """Every instruction of a fused group rounds to its op's storage type, so fusing changes no bit: the decoder
-    block with the fusion pass on (10 launches) and off (one launch per op)."""
+    block with the fusion pass on (7 launches) and off (one launch per op)."""
     fused = _block_outputs(ga, mm, dev, 32, 512, 768, seed=3)
     fused_rows = _block_outputs(ga, mm, dev, 640, 256, 512, seed=4)  # rows enough for the one-launch normalisation
     monkeypatch.setenv("GCMI_NO_POINTWISE_FUSION", "1")
