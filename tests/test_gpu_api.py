@@ -20,6 +20,17 @@ def ga(gc, dev):
     return importlib.import_module("graph_compiler_amd.graph_api")
 
 
+@pytest.fixture(autouse=True, params=["generated", "library"])
+def fused_kernels(request, monkeypatch):
+    """Every test of this file runs with the kernels generated for fused point-wise groups at compile time (a failure
+    to generate or compile one is an error) and with the library's generic kernels for such groups."""
+    if request.param == "library":
+        monkeypatch.setenv("GCMI_NO_GENERATED_KERNELS", "1")
+    else:
+        monkeypatch.setenv("GCMI_GENERATED_KERNELS_REQUIRED", "1")
+    return request.param
+
+
 def _res(name):
     return open(os.path.join(ROOT, "tests", "golden", name)).read()
 
