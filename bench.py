@@ -377,6 +377,19 @@ def main():
             run_block(i)
         torch.cuda.synchronize()
         t_blk = (time.perf_counter() - t0) * 1e3 / n
+        # the same through execute_async on torch's stream: launches only, one wait at the end (a serving loop that
+        # keeps its tensors on the GPU)
+        cur = torch.cuda.current_stream().cuda_stream
+        bound_async = [exe.bind(list(enumerate(st_)), [(10, o1), (11, o2)], stream=cur) for st_ in sets]
+        for i in range(3):
+            bound_async[i % nsets]()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n):
+            if bound_async[i % nsets]():
+                raise RuntimeError("execute_async failed")
+        torch.cuda.synchronize()
+        t_blk_async = (time.perf_counter() - t0) * 1e3 / n
         exe.close()
         comp.close()
         byts = 2.0 * (H * H + 3 * H * Fd) + 2.0 * 4 * T * H
@@ -386,9 +399,11 @@ def main():
                         "gated FFN, residual, RMSNorm; textual MLIR through compile_mlir/execute with device pointers; wall "
                         "clock per execute (returns after completion); algorithmic bytes = the four weights + activations once",
             "launches_per_execute": n_launch, "ms_per_execute": round(t_blk, 4),
+            "ms_per_execute_async_back_to_back": round(t_blk_async, 4),
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
-        log("mlir llama2 block: %.4f ms per execute, %d launches, %.0f GB/s of weights" % (t_blk, n_launch, gbs))
+        log("mlir llama2 block: %.4f ms per execute, %d launches, %.0f GB/s of weights; %.4f ms back to back through execute_async"
+            % (t_blk, n_launch, gbs, t_blk_async))
         del sets
         torch.cuda.empty_cache()
 

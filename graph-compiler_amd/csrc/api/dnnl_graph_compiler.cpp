@@ -139,6 +139,29 @@ extern "C" dnnl_status_t dnnl_graph_compiler_execute(const dnnl_graph_compiler_e
   }
 }
 
+extern "C" dnnl_status_t dnnl_graph_compiler_execute_async(const dnnl_graph_compiler_executable *exe,
+                                                           dnnl_graph_compiler_tensor *inputs,
+                                                           dnnl_graph_compiler_tensor *outputs, void *stream) {
+  if (!exe)
+    return dnnl_invalid_arguments;
+  try {
+    const_cast<dnnl_graph_compiler_executable *>(exe)->impl.execute_async(inputs, outputs, (hipStream_t)stream);
+    return dnnl_success;
+  } catch (const std::invalid_argument &e) {
+    remember(e.what());
+    return dnnl_invalid_arguments;
+  } catch (const std::bad_alloc &) {
+    remember("out of memory");
+    return dnnl_out_of_memory;
+  } catch (const std::exception &e) {
+    remember(e.what());
+    return dnnl_runtime_error;
+  } catch (...) {
+    remember("unknown error");
+    return dnnl_runtime_error;
+  }
+}
+
 // Introspection for tests: the launch plan of a compiled partition, one line
 // per kernel, written into buf (truncated to len-1 characters).
 extern "C" __attribute__((visibility("default"))) size_t gc_executable_describe(const dnnl_graph_compiler_executable *exe,

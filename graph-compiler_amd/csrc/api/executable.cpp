@@ -1519,6 +1519,22 @@ void Executable::launch(const Step &s) {
 
 // src/dnnl/dnnl_graph_compiler.cpp:64-103
 void Executable::execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs) {
+  run(inputs, outputs, true);
+}
+
+// The launches of execute() on a stream of the caller's, in its order with the caller's other work there; nothing is
+// waited for.  The executable's arena holds the intermediates, so calls on one executable must follow one another on
+// one stream (or be ordered by the caller), and host buffers cannot take part.
+void Executable::execute_async(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs, hipStream_t stream) {
+  struct Swap {
+    hipStream_t &slot, saved;
+    Swap(hipStream_t &s, hipStream_t v) : slot(s), saved(s) { slot = v; }
+    ~Swap() { slot = saved; }
+  } swap(stream_, stream);
+  run(inputs, outputs, false);
+}
+
+void Executable::run(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs, bool wait) {
   auto find = [](dnnl_graph_compiler_tensor *ts, size_t n, size_t i, size_t id) -> dnnl_graph_compiler_tensor * {
     if (!ts)
       throw std::invalid_argument("Tensor not found");
@@ -1547,6 +1563,8 @@ void Executable::execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler
     if (is_device_pointer(t->data)) {
       ptr_[(size_t)slot] = t->data;
     } else {
+      if (!wait)
+        throw std::invalid_argument("execute_async: input " + std::to_string(id) + " is not a device pointer");
       // a constant keeps its first contents: staged once
       const bool constant = g_.tensors.at(id).constant;
       if (const_staged_.size() < slots_.size())
@@ -1567,6 +1585,8 @@ void Executable::execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler
     if (!t->data)
       throw std::invalid_argument("Output tensor has no buffer");
     bool also_input = slots_[(size_t)slot].is_input;
+    if (!wait && !is_device_pointer(t->data))
+      throw std::invalid_argument("execute_async: output " + std::to_string(id) + " is not a device pointer");
     if (is_device_pointer(t->data) && !also_input)
       ptr_[(size_t)slot] = t->data;
     else
@@ -1584,7 +1604,8 @@ void Executable::execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler
     hipMemcpyKind kind = is_device_pointer(cb.first) ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost;
     hip_check(hipMemcpyAsync(cb.first, ptr_[(size_t)cb.second], slots_[(size_t)cb.second].bytes, kind, stream_), "copy result");
   }
-  hip_check(hipStreamSynchronize(stream_), "execute");
+  if (wait)
+    hip_check(hipStreamSynchronize(stream_), "execute");
 }
 
 std::string Executable::describe() const {

@@ -99,6 +99,8 @@ public:
   Executable &operator=(const Executable &) = delete;
 
   void execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs);
+  // the same launches on the caller's stream, without waiting for them: device pointers only
+  void execute_async(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs, hipStream_t stream);
 
   const Graph &graph() const { return g_; }
   const std::vector<Step> &steps() const { return steps_; }
@@ -138,6 +140,7 @@ private:
   void add_copy(int src_slot, DT src_dt, const std::vector<int64_t> &dims, const std::vector<int64_t> &strides,
                 int dst_slot, DT dst_dt);
   void launch(const Step &s);
+  void run(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs, bool wait);
   void build_generated_kernels();
 };
 

@@ -14,7 +14,7 @@ from . import lib, EXPORTS
 EXPORTS["dnnl_graph_compiler.h"] = [
     "dnnl_graph_compiler_get_version", "dnnl_graph_compiler_create", "dnnl_graph_compiler_destroy",
     "dnnl_graph_compiler_compile", "dnnl_graph_compiler_destroy_executable", "dnnl_graph_compiler_execute",
-    "dnnl_graph_compiler_explain", "dnnl_graph_compiler_last_error",
+    "dnnl_graph_compiler_execute_async", "dnnl_graph_compiler_explain", "dnnl_graph_compiler_last_error",
     "dnnl_graph_compiler_compile_mlir", "dnnl_graph_compiler_explain_mlir", "dnnl_graph_compiler_generated_source_mlir",
     "dnnl_graph_compiler_generated_kernel_launches"]
 
@@ -53,6 +53,8 @@ def api():
         L.dnnl_graph_compiler_destroy_executable.argtypes = [C.c_void_p]
         L.dnnl_graph_compiler_execute.restype = C.c_int
         L.dnnl_graph_compiler_execute.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor)]
+        L.dnnl_graph_compiler_execute_async.restype = C.c_int
+        L.dnnl_graph_compiler_execute_async.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.c_void_p]
         L.dnnl_graph_compiler_explain.restype = C.c_int
         L.dnnl_graph_compiler_explain.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t]
         L.dnnl_graph_compiler_last_error.restype = C.c_char_p
@@ -148,9 +150,11 @@ class Executable:
 
         return api().dnnl_graph_compiler_execute(self.h, pack(inputs), pack(outputs))
 
-    def bind(self, inputs, outputs):
+    def bind(self, inputs, outputs, stream=None):
         """The tensor arrays for execute(), built once: bind(...)() is then the C call alone, which is what a C or
-        C++ caller pays (building the ctypes structures for a dozen tensors costs more than a small module runs)."""
+        C++ caller pays (building the ctypes structures for a dozen tensors costs more than a small module runs).
+        With `stream` (a hipStream_t as an integer, e.g. torch.cuda.current_stream().cuda_stream) the call is
+        execute_async on that stream: launches only, device tensors only."""
         keep = []
 
         def pack(items):
@@ -161,10 +165,17 @@ class Executable:
                 arr[i] = t
             return arr
 
-        ins, outs, fn, h = pack(inputs), pack(outputs), api().dnnl_graph_compiler_execute, self.h
+        ins, outs, h = pack(inputs), pack(outputs), self.h
+        if stream is None:
+            fn = api().dnnl_graph_compiler_execute
 
-        def call(_keep=keep):
-            return fn(h, ins, outs)
+            def call(_keep=keep):
+                return fn(h, ins, outs)
+        else:
+            fn_async, sp = api().dnnl_graph_compiler_execute_async, C.c_void_p(stream)
+
+            def call(_keep=keep):
+                return fn_async(h, ins, outs, sp)
         return call
 
     def close(self):

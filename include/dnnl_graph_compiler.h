@@ -102,6 +102,19 @@ dnnl_status_t dnnl_graph_compiler_execute(const struct dnnl_graph_compiler_execu
                                           struct dnnl_graph_compiler_tensor *inputs,
                                           struct dnnl_graph_compiler_tensor *outputs);
 
+/* No counterpart in the reference, whose execute runs on CPU threads and returns
+ * when they are done.  For callers that keep their tensors on the GPU (a serving
+ * loop, a framework with its own streams): the launches of execute on `stream`
+ * (a hipStream_t; NULL is the default stream), ordered with the caller's other
+ * work there, without waiting for them.  Every tensor's data must be a device
+ * pointer (a host pointer: dnnl_invalid_arguments, and nothing is launched).
+ * An executable keeps its intermediates in one
+ * arena: calls on one executable must follow one another on one stream, or be
+ * ordered by the caller with events. */
+dnnl_status_t dnnl_graph_compiler_execute_async(const struct dnnl_graph_compiler_executable *exe,
+                                                struct dnnl_graph_compiler_tensor *inputs,
+                                                struct dnnl_graph_compiler_tensor *outputs, void *stream);
+
 /* Host-side stages only (parse, verify, fuse, plan): writes the kernel launch
  * plan of the partition, one line per launch, into buf (NUL terminated,
  * truncated to len) and returns the status compile would return for these

@@ -334,3 +334,35 @@ def test_bound_tensor_lists_execute_repeatedly(ga, dev):
         assert torch.equal(out, a + k)
     exe.close()
     gcomp.close()
+
+
+def test_execute_async_on_the_callers_stream(ga, dev):
+    """execute_async launches on the stream it is given and does not wait: two calls with different inputs follow one
+    another there, results are read after the caller's own synchronisation; host buffers are refused."""
+    import ctypes as C
+    M, K, N = 64, 96, 128
+    g = ga._graph([{"kind": "MatMul", "inputs": [ga._t(0, "f32", [M, K]), ga._t(1, "f32", [K, N])], "outputs": [ga._t(2, "f32", [M, N])]},
+                   {"kind": "ReLU", "inputs": [ga._t(2, "f32", [M, N])], "outputs": [ga._t(3, "f32", [M, N])]},
+                   {"kind": "Exp", "inputs": [ga._t(3, "f32", [M, N])], "outputs": [ga._t(4, "f32", [M, N])]},
+                   {"kind": "Multiply", "inputs": [ga._t(4, "f32", [M, N]), ga._t(3, "f32", [M, N])], "outputs": [ga._t(5, "f32", [M, N])]}],
+                  [0, 1], [5])
+    comp = ga.Compiler()
+    st, exe = comp.compile(g)
+    assert st == 0, ga.api().dnnl_graph_compiler_last_error().decode()
+    torch.manual_seed(21)
+    a = [torch.randn(M, K, device=dev) * 0.2 for _ in range(2)]
+    w = torch.randn(K, N, device=dev) * 0.2
+    outs = [torch.zeros(M, N, device=dev) for _ in range(2)]
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        calls = [exe.bind([(0, a[i]), (1, w)], [(5, outs[i])], stream=side.cuda_stream) for i in range(2)]
+        assert calls[0]() == 0 and calls[1]() == 0
+    side.synchronize()
+    for i in range(2):
+        r = torch.relu(a[i].double() @ w.double())
+        assert_close((torch.exp(r) * r).cpu().numpy(), outs[i].double().cpu().numpy(), 1e-4, "async call %d" % i)
+    host = np.zeros((M, N), np.float32)
+    bad = exe.bind([(0, a[0]), (1, w)], [(5, host)], stream=side.cuda_stream)
+    assert bad() == ga.INVALID_ARGUMENTS and b"device pointer" in ga.api().dnnl_graph_compiler_last_error()
+    exe.close()
+    comp.close()
