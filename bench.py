@@ -390,6 +390,29 @@ def main():
                 raise RuntimeError("execute_async failed")
         torch.cuda.synchronize()
         t_blk_async = (time.perf_counter() - t0) * 1e3 / n
+        # and recorded once per buffer set into a HIP graph, then replayed
+        side = torch.cuda.Stream()
+        graphs = []
+        with torch.cuda.stream(side):
+            for st_ in sets:
+                call = exe.bind(list(enumerate(st_)), [(10, o1), (11, o2)], stream=side.cuda_stream)
+                call()
+                side.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                gr.capture_begin()
+                call()
+                gr.capture_end()
+                graphs.append((gr, call))
+        side.synchronize()
+        for i in range(3):
+            graphs[i % nsets][0].replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n):
+            graphs[i % nsets][0].replay()
+        torch.cuda.synchronize()
+        t_blk_graph = (time.perf_counter() - t0) * 1e3 / n
+        del graphs
         exe.close()
         comp.close()
         byts = 2.0 * (H * H + 3 * H * Fd) + 2.0 * 4 * T * H
@@ -400,10 +423,11 @@ def main():
                         "clock per execute (returns after completion); algorithmic bytes = the four weights + activations once",
             "launches_per_execute": n_launch, "ms_per_execute": round(t_blk, 4),
             "ms_per_execute_async_back_to_back": round(t_blk_async, 4),
+            "ms_per_hip_graph_replay_back_to_back": round(t_blk_graph, 4),
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
-        log("mlir llama2 block: %.4f ms per execute, %d launches, %.0f GB/s of weights; %.4f ms back to back through execute_async"
-            % (t_blk, n_launch, gbs, t_blk_async))
+        log("mlir llama2 block: %.4f ms per execute, %d launches, %.0f GB/s of weights; back to back: %.4f ms through execute_async, %.4f ms as HIP graph replays"
+            % (t_blk, n_launch, gbs, t_blk_async, t_blk_graph))
         del sets
         torch.cuda.empty_cache()
 

@@ -478,3 +478,50 @@ def test_generated_kernels_give_the_bits_of_the_library_kernels(ga, mm, dev, mon
     assert ga.generated_kernel_launches() == before
     for (a0, a1), (b0, b1) in zip(gen, lib):
         assert torch.equal(a0, b0) and torch.equal(a1, b1)
+
+
+def test_execute_async_captured_in_a_hip_graph(ga, mm, dev):
+    """The launches of execute_async can be recorded into a HIP graph (no allocation, copy or memset is among them):
+    the decoder block -- split-K GEMMs with their workspace, residual epilogues, normalisations, the gate -- replayed
+    three times with new inputs, eager executes and synchronisations in between, gives the eager results bit for bit."""
+    T, H, F = 32, 512, 1024
+    bf = torch.bfloat16
+    torch.manual_seed(31)
+    r = lambda *s: torch.randn(*s, device=dev)  # noqa: E731
+    args = [r(1, T, H).to(bf), (r(H, H) / H ** 0.5).to(bf), r(1, T, H).to(bf), torch.full((1,), 1e-5, device=dev),
+            (1 + 0.1 * r(H)).to(bf), (r(F, H) / H ** 0.5).to(bf), (r(F, H) / H ** 0.5).to(bf), (r(H, F) / F ** 0.5).to(bf),
+            torch.full((1,), 1e-6, device=dev), (1 + 0.1 * r(H)).to(bf)]
+    o1 = torch.zeros(1, T, H, device=dev, dtype=bf)
+    o2 = torch.zeros_like(o1)
+    comp = ga.Compiler()
+    st, exe = comp.compile_mlir(mm.decoder_mlp_block(T, H, F))
+    assert st == 0, ga.api().dnnl_graph_compiler_last_error().decode()
+    try:
+        eager = exe.bind(list(enumerate(args)), [(10, o1), (11, o2)])
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            call = exe.bind(list(enumerate(args)), [(10, o1), (11, o2)], stream=side.cuda_stream)
+            assert call() == 0  # once outside the capture: modules and static buffers are resolved
+            side.synchronize()
+            graph.capture_begin()
+            rc = call()
+            graph.capture_end()
+            assert rc == 0
+        side.synchronize()
+        for k in range(3):
+            args[0].copy_(r(1, T, H).to(bf))
+            args[2].copy_(r(1, T, H).to(bf))
+            torch.cuda.synchronize()
+            assert eager() == 0
+            want = (o1.clone(), o2.clone())
+            o1.zero_()
+            o2.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(o1, want[0]) and torch.equal(o2, want[1]), "replay %d" % k
+        del graph
+    finally:
+        exe.close()
+        comp.close()
