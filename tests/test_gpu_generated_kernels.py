@@ -1,9 +1,12 @@
 """GPU: the kernels generated for fused point-wise groups against the library's generic kernels for the same groups,
 on seeded random programs -- random chains of the named unary and binary linalg ops over full-shape, row-broadcast
 and column-broadcast operands, storage types f32 / bf16 / f16, shapes inside and outside the four-elements-per-thread
-mode, optionally with a sum over the last or the first axis and a normalisation behind it.  The bar is bit equality
-(NaNs and infinities included: results are compared as integers), since both run the same expressions in the same order."""
+mode, optionally with a sum over the last or the first axis and a normalisation behind it.  The bar between the two
+is bit equality (NaNs and infinities included: results are compared as integers), since both run the same expressions
+in the same order.  Both share the planner, so the programs are also evaluated op by op with torch (f32 arithmetic,
+every result rounded to the storage type) and compared within a tolerance, NaNs and infinities in the same places."""
 import importlib
+import re
 
 import numpy as np
 import pytest
@@ -86,6 +89,44 @@ def random_module(rng, shape, dt):
     return text, [s for _, s in args], [shapes_of[t] for t in res_types]
 
 
+T_UNARY = {"abs": torch.abs, "ceil": torch.ceil, "floor": torch.floor, "negf": torch.neg, "exp": torch.exp, "tanh": torch.tanh,
+           "square": lambda x: x * x, "erf": torch.erf, "sqrt": torch.sqrt, "rsqrt": torch.rsqrt, "log": torch.log,
+           "reciprocal": torch.reciprocal,
+           "round": lambda x: torch.where(x >= 0, torch.floor(x + 0.5), torch.ceil(x - 0.5))}  # halves away from zero
+T_BINARY = {"add": torch.add, "sub": torch.sub, "mul": torch.mul, "div": torch.div,
+            "max": lambda a, b: torch.where(torch.isnan(a) | torch.isnan(b), a + b, torch.maximum(a, b)),
+            "min": lambda a, b: torch.where(torch.isnan(a) | torch.isnan(b), a + b, torch.minimum(a, b))}
+
+
+def torch_reference(text, ins, td, shape):
+    """The module of random_module(), line by line: f32 arithmetic, every op's result rounded to the storage type."""
+    env = dict(zip(["%x", "%y", "%r", "%c"], [t.float() for t in ins]))
+    env["%one"] = torch.ones((), device=ins[0].device)
+
+    def rnd(v):
+        return v.to(td).float()
+
+    for line in text.splitlines():
+        line = line.strip()
+        m = re.match(r"(%\w+) = linalg\.(\w+) ins\(([^:]+) :", line)
+        if line.startswith("%s = linalg.reduce"):
+            src = re.search(r"ins\((%\w+)", line).group(1)
+            env["%s"] = rnd(env[src].sum(int(re.search(r"dimensions = \[(\d+)\]", line).group(1))))
+        elif m and m.group(2) == "broadcast":
+            v = env[m.group(3).strip()]
+            for d in sorted(int(d) for d in re.search(r"dimensions = \[([^\]]*)\]", line).group(1).split(",")):
+                v = v.unsqueeze(d)
+            env[m.group(1)] = v.expand(*shape)
+        elif m and m.group(2) in T_UNARY:
+            env[m.group(1)] = rnd(T_UNARY[m.group(2)](env[m.group(3).strip()]))
+        elif m and m.group(2) in T_BINARY:
+            a, b = [t.strip() for t in m.group(3).split(",")]
+            env[m.group(1)] = rnd(T_BINARY[m.group(2)](env[a], env[b]))
+        elif line.startswith("return"):
+            return [env[n.strip()] for n in line[len("return"):].split(":")[0].split(",")]
+    raise AssertionError("no return in the module")
+
+
 def _run(ga, text, ins, outs):
     comp = ga.Compiler()
     try:
@@ -124,3 +165,15 @@ def test_random_groups_generated_equals_library(ga, dev, monkeypatch, seed):
     for a, b in zip(*runs):
         same = torch.equal(a.view(bits), b.view(bits))
         assert same, "%s\nfirst difference at %s" % (text, (a.view(bits) != b.view(bits)).nonzero()[:4].tolist())
+    # against torch: one rounding of slack per op of the chain, libm-grade device functions
+    tol = {"f32": 2e-4, "bf16": 3e-2, "f16": 4e-3}[dt]
+    for got, ref in zip(runs[0], torch_reference(text, ins, td, list(shape))):
+        got, ref = got.double(), ref.double().expand_as(got)
+        assert torch.equal(torch.isnan(got), torch.isnan(ref)), text
+        fin = torch.isfinite(ref) & torch.isfinite(got)
+        rest = ~fin & ~torch.isnan(ref)
+        assert torch.equal(got[rest], ref[rest]), text  # infinities, with their signs
+        if fin.any():
+            scale = torch.maximum(ref[fin].abs(), ref[fin].pow(2).mean().sqrt().clamp(max=1e300))
+            err = ((got[fin] - ref[fin]).abs() / scale).max().item()
+            assert err <= tol, "%s\nerror %g" % (text, err)
