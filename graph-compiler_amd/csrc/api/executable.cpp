@@ -1105,6 +1105,13 @@ void Executable::plan_fusion(std::vector<bool> &skip, const std::vector<bool> &c
       bool only_here = true;
       for (size_t c : consumers[r])
         only_here = only_here && std::find(s2.f_members.begin(), s2.f_members.end(), c) != s2.f_members.end();
+      // an op with several point-wise readers is a member of each reader's group (it is recomputed there): no other
+      // group may load r either (a layer normalisation reads the mean in the variance group and in the scaling)
+      for (auto &other : emit_at)
+        for (const Step &so : other.second)
+          if (other.first != i2 && so.kind == Step::Fused &&
+              std::find(so.f_in_tensor.begin(), so.f_in_tensor.end(), r) != so.f_in_tensor.end())
+            only_here = false;
       // the same non-unit dims, and r broadcast exactly along the summed ones
       const size_t nd = s1.dims.size();
       if (!only_here || s1.f_place.size() != nd || s2.dims.size() != nd)

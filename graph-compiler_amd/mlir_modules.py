@@ -139,6 +139,36 @@ def rmsnorm(tokens, hidden):
                    [ttype([1, tokens, hidden], "bf16")], f, [n])
 
 
+def layernorm(rows, hidden, dtype="f32", eps=1e-5):
+    """Layer normalisation over the last axis spelled with named linalg ops, two reductions: mean, then the variance
+    of the centred values; (x [rows,hidden], gamma [hidden], beta [hidden]) -> [rows,hidden].  Ids 0..2, result 3."""
+    full, col, vec = ttype([rows, hidden], dtype), ttype([rows], dtype), ttype([hidden], dtype)
+    f = _Fn()
+    e, er = _empty(f, [rows, hidden], dtype), _empty(f, [rows], dtype)
+    z = _zeros(f, [rows], dtype)
+
+    def op(name, ins, ty, outs):
+        return f.emit("linalg.%s ins(%s : %s) outs(%s : %s) -> %s" % (name, ", ".join(ins), ", ".join([ty] * len(ins)), outs, ty, ty))
+
+    def rowsum(v):
+        return f.emit("linalg.reduce { arith.addf } ins(%s : %s) outs(%s : %s) dimensions = [1]" % (v, full, z, col))
+
+    def along_row(v):
+        return f.emit("linalg.broadcast ins(%s : %s) outs(%s : %s) dimensions = [1]" % (v, col, e, full))
+
+    def along_col(v):
+        return f.emit("linalg.broadcast ins(%s : %s) outs(%s : %s) dimensions = [0]" % (v, vec, e, full))
+
+    n = _splat(f, float(hidden), [rows], dtype)
+    mean = op("div", [rowsum("%arg0"), n], col, er)
+    d = op("sub", ["%arg0", along_row(mean)], full, e)
+    var = op("div", [rowsum(op("square", [d], full, e)), n], col, er)
+    r = op("rsqrt", [op("add", [var, _splat(f, eps, [rows], dtype)], col, er)], col, er)
+    y = op("mul", [op("mul", [d, along_row(r)], full, e), along_col("%arg1")], full, e)
+    y = op("add", [y, along_col("%arg2")], full, e)
+    return _module([full, vec, vec], [full], f, [y])
+
+
 def decoder_mlp_block(tokens=32, hidden=4096, ffn=11008):
     """The second half of a llama-2 decoder layer, as test/benchgc/cases/llama2.mlir spells it:
 

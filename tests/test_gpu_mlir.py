@@ -525,3 +525,23 @@ def test_execute_async_captured_in_a_hip_graph(ga, mm, dev):
     finally:
         exe.close()
         comp.close()
+
+
+@pytest.mark.parametrize("rows,hidden,dtype", [(512, 1024, "f32"), (37, 300, "f32"), (2048, 768, "bf16"), (8, 4096, "bf16")])
+def test_layer_normalisation(ga, mm, dev, monkeypatch, rows, hidden, dtype):
+    """Mean, variance of the centred values, scaling: two launches, against torch and bit for bit against one launch
+    per op."""
+    td = torch.float32 if dtype == "f32" else torch.bfloat16
+    torch.manual_seed(rows + hidden)
+    x = (torch.randn(rows, hidden, device=dev) * 2 + 0.5).to(td)
+    g = (1 + 0.2 * torch.randn(hidden, device=dev)).to(td)
+    b = torch.randn(hidden, device=dev).to(td)
+    y = torch.zeros(rows, hidden, device=dev, dtype=td)
+    _run(ga, mm.layernorm(rows, hidden, dtype), [(0, x), (1, g), (2, b)], [(3, y)])
+    ref = torch.nn.functional.layer_norm(x.double(), (hidden,), g.double(), b.double(), 1e-5)
+    # bf16: every op of the chain rounds (the centred values, their squares, the statistics)
+    assert_close(ref.cpu().numpy(), y.double().cpu().numpy(), 1e-4 if dtype == "f32" else 5e-2, "layer norm " + dtype)
+    monkeypatch.setenv("GCMI_NO_POINTWISE_FUSION", "1")
+    y1 = torch.zeros_like(y)
+    _run(ga, mm.layernorm(rows, hidden, dtype), [(0, x), (1, g), (2, b)], [(3, y1)])
+    assert torch.equal(y, y1)

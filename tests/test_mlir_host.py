@@ -353,3 +353,14 @@ def test_ops_whose_operands_are_all_broadcasts(ga):
     st, plan = ga.explain_mlir(text)
     assert st == OK, plan
     assert _steps(plan) == ["eltwise: BroadcastTo (stride-0 copy)", "fused: Subtract+Add+Multiply", "fused: Maximum"], plan
+
+
+def test_layer_normalisation_plan(ga, mm):
+    """Two reductions: the mean is read by the variance group and by the scaling, so it is a kernel of its own; the
+    variance group and the scaling (which alone reads the reciprocal deviation) share a launch."""
+    st, plan = ga.explain_mlir(mm.layernorm(512, 1024))
+    assert st == OK, plan
+    assert _steps(plan) == ["reduce: Divide of ReduceSum",
+                            "reduce: Subtract+Multiply+Multiply+Add after Divide+Add+Rsqrt of ReduceSum of Subtract+Square"], plan
+    st, src = ga.generated_source_mlir(mm.layernorm(512, 1024, "bf16"), "gfx950")
+    assert st == OK and src.count('extern "C" __global__') == 2, src
