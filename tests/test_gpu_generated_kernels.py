@@ -59,26 +59,57 @@ def random_module(rng, shape, dt):
             values.append(emit(BINARY[int(rng.integers(len(BINARY)))], [a, b], full, "%e"))
     results, res_types = [values[-1]], [full]
     kind = rng.random()
-    if len(shape) > 1 and kind < 0.6:  # a sum over one axis, an op on the row values, and (sometimes) a normalisation
-        axis = len(shape) - 1 if kind < 0.45 else 0
+    if len(shape) > 1 and kind < 0.7:
+        # a sum over one axis and an op on the row values; then (sometimes) a normalisation by it, or a second sum
+        # over values centred by the first -- the shape of a layer normalisation: a row statistic with two readers
+        axis = len(shape) - 1 if kind < 0.5 else 0
         kept = [d for i, d in enumerate(shape) if i != axis]
         row = _t(kept, dt)
         lines.append("%er = tensor.empty() : " + row)
         lines.append("%c0 = arith.constant 0.0 : " + dt)
         lines.append("%z = linalg.fill ins(%c0 : " + dt + ") outs(%er : " + row + ") -> " + row)
-        lines.append("%s = linalg.reduce { arith.addf } ins(" + values[-1] + " : " + full + ") outs(%z : " + row + ") dimensions = [" +
-                     str(axis) + "]")
         lines.append("%one = arith.constant dense<1.000000e+00> : " + row)
-        s1 = emit("add", ["%s", "%one"], row, "%er")
+
+        def rowsum(v):
+            nonlocal n
+            n += 1
+            name = "%s" + str(n)
+            lines.append(name + " = linalg.reduce { arith.addf } ins(" + v + " : " + full + ") outs(%z : " + row + ") dimensions = [" +
+                         str(axis) + "]")
+            return name
+
+        def spread(v):
+            nonlocal n
+            n += 1
+            name = "%b" + str(n)
+            lines.append(name + " = linalg.broadcast ins(" + v + " : " + row + ") outs(%e : " + full + ") dimensions = [" + str(axis) + "]")
+            return name
+
+        s1 = emit("add", [rowsum(values[-1]), "%one"], row, "%er")
         results, res_types = [s1], [row]
-        if rng.random() < 0.7:
-            lines.append("%sb = linalg.broadcast ins(" + s1 + " : " + row + ") outs(%e : " + full + ") dimensions = [" + str(axis) + "]")
-            nrm = emit("div", [values[-1], "%sb"], full, "%e")
-            if rng.random() < 0.5 and len(shape) > 1:
+        form = rng.random()
+        if form < 0.45:
+            nrm = emit("div", [values[-1], spread(s1)], full, "%e")
+            if rng.random() < 0.5:
                 nrm = emit("mul", [nrm, "%rb"], full, "%e")
             results, res_types = [nrm], [full]
             if rng.random() < 0.5:
                 results, res_types = [s1, nrm], [row, full]
+        elif form < 0.85:
+            centred = emit("sub", [values[-1], spread(s1)], full, "%e")
+            spreadsq = emit(["square", "abs"][int(rng.integers(2))], [centred], full, "%e")
+            s2 = emit("add", [rowsum(spreadsq), "%one"], row, "%er")
+            if rng.random() < 0.5:
+                s2 = emit("sqrt", [s2], row, "%er")
+            out = emit("div", [centred, spread(s2)], full, "%e")
+            if rng.random() < 0.5:
+                out = emit("add", [emit("mul", [out, "%rb"], full, "%e"), "%rb"], full, "%e")
+            results, res_types = [out], [full]
+            pick = rng.random()
+            if pick < 0.25:
+                results, res_types = [s2, out], [row, full]
+            elif pick < 0.4:
+                results, res_types = [s1, out], [row, full]
     sig = ", ".join(a + ": " + _t(s, dt) for a, s in args)
     ret = ", ".join(results) + " : " + ", ".join(res_types)
     text = ("func.func @f(" + sig + ") -> (" + ", ".join(res_types) + ") {\n  " + "\n  ".join(lines) + "\n  return " + ret + "\n}")
@@ -108,10 +139,9 @@ def torch_reference(text, ins, td, shape):
 
     for line in text.splitlines():
         line = line.strip()
-        m = re.match(r"(%\w+) = linalg\.(\w+) ins\(([^:]+) :", line)
-        if line.startswith("%s = linalg.reduce"):
-            src = re.search(r"ins\((%\w+)", line).group(1)
-            env["%s"] = rnd(env[src].sum(int(re.search(r"dimensions = \[(\d+)\]", line).group(1))))
+        m = re.match(r"(%\w+) = linalg\.(\w+)(?: \{ arith\.addf \})? ins\(([^:]+) :", line)
+        if m and m.group(2) == "reduce":
+            env[m.group(1)] = rnd(env[m.group(3).strip()].sum(int(re.search(r"dimensions = \[(\d+)\]", line).group(1))))
         elif m and m.group(2) == "broadcast":
             v = env[m.group(3).strip()]
             for d in sorted(int(d) for d in re.search(r"dimensions = \[([^\]]*)\]", line).group(1).split(",")):
@@ -174,6 +204,6 @@ def test_random_groups_generated_equals_library(ga, dev, monkeypatch, seed):
         rest = ~fin & ~torch.isnan(ref)
         assert torch.equal(got[rest], ref[rest]), text  # infinities, with their signs
         if fin.any():
-            scale = torch.maximum(ref[fin].abs(), ref[fin].pow(2).mean().sqrt().clamp(max=1e300))
+            scale = torch.maximum(ref[fin].abs(), ref[fin].pow(2).mean().sqrt().clamp(max=1e300)).clamp(min=1e-30)
             err = ((got[fin] - ref[fin]).abs() / scale).max().item()
             assert err <= tol, "%s\nerror %g" % (text, err)
