@@ -1352,6 +1352,14 @@ std::vector<gcjit::FusedKernelSource> Executable::generated_kernels() const {
   std::vector<gcjit::FusedKernelSource> ks;
   for (size_t i = 0; i < steps_.size(); i++) {
     const Step &s = steps_[i];
+    if (s.kind == Step::Softmax && s.inner == 1) {
+      gcjit::FusedKernelSource k;
+      if (gcjit::generate_softmax(s.outer, s.len, s.a_dt, s.out_dt, "gcmi_fused_step" + std::to_string(i), k)) {
+        k.source = "// SoftMax\n" + k.source;
+        ks.push_back(std::move(k));
+      }
+      continue;
+    }
     if (s.kind != Step::Fused)
       continue;
     gcmi::FusedParams p{};
@@ -1516,6 +1524,16 @@ void Executable::launch(const Step &s) {
     break;
   }
   case Step::Softmax: {
+    if (s.jit_fn) {
+      const void *in = P(s.a);
+      void *out = P(s.out);
+      if (!s.jit_vectors || ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+        void *args[2] = {(void *)&in, (void *)&out};
+        hip_check(hipModuleLaunchKernel(s.jit_fn, s.jit_grid, 1, 1, s.jit_block, 1, 1, 0, stream_, args, nullptr), "SoftMax");
+        g_generated_launches++;
+        break;
+      }
+    }
     gcmi::SoftmaxParams p{};
     p.in = P(s.a), p.out = P(s.out), p.outer = s.outer, p.len = s.len, p.inner = s.inner, p.in_dt = s.a_dt, p.out_dt = s.out_dt;
     gc_check(gcmi_launch_softmax(&p, stream_) ? 5 : 0, "SoftMax");

@@ -36,6 +36,10 @@ struct FusedKernelSource {
 // Returns false when the program is not one the generator covers (the caller keeps the interpreter).
 bool generate_fused(const gcmi::FusedParams &p, const int *same_as, const std::string &name, FusedKernelSource &out);
 
+// The kernel for a softmax along the innermost axis of a [rows, len] view (arguments: in0, out).  Returns false for
+// rows too long to keep in registers (the library's kernel runs those).
+bool generate_softmax(int64_t rows, int64_t len, int in_dt, int out_dt, const std::string &name, FusedKernelSource &out);
+
 // A compiled set of kernels, loaded on the device that was current when it was built.
 class Module {
 public:

@@ -545,3 +545,30 @@ def test_layer_normalisation(ga, mm, dev, monkeypatch, rows, hidden, dtype):
     y1 = torch.zeros_like(y)
     _run(ga, mm.layernorm(rows, hidden, dtype), [(0, x), (1, g), (2, b)], [(3, y1)])
     assert torch.equal(y, y1)
+
+
+@pytest.mark.parametrize("shape,axis,dtype", [((1024, 4096), 1, "f32"), ((100, 37), 1, "f32"), ((512, 2048), 1, "bf16"),
+                                              ((6, 50, 520), 2, "f16"), ((16, 10000), 1, "f32"), ((3, 40000), 1, "f32"),
+                                              ((8, 96, 33), 1, "f32"), ((2, 3, 4, 64), 3, "bf16")])
+def test_softmax_alone(ga, dev, fused_kernels, shape, axis, dtype):
+    """linalg.softmax outside an attention pattern: rows of 33 to 40000 elements, innermost and middle axes, three
+    storage types.  Innermost-axis rows of up to 32768 elements get a generated kernel (a row is read once and kept
+    in registers); the rest run on the library's kernel."""
+    td = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[dtype]
+    t = "tensor<" + "".join("%dx" % d for d in shape) + dtype + ">"
+    text = ("func.func @f(%x: " + t + ") -> " + t + " {\n  %e = tensor.empty() : " + t + "\n"
+            "  %y = linalg.softmax dimension(" + str(axis) + ") ins(%x : " + t + ") outs(%e : " + t + ") -> " + t + "\n"
+            "  return %y : " + t + "\n}")
+    torch.manual_seed(len(shape) * 100 + shape[-1])
+    x = (torch.randn(shape, device=dev) * 3).to(td)
+    x.view(-1)[5] = float("-inf")  # one masked element: weight exactly 0
+    y = torch.full(shape, 7.0, device=dev, dtype=td)
+    before = ga.generated_kernel_launches()
+    _run(ga, text, [(0, x)], [(1, y)])
+    generated = ga.generated_kernel_launches() > before
+    assert generated == (fused_kernels == "generated" and axis == len(shape) - 1 and shape[axis] <= 32768)
+    ref = torch.softmax(x.double(), axis)
+    tol = {"f32": 1e-4, "bf16": 1e-2, "f16": 2e-3}[dtype]
+    assert_close(ref.cpu().numpy(), y.double().cpu().numpy(), tol, "softmax " + dtype)
+    assert y.view(-1)[5].item() == 0.0
+    assert_close(np.ones(ref.sum(axis).shape), y.double().sum(axis).cpu().numpy(), 10 * tol, "rows sum to one")
