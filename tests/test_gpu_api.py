@@ -366,3 +366,55 @@ def test_execute_async_on_the_callers_stream(ga, dev):
     assert bad() == ga.INVALID_ARGUMENTS and b"device pointer" in ga.api().dnnl_graph_compiler_last_error()
     exe.close()
     comp.close()
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_attention_partitions_against_torch(ga, dev, seed):
+    """Attention graphs with random sizes (also ones the fused kernel's fast path does not take), head dims 128 and
+    64, the scale as Multiply or Divide, and masks that are absent, shared ([Sq,Sk] / [1,1,Sq,Sk]: fused kernel) or
+    per batch ([B,1,Sq,Sk]: the matcher declines and the ops run one by one): all against torch with P rounded to
+    bf16 as in the graph."""
+    rng = np.random.default_rng(7000 + seed)
+    B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+    Sq, Sk = int(rng.choice([64, 128, 200, 256])), int(rng.choice([64, 128, 192, 200]))
+    D = 128 if seed % 4 else 64
+    scale_op = "Multiply" if rng.random() < 0.5 else "Divide"
+    mask_kind = ["none", "2d", "4d_shared", "per_batch"][int(rng.integers(4))]
+    s = [B, H, Sq, Sk]
+    mshape = {"none": None, "2d": [Sq, Sk], "4d_shared": [1, 1, Sq, Sk], "per_batch": [B, 1, Sq, Sk]}[mask_kind]
+    ops = [{"kind": "MatMul", "attrs": {"transpose_b": {"type": "bool", "value": 1}},
+            "inputs": [ga._t(0, "bf16", [B, H, Sq, D]), ga._t(1, "bf16", [B, H, Sk, D])], "outputs": [ga._t(5, "f32", s)]},
+           {"kind": scale_op, "inputs": [ga._t(5, "f32", s), ga._t(2, "f32", [1])], "outputs": [ga._t(6, "f32", s)]}]
+    cur, ins = 6, [0, 1, 2]
+    if mshape:
+        ops.append({"kind": "Add", "inputs": [ga._t(6, "f32", s), ga._t(3, "f32", mshape)], "outputs": [ga._t(7, "f32", s)]})
+        cur = 7
+        ins.append(3)
+    ops.append({"kind": "SoftMax", "attrs": {"axis": {"type": "s64", "value": -1}},
+                "inputs": [ga._t(cur, "f32", s)], "outputs": [ga._t(8, "bf16", s)]})
+    ops.append({"kind": "MatMul", "inputs": [ga._t(8, "bf16", s), ga._t(4, "bf16", [B, H, Sk, D])],
+                "outputs": [ga._t(9, "bf16", [B, H, Sq, D])]})
+    ins.append(4)
+    g = ga._graph(ops, ins, [9])
+    st, plan = ga.explain(g)
+    assert st == 0, plan
+    fused = plan.startswith("attention") or "\nattention" in plan
+    assert fused == (D == 128 and not (mask_kind == "per_batch" and B > 1)), plan
+    torch.manual_seed(seed)
+    Q = torch.randn(B, H, Sq, D).to(torch.bfloat16)
+    K = torch.randn(B, H, Sk, D).to(torch.bfloat16)
+    V = torch.randn(B, H, Sk, D).to(torch.bfloat16)
+    scale = 1.0 / D ** 0.5
+    sval = np.array([scale if scale_op == "Multiply" else 1.0 / scale], np.float32)
+    mask = None
+    if mshape:
+        mask = torch.where(torch.rand(mshape) < 0.3, torch.tensor(-30000.0), torch.zeros(())).float()
+        mask[..., 0] = 0  # no fully masked row
+    out = torch.zeros(B, H, Sq, D, dtype=torch.bfloat16)
+    tensors = [(0, Q), (1, K), (2, sval)] + ([(3, mask)] if mshape else []) + [(4, V)]
+    _run(ga, g, tensors, [(9, out)])
+    S = Q.double() @ K.double().transpose(-1, -2) * scale + (mask.double() if mshape else 0)
+    P = torch.softmax(S, -1)
+    ref = (P.to(torch.bfloat16).double() @ V.double()).to(torch.bfloat16).float().numpy()
+    mag = (P @ V.double().abs()).numpy()
+    assert_close(ref, out.float().numpy(), 1e-2, "attention %s D=%d mask=%s\n%s" % (s, D, mask_kind, plan), mag=mag)
