@@ -556,11 +556,17 @@ template <int ES, int KS, int WJ = 2, bool SPLIT = false, bool TB = false> struc
   static __device__ __forceinline__ void interleave_hint() {
     if (SPLIT)
       return;
-#pragma unroll
-    for (int i = 0; i < 4 * WJ; i++) {
+    // the fragment reads of the next k-step go out with the first MFMAs, two per MFMA, so that they have landed
+    // when the group ends and the wait in front of the next group finds little outstanding (1-4 % over one read
+    // per MFMA spread over the whole group)
+    constexpr int N_DS = 4 + (TB ? WJ : 2 * WJ);
+    static_for<0, 4 * WJ>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // 1 DS read
-    }
+      constexpr int left = N_DS - 2 * i;
+      if constexpr (left > 0)
+        __builtin_amdgcn_sched_group_barrier(0x100, left < 2 ? left : 2, 0); // DS reads
+    });
   }
 
   // wait until at most BEHIND later stages of this wave's DMA are still in flight
