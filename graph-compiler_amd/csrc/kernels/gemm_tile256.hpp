@@ -134,6 +134,15 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
 
 template <int ACT> __device__ __forceinline__ float act_const(float x) { return apply_act(x, ACT); }
 
+// two f32 -> two bf16 in one instruction (v_cvt_pk_bf16_f32: round to nearest even; not for NaNs, whose sign and
+// payload it keeps); lo in bits 0-15
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 // Epilogue shared by both kernels.  acc[j][i][r] holds
 //   m = m0 + wm*128 + i*32 + (lane & 31),  n = n0 + wn*64 + j*32 + 8*(r/4) + 4*(lane >> 5) + r%4.
 // Instantiated once per activation so that each copy unrolls completely.
@@ -146,12 +155,16 @@ static constexpr int G_STG_WAVE_BYTES = 128 * G_STG_PITCH; // 18 KiB per wave
 
 // WJ = MFMA tiles along n per wave: 2 (8 waves as 2 x 4, wave tile 128 x 64) or 4
 // (4 waves as 2 x 2, wave tile 128 x 128).
-template <int ES, bool EDGE, int ACT, bool STAGED, int WJ = 2>
+// LDSP (whole-tile kernels): the tile's 256 column parameters were laid out in LDS when the kernel started
+// (colp[0..255] bias as f32, -0.0 when there is none; [256..511] scale; [512..767] comp * colsum as s32), so a
+// lane fetches its four columns with one ds_read_b128 per array instead of scalar global loads behind a wait.
+template <int ES, bool EDGE, int ACT, bool STAGED, int WJ = 2, bool LDSP = false>
 __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[WJ][4],
                                                   int64_t m0, int64_t n0, int wm, int wn, int l32, int lh,
-                                                  char *stg) {
+                                                  char *stg, const float *colp = nullptr) {
   constexpr int PITCH = 64 * WJ + 16; // staging row: 32*WJ bf16 + 16 bytes of padding
-  const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
+  const int out_dt = STAGED ? (int)DT_BF16 : p.out_dt; // only bf16 results are staged
+  const int out_es = out_dt == DT_BF16 ? 2 : 4;
   char *Cb = reinterpret_cast<char *>(p.C);
   static_for<0, WJ>([&](auto jc) {
     constexpr int j = decltype(jc)::value;
@@ -159,18 +172,30 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
       constexpr int q = decltype(qc)::value;
       const int64_t n = n0 + wn * (32 * WJ) + j * 32 + 8 * q + 4 * lh;
       float bias4[4] = {0.f, 0.f, 0.f, 0.f}, scale4[4] = {1.f, 1.f, 1.f, 1.f};
-      int cs4[4] = {0, 0, 0, 0};
+      int cs4[4] = {0, 0, 0, 0}; // comp * colsum
+      if constexpr (LDSP) {
+        const int col = wn * (32 * WJ) + j * 32 + 8 * q + 4 * lh;
+        const f32x4_t b = *reinterpret_cast<const f32x4_t *>(colp + col);
+        bias4[0] = b[0], bias4[1] = b[1], bias4[2] = b[2], bias4[3] = b[3];
+        if (ES == 1) {
+          const f32x4_t sc = *reinterpret_cast<const f32x4_t *>(colp + 256 + col);
+          const i32x4_t cs = *reinterpret_cast<const i32x4_t *>(colp + 512 + col);
+          scale4[0] = sc[0], scale4[1] = sc[1], scale4[2] = sc[2], scale4[3] = sc[3];
+          cs4[0] = cs[0], cs4[1] = cs[1], cs4[2] = cs[2], cs4[3] = cs[3];
+        }
+      } else {
 #pragma unroll
-      for (int e = 0; e < 4; e++) {
-        if (!EDGE || n + e < p.N) {
-          if (p.bias)
-            bias4[e] = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n + e])
-                                            : reinterpret_cast<const float *>(p.bias)[n + e];
-          if (ES == 1) {
-            if (p.scale)
-              scale4[e] = p.scale[n + e];
-            if (p.colsum)
-              cs4[e] = p.colsum[n + e];
+        for (int e = 0; e < 4; e++) {
+          if (!EDGE || n + e < p.N) {
+            if (p.bias)
+              bias4[e] = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n + e])
+                                              : reinterpret_cast<const float *>(p.bias)[n + e];
+            if (ES == 1) {
+              if (p.scale)
+                scale4[e] = p.scale[n + e];
+              if (p.colsum)
+                cs4[e] = p.comp * p.colsum[n + e];
+            }
           }
         }
       }
@@ -181,6 +206,7 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
           return;
         uint32_t o32[4];
         uint16_t o16[4];
+        float xf[4] = {0.f, 0.f, 0.f, 0.f};
         float res4[4] = {0.f, 0.f, 0.f, 0.f};
         if (ES == 2 && p.residual) {
           const int64_t at = m * p.ldr + n;
@@ -206,22 +232,30 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
           if (ES == 1) {
             // s32 accumulator of (a ^ 0x80) * w; comp restores / applies the
             // zero-point term in exact integer arithmetic.
-            int c = (int)acc[j][i][4 * q + e] + p.comp * cs4[e];
-            if (p.out_dt == DT_S32) {
+            int c = (int)acc[j][i][4 * q + e] + cs4[e];
+            if (out_dt == DT_S32) {
               o32[e] = (uint32_t)c;
               o16[e] = 0;
             } else {
-              float x = (float)c * scale4[e];
-              if (p.bias)
-                x = x + bias4[e];
+              float x;
+              if constexpr (LDSP) { // an absent bias is -0.0: the fused multiply-add then equals the product
+                x = fmaf((float)c, scale4[e], bias4[e]);
+              } else {
+                x = (float)c * scale4[e];
+                if (p.bias)
+                  x = x + bias4[e];
+              }
               x = act_const<ACT>(x);
               o32[e] = __float_as_uint(x);
-              o16[e] = f32_to_bf16_bits(x);
+              if constexpr (LDSP && STAGED)
+                xf[e] = x; // converted in pairs below
+              else
+                o16[e] = f32_to_bf16_bits(x);
             }
           } else {
             float x = (float)acc[j][i][4 * q + e];
             const float r = res4[e];
-            if (p.out_dt == DT_BF16) {
+            if (out_dt == DT_BF16) {
               // bf16 graph: round after the matmul and after every bf16 op
               // (lib/gc/Transforms/Pipeline.cpp:79-95)
               x = round_bf16(x);
@@ -247,8 +281,21 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
           }
         }
         if (STAGED) {
-          *reinterpret_cast<uint2 *>(stg + (i * 32 + l32) * PITCH + j * 64 + q * 16 + lh * 8) =
-              make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
+          uint2 packed;
+          if constexpr (LDSP && ES == 1) {
+            // v_cvt_pk_bf16_f32 rounds to nearest even like the scalar routine but keeps a NaN's sign (the
+            // hardware's own invalid-operation NaN is negative), so four values with a NaN among them (their sum
+            // is one; so is the sum of opposite infinities) take the scalar routine: NaN -> 0x7FC0
+            const float any_nan = (xf[0] + xf[1]) + (xf[2] + xf[3]);
+            if (__builtin_expect(any_nan != any_nan, 0))
+              packed = make_uint2(f32_to_bf16_bits(xf[0]) | ((uint32_t)f32_to_bf16_bits(xf[1]) << 16),
+                                  f32_to_bf16_bits(xf[2]) | ((uint32_t)f32_to_bf16_bits(xf[3]) << 16));
+            else
+              packed = make_uint2(pack_bf16x2(xf[0], xf[1]), pack_bf16x2(xf[2], xf[3]));
+          } else {
+            packed = make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
+          }
+          *reinterpret_cast<uint2 *>(stg + (i * 32 + l32) * PITCH + j * 64 + q * 16 + lh * 8) = packed;
           return;
         }
         char *dst = Cb + (m * p.ldc + n) * out_es;
@@ -289,24 +336,25 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
   }
 }
 
-template <int ES, bool EDGE, bool STAGED, int WJ = 2>
+template <int ES, bool EDGE, bool STAGED, int WJ = 2, bool LDSP = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[WJ][4], int64_t m0,
-                                              int64_t n0, int wm, int wn, int l32, int lh, char *stg) {
+                                              int64_t n0, int wm, int wn, int l32, int lh, char *stg,
+                                              const float *colp = nullptr) {
   switch (p.act) {
   case ACT_RELU:
-    gemm_epilogue_act<ES, EDGE, ACT_RELU, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_RELU, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   case ACT_GELU_ERF:
-    gemm_epilogue_act<ES, EDGE, ACT_GELU_ERF, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_ERF, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   case ACT_GELU_TANH:
-    gemm_epilogue_act<ES, EDGE, ACT_GELU_TANH, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_TANH, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   case ACT_SIGMOID:
-    gemm_epilogue_act<ES, EDGE, ACT_SIGMOID, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_SIGMOID, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   default:
-    gemm_epilogue_act<ES, EDGE, ACT_NONE, STAGED, WJ>(p, acc, m0, n0, wm, wn, l32, lh, stg);
+    gemm_epilogue_act<ES, EDGE, ACT_NONE, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   }
 }
@@ -615,7 +663,11 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
   typedef typename FG::acc_t acc_t;
   constexpr int NST = FG::NST;
   // ring of NST stages (128 KiB); the epilogue reuses the whole array as 8 x 18 KiB staging regions
-  __shared__ __align__(1024) char smem[8 * G_STG_WAVE_BYTES];
+  // behind them the tile's column parameters for the epilogue: bias, scale, comp * colsum (see gemm_epilogue_act).
+  // One array on purpose: with a second LDS variable in the kernel the compiler puts a full vmcnt(0) wait in
+  // front of the fragment reads of every stage (it then treats every LDS read as a reader of the DMA's target).
+  __shared__ __align__(1024) char smem[8 * G_STG_WAVE_BYTES + (SPLIT ? 0 : 3 * G_BN * 4)];
+  float *colp = reinterpret_cast<float *>(smem + 8 * G_STG_WAVE_BYTES);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -708,10 +760,35 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
   const char *b_ptr = reinterpret_cast<const char *>(p.B) + (TB ? n0 * ldb_b : n0 * ES) + (int64_t)g0 * NST * b_step;
 
   uint4 a0[4], b0[WJ], a1[4], b1[WJ];
+  // column parameters of this tile: requested before the operand traffic, written to LDS in front of the
+  // prologue's barrier (which also publishes them to every wave)
+  float cp_bias = -0.0f, cp_scale = 1.0f;
+  int cp_cs = 0;
+  if constexpr (!SPLIT) {
+    if (tid < G_BN) {
+      const int64_t n = n0 + tid;
+      if (p.bias)
+        cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n])
+                                       : reinterpret_cast<const float *>(p.bias)[n];
+      if (ES == 1) {
+        if (p.scale)
+          cp_scale = p.scale[n];
+        if (p.colsum)
+          cp_cs = p.comp * p.colsum[n];
+      }
+    }
+  }
   // prologue: request k-blocks 0 .. NST-2 (KT is a positive multiple of NST), wait for block 0
 #pragma unroll
   for (int d = 0; d < NST - 1; d++)
     g.issue_loads(smem + d * FG::STAGE_BYTES, a_ptr + d * FG::KB, b_ptr + d * b_step);
+  if constexpr (!SPLIT) {
+    if (tid < G_BN) {
+      colp[tid] = cp_bias;
+      colp[G_BN + tid] = cp_scale;
+      reinterpret_cast<int *>(colp)[2 * G_BN + tid] = cp_cs;
+    }
+  }
   FG::template wait_dma<NST - 2>();
   __builtin_amdgcn_s_barrier();
   g.load_frags(smem, 0, a0, b0);
@@ -763,10 +840,12 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
     return; // the sum over slices and the epilogue are the second kernel's (a kernel boundary is the cheapest
             // way to make partial sums visible across XCDs: device-scope fences write back and invalidate whole L2s)
   }
-  if (p.out_dt == DT_BF16)
-    gemm_epilogue<ES, false, true, WJ>(p, acc, m0, n0, wm, wn, l32, lh, smem + wave * (128 * (64 * WJ + 16)));
-  else
-    gemm_epilogue<ES, false, false, WJ>(p, acc, m0, n0, wm, wn, l32, lh, nullptr);
+  if constexpr (!SPLIT) {
+    if (p.out_dt == DT_BF16)
+      gemm_epilogue<ES, false, true, WJ, true>(p, acc, m0, n0, wm, wn, l32, lh, smem + wave * (128 * (64 * WJ + 16)), colp);
+    else
+      gemm_epilogue<ES, false, false, WJ, true>(p, acc, m0, n0, wm, wn, l32, lh, nullptr, colp);
+  }
 }
 
 // Second pass of split-K: out = epilogue(sum over slices of the f32 partials), slices added in ascending

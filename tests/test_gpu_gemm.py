@@ -119,6 +119,38 @@ def test_int8_layer_matches_oracle(gc, orc, dev, M, N, K, act, zp):
     assert_close(yf, outf.cpu().numpy(), 1e-4, "int8 layer f32 out")
 
 
+@pytest.mark.parametrize("act", ["gelu_erf", "relu", None])
+def test_int8_layer_special_scales_and_biases(gc, orc, dev, act):
+    """Whole-tile shape (the kernel that converts to bf16 in pairs): NaNs of either sign and any payload,
+    infinities and overflowing products in scale and bias.  Every NaN of the result is the reference's 0x7FC0
+    (include/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmInterface.h:83-92), infinities keep their sign."""
+    M = N = K = 256
+    torch.manual_seed(0)
+    A = torch.randint(0, 256, (M, K), dtype=torch.int32).to(torch.uint8)
+    torch.manual_seed(1)
+    W = torch.randint(-127, 128, (K, N), dtype=torch.int32).to(torch.int8)
+    sc = (torch.rand(N) * 0.009 + 0.001).numpy()
+    bs = torch.randn(N).numpy()
+    sc_bits, bs_bits = sc.view(np.uint32), bs.view(np.uint32)
+    sc_bits[3], sc_bits[40] = 0xFFC12345, 0x7F800001          # negative quiet NaN with payload, signalling NaN
+    sc[7], sc[64], sc[65], sc[130] = np.inf, -np.inf, 3e38, -3e38
+    bs_bits[9], bs_bits[200] = 0xFFFFFFFF, 0x7FC00001
+    bs[11], bs[12], bs[7], bs[64] = np.inf, -np.inf, -np.inf, np.inf
+    _, y = orc.int8_layer(A.numpy(), W.numpy(), sc, bs, 128, act)
+    Wd = W.to(dev)
+    out = gc.gemm_int8(A.to(dev), Wd, gc.colsum_s8(Wd), 128, torch.from_numpy(sc).to(dev), torch.from_numpy(bs).to(dev),
+                       act, gc.BF16)
+    torch.cuda.synchronize()
+    got = out.view(torch.int16).cpu().numpy().view(np.uint16)
+    want = np.asarray(y).view(np.uint16).reshape(M, N)
+    special = (want & 0x7F80) == 0x7F80
+    assert special.any() and (want[special] == 0x7FC0).any() and (want[special] == 0x7F80).any()
+    bad = special & (got != want)
+    assert not bad.any(), sorted({(int(c), hex(int(g)), hex(int(w))) for c, g, w in
+                                  zip(np.nonzero(bad)[1], got[bad], want[bad])})[:12]
+    assert_close(orc.bf16_to_f32(want[~special]), orc.bf16_to_f32(got[~special]), 1e-2, "finite part")
+
+
 def test_int8_full_size_exact_checksums_and_rows(gc, orc, wl, dev):
     """BASELINE config 3 (4096 x 4096 x 11008).  Exactness of all 45M
     accumulators through integer checksums (row sums and column sums of the
