@@ -655,6 +655,18 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void mha_fwd_fast_kernel(
     }
     __builtin_amdgcn_s_barrier();
   }
+  if constexpr (NW == 8) {
+    // Make the compiler place its wait for the Q loads here.  Their first readers are the MFMAs inside the loop,
+    // and it knows nothing of the hand-written requests above and in the loop: left alone it puts
+    // "s_waitcnt vmcnt(7) .. vmcnt(0)" in front of those MFMAs in every trip, which in the real counter means
+    // "until the K/V blocks requested a moment ago have landed" and takes the ring's lead away.
+#pragma unroll
+    for (int ds = 0; ds < 8; ds++) {
+      i32x4_t t = {(int)qf[ds].x, (int)qf[ds].y, (int)qf[ds].z, (int)qf[ds].w};
+      asm volatile("" : "+v"(t));
+      qf[ds] = make_uint4((uint32_t)t[0], (uint32_t)t[1], (uint32_t)t[2], (uint32_t)t[3]);
+    }
+  }
 
   const float inv_scale = 1.0f / p.scale;
   // One visited key block: request the block NST-1 ahead into the stage that was
