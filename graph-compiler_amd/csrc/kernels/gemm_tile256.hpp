@@ -158,7 +158,10 @@ static constexpr int G_STG_WAVE_BYTES = 128 * G_STG_PITCH; // 18 KiB per wave
 // LDSP (whole-tile kernels): the tile's 256 column parameters were laid out in LDS when the kernel started
 // (colp[0..255] bias as f32, -0.0 when there is none; [256..511] scale; [512..767] comp * colsum as s32), so a
 // lane fetches its four columns with one ds_read_b128 per array instead of scalar global loads behind a wait.
-template <int ES, bool EDGE, int ACT, bool STAGED, int WJ = 2, bool LDSP = false>
+// MI16: the accumulators come from 16x16x32 MFMAs.  acc[j][i] still covers columns j*32.. and rows i*32.. of the wave
+// tile, as four 16 x 16 tiles: elements 4q..4q+3 belong to the tile at columns 16*(q/2), rows 16*(q%2), where a
+// lane holds columns 4*(lane/16)..+3 of row lane%16.
+template <int ES, bool EDGE, int ACT, bool STAGED, int WJ = 2, bool LDSP = false, bool MI16 = false>
 __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[WJ][4],
                                                   int64_t m0, int64_t n0, int wm, int wn, int l32, int lh,
                                                   char *stg, const float *colp = nullptr) {
@@ -170,11 +173,14 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
     constexpr int j = decltype(jc)::value;
     static_for<0, 4>([&](auto qc) {
       constexpr int q = decltype(qc)::value;
-      const int64_t n = n0 + wn * (32 * WJ) + j * 32 + 8 * q + 4 * lh;
+      // this lane's four columns and its row inside the 32 x 32 block (j, i)
+      const int n_off = MI16 ? 16 * (q >> 1) + 4 * (2 * lh + (l32 >> 4)) : 8 * q + 4 * lh;
+      const int m_off = MI16 ? 16 * (q & 1) + (l32 & 15) : l32;
+      const int64_t n = n0 + wn * (32 * WJ) + j * 32 + n_off;
       float bias4[4] = {0.f, 0.f, 0.f, 0.f}, scale4[4] = {1.f, 1.f, 1.f, 1.f};
       int cs4[4] = {0, 0, 0, 0}; // comp * colsum
       if constexpr (LDSP) {
-        const int col = wn * (32 * WJ) + j * 32 + 8 * q + 4 * lh;
+        const int col = wn * (32 * WJ) + j * 32 + n_off;
         const f32x4_t b = *reinterpret_cast<const f32x4_t *>(colp + col);
         bias4[0] = b[0], bias4[1] = b[1], bias4[2] = b[2], bias4[3] = b[3];
         if (ES == 1) {
@@ -201,7 +207,7 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
       }
       static_for<0, 4>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        const int64_t m = m0 + wm * 128 + i * 32 + l32;
+        const int64_t m = m0 + wm * 128 + i * 32 + m_off;
         if (EDGE && m >= p.M)
           return;
         uint32_t o32[4];
@@ -295,7 +301,7 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
           } else {
             packed = make_uint2(o16[0] | ((uint32_t)o16[1] << 16), o16[2] | ((uint32_t)o16[3] << 16));
           }
-          *reinterpret_cast<uint2 *>(stg + (i * 32 + l32) * PITCH + j * 64 + q * 16 + lh * 8) = packed;
+          *reinterpret_cast<uint2 *>(stg + (i * 32 + m_off) * PITCH + (j * 32 + n_off) * 2) = packed;
           return;
         }
         char *dst = Cb + (m * p.ldc + n) * out_es;
@@ -336,25 +342,25 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
   }
 }
 
-template <int ES, bool EDGE, bool STAGED, int WJ = 2, bool LDSP = false>
+template <int ES, bool EDGE, bool STAGED, int WJ = 2, bool LDSP = false, bool MI16 = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, typename MfmaOp<ES>::acc_t (&acc)[WJ][4], int64_t m0,
                                               int64_t n0, int wm, int wn, int l32, int lh, char *stg,
                                               const float *colp = nullptr) {
   switch (p.act) {
   case ACT_RELU:
-    gemm_epilogue_act<ES, EDGE, ACT_RELU, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
+    gemm_epilogue_act<ES, EDGE, ACT_RELU, STAGED, WJ, LDSP, MI16>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   case ACT_GELU_ERF:
-    gemm_epilogue_act<ES, EDGE, ACT_GELU_ERF, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_ERF, STAGED, WJ, LDSP, MI16>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   case ACT_GELU_TANH:
-    gemm_epilogue_act<ES, EDGE, ACT_GELU_TANH, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
+    gemm_epilogue_act<ES, EDGE, ACT_GELU_TANH, STAGED, WJ, LDSP, MI16>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   case ACT_SIGMOID:
-    gemm_epilogue_act<ES, EDGE, ACT_SIGMOID, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
+    gemm_epilogue_act<ES, EDGE, ACT_SIGMOID, STAGED, WJ, LDSP, MI16>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   default:
-    gemm_epilogue_act<ES, EDGE, ACT_NONE, STAGED, WJ, LDSP>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
+    gemm_epilogue_act<ES, EDGE, ACT_NONE, STAGED, WJ, LDSP, MI16>(p, acc, m0, n0, wm, wn, l32, lh, stg, colp);
     break;
   }
 }
@@ -848,6 +854,234 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
   }
 }
 
+// ---------------------------------------------------------------------------
+// The bf16 whole-tile kernel on v_mfma_f32_16x16x32_bf16 (B stored [K,N], no K slices).  Same tile, ring, DMA and
+// epilogue as gemm_tile256_fast_kernel<2, 2, 2>; what differs is the MFMA shape.  The board holds a power limit by
+// lowering the clock, and per multiply-accumulate the 16x16x32 form moves less register-file data (0.25 B of
+// accumulator + 0.25 B of operands against 0.5 B + 0.125 B): a loop of nothing but MFMAs sustains 2.13 PFLOP/s at
+// 2.29 GHz with it and 1.89 PFLOP/s at 2.11 GHz with 32x32x16.
+// One ring stage (64 bytes of K per row) is exactly one k-step of 32.  A wave's 128 x 64 tile is 8 x 4 tiles of
+// 16 x 16; the stage is computed in two halves of 16 MFMAs (row tiles 0-3, then 4-7).  Register fragments: the
+// A tiles of the half being computed and of the half to come (2 x 16 registers) and one set of B tiles (16).
+// First half: read the A tiles of the second half.  Barrier (next stage published).  Second half: read the next
+// stage's first-half A tiles, and each B tile as soon as its last MFMA of this stage has been issued.
+#ifndef G_FAST_MI16
+#define G_FAST_MI16 1
+#endif
+template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_kernel(GemmParams p) {
+  static_assert(ES == 2, "bf16 only");
+  typedef FastGemm<2, 2, 2, false, false> FG;
+  constexpr int NST = FG::NST;
+  // one array: the ring / epilogue staging, then the column parameters (see gemm_tile256_fast_kernel)
+  __shared__ __align__(1024) char smem[8 * G_STG_WAVE_BYTES + 3 * G_BN * 4];
+  float *colp = reinterpret_cast<float *>(smem + 8 * G_STG_WAVE_BYTES);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int l32 = lane & 31, lh = lane >> 5;
+  const int r16 = lane & 15, g16 = lane >> 4;
+
+  const int tiles_m = (int)(p.M / G_BM), tiles_n = (int)(p.N / G_BN);
+  int tm, tn;
+  tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
+  const int64_t m0 = (int64_t)tm * G_BM, n0 = (int64_t)tn * G_BN;
+  const int64_t lda_b = p.lda * 2, ldb_b = p.ldb * 2;
+  {
+    const int64_t bz = blockIdx.y; // strided batch
+    p.A = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * 2;
+    p.B = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * 2;
+    p.C = reinterpret_cast<char *>(p.C) + bz * p.c_bs * (p.out_dt == DT_BF16 ? 2 : 4);
+    if (p.residual)
+      p.residual = reinterpret_cast<const char *>(p.residual) + bz * p.c_bs * (p.residual_dt == DT_BF16 ? 2 : 4);
+  }
+
+  FG g;
+  g.wave_u = wave;
+  g.a_xor = 0;
+#pragma unroll
+  for (int i = 0; i < FG::NDMA; i++) { // as in gemm_tile256_fast_kernel
+    const int row = (wave * FG::NDMA + i) * FG::A_ROWS_PER_DMA + lane / FG::A_CPR;
+    const int c = (lane % FG::A_CPR) ^ FG::a_swz(row);
+    g.a_src[i] = (uint32_t)(row * lda_b + c * 16);
+    const int krow = (wave * FG::NDMA + i) * FG::B_ROWS_PER_DMA + lane / FG::B_CPR;
+    const int cb = (lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW);
+    g.b_src[i] = (uint32_t)(krow * ldb_b + cb * 16);
+  }
+  // A tile `it` (16 rows): lane -> row lane%16, k 8*(lane/16)..+7 = logical 16-byte chunk lane/16 of the row
+  const int row_a = wm * 128 + r16; // + 16*it: leaves the swizzle unchanged
+  const uint32_t a_ld = (uint32_t)(row_a * FG::KB + ((g16 ^ FG::a_swz(row_a)) << 4));
+  // B tile `jt` (16 columns): the 16 lanes of a group hand the transposing read a 4 (k) x 16 (n) block, lane ->
+  // k row lane%16/4, columns 4*(lane%4)..+3, and get back column lane%16 of those 4 k rows; group lane/16 takes
+  // k rows 8*(lane/16)..+3 and, 2048 bytes (4 k rows) on, ..+7
+  uint32_t b_ld[4];
+  {
+    const int kk = r16 >> 2, cc = r16 & 3;
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++) {
+      const int chunk = (wn * 4 + jt) * 2 + (cc >> 1);
+      b_ld[jt] = (uint32_t)(FG::A_BYTES + (8 * g16 + kk) * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + (cc & 1) * 8);
+    }
+  }
+
+  f32x4_t acc4[2][4][4]; // [j][i][q]: the 16 x 16 tile at columns 16*(q/2), rows 16*(q%2) of the 32 x 32 block (j, i)
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        acc4[j][i][q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int64_t b_step = (int64_t)FG::BK * ldb_b;
+  const int KT = (int)(p.K / FG::BK); // a positive multiple of NST (checked by the launcher)
+  const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b;
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * 2;
+
+  uint4 a_lo[4], a_hi[4], bb[4];
+  auto load_a = [&](const char *__restrict__ st, int half, uint4(&a)[4]) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ii++)
+      a[ii] = *reinterpret_cast<const uint4 *>(st + a_ld + (half * 4 + ii) * (16 * FG::KB));
+  };
+  auto load_b = [&](const char *__restrict__ st, uint4(&b)[4]) {
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++) {
+      const uint2 lo = MfmaOp<2>::tr_read(st + b_ld[jt]);
+      const uint2 hi = MfmaOp<2>::tr_read(st + b_ld[jt] + 4 * FG::B_ROW_BYTES);
+      b[jt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+    }
+  };
+  // 16 MFMAs: row tiles 4*HALF..+3 against the 4 column tiles; operand roles swapped as in the 32x32 kernels
+  // (first operand = B fragment), so a lane ends up with 4 consecutive columns of one row
+  auto mfma_half = [&](auto halfc, auto jt0c, auto jt1c, const uint4(&a)[4], const uint4(&b)[4]) {
+    constexpr int HALF = decltype(halfc)::value, JT0 = decltype(jt0c)::value, JT1 = decltype(jt1c)::value;
+    static_for<JT0, JT1>([&](auto jtc) {
+      constexpr int jt = decltype(jtc)::value;
+      static_for<0, 4>([&](auto iic) {
+        constexpr int it = HALF * 4 + decltype(iic)::value;
+        constexpr int j = jt >> 1, i = it >> 1, q = 2 * (jt & 1) + (it & 1);
+        acc4[j][i][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b[jt]),
+                                                                __builtin_bit_cast(bf16x8_t, a[it & 3]), acc4[j][i][q], 0, 0, 0);
+      });
+    });
+  };
+  // MFMA, two LDS reads, MFMA, two LDS reads ... until the group's reads are out, then the remaining MFMAs
+  auto hint = [&](auto ndsc, auto nmc) {
+    constexpr int N_DS = decltype(ndsc)::value, N_MFMA = decltype(nmc)::value;
+    static_for<0, N_MFMA>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      constexpr int left = N_DS - 2 * i;
+      if constexpr (left > 0)
+        __builtin_amdgcn_sched_group_barrier(0x100, left < 2 ? left : 2, 0);
+    });
+  };
+  // One stage (see FastGemm::stage for the ring).  MFMAs run column tile by column tile; a column tile's B fragment
+  // is dead after its four MFMAs of the second half and is reloaded from the next stage on the spot, so B needs one
+  // set of registers.
+  auto stage = [&](auto has_fill, auto has_next, auto behindc, char *__restrict__ cur, char *__restrict__ nxt,
+                   char *__restrict__ fill, const char *a_fill, const char *b_fill) {
+    constexpr bool HAS_FILL = decltype(has_fill)::value, HAS_NEXT = decltype(has_next)::value;
+    constexpr int BEHIND = decltype(behindc)::value;
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+    typedef std::integral_constant<int, 3> I3;
+    typedef std::integral_constant<int, 4> I4;
+    if constexpr (HAS_FILL)
+      g.issue_loads(fill, a_fill, b_fill);
+    load_a(cur, 1, a_hi);
+    mfma_half(I0{}, I0{}, I3{}, a_lo, bb); // 12 of the first half's 16
+    hint(I4{}, std::integral_constant<int, 12>{});
+    // The barrier sits three quarters into the first half: the reads above have returned by then (its wait covers
+    // them), and the four MFMAs left over cover the barrier's own latency.  Nothing may move across it.
+    __builtin_amdgcn_sched_barrier(0);
+    FG::template wait_dma<BEHIND>();
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_half(I0{}, I3{}, I4{}, a_lo, bb); // the last readers of a_lo
+    if constexpr (HAS_NEXT)
+      load_a(nxt, 0, a_lo);
+    static_for<0, 4>([&](auto jtc) {
+      constexpr int jt = decltype(jtc)::value;
+      mfma_half(I1{}, jtc, std::integral_constant<int, jt + 1>{}, a_hi, bb);
+      if constexpr (HAS_NEXT) {
+        const uint2 lo = MfmaOp<2>::tr_read(nxt + b_ld[jt]);
+        const uint2 hi = MfmaOp<2>::tr_read(nxt + b_ld[jt] + 4 * FG::B_ROW_BYTES);
+        bb[jt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+    });
+    // issue order after the barrier: the four MFMAs left of the first half; the next stage's first-half A tiles
+    // between the MFMAs of column tile 0; after each column tile its B fragment of the next stage
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    static_for<0, 4>([&](auto ic) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if constexpr (HAS_NEXT)
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    });
+    static_for<0, 4>([&](auto jtc) {
+      if constexpr (decltype(jtc)::value > 0)
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      if constexpr (HAS_NEXT)
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    });
+  };
+
+  // column parameters of this tile (see gemm_tile256_fast_kernel)
+  float cp_bias = -0.0f;
+  if (tid < G_BN && p.bias)
+    cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n0 + tid])
+                                   : reinterpret_cast<const float *>(p.bias)[n0 + tid];
+#pragma unroll
+  for (int d = 0; d < NST - 1; d++)
+    g.issue_loads(smem + d * FG::STAGE_BYTES, a_ptr + d * FG::KB, b_ptr + d * b_step);
+  if (tid < G_BN)
+    colp[tid] = cp_bias;
+  FG::template wait_dma<NST - 2>();
+  __builtin_amdgcn_s_barrier();
+  load_a(smem, 0, a_lo);
+  load_b(smem, bb);
+
+  typedef std::integral_constant<bool, true> T;
+  typedef std::integral_constant<bool, false> F;
+  int kt0 = 0;
+  for (; kt0 + 2 * NST <= KT; kt0 += NST) {
+    static_for<0, NST>([&](auto sc) {
+      constexpr int st = decltype(sc)::value;
+      constexpr int cur = st, nxt = (st + 1) % NST, fill = (st + NST - 1) % NST;
+      const int kf = kt0 + st + NST - 1;
+      stage(T{}, T{}, std::integral_constant<int, NST - 2>{}, smem + cur * FG::STAGE_BYTES, smem + nxt * FG::STAGE_BYTES, smem + fill * FG::STAGE_BYTES,
+            a_ptr + (int64_t)kf * FG::KB, b_ptr + kf * b_step);
+    });
+  }
+  static_for<0, NST>([&](auto sc) { // last group: only its first stage requests a block; the ring drains
+    constexpr int st = decltype(sc)::value;
+    constexpr int cur = st, nxt = (st + 1) % NST, fill = (st + NST - 1) % NST;
+    constexpr int behind = NST - 2 - st > 0 ? NST - 2 - st : 0;
+    const int kf = kt0 + st + NST - 1;
+    stage(std::integral_constant<bool, st == 0>{}, std::integral_constant<bool, (st < NST - 1)>{},
+          std::integral_constant<int, behind>{}, smem + cur * FG::STAGE_BYTES,
+          smem + nxt * FG::STAGE_BYTES, smem + fill * FG::STAGE_BYTES, a_ptr + (int64_t)kf * FG::KB, b_ptr + kf * b_step);
+  });
+
+  // the accumulators in the shape the epilogue takes: element 4q+e of block (j, i)
+  f32x16_t acc[2][4];
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          acc[j][i][4 * q + e] = acc4[j][i][q][e];
+  if (p.out_dt == DT_BF16)
+    gemm_epilogue<2, false, true, 2, true, true>(p, acc, m0, n0, wm, wn, l32, lh, smem + wave * G_STG_WAVE_BYTES, colp);
+  else
+    gemm_epilogue<2, false, false, 2, true, true>(p, acc, m0, n0, wm, wn, l32, lh, nullptr, colp);
+}
+
 // Second pass of split-K: out = epilogue(sum over slices of the f32 partials), slices added in ascending
 // order (deterministic), the same rounding points as the fused epilogue.  One thread per 4 columns; the
 // loads of eight slices are in flight together.
@@ -1012,6 +1246,12 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
                            stream, p);
       else
         hipLaunchKernelGGL((gemm_tile256_kernel<ES, true, true>), grid, block, 0, stream, p);
+      return hipGetLastError() == hipSuccess ? 0 : 5;
+    }
+  }
+  if constexpr (ES == 2) {
+    if (fast && G_FAST_MI16) {
+      hipLaunchKernelGGL(gemm_tile256_mi16_kernel<ES>, grid, dim3(512), 0, stream, p);
       return hipGetLastError() == hipSuccess ? 0 : 5;
     }
   }
