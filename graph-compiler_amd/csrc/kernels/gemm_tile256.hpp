@@ -855,8 +855,8 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
 }
 
 // ---------------------------------------------------------------------------
-// The bf16 whole-tile kernel on v_mfma_f32_16x16x32_bf16 (B stored [K,N], no K slices).  Same tile, ring, DMA and
-// epilogue as gemm_tile256_fast_kernel<2, 2, 2>; what differs is the MFMA shape.  The board holds a power limit by
+// The whole-tile kernel on v_mfma_f32_16x16x32_bf16 / v_mfma_i32_16x16x64_i8 (B stored [K,N], no K slices).  Same
+// tile, ring, DMA and epilogue as gemm_tile256_fast_kernel<ES, 2, 2>; what differs is the MFMA shape.  The board holds a power limit by
 // lowering the clock, and per multiply-accumulate the 16x16x32 form moves less register-file data (0.25 B of
 // accumulator + 0.25 B of operands against 0.5 B + 0.125 B): a loop of nothing but MFMAs sustains 2.13 PFLOP/s at
 // 2.29 GHz with it and 1.89 PFLOP/s at 2.11 GHz with 32x32x16.
@@ -869,8 +869,8 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
 #define G_FAST_MI16 1
 #endif
 template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_kernel(GemmParams p) {
-  static_assert(ES == 2, "bf16 only");
-  typedef FastGemm<2, 2, 2, false, false> FG;
+  typedef FastGemm<ES, 2, 2, false, false> FG;
+  typedef typename std::conditional<ES == 2, f32x4_t, i32x4_t>::type acc4_t;
   constexpr int NST = FG::NST;
   // one array: the ring / epilogue staging, then the column parameters (see gemm_tile256_fast_kernel)
   __shared__ __align__(1024) char smem[8 * G_STG_WAVE_BYTES + 3 * G_BN * 4];
@@ -887,11 +887,11 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
   int tm, tn;
   tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
   const int64_t m0 = (int64_t)tm * G_BM, n0 = (int64_t)tn * G_BN;
-  const int64_t lda_b = p.lda * 2, ldb_b = p.ldb * 2;
+  const int64_t lda_b = p.lda * ES, ldb_b = p.ldb * ES;
   {
     const int64_t bz = blockIdx.y; // strided batch
-    p.A = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * 2;
-    p.B = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * 2;
+    p.A = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * ES;
+    p.B = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * ES;
     p.C = reinterpret_cast<char *>(p.C) + bz * p.c_bs * (p.out_dt == DT_BF16 ? 2 : 4);
     if (p.residual)
       p.residual = reinterpret_cast<const char *>(p.residual) + bz * p.c_bs * (p.residual_dt == DT_BF16 ? 2 : 4);
@@ -899,7 +899,7 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
 
   FG g;
   g.wave_u = wave;
-  g.a_xor = 0;
+  g.a_xor = p.a_xor;
 #pragma unroll
   for (int i = 0; i < FG::NDMA; i++) { // as in gemm_tile256_fast_kernel
     const int row = (wave * FG::NDMA + i) * FG::A_ROWS_PER_DMA + lane / FG::A_CPR;
@@ -909,47 +909,55 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
     const int cb = (lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW);
     g.b_src[i] = (uint32_t)(krow * ldb_b + cb * 16);
   }
-  // A tile `it` (16 rows): lane -> row lane%16, k 8*(lane/16)..+7 = logical 16-byte chunk lane/16 of the row
+  // A tile `it` (16 rows): lane -> row lane%16, logical 16-byte chunk lane/16 of the row's 64 bytes (8 bf16 or
+  // 16 int8 of k)
   const int row_a = wm * 128 + r16; // + 16*it: leaves the swizzle unchanged
   const uint32_t a_ld = (uint32_t)(row_a * FG::KB + ((g16 ^ FG::a_swz(row_a)) << 4));
-  // B tile `jt` (16 columns): the 16 lanes of a group hand the transposing read a 4 (k) x 16 (n) block, lane ->
-  // k row lane%16/4, columns 4*(lane%4)..+3, and get back column lane%16 of those 4 k rows; group lane/16 takes
-  // k rows 8*(lane/16)..+3 and, 2048 bytes (4 k rows) on, ..+7
+  // B tile `jt` (16 columns): the 16 lanes of a group hand the transposing read an RG (k) x 16 (n) block of 8-byte
+  // pieces (bf16: k row lane%16/4, columns 4*(lane%4)..+3; int8: k row lane%16/2, columns 8*(lane%2)..+7) and get
+  // back column lane%16 of those RG k rows; group lane/16 takes k rows 2*RG*(lane/16)..+RG-1 and, 2048 bytes (RG
+  // k rows) on, the RG after them
   uint32_t b_ld[4];
   {
-    const int kk = r16 >> 2, cc = r16 & 3;
+    const int kk = ES == 2 ? (r16 >> 2) : (r16 >> 1);
+    const int cc = ES == 2 ? (r16 & 3) : (r16 & 1);
 #pragma unroll
     for (int jt = 0; jt < 4; jt++) {
-      const int chunk = (wn * 4 + jt) * 2 + (cc >> 1);
-      b_ld[jt] = (uint32_t)(FG::A_BYTES + (8 * g16 + kk) * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + (cc & 1) * 8);
+      const int chunk = ES == 2 ? (wn * 4 + jt) * 2 + (cc >> 1) : (wn * 4 + jt);
+      const int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
+      b_ld[jt] = (uint32_t)(FG::A_BYTES + (2 * FG::RG * g16 + kk) * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + sub);
     }
   }
 
-  f32x4_t acc4[2][4][4]; // [j][i][q]: the 16 x 16 tile at columns 16*(q/2), rows 16*(q%2) of the 32 x 32 block (j, i)
+  acc4_t acc4[2][4][4]; // [j][i][q]: the 16 x 16 tile at columns 16*(q/2), rows 16*(q%2) of the 32 x 32 block (j, i)
 #pragma unroll
   for (int j = 0; j < 2; j++)
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
       for (int q = 0; q < 4; q++)
-        acc4[j][i][q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        acc4[j][i][q] = acc4_t{0, 0, 0, 0};
 
   const int64_t b_step = (int64_t)FG::BK * ldb_b;
   const int KT = (int)(p.K / FG::BK); // a positive multiple of NST (checked by the launcher)
   const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b;
-  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * 2;
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * ES;
 
   uint4 a_lo[4], a_hi[4], bb[4];
   auto load_a = [&](const char *__restrict__ st, int half, uint4(&a)[4]) {
 #pragma unroll
-    for (int ii = 0; ii < 4; ii++)
-      a[ii] = *reinterpret_cast<const uint4 *>(st + a_ld + (half * 4 + ii) * (16 * FG::KB));
+    for (int ii = 0; ii < 4; ii++) {
+      uint4 v = *reinterpret_cast<const uint4 *>(st + a_ld + (half * 4 + ii) * (16 * FG::KB));
+      if (ES == 1) // u8 activations: a - 128 as s8 == a ^ 0x80
+        v = make_uint4(v.x ^ g.a_xor, v.y ^ g.a_xor, v.z ^ g.a_xor, v.w ^ g.a_xor);
+      a[ii] = v;
+    }
   };
   auto load_b = [&](const char *__restrict__ st, uint4(&b)[4]) {
 #pragma unroll
     for (int jt = 0; jt < 4; jt++) {
-      const uint2 lo = MfmaOp<2>::tr_read(st + b_ld[jt]);
-      const uint2 hi = MfmaOp<2>::tr_read(st + b_ld[jt] + 4 * FG::B_ROW_BYTES);
+      const uint2 lo = MfmaOp<ES>::tr_read(st + b_ld[jt]);
+      const uint2 hi = MfmaOp<ES>::tr_read(st + b_ld[jt] + FG::RG * FG::B_ROW_BYTES);
       b[jt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
     }
   };
@@ -962,8 +970,12 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
       static_for<0, 4>([&](auto iic) {
         constexpr int it = HALF * 4 + decltype(iic)::value;
         constexpr int j = jt >> 1, i = it >> 1, q = 2 * (jt & 1) + (it & 1);
-        acc4[j][i][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b[jt]),
-                                                                __builtin_bit_cast(bf16x8_t, a[it & 3]), acc4[j][i][q], 0, 0, 0);
+        if constexpr (ES == 2)
+          acc4[j][i][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b[jt]),
+                                                                  __builtin_bit_cast(bf16x8_t, a[it & 3]), acc4[j][i][q], 0, 0, 0);
+        else
+          acc4[j][i][q] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4_t, b[jt]),
+                                                                __builtin_bit_cast(i32x4_t, a[it & 3]), acc4[j][i][q], 0, 0, 0);
       });
     });
   };
@@ -1007,8 +1019,8 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
       constexpr int jt = decltype(jtc)::value;
       mfma_half(I1{}, jtc, std::integral_constant<int, jt + 1>{}, a_hi, bb);
       if constexpr (HAS_NEXT) {
-        const uint2 lo = MfmaOp<2>::tr_read(nxt + b_ld[jt]);
-        const uint2 hi = MfmaOp<2>::tr_read(nxt + b_ld[jt] + 4 * FG::B_ROW_BYTES);
+        const uint2 lo = MfmaOp<ES>::tr_read(nxt + b_ld[jt]);
+        const uint2 hi = MfmaOp<ES>::tr_read(nxt + b_ld[jt] + FG::RG * FG::B_ROW_BYTES);
         bb[jt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
       }
     });
@@ -1029,15 +1041,27 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
   };
 
   // column parameters of this tile (see gemm_tile256_fast_kernel)
-  float cp_bias = -0.0f;
-  if (tid < G_BN && p.bias)
-    cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n0 + tid])
-                                   : reinterpret_cast<const float *>(p.bias)[n0 + tid];
+  float cp_bias = -0.0f, cp_scale = 1.0f;
+  int cp_cs = 0;
+  if (tid < G_BN) {
+    if (p.bias)
+      cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n0 + tid])
+                                     : reinterpret_cast<const float *>(p.bias)[n0 + tid];
+    if (ES == 1) {
+      if (p.scale)
+        cp_scale = p.scale[n0 + tid];
+      if (p.colsum)
+        cp_cs = p.comp * p.colsum[n0 + tid];
+    }
+  }
 #pragma unroll
   for (int d = 0; d < NST - 1; d++)
     g.issue_loads(smem + d * FG::STAGE_BYTES, a_ptr + d * FG::KB, b_ptr + d * b_step);
-  if (tid < G_BN)
+  if (tid < G_BN) {
     colp[tid] = cp_bias;
+    colp[G_BN + tid] = cp_scale;
+    reinterpret_cast<int *>(colp)[2 * G_BN + tid] = cp_cs;
+  }
   FG::template wait_dma<NST - 2>();
   __builtin_amdgcn_s_barrier();
   load_a(smem, 0, a_lo);
@@ -1066,7 +1090,7 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
   });
 
   // the accumulators in the shape the epilogue takes: element 4q+e of block (j, i)
-  f32x16_t acc[2][4];
+  typename MfmaOp<ES>::acc_t acc[2][4];
 #pragma unroll
   for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -1077,9 +1101,9 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
         for (int e = 0; e < 4; e++)
           acc[j][i][4 * q + e] = acc4[j][i][q][e];
   if (p.out_dt == DT_BF16)
-    gemm_epilogue<2, false, true, 2, true, true>(p, acc, m0, n0, wm, wn, l32, lh, smem + wave * G_STG_WAVE_BYTES, colp);
+    gemm_epilogue<ES, false, true, 2, true, true>(p, acc, m0, n0, wm, wn, l32, lh, smem + wave * G_STG_WAVE_BYTES, colp);
   else
-    gemm_epilogue<2, false, false, 2, true, true>(p, acc, m0, n0, wm, wn, l32, lh, nullptr, colp);
+    gemm_epilogue<ES, false, false, 2, true, true>(p, acc, m0, n0, wm, wn, l32, lh, nullptr, colp);
 }
 
 // Second pass of split-K: out = epilogue(sum over slices of the f32 partials), slices added in ascending
@@ -1249,11 +1273,9 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
       return hipGetLastError() == hipSuccess ? 0 : 5;
     }
   }
-  if constexpr (ES == 2) {
-    if (fast && G_FAST_MI16) {
-      hipLaunchKernelGGL(gemm_tile256_mi16_kernel<ES>, grid, dim3(512), 0, stream, p);
-      return hipGetLastError() == hipSuccess ? 0 : 5;
-    }
+  if (fast && G_FAST_MI16) {
+    hipLaunchKernelGGL(gemm_tile256_mi16_kernel<ES>, grid, dim3(512), 0, stream, p);
+    return hipGetLastError() == hipSuccess ? 0 : 5;
   }
   if (fast)
     hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ>), grid, dim3(1024 / G_FAST_WJ), 0, stream, p);
