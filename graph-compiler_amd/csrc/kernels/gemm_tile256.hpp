@@ -868,8 +868,13 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
 #ifndef G_FAST_MI16
 #define G_FAST_MI16 1
 #endif
-template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_kernel(GemmParams p) {
-  typedef FastGemm<ES, 2, 2, false, false> FG;
+#ifndef G_MI16_SPLIT
+#define G_MI16_SPLIT 3
+#endif
+// TB: B stored [N,K]; its tile is staged and read like the A tile (plain 16-byte fragment reads).
+template <int ES, bool TB = false> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_kernel(GemmParams p) {
+  static_assert(!TB || ES == 2, "B stored [N,K]: bf16 only");
+  typedef FastGemm<ES, 2, 2, false, TB> FG;
   typedef typename std::conditional<ES == 2, f32x4_t, i32x4_t>::type acc4_t;
   constexpr int NST = FG::NST;
   // one array: the ring / epilogue staging, then the column parameters (see gemm_tile256_fast_kernel)
@@ -907,7 +912,7 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
     g.a_src[i] = (uint32_t)(row * lda_b + c * 16);
     const int krow = (wave * FG::NDMA + i) * FG::B_ROWS_PER_DMA + lane / FG::B_CPR;
     const int cb = (lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW);
-    g.b_src[i] = (uint32_t)(krow * ldb_b + cb * 16);
+    g.b_src[i] = TB ? (uint32_t)(row * ldb_b + c * 16) : (uint32_t)(krow * ldb_b + cb * 16);
   }
   // A tile `it` (16 rows): lane -> row lane%16, logical 16-byte chunk lane/16 of the row's 64 bytes (8 bf16 or
   // 16 int8 of k)
@@ -926,6 +931,10 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
       const int chunk = ES == 2 ? (wn * 4 + jt) * 2 + (cc >> 1) : (wn * 4 + jt);
       const int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
       b_ld[jt] = (uint32_t)(FG::A_BYTES + (2 * FG::RG * g16 + kk) * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + sub);
+      if (TB) { // row of the [N,K] tile = column of C; chunk and swizzle as for A
+        const int row_b = wn * 64 + jt * 16 + r16;
+        b_ld[jt] = (uint32_t)(FG::A_BYTES + row_b * FG::KB + ((g16 ^ FG::a_swz(row_b)) << 4));
+      }
     }
   }
 
@@ -938,10 +947,10 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
       for (int q = 0; q < 4; q++)
         acc4[j][i][q] = acc4_t{0, 0, 0, 0};
 
-  const int64_t b_step = (int64_t)FG::BK * ldb_b;
+  const int64_t b_step = TB ? (int64_t)FG::KB : (int64_t)FG::BK * ldb_b;
   const int KT = (int)(p.K / FG::BK); // a positive multiple of NST (checked by the launcher)
   const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b;
-  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * ES;
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + (TB ? n0 * ldb_b : n0 * ES);
 
   uint4 a_lo[4], a_hi[4], bb[4];
   auto load_a = [&](const char *__restrict__ st, int half, uint4(&a)[4]) {
@@ -953,13 +962,19 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
       a[ii] = v;
     }
   };
-  auto load_b = [&](const char *__restrict__ st, uint4(&b)[4]) {
-#pragma unroll
-    for (int jt = 0; jt < 4; jt++) {
+  auto load_b_tile = [&](const char *__restrict__ st, int jt) -> uint4 {
+    if constexpr (TB) {
+      return *reinterpret_cast<const uint4 *>(st + b_ld[jt]);
+    } else {
       const uint2 lo = MfmaOp<ES>::tr_read(st + b_ld[jt]);
       const uint2 hi = MfmaOp<ES>::tr_read(st + b_ld[jt] + FG::RG * FG::B_ROW_BYTES);
-      b[jt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      return make_uint4(lo.x, lo.y, hi.x, hi.y);
     }
+  };
+  auto load_b = [&](const char *__restrict__ st, uint4(&b)[4]) {
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++)
+      b[jt] = load_b_tile(st, jt);
   };
   // 16 MFMAs: row tiles 4*HALF..+3 against the 4 column tiles; operand roles swapped as in the 32x32 kernels
   // (first operand = B fragment), so a lane ends up with 4 consecutive columns of one row
@@ -999,13 +1014,13 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
     constexpr int BEHIND = decltype(behindc)::value;
     typedef std::integral_constant<int, 0> I0;
     typedef std::integral_constant<int, 1> I1;
-    typedef std::integral_constant<int, 3> I3;
+    typedef std::integral_constant<int, G_MI16_SPLIT> I3; // column tiles of the first half in front of the barrier
     typedef std::integral_constant<int, 4> I4;
     if constexpr (HAS_FILL)
       g.issue_loads(fill, a_fill, b_fill);
     load_a(cur, 1, a_hi);
     mfma_half(I0{}, I0{}, I3{}, a_lo, bb); // 12 of the first half's 16
-    hint(I4{}, std::integral_constant<int, 12>{});
+    hint(I4{}, std::integral_constant<int, 4 * G_MI16_SPLIT>{});
     // The barrier sits three quarters into the first half: the reads above have returned by then (its wait covers
     // them), and the four MFMAs left over cover the barrier's own latency.  Nothing may move across it.
     __builtin_amdgcn_sched_barrier(0);
@@ -1018,15 +1033,13 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
     static_for<0, 4>([&](auto jtc) {
       constexpr int jt = decltype(jtc)::value;
       mfma_half(I1{}, jtc, std::integral_constant<int, jt + 1>{}, a_hi, bb);
-      if constexpr (HAS_NEXT) {
-        const uint2 lo = MfmaOp<ES>::tr_read(nxt + b_ld[jt]);
-        const uint2 hi = MfmaOp<ES>::tr_read(nxt + b_ld[jt] + FG::RG * FG::B_ROW_BYTES);
-        bb[jt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
-      }
+      if constexpr (HAS_NEXT)
+        bb[jt] = load_b_tile(nxt, jt);
     });
     // issue order after the barrier: the four MFMAs left of the first half; the next stage's first-half A tiles
     // between the MFMAs of column tile 0; after each column tile its B fragment of the next stage
-    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    if constexpr (G_MI16_SPLIT < 4)
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * (4 - G_MI16_SPLIT), 0);
     static_for<0, 4>([&](auto ic) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       if constexpr (HAS_NEXT)
@@ -1036,7 +1049,7 @@ template <int ES> __global__ __launch_bounds__(512, 1) void gemm_tile256_mi16_ke
       if constexpr (decltype(jtc)::value > 0)
         __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
       if constexpr (HAS_NEXT)
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, TB ? 1 : 2, 0);
     });
   };
 
@@ -1265,7 +1278,9 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   dim3 grid((unsigned)nblk, (unsigned)nbatch), block(G_THREADS);
   if constexpr (ES == 2) {
     if (p.trans_b) {
-      if (fast)
+      if (fast && G_FAST_MI16)
+        hipLaunchKernelGGL((gemm_tile256_mi16_kernel<ES, true>), grid, dim3(512), 0, stream, p);
+      else if (fast)
         hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, false, true>), grid, dim3(1024 / G_FAST_WJ), 0,
                            stream, p);
       else
