@@ -863,8 +863,8 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
 // One ring stage (64 bytes of K per row) is exactly one k-step of 32.  A wave's 128 x 64 tile is 8 x 4 tiles of
 // 16 x 16; the stage is computed in two halves of 16 MFMAs (row tiles 0-3, then 4-7).  Register fragments: the
 // A tiles of the half being computed and of the half to come (2 x 16 registers) and one set of B tiles (16).
-// First half: read the A tiles of the second half.  Barrier (next stage published).  Second half: read the next
-// stage's first-half A tiles, and each B tile as soon as its last MFMA of this stage has been issued.
+// First half: read the A tiles of the second half (and B tile 3).  Barrier (next stage published).  Second half:
+// read the next stage's first-half A tiles, and B tiles 0-2 as soon as their last MFMAs of this stage are issued.
 #ifndef G_FAST_MI16
 #define G_FAST_MI16 1
 #endif
@@ -1019,8 +1019,11 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(512, 1) void gem
     if constexpr (HAS_FILL)
       g.issue_loads(fill, a_fill, b_fill);
     load_a(cur, 1, a_hi);
+    // the last column tile's B fragment is first read behind the barrier: fetched here rather than at the very end
+    // of the previous stage, where the (full) LDS wait in front of this half would have to sit it out
+    bb[3] = load_b_tile(cur, 3);
     mfma_half(I0{}, I0{}, I3{}, a_lo, bb); // 12 of the first half's 16
-    hint(I4{}, std::integral_constant<int, 4 * G_MI16_SPLIT>{});
+    hint(std::integral_constant<int, TB ? 5 : 6>{}, std::integral_constant<int, 4 * G_MI16_SPLIT>{});
     // The barrier sits three quarters into the first half: the reads above have returned by then (its wait covers
     // them), and the four MFMAs left over cover the barrier's own latency.  Nothing may move across it.
     __builtin_amdgcn_sched_barrier(0);
@@ -1033,7 +1036,7 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(512, 1) void gem
     static_for<0, 4>([&](auto jtc) {
       constexpr int jt = decltype(jtc)::value;
       mfma_half(I1{}, jtc, std::integral_constant<int, jt + 1>{}, a_hi, bb);
-      if constexpr (HAS_NEXT)
+      if constexpr (HAS_NEXT && jt < 3)
         bb[jt] = load_b_tile(nxt, jt);
     });
     // issue order after the barrier: the four MFMAs left of the first half; the next stage's first-half A tiles
@@ -1048,7 +1051,7 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(512, 1) void gem
     static_for<0, 4>([&](auto jtc) {
       if constexpr (decltype(jtc)::value > 0)
         __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-      if constexpr (HAS_NEXT)
+      if constexpr (HAS_NEXT && decltype(jtc)::value < 3)
         __builtin_amdgcn_sched_group_barrier(0x100, TB ? 1 : 2, 0);
     });
   };
