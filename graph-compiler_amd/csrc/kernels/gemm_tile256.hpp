@@ -233,6 +233,52 @@ __device__ __forceinline__ void gemm_epilogue_act(const GemmParams &p, typename 
                                                    : reinterpret_cast<const float *>(p.residual)[at + e];
           }
         }
+        if constexpr (ES == 2 && LDSP && STAGED) {
+          // bf16 graph, whole tiles: the same rounding points as below (after the matmul and after every bf16 op,
+          // lib/gc/Transforms/Pipeline.cpp:79-95), rounded in pairs by v_cvt_pk_bf16_f32.  A NaN stays a NaN
+          // through the ops that follow, so only the last conversion has to give it the reference's 0x7FC0.
+          float x[4] = {(float)acc[j][i][4 * q], (float)acc[j][i][4 * q + 1], (float)acc[j][i][4 * q + 2],
+                        (float)acc[j][i][4 * q + 3]};
+          uint32_t p0, p1;
+          auto rnd = [&]() {
+            p0 = pack_bf16x2(x[0], x[1]), p1 = pack_bf16x2(x[2], x[3]);
+            x[0] = __uint_as_float(p0 << 16), x[1] = __uint_as_float(p0 & 0xffff0000u);
+            x[2] = __uint_as_float(p1 << 16), x[3] = __uint_as_float(p1 & 0xffff0000u);
+          };
+          rnd();
+          if (p.bias) {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              x[e] = x[e] + bias4[e];
+            rnd();
+          }
+          if (ACT != ACT_NONE) {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              x[e] = act_const<ACT>(x[e]);
+            if (ACT == ACT_RELU) { // max(x, 0) of a bf16 value is a bf16 value: nothing to round
+              p0 = (__float_as_uint(x[0]) >> 16) | (__float_as_uint(x[1]) & 0xffff0000u);
+              p1 = (__float_as_uint(x[2]) >> 16) | (__float_as_uint(x[3]) & 0xffff0000u);
+            } else {
+              rnd();
+            }
+          }
+          if (p.residual) {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              x[e] = x[e] + res4[e];
+            rnd();
+          }
+          const float any_nan = (x[0] + x[1]) + (x[2] + x[3]); // a NaN if one of them is (or opposite infinities)
+          if (__builtin_expect(any_nan != any_nan, 0)) {
+            if (x[0] != x[0]) p0 = (p0 & 0xffff0000u) | 0x7FC0u;
+            if (x[1] != x[1]) p0 = (p0 & 0x0000ffffu) | 0x7FC00000u;
+            if (x[2] != x[2]) p1 = (p1 & 0xffff0000u) | 0x7FC0u;
+            if (x[3] != x[3]) p1 = (p1 & 0x0000ffffu) | 0x7FC00000u;
+          }
+          *reinterpret_cast<uint2 *>(stg + (i * 32 + m_off) * PITCH + (j * 32 + n_off) * 2) = make_uint2(p0, p1);
+          return;
+        }
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           if (ES == 1) {

@@ -35,6 +35,39 @@ def test_bf16_gemm_matches_oracle(gc, orc, wl, dev, M, N, K, epi):
     assert_close(ref, out.float().cpu().numpy(), rtol, "bf16 %dx%dx%d %s" % (M, N, K, epi), mag=mm)
 
 
+@pytest.mark.parametrize("epi", ["none", "bias", "bias_relu", "gelu"])
+def test_bf16_gemm_special_values_whole_tiles(gc, orc, wl, dev, epi):
+    """Whole tiles (the kernel that rounds to bf16 in pairs): NaNs of either sign in A, infinities in A and in the
+    bias.  Where the reference has a NaN the result is its 0x7FC0
+    (include/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmInterface.h:83-92), infinities agree bit for bit."""
+    M, N, K = 256, 512, 256
+    torch.manual_seed(0)
+    A = wl.bf16_bits((torch.randn(M, K) * 0.5).to(torch.bfloat16)).copy()
+    torch.manual_seed(1)
+    B = (torch.randn(K, N) * 0.5).to(torch.bfloat16)
+    A[3, 5], A[40, 7], A[41, 0] = 0xFFC1, 0x7FC0, 0x7F81       # NaNs: negative with payload, canonical, signalling
+    A[100, 9], A[101, 9] = 0x7F80, 0xFF80                      # +inf, -inf: whole rows of +-inf
+    A[102, 1], A[102, 2] = 0x7F80, 0xFF80                      # both in one row: inf - inf
+    bias = None
+    if "bias" in epi:
+        torch.manual_seed(2)
+        bias = wl.bf16_bits(torch.randn(N).to(torch.bfloat16)).copy()
+        bias[17], bias[18], bias[300] = 0x7F80, 0xFF80, 0xFFFF
+    act = {"none": None, "bias": None, "bias_relu": "relu", "gelu": "gelu_erf"}[epi]
+    want = np.asarray(orc.matmul_bf16(A, wl.bf16_bits(B), bias, act)).view(np.uint16).reshape(M, N)
+    At = torch.from_numpy(A.view(np.int16)).view(torch.bfloat16)
+    bt = None if bias is None else torch.from_numpy(bias.view(np.int16)).view(torch.bfloat16).to(dev)
+    out = gc.gemm_bf16(At.to(dev), B.to(dev), bt, act)
+    torch.cuda.synchronize()
+    got = out.view(torch.int16).cpu().numpy().view(np.uint16)
+    special = (want & 0x7F80) == 0x7F80
+    assert (want[special] == 0x7FC0).any() and (want[special] != 0x7FC0).any()
+    bad = special & (got != want)
+    assert not bad.any(), sorted({(int(r), int(c), hex(int(g)), hex(int(w))) for r, c, g, w in
+                                  zip(*np.nonzero(bad), got[bad], want[bad])})[:12]
+    assert_close(orc.bf16_to_f32(want[~special]), orc.bf16_to_f32(got[~special]), 2e-2, "finite part")
+
+
 def test_bf16_gemm_f32_out_and_strided_operands(gc, orc, wl, dev):
     M, N, K = 260, 264, 200
     torch.manual_seed(0)
