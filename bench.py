@@ -83,9 +83,9 @@ def time_launches(torch, fn, nsets, steps, warmup):
 # --copy-calibration: a 1 GiB copy reads FETCH_SIZE = 524304 KiB (scale 2.0)
 # and WRITE_SIZE = 1048580 KiB (scale 1.0).
 TRAFFIC = {
-    "gemm": int((98556.8 * 2.0 + 32782.2) * 1024),    # algorithmic 64 MiB read + 32 MiB written
-    "int8": int((144087.1 * 2.0 + 88144.0) * 1024),   # algorithmic 59 MiB read + 86 MiB written
-    "mha": int((154703.8 * 2.0 + 65806.9) * 1024),    # algorithmic 208 MiB read + 64 MiB written (default mode)
+    "gemm": int((98541.8 * 2.0 + 32791.1) * 1024),    # algorithmic 64 MiB read + 32 MiB written
+    "int8": int((144003.5 * 2.0 + 88175.4) * 1024),   # algorithmic 59 MiB read + 86 MiB written
+    "mha": int((129697.3 * 2.0 + 65681.9) * 1024),    # algorithmic 208 MiB read + 64 MiB written (default mode)
 }
 
 
