@@ -184,6 +184,7 @@ Executable::Executable(Graph g, bool dry) : g_(std::move(g)) { init(dry); }
 void Executable::init(bool dry) {
   verify_graph(g_);
   plan();
+  plan_workspaces();
   layout_arena();
   if (dry)
     return;
@@ -194,6 +195,22 @@ void Executable::init(bool dry) {
       hip_check(hipMemcpy(arena_ + s.offset, s.init.data(), s.init.size(), hipMemcpyHostToDevice), "upload constants");
   ptr_.resize(slots_.size());
   build_generated_kernels();
+}
+
+// Scratch of the steps whose kernels need some (partial sums of K-sliced GEMMs, mask tile classes of attention): a
+// slot of the step's own, alive for that step only, so it shares arena space with other temporaries.  Nothing is
+// shared between executables or streams: two executables may run side by side, as the reference's may
+// (thread-local scratch, lib/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmOnednn.cpp:70).
+void Executable::plan_workspaces() {
+  for (Step &s : steps_) {
+    size_t bytes = 0;
+    if (s.kind == Step::GemmBf16 && s.batch <= 1)
+      bytes = gcmi_gemm_bf16_workspace_bytes(s.M, s.N, s.K, s.tb ? 1 : 0);
+    else if (s.kind == Step::Mha && s.mask >= 0)
+      bytes = gcmi_mha_fwd_workspace_bytes(s.Sq, s.Sk, s.D, 1);
+    if (bytes)
+      s.ws = new_slot(bytes);
+  }
 }
 
 // One allocation per executable, temporaries with disjoint lifetimes share memory: the tick-based merge
@@ -214,7 +231,7 @@ void Executable::layout_arena() {
   };
   for (int i = 0; i < (int)steps_.size(); i++) {
     const Step &s = steps_[i];
-    for (int slot : {s.a, s.b, s.c, s.out, s.bias, s.mask, s.aux, s.scale_slot, s.scales_slot, s.zps_slot})
+    for (int slot : {s.a, s.b, s.c, s.out, s.bias, s.mask, s.aux, s.ws, s.scale_slot, s.scales_slot, s.zps_slot})
       touch(slot, i);
     for (int slot : s.f_in)
       touch(slot, i);
@@ -264,6 +281,8 @@ void Executable::layout_arena() {
 }
 
 Executable::~Executable() {
+  if (once_done_)
+    (void)hipEventDestroy(once_done_);
   if (stream_)
     (void)hipStreamDestroy(stream_);
   if (arena_)
@@ -1418,11 +1437,11 @@ void Executable::launch(const Step &s) {
     break;
   case Step::GemmBf16:
     // s.c: the residual tensor (same shape as the result), s.b_dt its type
-    gc_check(gcmi_gemm_bf16_residual(P(s.a) + s.a_off * 2, P(s.b) + s.b_off * 2,
-                                     P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4), s.batch, s.M, s.N, s.K, s.lda,
-                                     s.ldb, s.ldc, s.a_bs, s.b_bs, s.c_bs, s.tb ? 1 : 0, P(s.bias),
-                                     s.bias_dt ? s.bias_dt : GCMI_BF16, s.act, P(s.c), s.N, s.b_dt ? s.b_dt : GCMI_BF16,
-                                     s.out_dt, stream_),
+    gc_check(gcmi_gemm_bf16_ws(P(s.a) + s.a_off * 2, P(s.b) + s.b_off * 2,
+                               P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4), s.batch, s.M, s.N, s.K, s.lda, s.ldb,
+                               s.ldc, s.a_bs, s.b_bs, s.c_bs, s.tb ? 1 : 0, P(s.bias), s.bias_dt ? s.bias_dt : GCMI_BF16,
+                               s.act, P(s.c), s.N, s.b_dt ? s.b_dt : GCMI_BF16, s.out_dt, P(s.ws),
+                               s.ws >= 0 ? slots_[(size_t)s.ws].bytes : 0, stream_),
              "MatMul bf16");
     break;
   case Step::ColSum:
@@ -1449,8 +1468,8 @@ void Executable::launch(const Step &s) {
       memcpy(&v, &raw, 4);
       scale = s.scale_div ? 1.0f / v : v;
     }
-    gc_check(gcmi_mha_fwd_bf16(P(s.a), P(s.b), P(s.c), (const float *)P(s.mask), s.mask_ld, P(s.out), s.BH, s.Sq, s.Sk, s.D,
-                               scale, stream_),
+    gc_check(gcmi_mha_fwd_bf16_ws(P(s.a), P(s.b), P(s.c), (const float *)P(s.mask), s.mask_ld, P(s.out), s.BH, s.Sq, s.Sk,
+                                  s.D, scale, 1, P(s.ws), s.ws >= 0 ? slots_[(size_t)s.ws].bytes : 0, stream_),
              "attention");
     break;
   }
@@ -1544,6 +1563,7 @@ void Executable::launch(const Step &s) {
 
 // src/dnnl/dnnl_graph_compiler.cpp:64-103
 void Executable::execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs) {
+  std::lock_guard<std::mutex> turn(run_mu_); // held until the stream has drained: the arena is this call's
   run(inputs, outputs, true);
 }
 
@@ -1551,6 +1571,11 @@ void Executable::execute(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler
 // waited for.  The executable's arena holds the intermediates, so calls on one executable must follow one another on
 // one stream (or be ordered by the caller), and host buffers cannot take part.
 void Executable::execute_async(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_tensor *outputs, hipStream_t stream) {
+  for (const Step &s : steps_)
+    if (s.kind == Step::Mha && s.scale_slot >= 0)
+      throw std::invalid_argument("execute_async: the attention scale of this partition is a tensor that has to be read "
+                                  "back to the host (a wait); use execute, or give the scale as a constant");
+  std::lock_guard<std::mutex> turn(run_mu_);
   struct Swap {
     hipStream_t &slot, saved;
     Swap(hipStream_t &s, hipStream_t v) : slot(s), saved(s) { slot = v; }
@@ -1619,18 +1644,32 @@ void Executable::run(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_ten
   }
   if (step_done_.size() < steps_.size())
     step_done_.resize(steps_.size(), 0);
+  // what an earlier call computed once (steps over constant tensors, column sums of constant weights) may still be
+  // in flight on that call's stream
+  if (once_recorded_ && once_stream_ != stream_)
+    hip_check(hipStreamWaitEvent(stream_, once_done_, 0), "wait for constant results");
   for (size_t i = 0; i < steps_.size(); i++) {
     if (steps_[i].once && step_done_[i])
       continue;
+    const bool keeps = steps_[i].once || (steps_[i].kind == Step::ColSum && steps_[i].op == 1 && !colsum_valid_[steps_[i].out]);
     launch(steps_[i]);
     step_done_[i] = steps_[i].once;
+    if (keeps) { // record behind the last of them (re-recorded per step: cheap, and only in the first calls)
+      if (!once_done_)
+        hip_check(hipEventCreateWithFlags(&once_done_, hipEventDisableTiming), "hipEventCreate");
+      hip_check(hipEventRecord(once_done_, stream_), "hipEventRecord");
+      once_recorded_ = true, once_stream_ = stream_;
+    }
   }
   for (auto &cb : copy_back) {
     hipMemcpyKind kind = is_device_pointer(cb.first) ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost;
     hip_check(hipMemcpyAsync(cb.first, ptr_[(size_t)cb.second], slots_[(size_t)cb.second].bytes, kind, stream_), "copy result");
   }
-  if (wait)
+  if (wait) {
     hip_check(hipStreamSynchronize(stream_), "execute");
+    if (once_stream_ == stream_)
+      once_recorded_ = false; // those results are final now: nobody has to wait for them again
+  }
 }
 
 std::string Executable::describe() const {

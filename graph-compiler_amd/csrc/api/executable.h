@@ -17,6 +17,7 @@
 
 #include <cstdint>
 #include <map>
+#include <mutex>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -33,6 +34,7 @@ struct Step {
   bool once = false; // depends on constant tensors only: runs in the first execute, its result is kept
   // operands are arena slot indices (-1 = none)
   int a = -1, b = -1, c = -1, out = -1, bias = -1, mask = -1, aux = -1;
+  int ws = -1; // scratch of this step alone (partial sums of a K-sliced GEMM, mask tile classes of attention)
   int64_t M = 0, N = 0, K = 0, lda = 0, ldb = 0, ldc = 0;
   int64_t a_off = 0, b_off = 0, out_off = 0; // element offsets (batched fallbacks)
   int64_t batch = 1, a_bs = 0, b_bs = 0, c_bs = 0; // strided batch in one launch (0 stride: shared operand)
@@ -115,7 +117,14 @@ private:
   std::vector<Step> steps_;
   std::vector<Slot> slots_;
   std::unordered_map<size_t, int> slot_of_tensor_;
-  std::vector<void *> ptr_; // per-slot device pointer during execute
+  std::vector<void *> ptr_; // per-slot device pointer during execute (guarded by run_mu_)
+  // execute() may be called from several host threads (the reference's execute is const and re-entrant,
+  // src/dnnl/dnnl_graph_compiler.cpp:214-226): calls on one executable take turns, since they share its arena
+  std::mutex run_mu_;
+  // results of once-only steps: computed on the stream of the first call, waited for by calls on other streams
+  hipEvent_t once_done_ = nullptr;
+  hipStream_t once_stream_ = nullptr;
+  bool once_recorded_ = false;
   char *arena_ = nullptr;
   size_t arena_bytes_ = 0;
   size_t arena_bytes_no_reuse_ = 0; // what one region per slot would take
@@ -130,6 +139,7 @@ private:
   int const_slot(const void *data, size_t bytes);
   void init(bool dry);
   void plan();
+  void plan_workspaces();
   void layout_arena();
   void plan_generic(const Op &op);
   void plan_fusion(std::vector<bool> &skip, const std::vector<bool> &claimed, std::map<size_t, std::vector<Step>> &emit_at,

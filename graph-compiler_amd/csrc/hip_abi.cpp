@@ -1,7 +1,8 @@
 // The thin C-ABI layer between host code and the HIP kernels: argument
 // validation, parameter-block assembly, launches.  This and the kernels' own
 // launch stubs are the only translation units that touch the HIP runtime for
-// compute; nothing here allocates device memory.
+// compute.  Device memory is allocated in one place only: the library workspace of the entry points that take no
+// workspace argument (LibraryWorkspace below).
 #include <hip/hip_runtime_api.h>
 
 #include <cstdarg>
@@ -26,6 +27,8 @@ int gcmi_launch_brgemm(const void *A, const void *B, void *C, int64_t M, int64_t
                        int64_t LDB, int64_t LDC, int64_t stride_a, int64_t stride_b, int num, int beta_zero, int dtA,
                        int dtB, hipStream_t stream);
 int gcmi_launch_mha_fwd(const MhaParams *p, hipStream_t stream);
+int64_t gcmi_launch_gemm_bf16_workspace(const GemmParams *p);
+int64_t gcmi_launch_mha_workspace(const MhaParams *p);
 }
 
 namespace {
@@ -47,6 +50,64 @@ int launched(int rc, const char *what) {
 
 extern "C" const char *gcmi_last_error(void) { return g_err; }
 
+namespace {
+// Where a call's scratch (partial sums of K-sliced GEMMs, mask tile classes of attention) comes from.
+enum class Ws { Library, Caller };
+
+// Scratch of the entry points that take no workspace argument: one buffer per device, allocated at the first call
+// that needs it and grown on demand.  Every call on the device shares it, so its users are put in order: the mutex
+// is held while a call's kernels are enqueued, an event is recorded behind them, and a call on another stream
+// waits for that event first.
+struct LibraryWorkspace {
+  std::mutex mu;
+  void *ptr = nullptr;
+  size_t cap = 0;
+  hipEvent_t done = nullptr;
+  hipStream_t last = nullptr;
+  bool used = false;
+};
+LibraryWorkspace g_ws[64];
+
+// Takes the device's buffer (at least `bytes`) for one call on `stream`; the lock is held until release().
+int ws_acquire(size_t bytes, hipStream_t stream, LibraryWorkspace **out, void **ptr) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    return fail(ST_RUNTIME, "workspace: no current device");
+  LibraryWorkspace &w = g_ws[dev];
+  w.mu.lock();
+  if (w.cap < bytes) {
+    if (w.ptr) { // kernels of earlier calls may still read it
+      (void)hipDeviceSynchronize();
+      (void)hipFree(w.ptr);
+      w.ptr = nullptr, w.cap = 0, w.used = false;
+    }
+    const size_t want = bytes < ((size_t)8 << 20) ? ((size_t)8 << 20) : bytes;
+    if (hipMalloc(&w.ptr, want) != hipSuccess) {
+      w.ptr = nullptr;
+      w.mu.unlock();
+      return fail(1, "workspace: hipMalloc of %zu bytes failed", want);
+    }
+    w.cap = want;
+  }
+  if (!w.done && hipEventCreateWithFlags(&w.done, hipEventDisableTiming) != hipSuccess) {
+    w.done = nullptr;
+    w.mu.unlock();
+    return fail(ST_RUNTIME, "workspace: hipEventCreate failed");
+  }
+  if (w.used && w.last != stream && hipStreamWaitEvent(stream, w.done, 0) != hipSuccess) {
+    w.mu.unlock();
+    return fail(ST_RUNTIME, "workspace: hipStreamWaitEvent failed");
+  }
+  *out = &w, *ptr = w.ptr;
+  return ST_OK;
+}
+void ws_release(LibraryWorkspace *w, hipStream_t stream) {
+  if (hipEventRecord(w->done, stream) == hipSuccess)
+    w->used = true, w->last = stream;
+  w->mu.unlock();
+}
+} // namespace
+
 extern "C" int gcmi_init(int device) {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess || n <= 0)
@@ -67,7 +128,8 @@ namespace {
 int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream,
                   int64_t batch = 1, int64_t a_bs = 0, int64_t b_bs = 0, int64_t c_bs = 0, const void *residual = nullptr,
-                  int64_t ldr = 0, int residual_dtype = 0);
+                  int64_t ldr = 0, int residual_dtype = 0, Ws ws_from = Ws::Library, void *ws = nullptr,
+                  size_t ws_bytes = 0);
 }
 
 extern "C" int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -125,7 +187,7 @@ namespace {
 int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream,
                   int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs, const void *residual, int64_t ldr,
-                  int residual_dtype) {
+                  int residual_dtype, Ws ws_from, void *ws, size_t ws_bytes) {
   if (M < 0 || N < 0 || K < 0)
     return fail(ST_INVALID, "gemm_bf16: negative size");
   if (M == 0 || N == 0)
@@ -147,9 +209,62 @@ int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M
   p.trans_b = trans_b ? 1 : 0;
   p.batch = batch, p.a_bs = a_bs, p.b_bs = b_bs, p.c_bs = c_bs;
   p.residual = residual, p.ldr = ldr, p.residual_dt = residual_dtype;
-  return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
+  // K-sliced shapes (a short A against wide weights) pass f32 partial sums through a workspace
+  const int64_t want = gcmi_launch_gemm_bf16_workspace(&p);
+  if (want <= 0)
+    return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
+  if (ws_from == Ws::Caller) { // what the caller brought, however little: the launcher cuts fewer slices, or none
+    if (ws && (reinterpret_cast<uintptr_t>(ws) & 15) != 0)
+      return fail(ST_INVALID, "gemm_bf16: workspace is not 16-byte aligned");
+    p.partial = ws_bytes >= 4 ? (float *)ws : nullptr, p.partial_cap = (int64_t)(ws_bytes / 4);
+    return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
+  }
+  LibraryWorkspace *lw = nullptr;
+  void *lp = nullptr;
+  if (int rc = ws_acquire((size_t)want * 4, (hipStream_t)stream, &lw, &lp))
+    return rc;
+  p.partial = (float *)lp, p.partial_cap = want;
+  const int rc = launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
+  ws_release(lw, (hipStream_t)stream);
+  return rc;
 }
 } // namespace
+
+extern "C" size_t gcmi_gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_b) {
+  if (M <= 0 || N <= 0 || K <= 0)
+    return 0;
+  GemmParams p{};
+  // aligned stand-ins: the question is what the shape could use
+  p.A = p.B = (const void *)(uintptr_t)256, p.C = (void *)(uintptr_t)256;
+  p.M = M, p.N = N, p.K = K, p.lda = K, p.ldb = trans_b ? K : N, p.ldc = N;
+  p.bias_dt = GCMI_BF16, p.out_dt = GCMI_BF16, p.trans_b = trans_b ? 1 : 0, p.batch = 1;
+  const int64_t want = gcmi_launch_gemm_bf16_workspace(&p);
+  return want > 0 ? (size_t)want * 4 : 0;
+}
+
+extern "C" int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                 int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b,
+                                 int64_t stride_c, int trans_b, const void *bias, int bias_dtype, int act,
+                                 const void *residual, int64_t ldr, int residual_dtype, int out_dtype, void *workspace,
+                                 size_t workspace_bytes, void *stream) {
+  if (batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0)
+    return fail(ST_INVALID, "gemm_bf16_ws: negative batch count or stride");
+  if (batch == 0)
+    return ST_OK;
+  if (batch > 65535)
+    return fail(ST_UNIMPL, "gemm_bf16_ws: more than 65535 batches in one call");
+  if (batch > 1 && stride_c < (M - 1) * ldc + N)
+    return fail(ST_INVALID, "gemm_bf16_ws: results of different batches would overlap");
+  if (residual) {
+    if (residual_dtype != GCMI_BF16 && residual_dtype != GCMI_F32)
+      return fail(ST_UNIMPL, "gemm_bf16_ws: residual_dtype %d", residual_dtype);
+    if (ldr < N || (batch > 1 && stride_c < (M - 1) * ldr + N))
+      return fail(ST_INVALID, "gemm_bf16_ws: residual rows or batches overlap (ldr %lld)", (long long)ldr);
+  }
+  return gemm_bf16_any(trans_b != 0, A, B, C, M, N, K, lda, ldb, ldc, bias, bias_dtype, act, out_dtype, stream, batch,
+                       stride_a, stride_b, stride_c, residual, ldr, residual_dtype, Ws::Caller, workspace,
+                       workspace_bytes);
+}
 
 extern "C" int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K,
                               int64_t lda, int64_t ldb, int64_t ldc, const int32_t *colsum, int32_t zp_a,
@@ -236,9 +351,39 @@ extern "C" int gcmi_mha_fwd_bf16(const void *Q, const void *K, const void *V, co
   return gcmi_mha_fwd_bf16_opt(Q, K, V, mask, mask_ld, O, BH, Sq, Sk, D, scale, 1, stream);
 }
 
+namespace {
+int mha_any(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld, void *O, int64_t BH,
+            int64_t Sq, int64_t Sk, int64_t D, float scale, int skip_masked, void *stream, Ws ws_from, void *ws,
+            size_t ws_bytes);
+}
+
 extern "C" int gcmi_mha_fwd_bf16_opt(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld,
                                      void *O, int64_t BH, int64_t Sq, int64_t Sk, int64_t D, float scale,
                                      int skip_masked, void *stream) {
+  return mha_any(Q, K, V, mask, mask_ld, O, BH, Sq, Sk, D, scale, skip_masked, stream, Ws::Library, nullptr, 0);
+}
+
+extern "C" int gcmi_mha_fwd_bf16_ws(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld,
+                                    void *O, int64_t BH, int64_t Sq, int64_t Sk, int64_t D, float scale, int skip_masked,
+                                    void *workspace, size_t workspace_bytes, void *stream) {
+  return mha_any(Q, K, V, mask, mask_ld, O, BH, Sq, Sk, D, scale, skip_masked, stream, Ws::Caller, workspace,
+                 workspace_bytes);
+}
+
+extern "C" size_t gcmi_mha_fwd_workspace_bytes(int64_t Sq, int64_t Sk, int64_t D, int has_mask) {
+  if (!has_mask || Sq <= 0 || Sk <= 0 || Sq > 0x7fffffff || Sk > 0x7fffffff)
+    return 0;
+  MhaParams p{};
+  p.mask = (const float *)(uintptr_t)256;
+  p.Sq = (int)Sq, p.Sk = (int)Sk, p.D = (int)D;
+  const int64_t want = gcmi_launch_mha_workspace(&p);
+  return want > 0 ? (size_t)want : 0;
+}
+
+namespace {
+int mha_any(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld, void *O, int64_t BH,
+            int64_t Sq, int64_t Sk, int64_t D, float scale, int skip_masked, void *stream, Ws ws_from, void *ws,
+            size_t ws_bytes) {
   if (BH < 0 || Sq < 0 || Sk < 0)
     return fail(ST_INVALID, "mha_fwd: negative size");
   if (D != 128)
@@ -257,11 +402,25 @@ extern "C" int gcmi_mha_fwd_bf16_opt(const void *Q, const void *K, const void *V
   p.Q = Q, p.K = K, p.V = V, p.O = O, p.mask = mask, p.mask_ld = mask_ld;
   p.BH = (int)BH, p.Sq = (int)Sq, p.Sk = (int)Sk, p.D = (int)D, p.scale = scale;
   p.skip_masked = skip_masked ? 1 : 0;
+  // the classes of the mask's tiles (constant 0, constant -inf, general) go through a small workspace
+  const int64_t want = gcmi_launch_mha_workspace(&p);
+  LibraryWorkspace *lw = nullptr;
+  if (want > 0 && ws_from == Ws::Caller) {
+    p.tile_class = (uint8_t *)ws, p.tile_class_cap = (int64_t)ws_bytes;
+  } else if (want > 0) {
+    void *lp = nullptr;
+    if (int rc = ws_acquire((size_t)want, (hipStream_t)stream, &lw, &lp))
+      return rc;
+    p.tile_class = (uint8_t *)lp, p.tile_class_cap = want;
+  }
   int rc = gcmi_launch_mha_fwd(&p, (hipStream_t)stream);
+  if (lw)
+    ws_release(lw, (hipStream_t)stream);
   if (rc == 2)
     return fail(ST_INVALID, "mha_fwd: Q/K/V/O must be 16-byte aligned");
   return launched(rc, "mha_fwd");
 }
+} // namespace
 
 // ---------------------------------------------------------------------------
 // Microkernel ABI: dispatch-once / execute-many, as the reference's runtime

@@ -276,11 +276,9 @@ template <bool HAS_MASK, bool EDGE> __global__ __launch_bounds__(FA_THREADS, 2) 
 // may be skipped altogether: it contributes exp(-inf) = 0 to every sum and
 // leaves the running maximum unchanged.
 enum : uint8_t { FA_TILE_GENERAL = 0, FA_TILE_ZERO = 1, FA_TILE_NEG_INF = 2 };
+// The classes live in a buffer the caller brings (MhaParams::tile_class, one byte per tile); without one every tile
+// is read from the mask and nothing is skipped.
 static constexpr int FA_MAX_TILES = 1 << 20;
-// Workspace of the classification pass.  One copy per device, shared by all
-// calls on that device: calls on different streams of one device must not
-// overlap (calls on one stream are ordered).
-static __device__ __align__(256) uint8_t fa_tile_class_ws[FA_MAX_TILES];
 
 __global__ __launch_bounds__(64) void mha_classify_mask_kernel(const float *mask, int64_t mask_ld, int n_kb, uint8_t *cls) {
   const int qt = blockIdx.y, kb = blockIdx.x, lane = threadIdx.x;
@@ -727,6 +725,14 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void mha_fwd_fast_kernel(
 
 using namespace gcmi;
 
+// bytes of workspace (MhaParams::tile_class) a masked call of this shape can use; 0: none
+extern "C" int64_t gcmi_launch_mha_workspace(const MhaParams *p) {
+  if (!p->mask || p->D != FA_D || p->Sq <= 0 || p->Sk <= 0 || p->Sq % FA_BQ != 0 || p->Sk % FA_BK != 0)
+    return 0;
+  const int64_t n_qt = p->Sq / 32, n_kb = p->Sk / FA_BK;
+  return (n_qt * n_kb <= FA_MAX_TILES && n_qt <= 65535) ? n_qt * n_kb : 0;
+}
+
 extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
   MhaParams p = *pp;
   if (p.D != FA_D)
@@ -743,13 +749,11 @@ extern "C" int gcmi_launch_mha_fwd(const MhaParams *pp, hipStream_t stream) {
               (!p.mask || (al16(p.mask) && p.mask_ld % 4 == 0));
   if (!(al16(p.Q) && al16(p.K) && al16(p.V) && al16(p.O)))
     return 2; // rows are 256 bytes: a 16-byte aligned base is required
+  uint8_t *const ws = p.tile_class;
   p.tile_class = nullptr;
-  if (p.mask && fast) {
+  if (p.mask && fast && ws) {
     const int64_t n_qt = p.Sq / 32, n_kb = p.Sk / FA_BK;
-    if (n_qt * n_kb <= FA_MAX_TILES && n_qt <= 65535) {
-      uint8_t *ws = nullptr;
-      if (hipGetSymbolAddress((void **)&ws, HIP_SYMBOL(fa_tile_class_ws)) != hipSuccess)
-        return 5;
+    if (n_qt * n_kb <= FA_MAX_TILES && n_qt <= 65535 && n_qt * n_kb <= p.tile_class_cap) {
       hipLaunchKernelGGL(mha_classify_mask_kernel, dim3((unsigned)n_kb, (unsigned)n_qt), dim3(64), 0, stream, p.mask,
                          p.mask_ld, (int)n_kb, ws);
       p.tile_class = ws;

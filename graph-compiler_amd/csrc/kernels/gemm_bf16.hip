@@ -8,3 +8,12 @@ extern "C" int gcmi_launch_gemm_bf16(const gcmi::GemmParams *p, hipStream_t stre
     return rc;
   return gcmi::launch_tile256<2>(p, stream);
 }
+
+// floats of workspace (GemmParams::partial) the launch above would use for this call: 0 when K is not sliced
+extern "C" int64_t gcmi_launch_gemm_bf16_workspace(const gcmi::GemmParams *p) {
+  int64_t want = 0;
+  if (gcmi::launch_skinny_nt(p, nullptr, &want) >= 0)
+    return want;
+  gcmi::launch_tile256<2>(p, nullptr, &want);
+  return want;
+}

@@ -23,7 +23,9 @@ struct GemmParams {
   // and writes its f32 partial sums [M x N] to partial + slice * M * N; a second kernel sums the slices and
   // runs the epilogue
   int32_t splits;        // 0 or 1: off
+  // workspace of the f32 partial sums: brought by the caller (partial_cap floats; without one K is not sliced)
   float *partial;
+  int64_t partial_cap;
   int32_t trans_b;       // bf16 only: B is stored [N,K] (k contiguous), ldb elements between its rows
   // strided batch (bf16 tile kernels): blockIdx.y is the batch index, operands advance by these element strides
   // (0 = the operand is shared by all batches).  batch <= 1: a single GEMM.
@@ -55,8 +57,11 @@ struct MhaParams {
   int64_t mask_ld;
   int32_t BH, Sq, Sk, D;
   float scale;
-  // fast path only: class of every (32 query rows x 64 keys) mask tile, [Sq/32][Sk/64], or null
-  const uint8_t *tile_class;
+  // fast path only: class of every (32 query rows x 64 keys) mask tile, [Sq/32][Sk/64].  The caller brings the
+  // buffer (tile_class_cap bytes); the launcher fills it with a classification pass.  Null: no classes (every tile is
+  // read from the mask, nothing is skipped)
+  uint8_t *tile_class;
+  int64_t tile_class_cap;
   int32_t skip_masked; // 1: tiles whose mask is all -inf are not computed (the result is the same)
 };
 

@@ -163,8 +163,12 @@ template <int MT> __global__ __launch_bounds__(SK_WAVES * 64, 2) void gemm_skinn
 }
 
 // Takes the call when the shape is this kernel's (returns -1 otherwise: the tile kernels handle it).
-static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream) {
+// want != null: nothing is launched; *want receives the floats of workspace this call would use if it had them.
+static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream, int64_t *want = nullptr) {
   GemmParams p = *pp;
+  if (want)
+    *want = 0;
+  const int64_t ws_cap = want ? INT64_MAX : (p.partial ? p.partial_cap : 0);
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
   if (!p.trans_b || p.batch > 1 || p.M < 1 || p.M > 64 || p.N % 32 != 0 || p.K % 64 != 0 || p.K < 256 || !al16(p.A) || !al16(p.B) ||
@@ -183,7 +187,7 @@ static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream) {
   int best = 1;
   double best_score = -1.0;
   for (int s = 1; s <= 16; s++) {
-    if (steps / (s * SK_WAVES) < 2 || (int64_t)s * p.M * p.N > G_SPLITK_WS_FLOATS)
+    if (steps / (s * SK_WAVES) < 2 || (s > 1 && (int64_t)s * p.M * p.N > ws_cap))
       break;
     const double rounds = (double)nblocks * s / (double)n_cu;
     const double fill = rounds / (double)(int64_t)(rounds + 0.999999);
@@ -194,11 +198,11 @@ static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream) {
   }
   if (steps / (best * SK_WAVES) < 2)
     return -1;
-  float *ws = nullptr;
-  if (hipGetSymbolAddress((void **)&ws, HIP_SYMBOL(gemm_splitk_ws)) != hipSuccess)
-    return 5;
+  if (want) {
+    *want = best > 1 ? (int64_t)best * p.M * p.N : 0;
+    return 0;
+  }
   p.splits = best;
-  p.partial = ws;
   const dim3 grid((unsigned)(nblocks * best)), block(SK_WAVES * 64);
   if (mt == 1)
     hipLaunchKernelGGL(gemm_skinny_nt_kernel<1>, grid, block, 0, stream, p);

@@ -32,6 +32,7 @@
 //                                        16-bit, 8 for 8-bit), CW = 16-byte
 //                                        chunks one read touches per row
 #pragma once
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.hpp"
@@ -1168,6 +1169,363 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(512, 1) void gem
     gemm_epilogue<ES, false, false, 2, true, true>(p, acc, m0, n0, wm, wn, l32, lh, nullptr, colp);
 }
 
+// ---------------------------------------------------------------------------
+// The whole-tile kernel with one wave per SIMD: 4 waves as 2 x 2, each owning 128 x 128 of the 256 x 256 tile as
+// 8 x 8 tiles of 16 x 16 (v_mfma_f32_16x16x32_bf16 / v_mfma_i32_16x16x64_i8), 256 accumulator registers.  Against
+// the 8-wave kernel a multiply-accumulate costs a third less LDS read traffic (per k-step a wave reads 8 KiB of A
+// and 8 KiB of B for 64 MFMAs, not 8 + 4 KiB for 32), which is what counts on a board that holds its power limit
+// by lowering the clock.  With a single wave per SIMD nothing hides a stall, so every fragment is fetched a whole
+// stage ahead:
+//   stage s computes k-block s entirely from registers: A tiles in one of two register sets, B tiles in one set;
+//   its MFMAs run column tile by column tile, and between them the wave reads k-block s+1: one A tile per column
+//   tile into the other A set, and the B tile of a column as soon as that column's MFMAs are issued (column 7's
+//   goes to a spare register set, alternating by stage, so it can be fetched early as well).
+// Because a k-block sits in registers for the whole of its stage, its LDS slot is free during the stage: the ring
+// of 4 slots carries k-blocks s+1 .. s+4, and the DMA of block s+4 is issued at the start of stage s, three full
+// stages (about 3000 cycles) before the barrier that publishes it.  One barrier per stage, at its start:
+//   s_waitcnt vmcnt(2 stages) lgkmcnt(0)   own share of block s+1 has landed; own reads of block s have returned
+//   s_barrier                              block s+1 is visible to all; slot s may be overwritten
+// The main loop is assembly text written by gen_gemm_w4_mainloop.py (registers and issue order fixed by hand: the
+// compiler's allocator does not hold 64 accumulator tiles and three fragment sets without copies and spills);
+// set-up and epilogue are the C++ below.
+#include "gemm_w4_mainloop.inc"
+
+// Epilogue of gemm_tile256_w4_kernel.  The main loop's assembly ends by writing the raw accumulators of column
+// tiles 0-3 (the left 64 columns of the wave's 128 x 128) to a wave-private LDS region, 128 rows of 256 bytes at a
+// pitch of 272; a second, small assembly statement does the same for column tiles 4-7 once the first half has been
+// consumed.  What is left for this code is a rolled loop over rows: a lane reads four consecutive columns of a row
+// (16 bytes, 16 lanes per row, 4 rows per instruction), applies the epilogue and stores 8 (bf16) or 16 bytes, so a
+// row leaves as one or two whole 128-byte lines.  Unrolled over the 64 accumulator tiles in place of the loop, the
+// same work was ten times the code, all of it executed once per workgroup and fetched cold: 12 us of a 100 us
+// kernel went into instruction-cache misses.
+static constexpr int W4_DUMP_PITCH = 272;                   // 64 f32 / s32 + 16 bytes: conflict-free for the 16-byte writes
+static constexpr int W4_DUMP_WAVE_BYTES = 128 * W4_DUMP_PITCH; // 34816 per wave, 139264 per workgroup
+
+// Four results of one row: c = the raw accumulators of columns n .. n+3 of row m.  HAS_BIAS / HAS_RES are
+// compile-time so that the eight rows of an unrolled group are straight-line code (their LDS reads go out together).
+template <int ES, int ACT, int OUT, bool HAS_BIAS, bool HAS_RES, typename acc4_t>
+__device__ __forceinline__ void w4_epilogue_row(const GemmParams &p, const acc4_t &c, int64_t m, int64_t n,
+                                                const f32x4_t &bias4, const f32x4_t &scale4, const i32x4_t &cs4) {
+  char *Cb = reinterpret_cast<char *>(p.C);
+  float x[4];
+  uint32_t p0 = 0, p1 = 0; // bf16 results, two per register
+  if constexpr (ES == 1) {
+    int ci[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      ci[e] = (int)c[e] + cs4[e]; // exact: the zero-point term in integer arithmetic
+    if constexpr (OUT == DT_S32) {
+      *reinterpret_cast<i32x4_t *>(Cb + (m * p.ldc + n) * 4) = i32x4_t{ci[0], ci[1], ci[2], ci[3]};
+      return;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      x[e] = act_const<ACT>(fmaf((float)ci[e], scale4[e], bias4[e])); // an absent bias is -0.0: the product itself
+    if constexpr (OUT == DT_F32) {
+      *reinterpret_cast<f32x4_t *>(Cb + (m * p.ldc + n) * 4) = f32x4_t{x[0], x[1], x[2], x[3]};
+      return;
+    }
+    // v_cvt_pk_bf16_f32 rounds to nearest even but keeps a NaN's sign and payload; a NaN among the four (their
+    // sum is one; so is the sum of opposite infinities) sends them through the scalar rule: NaN -> 0x7FC0
+    const float any_nan = (x[0] + x[1]) + (x[2] + x[3]);
+    if (__builtin_expect(any_nan != any_nan, 0)) {
+      p0 = f32_to_bf16_bits(x[0]) | ((uint32_t)f32_to_bf16_bits(x[1]) << 16);
+      p1 = f32_to_bf16_bits(x[2]) | ((uint32_t)f32_to_bf16_bits(x[3]) << 16);
+    } else {
+      p0 = pack_bf16x2(x[0], x[1]), p1 = pack_bf16x2(x[2], x[3]);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      x[e] = (float)c[e];
+    float res4[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (HAS_RES) { // 16-byte aligned rows (checked by the launcher)
+      const int64_t at = m * p.ldr + n;
+      if (p.residual_dt == DT_BF16) {
+        const uint2 v = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.residual) + at);
+        res4[0] = __uint_as_float(v.x << 16), res4[1] = __uint_as_float(v.x & 0xffff0000u);
+        res4[2] = __uint_as_float(v.y << 16), res4[3] = __uint_as_float(v.y & 0xffff0000u);
+      } else {
+        const f32x4_t v = *reinterpret_cast<const f32x4_t *>(reinterpret_cast<const float *>(p.residual) + at);
+        res4[0] = v[0], res4[1] = v[1], res4[2] = v[2], res4[3] = v[3];
+      }
+    }
+    if constexpr (OUT == DT_F32) { // no intermediate rounding
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if constexpr (HAS_BIAS)
+          x[e] = x[e] + bias4[e];
+        x[e] = act_const<ACT>(x[e]);
+        if constexpr (HAS_RES) { // kept apart from the activation's last multiply: the sum equals a separate add
+#pragma clang fp contract(off)
+          x[e] = x[e] + res4[e];
+        }
+      }
+      *reinterpret_cast<f32x4_t *>(Cb + (m * p.ldc + n) * 4) = f32x4_t{x[0], x[1], x[2], x[3]};
+      return;
+    }
+    // bf16 graph: rounded after the matmul and after every bf16 op (lib/gc/Transforms/Pipeline.cpp:79-95), in
+    // pairs.  A NaN stays a NaN through the ops that follow, so only the last conversion gives it 0x7FC0.
+    auto rnd = [&]() {
+      p0 = pack_bf16x2(x[0], x[1]), p1 = pack_bf16x2(x[2], x[3]);
+      x[0] = __uint_as_float(p0 << 16), x[1] = __uint_as_float(p0 & 0xffff0000u);
+      x[2] = __uint_as_float(p1 << 16), x[3] = __uint_as_float(p1 & 0xffff0000u);
+    };
+    constexpr bool LAST_IS_MATMUL = !HAS_BIAS && ACT == ACT_NONE && !HAS_RES;
+    if constexpr (LAST_IS_MATMUL) { // nothing follows the first rounding: no need to widen again
+      p0 = pack_bf16x2(x[0], x[1]), p1 = pack_bf16x2(x[2], x[3]);
+    } else {
+      rnd();
+    }
+    if constexpr (HAS_BIAS) {
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        x[e] = x[e] + bias4[e];
+      rnd();
+    }
+    if constexpr (ACT != ACT_NONE) {
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        x[e] = act_const<ACT>(x[e]);
+      if constexpr (ACT == ACT_RELU) { // max(x, 0) of a bf16 value is a bf16 value: nothing to round
+        p0 = (__float_as_uint(x[0]) >> 16) | (__float_as_uint(x[1]) & 0xffff0000u);
+        p1 = (__float_as_uint(x[2]) >> 16) | (__float_as_uint(x[3]) & 0xffff0000u);
+      } else {
+        rnd();
+      }
+    }
+    if constexpr (HAS_RES) {
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        x[e] = x[e] + res4[e];
+      rnd();
+    }
+    const float any_nan = (x[0] + x[1]) + (x[2] + x[3]);
+    if (__builtin_expect(any_nan != any_nan, 0)) {
+      if (x[0] != x[0]) p0 = (p0 & 0xffff0000u) | 0x7FC0u;
+      if (x[1] != x[1]) p0 = (p0 & 0x0000ffffu) | 0x7FC00000u;
+      if (x[2] != x[2]) p1 = (p1 & 0xffff0000u) | 0x7FC0u;
+      if (x[3] != x[3]) p1 = (p1 & 0x0000ffffu) | 0x7FC00000u;
+    }
+  }
+  typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+  const u32x2_t vv = {p0, p1};
+  __builtin_nontemporal_store(vv, reinterpret_cast<u32x2_t *>(Cb + (m * p.ldc + n) * 2));
+}
+
+// One half (64 columns) of the wave tile.  OUT = DT_BF16 / DT_F32 / DT_S32.
+template <int ES, int ACT, int OUT>
+__device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, int64_t m0, int64_t n0, int wm, int wn,
+                                                 int lane, const char *dump, const float *colp) {
+  typedef typename std::conditional<ES == 2, float, int>::type acc_e;
+  typedef acc_e acc4_t __attribute__((ext_vector_type(4)));
+  const int rr = lane >> 4, cc = lane & 15;
+  const int col = wn * 128 + half * 64 + 4 * cc; // this lane's four columns inside the workgroup tile
+  const int64_t n = n0 + col;
+  const f32x4_t bias4 = *reinterpret_cast<const f32x4_t *>(colp + col); // -0.0 where there is no bias
+  f32x4_t scale4 = {1.f, 1.f, 1.f, 1.f};
+  i32x4_t cs4 = {0, 0, 0, 0}; // comp * colsum
+  if constexpr (ES == 1) {
+    scale4 = *reinterpret_cast<const f32x4_t *>(colp + 256 + col);
+    cs4 = *reinterpret_cast<const i32x4_t *>(colp + 512 + col);
+  }
+  const bool has_bias = ES == 2 && p.bias != nullptr, has_res = ES == 2 && p.residual != nullptr;
+  constexpr int U = 8; // rows in flight per lane
+#pragma unroll 1
+  for (int i0 = 0; i0 < 32; i0 += U) {
+    acc4_t c[U];
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      c[u] = *reinterpret_cast<const acc4_t *>(dump + ((i0 + u) * 4 + rr) * W4_DUMP_PITCH + cc * 16);
+    auto rows = [&](auto hb, auto hr) {
+#pragma unroll
+      for (int u = 0; u < U; u++)
+        w4_epilogue_row<ES, ACT, OUT, decltype(hb)::value, decltype(hr)::value>(
+            p, c[u], m0 + wm * 128 + (i0 + u) * 4 + rr, n, bias4, scale4, cs4);
+    };
+    typedef std::integral_constant<bool, true> T;
+    typedef std::integral_constant<bool, false> F;
+    if constexpr (ES == 1) {
+      rows(F{}, F{});
+    } else {
+      if (has_bias) {
+        if (has_res)
+          rows(T{}, T{});
+        else
+          rows(T{}, F{});
+      } else {
+        if (has_res)
+          rows(F{}, T{});
+        else
+          rows(F{}, F{});
+      }
+    }
+  }
+}
+
+// kind = act + 8 * (0: bf16, 1: f32, 2: s32)
+template <int ES>
+__device__ __forceinline__ void w4_epilogue_half_any(const GemmParams &p, int kind, int half, int64_t m0, int64_t n0,
+                                                     int wm, int wn, int lane, const char *dump, const float *colp) {
+#define GCMI_W4_CASE(ACT, OUT, K)                                                                                     \
+  case (int)ACT + 8 * K:                                                                                              \
+    w4_epilogue_half<ES, ACT, OUT>(p, half, m0, n0, wm, wn, lane, dump, colp);                                        \
+    break;
+  switch (kind) {
+    GCMI_W4_CASE(ACT_RELU, DT_BF16, 0)
+    GCMI_W4_CASE(ACT_GELU_ERF, DT_BF16, 0)
+    GCMI_W4_CASE(ACT_GELU_TANH, DT_BF16, 0)
+    GCMI_W4_CASE(ACT_SIGMOID, DT_BF16, 0)
+    GCMI_W4_CASE(ACT_NONE, DT_F32, 1)
+    GCMI_W4_CASE(ACT_RELU, DT_F32, 1)
+    GCMI_W4_CASE(ACT_GELU_ERF, DT_F32, 1)
+    GCMI_W4_CASE(ACT_GELU_TANH, DT_F32, 1)
+    GCMI_W4_CASE(ACT_SIGMOID, DT_F32, 1)
+    GCMI_W4_CASE(ACT_NONE, DT_S32, 2)
+  default:
+    w4_epilogue_half<ES, ACT_NONE, DT_BF16>(p, half, m0, n0, wm, wn, lane, dump, colp);
+    break;
+  }
+#undef GCMI_W4_CASE
+}
+
+template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gemm_tile256_w4_kernel(GemmParams p) {
+  static_assert(!TB || ES == 2, "B stored [N,K]: bf16 only");
+  typedef FastGemm<ES, 2, 4, false, TB> FG; // 4 waves: 4 DMA instructions per operand, wave and stage
+  static_assert(FG::NST == 4 && FG::NDMA == 4 && FG::STAGE_BYTES == 32768 && FG::A_BYTES == 16384, "the assembly's ring");
+#ifdef GCMI_W4_TIMING
+  const long long wall_entry = wall_clock64();
+  float *const timing_out = p.partial;
+#endif
+  // one array: the ring (128 KiB; the epilogue's 4 x 34 KiB of accumulators afterwards), then the column parameters
+  __shared__ __align__(1024) char smem[8 * G_STG_WAVE_BYTES + 3 * G_BN * 4];
+  static_assert(4 * W4_DUMP_WAVE_BYTES <= 8 * G_STG_WAVE_BYTES, "accumulator regions overlap the column parameters");
+  float *colp = reinterpret_cast<float *>(smem + 8 * G_STG_WAVE_BYTES);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int r16 = lane & 15, g16 = lane >> 4;
+
+  const int tiles_m = (int)(p.M / G_BM), tiles_n = (int)(p.N / G_BN);
+  int tm, tn;
+  tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
+  // integer division runs on the vector unit; the operand addresses below must be in scalar registers
+  tm = __builtin_amdgcn_readfirstlane(tm), tn = __builtin_amdgcn_readfirstlane(tn);
+  const int64_t m0 = (int64_t)tm * G_BM, n0 = (int64_t)tn * G_BN;
+  const int64_t lda_b = p.lda * ES, ldb_b = p.ldb * ES;
+  {
+    const int64_t bz = blockIdx.y; // strided batch
+    p.A = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * ES;
+    p.B = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * ES;
+    p.C = reinterpret_cast<char *>(p.C) + bz * p.c_bs * (p.out_dt == DT_BF16 ? 2 : 4);
+    if (p.residual)
+      p.residual = reinterpret_cast<const char *>(p.residual) + bz * p.c_bs * (p.residual_dt == DT_BF16 ? 2 : 4);
+  }
+
+  // per-lane source offsets of the wave's DMA instructions, as in gemm_tile256_fast_kernel
+  i32x4_t a_off, b_off;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int row = (wave * 4 + i) * FG::A_ROWS_PER_DMA + lane / FG::A_CPR;
+    const int c = (lane % FG::A_CPR) ^ FG::a_swz(row);
+    a_off[i] = (int)(row * lda_b + c * 16);
+    const int krow = (wave * 4 + i) * FG::B_ROWS_PER_DMA + lane / FG::B_CPR;
+    const int cb = (lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW);
+    b_off[i] = TB ? (int)(row * ldb_b + c * 16) : (int)(krow * ldb_b + cb * 16);
+  }
+  // fragment addresses as in gemm_tile256_mi16_kernel: A tile `it` = rows wm*128 + 16*it .., B tile `jt` = columns
+  // wn*128 + 16*jt ..; slots 2 and 3 through a second base (an instruction's offset field has 16 bits)
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(GCMI_LDS char *)smem;
+  typedef int i32x8_t __attribute__((ext_vector_type(8)));
+  i32x2_t a_ld;
+  i32x8_t b_ld0, b_ld2;
+  {
+    const int row_a = wm * 128 + r16;
+    a_ld[0] = (int)(lds0 + row_a * FG::KB + ((g16 ^ FG::a_swz(row_a)) << 4));
+    a_ld[1] = a_ld[0] + 65536;
+    const int kk = ES == 2 ? (r16 >> 2) : (r16 >> 1);
+    const int cc = ES == 2 ? (r16 & 3) : (r16 & 1);
+#pragma unroll
+    for (int jt = 0; jt < 8; jt++) {
+      const int chunk = ES == 2 ? (wn * 8 + jt) * 2 + (cc >> 1) : (wn * 8 + jt);
+      const int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
+      int at = FG::A_BYTES + (2 * FG::RG * g16 + kk) * FG::B_ROW_BYTES + ((chunk ^ (kk * FG::CW)) << 4) + sub;
+      if (TB) {
+        const int row_b = wn * 128 + jt * 16 + r16;
+        at = FG::A_BYTES + row_b * FG::KB + ((g16 ^ FG::a_swz(row_b)) << 4);
+      }
+      b_ld0[jt] = (int)(lds0 + at);
+      b_ld2[jt] = (int)(lds0 + at + 65536);
+    }
+  }
+
+  // column parameters of this tile (see gemm_tile256_fast_kernel): 256 threads, one column each
+  float cp_bias = -0.0f, cp_scale = 1.0f;
+  int cp_cs = 0;
+  if (p.bias)
+    cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n0 + tid])
+                                   : reinterpret_cast<const float *>(p.bias)[n0 + tid];
+  if (ES == 1) {
+    if (p.scale)
+      cp_scale = p.scale[n0 + tid];
+    if (p.colsum)
+      cp_cs = p.comp * p.colsum[n0 + tid];
+  }
+
+  uint64_t a_ptr = (uint64_t)(reinterpret_cast<const char *>(p.A) + m0 * lda_b);
+  uint64_t b_ptr = (uint64_t)(reinterpret_cast<const char *>(p.B) + (TB ? n0 * ldb_b : n0 * ES));
+  uint64_t b_step = TB ? (uint64_t)FG::KB : (uint64_t)(FG::BK * ldb_b);
+  int trips = (int)(p.K / FG::BK) / 4 - 1; // k-blocks: a positive multiple of 4 (checked by the launcher)
+  const uint32_t dma_lds = lds0 + (uint32_t)wave * 4096u;
+  const uint32_t a_xor = p.a_xor;
+  // where this lane writes its accumulators for the epilogue: row lane%16 (+ 16*it), 16-byte chunk lane/16 (+ 4*jt)
+  // of the wave's region
+  const uint32_t dump_ld = lds0 + (uint32_t)wave * W4_DUMP_WAVE_BYTES + (uint32_t)(r16 * W4_DUMP_PITCH + g16 * 16);
+
+#define GCMI_W4_OPERANDS                                                                                              \
+  : "+{s[40:41]}"(a_ptr), "+{s[42:43]}"(b_ptr), "+{s46}"(trips)                                                       \
+  : "{v[0:3]}"(a_off), "{v[4:7]}"(b_off), "{v[8:9]}"(a_ld), "{v[10:17]}"(b_ld0), "{v[18:25]}"(b_ld2),                \
+    "{s[44:45]}"(b_step), "{s47}"(dma_lds), "{s48}"(a_xor), "{v26}"(dump_ld)                                        \
+  : "memory", "scc", "s49", GCMI_W4_CLOBBERS
+#ifdef GCMI_W4_TIMING // measurement builds: core clock cycles and 100 MHz ticks spent in the main loop
+  const long long tick0 = clock64(), wall0 = wall_clock64();
+#endif
+  if constexpr (ES == 1)
+    asm volatile(GCMI_W4_ASM_I8 GCMI_W4_OPERANDS);
+  else if constexpr (TB)
+    asm volatile(GCMI_W4_ASM_BF16_TB GCMI_W4_OPERANDS);
+  else
+    asm volatile(GCMI_W4_ASM_BF16 GCMI_W4_OPERANDS);
+#undef GCMI_W4_OPERANDS
+#ifdef GCMI_W4_TIMING
+  const long long tick1 = clock64(), wall1 = wall_clock64();
+#endif
+  // the column parameters were requested before the main loop and are first needed here
+  colp[tid] = cp_bias;
+  colp[G_BN + tid] = cp_scale;
+  reinterpret_cast<int *>(colp)[2 * G_BN + tid] = cp_cs;
+  __syncthreads();
+
+  const int out_kind = p.out_dt == DT_BF16 ? 0 : ((ES == 1 && p.out_dt == DT_S32) ? 2 : 1);
+  const int kind = (out_kind == 2 ? (int)ACT_NONE : p.act) + 8 * out_kind;
+  const char *dump = smem + wave * W4_DUMP_WAVE_BYTES;
+  w4_epilogue_half_any<ES>(p, kind, 0, m0, n0, wm, wn, lane, dump, colp);
+  // the right half: the accumulators of column tiles 4-7 are still where the main loop left them
+  asm volatile(GCMI_W4_ASM_DUMP_HI : : "{v26}"(dump_ld) : "memory");
+  w4_epilogue_half_any<ES>(p, kind, 1, m0, n0, wm, wn, lane, dump, colp);
+#ifdef GCMI_W4_TIMING
+  const long long wall_issued = wall_clock64();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (timing_out && tid == 0 && blockIdx.x < 256) {
+    long long *t = reinterpret_cast<long long *>(timing_out) + 8 * blockIdx.x;
+    t[0] = tick1 - tick0, t[1] = wall1 - wall0, t[2] = wall0 - wall_entry, t[3] = wall_issued - wall1, t[4] = wall_clock64() - wall_issued;
+    t[5] = wall_entry;
+  }
+#endif
+}
+
 // Second pass of split-K: out = epilogue(sum over slices of the f32 partials), slices added in ascending
 // order (deterministic), the same rounding points as the fused epilogue.  One thread per 4 columns; the
 // loads of eight slices are in flight together.
@@ -1234,11 +1592,6 @@ template <int ACT> __global__ __launch_bounds__(256) void gemm_splitk_reduce_ker
     *reinterpret_cast<f32x4_t *>(reinterpret_cast<float *>(p.C) + m * p.ldc + n) = f32x4_t{o32[0], o32[1], o32[2], o32[3]};
 }
 
-// Workspace of the split-K partial sums.  One copy per device, shared by all calls: calls on different
-// streams of one device must not overlap.
-static constexpr int64_t G_SPLITK_WS_FLOATS = (int64_t)8 << 20; // 32 MiB
-static __device__ __align__(256) float gemm_splitk_ws[G_SPLITK_WS_FLOATS];
-
 // second pass of every K-sliced GEMM: one thread per four outputs, the activation as a template argument
 static void launch_splitk_reduce(const GemmParams &p, hipStream_t stream) {
   const dim3 grid((unsigned)((p.M * (p.N / 4) + 255) / 256)), block(256);
@@ -1262,8 +1615,13 @@ static void launch_splitk_reduce(const GemmParams &p, hipStream_t stream) {
 }
 
 // Host-side launch of the 256x256 tile kernels for one element size.
-template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t stream) {
+// want != null: nothing is launched; *want receives the floats of workspace this call would use if it had them.
+template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *want = nullptr) {
   GemmParams p = *pp;
+  if (want)
+    *want = 0;
+  const int64_t ws_cap = want ? INT64_MAX : (p.partial ? p.partial_cap : 0);
+  float *const ws = p.partial;
   const int tiles_m = (int)((p.M + G_BM - 1) / G_BM), tiles_n = (int)((p.N + G_BN - 1) / G_BN);
   const int64_t nblk = (int64_t)tiles_m * tiles_n;
   if (nblk <= 0 || nblk > 0x7fffffff)
@@ -1302,12 +1660,14 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
     const int groups = (int)(p.K / KGROUP);
     int splits = (n_cu + tiles_n - 1) / tiles_n;
     splits = splits < groups ? splits : groups;
-    while (splits > 1 && (int64_t)splits * p.M * p.N > G_SPLITK_WS_FLOATS)
+    if (want) {
+      if (splits > 1 && tiles_n * 2 <= n_cu)
+        *want = (int64_t)splits * p.M * p.N;
+      return 0;
+    }
+    while (splits > 1 && (int64_t)splits * p.M * p.N > ws_cap)
       splits--;
     if (splits > 1 && tiles_n * 2 <= n_cu) {
-      float *ws = nullptr;
-      if (hipGetSymbolAddress((void **)&ws, HIP_SYMBOL(gemm_splitk_ws)) != hipSuccess)
-        return 5;
       p.splits = splits;
       p.partial = ws;
       if constexpr (ES == 2) {
@@ -1322,9 +1682,23 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
       return hipGetLastError() == hipSuccess ? 0 : 5;
     }
   }
+  if (want)
+    return 0;
   if (p.group_m <= 0)
     p.group_m = 4;
   dim3 grid((unsigned)nblk, (unsigned)nbatch), block(G_THREADS);
+  const char *w4_env = getenv("GCMI_GEMM_W4");
+  const int use_w4 = w4_env ? atoi(w4_env) : 1;
+  if (fast && use_w4 && (ES == 2 || p.out_dt == DT_BF16)) {
+    if constexpr (ES == 2) {
+      if (p.trans_b) {
+        hipLaunchKernelGGL((gemm_tile256_w4_kernel<ES, true>), grid, dim3(256), 0, stream, p);
+        return hipGetLastError() == hipSuccess ? 0 : 5;
+      }
+    }
+    hipLaunchKernelGGL(gemm_tile256_w4_kernel<ES>, grid, dim3(256), 0, stream, p);
+    return hipGetLastError() == hipSuccess ? 0 : 5;
+  }
   if constexpr (ES == 2) {
     if (p.trans_b) {
       if (fast && G_FAST_MI16)

@@ -61,6 +61,37 @@ def bf16_mlp_chain(M=4096, K=4096, H=11008, seed=0):
     return x, W1, W2, b2
 
 
+def benchgc_matmul_fill(name, shape, dtype, dst_dtype, amp):
+    """Default fill of the reference harness's matmul driver
+    (test/benchgc/src/benchgc/arg/matmul.py:104-148): integer-valued data, dense
+    for the source, and for the weight of a density that keeps every sum exactly
+    representable in the result type -- the fill under which its strict
+    point-to-point compare (thresholds 1e-6 f32 / eps(bf16), :160-173) can be met.
+    name "src" | "wei"; amp = the reduction length K (:64-102).  Ranges: src
+    [-64,64) f32 / [-4,4) bf16,f16; wei [-128,128) f32 / [-8,8) bf16 / [-2,2) f16;
+    seeds 0 (src) and 1 (wei) (:141, util.py:163-171 with the default --seed 0)."""
+    rng = [{torch.float32: (-64, 64), torch.bfloat16: (-4, 4), torch.float16: (-4, 4)},
+           {torch.float32: (-128, 128), torch.bfloat16: (-8, 8), torch.float16: (-2, 2)}]
+    digits = {torch.float32: 24, torch.bfloat16: 8, torch.float16: 11}
+    src_min, src_max = rng[0][dtype]
+    wei_min, wei_max = rng[1][dtype]
+    max_value = max(abs(src_min), abs(src_max)) * max(abs(wei_min), abs(wei_max))
+    safe_n_acc = (1 << min(24, digits[dst_dtype])) // max_value
+    if name == "src":
+        lo, hi = src_min, src_max
+        density = 1.0
+    elif name == "wei":
+        lo, hi = wei_min, wei_max
+        density = min(safe_n_acc / int(amp), 1.0)
+    else:
+        raise ValueError(name)
+    torch.manual_seed(0 if name == "src" else 1)
+    value = torch.bernoulli(torch.full(tuple(shape), density)) * torch.randint(lo, hi, tuple(shape))
+    while value.flatten()[0] <= 0:
+        value.flatten()[0] = torch.randint(lo, hi + 1, size=[1])[0].item()
+    return value.to(dtype)
+
+
 def causal_mask(Sq, Sk, value=float("-inf")):
     """Additive mask: 0 on and below the diagonal, `value` above."""
     return torch.triu(torch.full((Sq, Sk), value, dtype=torch.float32), diagonal=1)

@@ -3,7 +3,22 @@
  * compiler's contraction hot path.  Every pointer is a DEVICE pointer unless
  * stated otherwise; sizes and leading dimensions are in elements; `stream` is a
  * hipStream_t passed as void* (NULL = the default stream).  Calls are
- * asynchronous on `stream`.  No function allocates device memory.
+ * asynchronous on `stream`.
+ *
+ * Scratch memory.  Two kinds of call need device memory beyond their operands:
+ * K-sliced GEMMs (a short A against wide weights: f32 partial sums) and masked
+ * attention (one byte per mask tile).  Each entry point says where it comes
+ * from:
+ *   - plain entry points (gcmi_gemm_bf16, gcmi_mha_fwd_bf16, ...): a workspace
+ *     the library allocates per device at the first call that needs one and
+ *     grows on demand (hipMalloc under a lock).  Calls that use it are put in
+ *     order across streams (an event behind each, waited for by the next call
+ *     on another stream), so they are safe from any number of host threads;
+ *   - *_ws entry points: a workspace the caller brings (size from the
+ *     *_workspace_bytes query).  Nothing is shared: calls with different
+ *     workspaces may overlap on different streams.  This is what a compiled
+ *     partition uses (its arena holds the workspace);
+ * Everything else needs no scratch and allocates nothing.
  *
  * Return value: a dnnl_status_t-compatible int (0 success, 2 invalid
  * arguments, 3 unimplemented, 5 runtime error); gcmi_last_error() gives text.
@@ -14,6 +29,7 @@
 #ifndef GC_HIP_KERNELS_H
 #define GC_HIP_KERNELS_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -49,8 +65,7 @@ const char *gcmi_last_error(void);
  * When A has at most 256 rows and N is narrow (fewer column tiles than half the
  * compute units), K is cut into slices over workgroups and a second kernel adds
  * the f32 partial sums in a fixed order (results do not vary from run to run).
- * The partial sums live in a 32 MiB per-device static buffer: such calls on
- * different streams of one device must not overlap.
+ * The partial sums go through the library workspace (see "Scratch memory").
  */
 int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                    int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream);
@@ -97,6 +112,22 @@ int gcmi_gemm_bf16_residual(const void *A, const void *B, void *C, int64_t batch
                             int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
                             int trans_b, const void *bias, int bias_dtype, int act, const void *residual, int64_t ldr,
                             int residual_dtype, int out_dtype, void *stream);
+
+/*
+ * gcmi_gemm_bf16_residual with the workspace as an argument: `workspace`
+ * (16-byte aligned, workspace_bytes long; NULL / 0: K is not sliced) holds the
+ * partial sums of a K-sliced call.  gcmi_gemm_bf16_workspace_bytes gives the
+ * size the shape can use (0: the shape is never sliced); with less, fewer
+ * slices are cut.  The result does not depend on the workspace's address, and
+ * for a given size it does not vary from run to run.  No counterpart in the
+ * reference, whose K-sliced partial sums live in a buffer its generated code
+ * allocates (lib/gc/Transforms/DeepTileContractionOp.cpp:988-996).
+ */
+size_t gcmi_gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_b);
+int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                      int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                      int trans_b, const void *bias, int bias_dtype, int act, const void *residual, int64_t ldr,
+                      int residual_dtype, int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * 8-bit matmul with s32 accumulation and fused dequantise epilogue.
@@ -158,12 +189,23 @@ int gcmi_mha_fwd_bf16(const void *Q, const void *K, const void *V, const float *
  * it contributes exp(-inf) = 0 to every sum, so the result is bit-identical.
  * skip_masked == 0: every block is computed (the dense 4*BH*Sq*Sk*D operation
  * count).  scale must be > 0 for the fast kernel (otherwise a slower, general
- * kernel runs).  The tile classes live in a per-device static buffer: calls on
- * different streams of one device must not overlap.
+ * kernel runs).  The tile classes go through the library workspace (see
+ * "Scratch memory").
  * No counterpart in the reference.
  */
 int gcmi_mha_fwd_bf16_opt(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld, void *O,
                           int64_t BH, int64_t Sq, int64_t Sk, int64_t D, float scale, int skip_masked, void *stream);
+
+/*
+ * The same with the workspace as an argument: one byte per (32 query rows x 64
+ * keys) mask tile, gcmi_mha_fwd_workspace_bytes in all (0: the shape has no
+ * use for one).  With NULL or too small a workspace every tile is read from
+ * the mask and nothing is skipped; the result is the same.
+ */
+size_t gcmi_mha_fwd_workspace_bytes(int64_t Sq, int64_t Sk, int64_t D, int has_mask);
+int gcmi_mha_fwd_bf16_ws(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld, void *O,
+                         int64_t BH, int64_t Sq, int64_t Sk, int64_t D, float scale, int skip_masked, void *workspace,
+                         size_t workspace_bytes, void *stream);
 
 #pragma GCC visibility pop
 #ifdef __cplusplus

@@ -92,3 +92,28 @@ def assert_close(ref, res, rtol, what="", mag=None):
     bad, md = close_report(ref, res, rtol, mag)
     assert bad == 0, "%s: %d elements beyond rtol %g (max scaled error %.3e)" % (what, bad, rtol, md)
     return md
+
+
+def strict_failures(orc, ref, res, thr):
+    """The reference harness's own point-to-point rule (test/benchgc/src/benchgc/arg/compare.py:60-137) applied
+    element by element: d = |ref-res|/|ref| where |ref| > 1e-5, else |ref-res|; pass iff d <= thr, or both NaN, or
+    the same infinity.  Returns the boolean mask of failing elements; its count is checked against the oracle's
+    gco_compare_p2p on the same data."""
+    r = np.asarray(ref, np.float32)
+    s = np.asarray(res, np.float32)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        a = np.abs(r)
+        d = np.where(a > np.float32(1e-5), np.abs(r - s) / a, np.abs(r - s))
+    ok = (d <= np.float32(thr)) | (np.isnan(r) & np.isnan(s)) | (np.isinf(r) & np.isinf(s) & ((r > 0) == (s > 0)))
+    bad = ~ok
+    n_oracle, _ = orc.compare_p2p(r, s, thr)
+    assert int(bad.sum()) == n_oracle, "numpy restatement (%d) and gco_compare_p2p (%d) disagree" % (bad.sum(), n_oracle)
+    return bad
+
+
+def mistrusted(res, zero_percent):
+    """benchgc's mistrust check (compare.py:112-119): too many zeros in the result make a pass meaningless."""
+    res = np.asarray(res)
+    if res.size < 10:
+        return False
+    return (res.size - np.count_nonzero(res)) * 100.0 / res.size > zero_percent

@@ -156,7 +156,7 @@ def test_arena_shares_memory_between_temporaries_with_disjoint_lifetimes(ga):
     allocations by lifetime ticks, lib/gc/Transforms/MergeAllocTickBased.cpp).  The plan reports both sizes."""
     import json
     import re
-    M = 256
+    M = 512  # two tile rows: these matmuls are not K-sliced and need no scratch
     ops = []
     for i in range(4):
         src = 0 if i == 0 else 10 + i - 1
@@ -170,3 +170,23 @@ def test_arena_shares_memory_between_temporaries_with_disjoint_lifetimes(ga):
     one = M * M * 2
     assert naive == 9 * one          # 5 inputs + 3 temporaries + 1 output
     assert shared == 8 * one         # t3 reuses t1's region
+
+
+def test_k_sliced_matmuls_get_scratch_of_their_own_in_the_arena(ga, gc):
+    """A short A against a wide weight is K-sliced: its partial sums live in a slot of the executable's arena, alive
+    for that step only (two such steps share the space), not in anything shared between executables."""
+    import re
+    M, K, N = 32, 4096, 4096
+    ops = [{"kind": "MatMul", "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [K, N])],
+            "outputs": [ga._t(10, "bf16", [M, N])]},
+           {"kind": "MatMul", "inputs": [ga._t(10, "bf16", [M, N]), ga._t(2, "bf16", [N, K])],
+            "outputs": [ga._t(11, "bf16", [M, K])]}]
+    st, plan = ga.explain(ga._graph(ops, [0, 1, 2], [11]))
+    assert st == 0, plan
+    m = re.search(r"arena: (\d+) bytes \((\d+) with one region per buffer\)", plan)
+    shared, naive = int(m.group(1)), int(m.group(2))
+    ws = gc.lib().gcmi_gemm_bf16_workspace_bytes(M, N, K, 0)
+    assert ws >= 2 * M * N * 4      # at least two slices of f32 partial sums
+    tensors = 2 * M * K * 2 + 2 * K * N * 2 + M * N * 2
+    assert naive == tensors + 2 * ws
+    assert shared == tensors + ws   # the second step's scratch takes the place of the first's

@@ -418,3 +418,96 @@ def test_random_attention_partitions_against_torch(ga, dev, seed):
     ref = (P.to(torch.bfloat16).double() @ V.double()).to(torch.bfloat16).float().numpy()
     mag = (P @ V.double().abs()).numpy()
     assert_close(ref, out.float().numpy(), 1e-2, "attention %s D=%d mask=%s\n%s" % (s, D, mask_kind, plan), mag=mag)
+
+
+def test_two_executables_interleaved_on_two_streams_match_serial_runs(ga, wl, dev):
+    """The reference's execute is re-entrant (src/dnnl/dnnl_graph_compiler.cpp:214-226; scratch is thread-local,
+    lib/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmOnednn.cpp:70).  Here the scratch of K-sliced GEMMs and of
+    masked attention is part of each executable's arena: two executables launched alternately on two streams,
+    with nothing ordering one stream against the other, give the bits of serial execution."""
+    M, K, N = 32, 4096, 4096   # a short A against a wide weight: K-sliced, partial sums in the workspace
+    B, H, S, D = 1, 8, 512, 128
+    comp = ga.Compiler()
+    g_mm = ga._graph([{"kind": "MatMul", "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [K, N])],
+                       "outputs": [ga._t(2, "bf16", [M, N])]}], [0, 1], [2])
+    exes = []
+    for _ in range(2):
+        st, e = comp.compile(g_mm)
+        assert st == 0, ga.api().dnnl_graph_compiler_last_error().decode()
+        exes.append(e)
+    st, e_att = comp.compile(ga.mha_json(B, H, S, S, D, True, "Multiply"))
+    assert st == 0, ga.api().dnnl_graph_compiler_last_error().decode()
+    assert b"attention" in ga.explain(ga.mha_json(B, H, S, S, D, True, "Multiply"))[1].encode()
+    torch.manual_seed(5)
+    A = [(torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev) for _ in range(2)]
+    W = [(torch.randn(K, N) * 0.05).to(torch.bfloat16).to(dev) for _ in range(2)]
+    Q, Kt, V, mask, scale = wl.bf16_mha(B, H, S, D)
+    Q, Kt, V, mask = Q.to(dev), Kt.to(dev), V.to(dev), mask.to(dev)
+    sval = torch.tensor([scale], dtype=torch.float32)
+
+    # serial: one executable after the other, each waited for
+    want = [torch.zeros(M, N, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+    for i in range(2):
+        assert exes[i].execute([(0, A[i]), (1, W[i])], [(2, want[i])]) == 0
+    want_att = torch.zeros(B, H, S, D, dtype=torch.bfloat16, device=dev)
+    assert e_att.execute([(0, Q), (1, Kt), (2, sval.numpy()), (3, mask), (4, V)], [(9, want_att)]) == 0
+
+    # interleaved: stream i runs executable i, twenty rounds back to back; the raw attention entry point (library
+    # workspace, ordered across streams by the library) alternates with them on both streams
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [[torch.zeros(M, N, dtype=torch.bfloat16, device=dev) for _ in range(20)] for _ in range(2)]
+    got_att = [torch.zeros(B, H, S, D, dtype=torch.bfloat16, device=dev) for _ in range(20)]
+    calls = [[exes[i].bind([(0, A[i]), (1, W[i])], [(2, got[i][r])], stream=streams[i].cuda_stream) for r in range(20)]
+             for i in range(2)]
+    gcm = __import__("sys").modules["graph_compiler_amd"]
+    torch.cuda.synchronize()
+    for r in range(20):
+        for i in range(2):
+            assert calls[i][r]() == 0
+        with torch.cuda.stream(streams[r % 2]):
+            gcm.mha_fwd_bf16(Q, Kt, V, mask, scale, out=got_att[r])
+    torch.cuda.synchronize()
+    for i in range(2):
+        for r in range(20):
+            assert torch.equal(got[i][r].view(torch.int16), want[i].view(torch.int16)), (i, r)
+    for r in range(20):
+        assert torch.equal(got_att[r].view(torch.int16), want_att.view(torch.int16)), r
+    for e in exes + [e_att]:
+        e.close()
+    comp.close()
+
+
+def test_execute_from_two_host_threads_on_one_executable(ga, dev):
+    """Calls on one executable take turns (they share its arena): two threads calling execute at once both get
+    correct results."""
+    import threading
+    M, K, N = 32, 2048, 4096
+    comp = ga.Compiler()
+    g = ga._graph([{"kind": "MatMul", "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [K, N])],
+                    "outputs": [ga._t(2, "bf16", [M, N])]},
+                   {"kind": "ReLU", "inputs": [ga._t(2, "bf16", [M, N])], "outputs": [ga._t(3, "bf16", [M, N])]}], [0, 1], [3])
+    st, exe = comp.compile(g)
+    assert st == 0, ga.api().dnnl_graph_compiler_last_error().decode()
+    torch.manual_seed(6)
+    W = (torch.randn(K, N) * 0.05).to(torch.bfloat16).to(dev)
+    A = [(torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev) for _ in range(2)]
+    ref = [torch.relu((A[i].float() @ W.float()).to(torch.bfloat16)) for i in range(2)]
+    errs = []
+
+    def work(i):
+        for _ in range(10):
+            out = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+            if exe.execute([(0, A[i]), (1, W)], [(3, out)]) != 0:
+                errs.append("status")
+            d = (out.float() - ref[i].float()).abs().max().item()
+            if d > 0.25:
+                errs.append("thread %d off by %g" % (i, d))
+
+    ts = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    assert not errs, errs
+    exe.close()
+    comp.close()
