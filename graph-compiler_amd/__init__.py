@@ -22,6 +22,7 @@ ACT = {None: 0, "none": 0, "relu": 1, "gelu_erf": 2, "gelu_tanh": 3, "sigmoid": 
 EXPORTS = {
     "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_bf16_nt", "gcmi_gemm_bf16_batched", "gcmi_gemm_bf16_residual", "gcmi_gemm_f32_batched",
                          "gcmi_gemm_bf16_ws", "gcmi_gemm_bf16_workspace_bytes", "gcmi_mha_fwd_bf16_ws", "gcmi_mha_fwd_workspace_bytes",
+                         "gcmi_gemm_bf16_noalloc", "gcmi_noalloc_scratch_bytes",
                          "gcmi_gemm_int8", "gcmi_colsum_s8",
                          "gcmi_gemm_f32", "gcmi_mha_fwd_bf16", "gcmi_mha_fwd_bf16_opt"],
     "gc_brgemm.h": ["dnnl_brgemm_dispatch", "dnnl_brgemm_tileconfig", "dnnl_brgemm_tilerelease",
@@ -64,6 +65,10 @@ def lib():
     L.gcmi_mha_fwd_workspace_bytes.argtypes = [i64, i64, i64, ci]
     L.gcmi_mha_fwd_bf16_ws.restype = ci
     L.gcmi_mha_fwd_bf16_ws.argtypes = [vp, vp, vp, vp, i64, vp, i64, i64, i64, i64, f32, ci, vp, C.c_size_t, vp]
+    L.gcmi_gemm_bf16_noalloc.restype = ci
+    L.gcmi_gemm_bf16_noalloc.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp, ci, ci, ci, vp]
+    L.gcmi_noalloc_scratch_bytes.restype = C.c_size_t
+    L.gcmi_noalloc_scratch_bytes.argtypes = []
     L.gcmi_gemm_f32_batched.restype = ci
     L.gcmi_gemm_f32_batched.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, ci, vp, ci, vp]
     L.gcmi_gemm_bf16_nt.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, ci, ci, ci, vp]

@@ -29,6 +29,7 @@ int gcmi_launch_brgemm(const void *A, const void *B, void *C, int64_t M, int64_t
 int gcmi_launch_mha_fwd(const MhaParams *p, hipStream_t stream);
 int64_t gcmi_launch_gemm_bf16_workspace(const GemmParams *p);
 int64_t gcmi_launch_mha_workspace(const MhaParams *p);
+int gcmi_noalloc_scratch(void **ptr, size_t *bytes);
 }
 
 namespace {
@@ -52,7 +53,7 @@ extern "C" const char *gcmi_last_error(void) { return g_err; }
 
 namespace {
 // Where a call's scratch (partial sums of K-sliced GEMMs, mask tile classes of attention) comes from.
-enum class Ws { Library, Caller };
+enum class Ws { Library, Caller, Static };
 
 // Scratch of the entry points that take no workspace argument: one buffer per device, allocated at the first call
 // that needs it and grown on demand.  Every call on the device shares it, so its users are put in order: the mutex
@@ -121,6 +122,11 @@ extern "C" int gcmi_init(int device) {
     return fail(ST_RUNTIME, "hipGetDeviceProperties failed");
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(ST_UNIMPL, "device is %s; these kernels are built for gfx950 only", prop.gcnArchName);
+  // the device address of the static scratch array (gcmi_gemm_bf16_noalloc), once per device
+  void *sp = nullptr;
+  size_t sb = 0;
+  if (gcmi_noalloc_scratch(&sp, &sb) != 0)
+    return fail(ST_RUNTIME, "hipGetSymbolAddress(scratch) failed on device %d", device);
   return ST_OK;
 }
 
@@ -219,6 +225,19 @@ int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M
     p.partial = ws_bytes >= 4 ? (float *)ws : nullptr, p.partial_cap = (int64_t)(ws_bytes / 4);
     return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
   }
+  if (ws_from == Ws::Static) {
+    void *sp = nullptr;
+    size_t sb = 0;
+    if (gcmi_noalloc_scratch(&sp, &sb) != 0)
+      return fail(ST_RUNTIME, "gemm_bf16_noalloc: the address of the static scratch array is not available");
+    if ((size_t)want * 4 > sb)
+      return fail(ST_INVALID,
+                  "gemm_bf16_noalloc: %lld x %lld x %lld needs %lld bytes of scratch for its K slices, the static "
+                  "buffer holds %zu; use gcmi_gemm_bf16 (library workspace) or gcmi_gemm_bf16_ws",
+                  (long long)M, (long long)N, (long long)K, (long long)want * 4, sb);
+    p.partial = (float *)sp, p.partial_cap = (int64_t)(sb / 4);
+    return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16_noalloc");
+  }
   LibraryWorkspace *lw = nullptr;
   void *lp = nullptr;
   if (int rc = ws_acquire((size_t)want * 4, (hipStream_t)stream, &lw, &lp))
@@ -264,6 +283,19 @@ extern "C" int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t 
   return gemm_bf16_any(trans_b != 0, A, B, C, M, N, K, lda, ldb, ldc, bias, bias_dtype, act, out_dtype, stream, batch,
                        stride_a, stride_b, stride_c, residual, ldr, residual_dtype, Ws::Caller, workspace,
                        workspace_bytes);
+}
+
+extern "C" size_t gcmi_noalloc_scratch_bytes(void) {
+  void *p = nullptr;
+  size_t b = 0;
+  return gcmi_noalloc_scratch(&p, &b) == 0 ? b : 0;
+}
+
+extern "C" int gcmi_gemm_bf16_noalloc(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                                      int64_t lda, int64_t ldb, int64_t ldc, int trans_b, const void *bias,
+                                      int bias_dtype, int act, int out_dtype, void *stream) {
+  return gemm_bf16_any(trans_b != 0, A, B, C, M, N, K, lda, ldb, ldc, bias, bias_dtype, act, out_dtype, stream, 1, 0, 0,
+                       0, nullptr, 0, 0, Ws::Static);
 }
 
 extern "C" int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K,

@@ -17,3 +17,25 @@ extern "C" int64_t gcmi_launch_gemm_bf16_workspace(const gcmi::GemmParams *p) {
   gcmi::launch_tile256<2>(p, nullptr, &want);
   return want;
 }
+
+// Scratch of the entry point that allocates nothing (gcmi_gemm_bf16_noalloc): the partial sums of K-sliced calls.
+// Each device the library runs on holds its own copy until the process ends.  `scratch` is only a host-side
+// stand-in here: its device address is asked for once per device and kept.
+static constexpr size_t GCMI_NOALLOC_SCRATCH_BYTES = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[GCMI_NOALLOC_SCRATCH_BYTES];
+
+extern "C" int gcmi_noalloc_scratch(void **ptr, size_t *bytes) {
+  static void *dev_ptr[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    return 5;
+  void *q = __atomic_load_n(&dev_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!q) {
+    if (hipGetSymbolAddress(&q, HIP_SYMBOL(scratch)) != hipSuccess || !q)
+      return 5;
+    __atomic_store_n(&dev_ptr[dev], q, __ATOMIC_RELEASE); // the same value from every thread that gets here
+  }
+  *ptr = q;
+  *bytes = GCMI_NOALLOC_SCRATCH_BYTES;
+  return 0;
+}

@@ -18,6 +18,7 @@
  *     *_workspace_bytes query).  Nothing is shared: calls with different
  *     workspaces may overlap on different streams.  This is what a compiled
  *     partition uses (its arena holds the workspace);
+ *   - gcmi_gemm_bf16_noalloc: a static device array; allocates nothing.
  * Everything else needs no scratch and allocates nothing.
  *
  * Return value: a dnnl_status_t-compatible int (0 success, 2 invalid
@@ -128,6 +129,24 @@ int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int6
                       int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
                       int trans_b, const void *bias, int bias_dtype, int act, const void *residual, int64_t ldr,
                       int residual_dtype, int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * gcmi_gemm_bf16 / gcmi_gemm_bf16_nt (trans_b) for callers that cannot
+ * allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  The
+ * partial sums of a K-sliced call go to a static device array of
+ * gcmi_noalloc_scratch_bytes() = 32 MiB that every device the library runs on
+ * holds until the process ends; the call allocates nothing and frees nothing.
+ * A shape whose K slices need more than that (gcmi_gemm_bf16_workspace_bytes)
+ * is refused with status 2 and a message; shapes that are not K-sliced need no
+ * scratch and are never refused.  Every call on a device shares that device's
+ * array: calls that overlap in time on one device (different streams) race;
+ * calls on one stream are safe.  Results equal gcmi_gemm_bf16's bit for bit.
+ */
+size_t gcmi_noalloc_scratch_bytes(void);
+int gcmi_gemm_bf16_noalloc(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                           int64_t ldb, int64_t ldc, int trans_b, const void *bias, int bias_dtype, int act,
+                           int out_dtype, void *stream);
 
 /*
  * 8-bit matmul with s32 accumulation and fused dequantise epilogue.
