@@ -22,7 +22,7 @@ ACT = {None: 0, "none": 0, "relu": 1, "gelu_erf": 2, "gelu_tanh": 3, "sigmoid": 
 EXPORTS = {
     "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_bf16_nt", "gcmi_gemm_bf16_batched", "gcmi_gemm_bf16_residual", "gcmi_gemm_f32_batched",
                          "gcmi_gemm_bf16_ws", "gcmi_gemm_bf16_workspace_bytes", "gcmi_mha_fwd_bf16_ws", "gcmi_mha_fwd_workspace_bytes",
-                         "gcmi_gemm_bf16_noalloc", "gcmi_noalloc_scratch_bytes",
+                         "gcmi_gemm_bf16_noalloc", "gcmi_noalloc_scratch_bytes", "gcmi_gemm_int8_cfg", "gcmi_gemm_tile_config_query",
                          "gcmi_gemm_int8", "gcmi_colsum_s8",
                          "gcmi_gemm_f32", "gcmi_mha_fwd_bf16", "gcmi_mha_fwd_bf16_opt"],
     "gc_brgemm.h": ["dnnl_brgemm_dispatch", "dnnl_brgemm_tileconfig", "dnnl_brgemm_tilerelease",
@@ -60,7 +60,11 @@ def lib():
     L.gcmi_gemm_bf16_workspace_bytes.restype = C.c_size_t
     L.gcmi_gemm_bf16_workspace_bytes.argtypes = [i64, i64, i64, ci]
     L.gcmi_gemm_bf16_ws.restype = ci
-    L.gcmi_gemm_bf16_ws.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, vp, ci, ci, vp, i64, ci, ci, vp, C.c_size_t, vp]
+    L.gcmi_gemm_bf16_ws.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, vp, ci, ci, vp, i64, ci, ci, vp, C.c_size_t, vp, vp]
+    L.gcmi_gemm_int8_cfg.restype = ci
+    L.gcmi_gemm_int8_cfg.argtypes = [vp, ci, vp, vp, i64, i64, i64, i64, i64, i64, vp, C.c_int32, vp, vp, ci, ci, vp, vp]
+    L.gcmi_gemm_tile_config_query.restype = ci
+    L.gcmi_gemm_tile_config_query.argtypes = [ci, i64, i64, i64, ci, ci, vp, vp, C.c_char_p, C.c_size_t]
     L.gcmi_mha_fwd_workspace_bytes.restype = C.c_size_t
     L.gcmi_mha_fwd_workspace_bytes.argtypes = [i64, i64, i64, ci]
     L.gcmi_mha_fwd_bf16_ws.restype = ci
@@ -92,6 +96,27 @@ def lib():
     L.dnnl_brgemm_execute.argtypes = [i64, vp, u64, vp, u64, vp, u64, ci]
     _lib = L
     return L
+
+
+class TileConfig(C.Structure):
+    """gcmi_gemm_tile_config of include/gc_hip_kernels.h"""
+    _fields_ = [(n, C.c_int32) for n in ("kernel", "bm", "bn", "kbytes", "stages", "waves_m", "waves_n", "wave_m", "wave_n",
+                                         "mfma_m", "mfma_n", "mfma_k", "split_k", "group_m", "workgroups", "from_attrs")]
+
+
+MATMUL_CONFIG_NAMES = ("MThreads", "NThreads", "KThreads", "MBlock", "NBlock", "KBlock", "innermostMBlock",
+                       "innermostNBlock", "innermostKBlock")
+
+
+def tile_config(M, N, K, a_dtype=BF16, trans_b=False, out_dtype=BF16, matmul_config=None):
+    """What the launcher chooses for this GEMM (no GPU needed).  matmul_config: the nine MatmulConfig integers in
+    MATMUL_CONFIG_NAMES order, or None.  Returns (TileConfig, note)."""
+    c = TileConfig()
+    note = C.create_string_buffer(200)
+    arr = None if matmul_config is None else (C.c_int64 * 9)(*matmul_config)
+    check(lib().gcmi_gemm_tile_config_query(a_dtype, M, N, K, int(trans_b), out_dtype, arr, C.byref(c), note, 200),
+          "gcmi_gemm_tile_config_query")
+    return c, note.value.decode()
 
 
 class GcError(RuntimeError):

@@ -177,6 +177,21 @@ void Executable::add_copy(int src, DT sdt, const std::vector<int64_t> &dims, con
   steps_.push_back(std::move(s));
 }
 
+// The nine MatmulConfig attributes of a matmul op, in the order the kernels' ABI takes them; empty unless all nine
+// are integer attributes (the reference uses a config only when it is complete, MatmulConfigAnalysis.cpp:368-404).
+static std::vector<int64_t> matmul_config_attrs(const Op &op) {
+  static const char *names[9] = {"MThreads", "NThreads", "KThreads", "MBlock", "NBlock", "KBlock",
+                                 "innermostMBlock", "innermostNBlock", "innermostKBlock"};
+  std::vector<int64_t> v;
+  for (const char *n : names) {
+    auto it = op.attrs.find(n);
+    if (it == op.attrs.end() || it->second.type != Attr::S64)
+      return {};
+    v.push_back(it->second.i);
+  }
+  return v;
+}
+
 // ---------------------------------------------------------------------------
 Executable::Executable(const char *json, bool dry) : g_(parse_graph(json)) { init(dry); }
 Executable::Executable(Graph g, bool dry) : g_(std::move(g)) { init(dry); }
@@ -576,6 +591,7 @@ void Executable::plan() {
       s.a_dt = dt_dnnl(qa.dt), s.zp = zpA, s.aux = cs_slot, s.scales_slot = sc_slot;
       s.bias = bias_t >= 0 ? slot_for((size_t)bias_t) : -1;
       s.act = act, s.out_dt = dt_dnnl(T(cur).dt);
+      s.mm_cfg = matmul_config_attrs(mm);
       v.push_back(s);
       skip[dq_a] = skip[dq_w] = claimed[dq_a] = claimed[dq_w] = true;
     } else {
@@ -651,6 +667,7 @@ void Executable::plan() {
           s.a_bs = ba == bo ? a_mat : 0, s.b_bs = bb == bo ? b_mat : 0, s.c_bs = M * N;
         }
         s.a = sa_slot, s.b = sb_slot, s.out = out_slot;
+        s.mm_cfg = matmul_config_attrs(mm);
         s.M = flatten ? M * nb : M, s.N = N, s.K = K;
         s.lda = as[Ra - 1], s.ldb = bs[Rb - 1], s.ldc = N;
         s.ta = tA, s.tb = tB;
@@ -1441,7 +1458,8 @@ void Executable::launch(const Step &s) {
                                P(s.out) + s.out_off * (s.out_dt == GCMI_BF16 ? 2 : 4), s.batch, s.M, s.N, s.K, s.lda, s.ldb,
                                s.ldc, s.a_bs, s.b_bs, s.c_bs, s.tb ? 1 : 0, P(s.bias), s.bias_dt ? s.bias_dt : GCMI_BF16,
                                s.act, P(s.c), s.N, s.b_dt ? s.b_dt : GCMI_BF16, s.out_dt, P(s.ws),
-                               s.ws >= 0 ? slots_[(size_t)s.ws].bytes : 0, stream_),
+                               s.ws >= 0 ? slots_[(size_t)s.ws].bytes : 0, s.mm_cfg.size() == 9 ? s.mm_cfg.data() : nullptr,
+                               stream_),
              "MatMul bf16");
     break;
   case Step::ColSum:
@@ -1451,8 +1469,9 @@ void Executable::launch(const Step &s) {
     colsum_valid_[s.out] = true;
     break;
   case Step::GemmInt8:
-    gc_check(gcmi_gemm_int8(P(s.a), s.a_dt, P(s.b), P(s.out), s.M, s.N, s.K, s.lda, s.ldb, s.ldc, (const int32_t *)P(s.aux),
-                            s.zp, (const float *)P(s.scales_slot), (const float *)P(s.bias), s.act, s.out_dt, stream_),
+    gc_check(gcmi_gemm_int8_cfg(P(s.a), s.a_dt, P(s.b), P(s.out), s.M, s.N, s.K, s.lda, s.ldb, s.ldc, (const int32_t *)P(s.aux),
+                                s.zp, (const float *)P(s.scales_slot), (const float *)P(s.bias), s.act, s.out_dt,
+                                s.mm_cfg.size() == 9 ? s.mm_cfg.data() : nullptr, stream_),
              "MatMul int8");
     break;
   case Step::Mha: {
@@ -1675,8 +1694,31 @@ void Executable::run(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_ten
 std::string Executable::describe() const {
   static const char *names[] = {"gemm_f32", "gemm_bf16", "gemm_int8", "colsum", "attention", "eltwise", "reduce", "softmax"};
   std::ostringstream os;
-  for (auto &s : steps_)
+  static const char *kernels[] = {"bounds-checked tile", "whole tiles, 8 waves", "whole tiles, 4 waves (one per SIMD)",
+                                  "K slices + second pass", "weight streaming (+ second pass)"};
+  for (auto &s : steps_) {
     os << (s.kind == Step::Fused ? (s.sum_ins >= 0 ? "reduce" : "fused") : names[(int)s.kind]) << ": " << s.note << "\n";
+    if ((s.kind == Step::GemmBf16 && s.batch <= 1 && !s.ta) || s.kind == Step::GemmInt8) {
+      // the tile descriptor the launcher will choose for this shape (the counterpart of the reference's MatmulConfig)
+      gcmi_gemm_tile_config c{};
+      char why[160] = "";
+      const int a_dt = s.kind == Step::GemmInt8 ? s.a_dt : GCMI_BF16;
+      if (gcmi_gemm_tile_config_query(a_dt, s.M, s.N, s.K, s.tb ? 1 : 0, s.out_dt, s.mm_cfg.size() == 9 ? s.mm_cfg.data() : nullptr,
+                                      &c, why, sizeof(why)) == 0) {
+        os << "  tile: " << kernels[c.kernel] << ", " << c.bm << "x" << c.bn << " per workgroup, " << c.kbytes
+           << " B of K per stage x " << c.stages << " stages, waves " << c.waves_m << "x" << c.waves_n << " of " << c.wave_m << "x"
+           << c.wave_n << ", mfma " << c.mfma_m << "x" << c.mfma_n << "x" << c.mfma_k << ", split_k " << c.split_k << ", "
+           << c.workgroups << " workgroups";
+        if (c.from_attrs)
+          os << " [MatmulConfig attributes applied]";
+        else if (why[0])
+          os << " [" << why << "]";
+        else if (s.mm_cfg.size() == 9)
+          os << " [MatmulConfig attributes leave the default]";
+        os << "\n";
+      }
+    }
+  }
   if (!g_.target_hints.empty()) {
     os << "target hints (CPU, not used):";
     for (auto &h : g_.target_hints)

@@ -34,6 +34,9 @@ struct Step {
   bool once = false; // depends on constant tensors only: runs in the first execute, its result is kept
   // operands are arena slot indices (-1 = none)
   int a = -1, b = -1, c = -1, out = -1, bias = -1, mask = -1, aux = -1;
+  // the op's MatmulConfig attributes {MThreads, NThreads, KThreads, MBlock, NBlock, KBlock, innermostMBlock,
+  // innermostNBlock, innermostKBlock} when all nine are there (lib/gc/Analysis/MatmulConfigAnalysis.cpp:368-404)
+  std::vector<int64_t> mm_cfg;
   int ws = -1; // scratch of this step alone (partial sums of a K-sliced GEMM, mask tile classes of attention)
   int64_t M = 0, N = 0, K = 0, lda = 0, ldb = 0, ldc = 0;
   int64_t a_off = 0, b_off = 0, out_off = 0; // element offsets (batched fallbacks)

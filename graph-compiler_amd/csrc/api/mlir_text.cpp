@@ -658,6 +658,24 @@ void parse_op(Cursor &c, Builder &b, const std::string &res, const std::string &
       o.attrs["transpose_a"] = attr_bool(true);
     if (op.find("transpose_b") != std::string::npos)
       o.attrs["transpose_b"] = attr_bool(true);
+    // the tuning attributes the reference reads from the op ({MThreads = 4 : i32, ...},
+    // lib/gc/Analysis/MatmulConfigAnalysis.cpp:368-404; test/mlir/test/gc/Transforms/deepTileContractionNamedOp.mlir:33)
+    for (const char *n : {"MThreads", "NThreads", "KThreads", "MBlock", "NBlock", "KBlock", "innermostMBlock",
+                          "innermostNBlock", "innermostKBlock"}) {
+      const std::string key = n;
+      size_t at = 0;
+      while ((at = brace.find(key, at)) != std::string::npos) {
+        const bool starts = at == 0 || !(isalnum((unsigned char)brace[at - 1]) || brace[at - 1] == '_');
+        size_t q = at + key.size();
+        while (q < brace.size() && isspace((unsigned char)brace[q]))
+          q++;
+        if (starts && q < brace.size() && brace[q] == '=') {
+          o.attrs[key] = attr_int(strtoll(brace.c_str() + q + 1, nullptr, 10));
+          break;
+        }
+        at += key.size();
+      }
+    }
     size_t id = result(rt);
     b.g.ops.back().out = {id};
     return;

@@ -5,6 +5,7 @@
 // workspace argument (LibraryWorkspace below).
 #include <hip/hip_runtime_api.h>
 
+#include <climits>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -28,6 +29,8 @@ int gcmi_launch_brgemm(const void *A, const void *B, void *C, int64_t M, int64_t
                        int dtB, hipStream_t stream);
 int gcmi_launch_mha_fwd(const MhaParams *p, hipStream_t stream);
 int64_t gcmi_launch_gemm_bf16_workspace(const GemmParams *p);
+int gcmi_launch_gemm_bf16_config(const GemmParams *p, GemmTileConfig *cfg);
+int gcmi_launch_gemm_int8_config(const GemmParams *p, GemmTileConfig *cfg);
 int64_t gcmi_launch_mha_workspace(const MhaParams *p);
 int gcmi_noalloc_scratch(void **ptr, size_t *bytes);
 }
@@ -131,11 +134,50 @@ extern "C" int gcmi_init(int device) {
 }
 
 namespace {
+// The reference reads a MatmulConfig from nine integer attributes of the matmul op -- all nine or none
+// (readConfigFromAttrs, lib/gc/Analysis/MatmulConfigAnalysis.cpp:368-404) -- and drops it when validateConfig
+// (:40-65) fails.  Here the nine are {MThreads, NThreads, KThreads, MBlock, NBlock, KBlock, innermostMBlock,
+// innermostNBlock, innermostKBlock}; what they can steer on the GPU: the workgroup tile (MBlock x NBlock: 256 x 256
+// is the one that is built), the tile of one wave (innermostMBlock x innermostNBlock: 128 x 128 = 4 waves per
+// workgroup, 128 x 64 = 8 waves) and the number of K slices (KThreads).  MThreads x NThreads is the reference's
+// thread grid; the GPU's grid follows from the tile.  Returns false, with the reason, when the config is not used.
+bool apply_matmul_config(const int64_t *c, int64_t M, int64_t N, int64_t K, GemmParams &p, const char **why) {
+  const int64_t MThreads = c[0], NThreads = c[1], KThreads = c[2], MBlock = c[3], NBlock = c[4], KBlock = c[5], iM = c[6],
+                iN = c[7], iK = c[8];
+  *why = "";
+  for (int i = 0; i < 9; i++)
+    if (c[i] <= 0) {
+      *why = "invalid (a field is not positive)";
+      return false;
+    }
+  (void)MThreads, (void)NThreads;
+  if (MBlock % iM != 0 || NBlock % iN != 0 || KBlock % iK != 0) {
+    *why = "invalid (a block is not a multiple of its innermost block)";
+    return false;
+  }
+  if ((K + KBlock - 1) / KBlock < KThreads) {
+    *why = "invalid (fewer K blocks than KThreads)";
+    return false;
+  }
+  if (MBlock != 256 || NBlock != 256) {
+    *why = "not built (the workgroup tile is 256 x 256)";
+    return false;
+  }
+  if (iM != 128 || (iN != 128 && iN != 64)) {
+    *why = "not built (a wave's tile is 128 x 128 or 128 x 64)";
+    return false;
+  }
+  (void)M, (void)N;
+  p.cfg_waves = iN == 128 ? 4 : 8;
+  p.cfg_split_k = (int32_t)(KThreads > 1024 ? 1024 : KThreads);
+  return true;
+}
+
 int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream,
                   int64_t batch = 1, int64_t a_bs = 0, int64_t b_bs = 0, int64_t c_bs = 0, const void *residual = nullptr,
                   int64_t ldr = 0, int residual_dtype = 0, Ws ws_from = Ws::Library, void *ws = nullptr,
-                  size_t ws_bytes = 0);
+                  size_t ws_bytes = 0, const int64_t *matmul_config = nullptr);
 }
 
 extern "C" int gcmi_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -193,7 +235,7 @@ namespace {
 int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldb, int64_t ldc, const void *bias, int bias_dtype, int act, int out_dtype, void *stream,
                   int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs, const void *residual, int64_t ldr,
-                  int residual_dtype, Ws ws_from, void *ws, size_t ws_bytes) {
+                  int residual_dtype, Ws ws_from, void *ws, size_t ws_bytes, const int64_t *matmul_config) {
   if (M < 0 || N < 0 || K < 0)
     return fail(ST_INVALID, "gemm_bf16: negative size");
   if (M == 0 || N == 0)
@@ -215,6 +257,10 @@ int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M
   p.trans_b = trans_b ? 1 : 0;
   p.batch = batch, p.a_bs = a_bs, p.b_bs = b_bs, p.c_bs = c_bs;
   p.residual = residual, p.ldr = ldr, p.residual_dt = residual_dtype;
+  if (matmul_config) {
+    const char *why;
+    (void)apply_matmul_config(matmul_config, M, N, K, p, &why); // not usable: ignored, as in the reference
+  }
   // K-sliced shapes (a short A against wide weights) pass f32 partial sums through a workspace
   const int64_t want = gcmi_launch_gemm_bf16_workspace(&p);
   if (want <= 0)
@@ -265,7 +311,7 @@ extern "C" int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t 
                                  int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b,
                                  int64_t stride_c, int trans_b, const void *bias, int bias_dtype, int act,
                                  const void *residual, int64_t ldr, int residual_dtype, int out_dtype, void *workspace,
-                                 size_t workspace_bytes, void *stream) {
+                                 size_t workspace_bytes, const int64_t *matmul_config, void *stream) {
   if (batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0)
     return fail(ST_INVALID, "gemm_bf16_ws: negative batch count or stride");
   if (batch == 0)
@@ -282,7 +328,37 @@ extern "C" int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t 
   }
   return gemm_bf16_any(trans_b != 0, A, B, C, M, N, K, lda, ldb, ldc, bias, bias_dtype, act, out_dtype, stream, batch,
                        stride_a, stride_b, stride_c, residual, ldr, residual_dtype, Ws::Caller, workspace,
-                       workspace_bytes);
+                       workspace_bytes, matmul_config);
+}
+
+extern "C" int gcmi_gemm_tile_config_query(int a_dtype, int64_t M, int64_t N, int64_t K, int trans_b, int out_dtype,
+                                           const int64_t *matmul_config, gcmi_gemm_tile_config *out, char *note,
+                                           size_t note_len) {
+  if (note && note_len)
+    note[0] = 0;
+  if (!out || M <= 0 || N <= 0 || K <= 0)
+    return fail(ST_INVALID, "gemm_tile_config_query: bad arguments");
+  const bool i8 = a_dtype == GCMI_S8 || a_dtype == GCMI_U8;
+  if (!i8 && a_dtype != GCMI_BF16)
+    return fail(ST_UNIMPL, "gemm_tile_config_query: a_dtype %d", a_dtype);
+  GemmParams p{};
+  // aligned stand-ins and every workspace the shape could use: the question is what the shape gets
+  p.A = p.B = (const void *)(uintptr_t)256, p.C = (void *)(uintptr_t)256;
+  p.M = M, p.N = N, p.K = K, p.lda = K, p.ldb = trans_b ? K : N, p.ldc = N;
+  p.bias_dt = GCMI_BF16, p.out_dt = out_dtype, p.trans_b = trans_b ? 1 : 0, p.batch = 1;
+  p.partial = (float *)(uintptr_t)256, p.partial_cap = INT64_MAX;
+  if (matmul_config) {
+    const char *why = "";
+    if (!apply_matmul_config(matmul_config, M, N, K, p, &why) && note && note_len)
+      snprintf(note, note_len, "MatmulConfig attributes ignored: %s", why);
+  }
+  GemmTileConfig c{};
+  const int rc = i8 ? gcmi_launch_gemm_int8_config(&p, &c) : gcmi_launch_gemm_bf16_config(&p, &c);
+  if (rc)
+    return fail(rc, "gemm_tile_config_query: no kernel takes this call");
+  static_assert(sizeof(gcmi_gemm_tile_config) == sizeof(GemmTileConfig), "the public struct mirrors GemmTileConfig");
+  memcpy(out, &c, sizeof(c));
+  return ST_OK;
 }
 
 extern "C" size_t gcmi_noalloc_scratch_bytes(void) {
@@ -301,6 +377,14 @@ extern "C" int gcmi_gemm_bf16_noalloc(const void *A, const void *B, void *C, int
 extern "C" int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K,
                               int64_t lda, int64_t ldb, int64_t ldc, const int32_t *colsum, int32_t zp_a,
                               const float *scale, const float *bias, int act, int out_dtype, void *stream) {
+  return gcmi_gemm_int8_cfg(A, a_dtype, W, C, M, N, K, lda, ldb, ldc, colsum, zp_a, scale, bias, act, out_dtype, nullptr,
+                            stream);
+}
+
+extern "C" int gcmi_gemm_int8_cfg(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K,
+                                  int64_t lda, int64_t ldb, int64_t ldc, const int32_t *colsum, int32_t zp_a,
+                                  const float *scale, const float *bias, int act, int out_dtype,
+                                  const int64_t *matmul_config, void *stream) {
   if (M < 0 || N < 0 || K < 0)
     return fail(ST_INVALID, "gemm_int8: negative size");
   if (M == 0 || N == 0)
@@ -328,6 +412,10 @@ extern "C" int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C
   p.bias = bias, p.bias_dt = GCMI_F32, p.scale = scale, p.colsum = comp ? colsum : nullptr, p.comp = comp;
   p.a_xor = a_dtype == GCMI_U8 ? 0x80808080u : 0u;
   p.act = out_dtype == GCMI_S32 ? GCMI_ACT_NONE : act, p.out_dt = out_dtype;
+  if (matmul_config) {
+    const char *why;
+    (void)apply_matmul_config(matmul_config, M, N, K, p, &why); // not usable: ignored, as in the reference
+  }
   return launched(gcmi_launch_gemm_int8(&p, (hipStream_t)stream), "gemm_int8");
 }
 

@@ -18,6 +18,13 @@ extern "C" int64_t gcmi_launch_gemm_bf16_workspace(const gcmi::GemmParams *p) {
   return want;
 }
 
+// what the launch above would choose (nothing is launched)
+extern "C" int gcmi_launch_gemm_bf16_config(const gcmi::GemmParams *p, gcmi::GemmTileConfig *cfg) {
+  if (gcmi::launch_skinny_nt(p, (hipStream_t)-1, nullptr, cfg) >= 0)
+    return 0;
+  return gcmi::launch_tile256<2>(p, (hipStream_t)-1, nullptr, cfg);
+}
+
 // Scratch of the entry point that allocates nothing (gcmi_gemm_bf16_noalloc): the partial sums of K-sliced calls.
 // Each device the library runs on holds its own copy until the process ends.  `scratch` is only a host-side
 // stand-in here: its device address is asked for once per device and kept.

@@ -32,6 +32,10 @@ using namespace gcmi;
 
 extern "C" int gcmi_launch_gemm_int8(const GemmParams *p, hipStream_t stream) { return launch_tile256<1>(p, stream); }
 
+extern "C" int gcmi_launch_gemm_int8_config(const GemmParams *p, GemmTileConfig *cfg) {
+  return launch_tile256<1>(p, (hipStream_t)-1, nullptr, cfg);
+}
+
 extern "C" int gcmi_launch_colsum_s8(const void *W, int64_t K, int64_t N, int64_t ldw, void *out, hipStream_t stream) {
   if (N <= 0)
     return 0;

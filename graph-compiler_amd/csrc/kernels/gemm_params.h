@@ -35,6 +35,33 @@ struct GemmParams {
   const void *residual; // null: none
   int64_t ldr;          // elements between its rows
   int32_t residual_dt;  // DT_BF16 or DT_F32
+  // wishes of the caller (the op's MatmulConfig attributes, translated): 0 = the launcher's own choice
+  int32_t cfg_waves;    // 4 or 8 waves per workgroup on whole tiles
+  int32_t cfg_split_k;  // number of K slices (1: none) where the shape can be sliced
+};
+
+// What the launcher decides for one GEMM call: the GPU's counterpart of the reference's MatmulConfig
+// (include/gc/Analysis/MatmulConfigAnalysis.h:25-34: thread split, L2 block, innermost block per dim), chosen per
+// (M, N, K, element type, layout) instead of by the CPU cost model.  Reported by dnnl_graph_compiler_explain.
+struct GemmTileConfig {
+  int32_t kernel;          // GemmKernel
+  int32_t bm, bn;          // workgroup tile (the reference's MBlock / NBlock)
+  int32_t kbytes;          // bytes of K per LDS stage and row (KBlock * element size)
+  int32_t stages;          // slots of the LDS ring
+  int32_t waves_m, waves_n; // waves of a workgroup along m and n
+  int32_t wave_m, wave_n;  // tile of one wave (the reference's innermost block: what one microkernel call covers)
+  int32_t mfma_m, mfma_n, mfma_k; // shape of the matrix instruction
+  int32_t split_k;         // K slices (the reference's KThreads); 1: none
+  int32_t group_m;         // tile rows an XCD walks before moving on (L2 locality)
+  int32_t workgroups;      // launched
+  int32_t from_attrs;      // 1: MatmulConfig attributes of the op were applied
+};
+enum GemmKernel : int32_t {
+  GK_EDGE = 0,    // bounds-checked 256x256 tile, 8 waves, 32x32 MFMAs: any shape and alignment
+  GK_WAVES8 = 1,  // whole tiles, 8 waves of 128 x 64, 16x16 MFMAs
+  GK_WAVES4 = 2,  // whole tiles, 4 waves of 128 x 128 (one per SIMD), 16x16 MFMAs, hand-placed main loop
+  GK_SPLITK = 3,  // one tile row: K slices over workgroups + second pass
+  GK_STREAM = 4,  // a short A against [N,K] weights: weight-streaming kernel (+ second pass)
 };
 
 struct F32GemmParams {

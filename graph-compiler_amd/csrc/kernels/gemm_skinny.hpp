@@ -164,10 +164,11 @@ template <int MT> __global__ __launch_bounds__(SK_WAVES * 64, 2) void gemm_skinn
 
 // Takes the call when the shape is this kernel's (returns -1 otherwise: the tile kernels handle it).
 // want != null: nothing is launched; *want receives the floats of workspace this call would use if it had them.
-static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream, int64_t *want = nullptr) {
+static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream, int64_t *want = nullptr, GemmTileConfig *cfg = nullptr) {
   GemmParams p = *pp;
   if (want)
     *want = 0;
+  const bool dry = want != nullptr || (cfg != nullptr && stream == (hipStream_t)-1);
   const int64_t ws_cap = want ? INT64_MAX : (p.partial ? p.partial_cap : 0);
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const int out_es = p.out_dt == DT_BF16 ? 2 : 4;
@@ -196,12 +197,25 @@ static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream, int64_t *w
     if (score > best_score + 1e-9)
       best_score = score, best = s;
   }
+  if (p.cfg_split_k > 0) { // the caller's slice count (its KThreads), as far as the shape and the workspace allow
+    int s = (p.cfg_split_k + SK_WAVES - 1) / SK_WAVES;
+    while (s > 1 && (steps / (s * SK_WAVES) < 2 || (int64_t)s * p.M * p.N > ws_cap))
+      s--;
+    best = s;
+  }
   if (steps / (best * SK_WAVES) < 2)
     return -1;
-  if (want) {
+  if (want)
     *want = best > 1 ? (int64_t)best * p.M * p.N : 0;
-    return 0;
+  if (cfg) {
+    GemmTileConfig c{};
+    c.kernel = GK_STREAM, c.bm = 32 * mt, c.bn = 32, c.kbytes = 128, c.stages = mt == 1 ? SK_DEPTH : 4;
+    c.waves_m = 1, c.waves_n = 1, c.wave_m = 32 * mt, c.wave_n = 32, c.mfma_m = c.mfma_n = 32, c.mfma_k = 16;
+    c.split_k = best * SK_WAVES, c.group_m = 1, c.workgroups = nblocks * best;
+    *cfg = c;
   }
+  if (dry)
+    return 0;
   p.splits = best;
   const dim3 grid((unsigned)(nblocks * best)), block(SK_WAVES * 64);
   if (mt == 1)

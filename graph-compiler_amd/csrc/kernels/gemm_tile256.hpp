@@ -32,7 +32,6 @@
 //                                        16-bit, 8 for 8-bit), CW = 16-byte
 //                                        chunks one read touches per row
 #pragma once
-#include <cstdlib>
 #include <type_traits>
 
 #include "common.hpp"
@@ -1616,10 +1615,13 @@ static void launch_splitk_reduce(const GemmParams &p, hipStream_t stream) {
 
 // Host-side launch of the 256x256 tile kernels for one element size.
 // want != null: nothing is launched; *want receives the floats of workspace this call would use if it had them.
-template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *want = nullptr) {
+// cfg != null: receives what was (or would be) chosen.
+template <int ES>
+static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *want = nullptr, GemmTileConfig *cfg = nullptr) {
   GemmParams p = *pp;
   if (want)
     *want = 0;
+  const bool dry = want != nullptr || (cfg != nullptr && stream == (hipStream_t)-1);
   const int64_t ws_cap = want ? INT64_MAX : (p.partial ? p.partial_cap : 0);
   float *const ws = p.partial;
   const int tiles_m = (int)((p.M + G_BM - 1) / G_BM), tiles_n = (int)((p.N + G_BN - 1) / G_BN);
@@ -1644,9 +1646,6 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   bool fast = fast_but_m && p.M % G_BM == 0;
   p.splits = 0;
   p.partial = nullptr;
-  // One tile row and too few column tiles to fill the GPU (decode-style shapes such as 32 x 4096 x 4096): the
-  // weights have to stream from HBM through all compute units, so K is cut into slices, one workgroup per
-  // (column tile, slice); partial sums go through the workspace and a small second kernel.
   const int64_t nbatch = p.batch > 1 ? p.batch : 1;
   if (nbatch > 65535)
     return 2;
@@ -1655,19 +1654,40 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   else if (!((p.a_bs * ES) % 16 == 0 && (p.b_bs * ES) % 16 == 0 && (p.c_bs * out_es) % 16 == 0 &&
              (!p.residual || (p.c_bs * res_es) % 16 == 0)))
     fast = false; // every batch's operands must keep the alignment the fast path loads with
+  if (p.group_m <= 0)
+    p.group_m = 4;
+  GemmTileConfig c{};
+  c.bm = G_BM, c.bn = G_BN, c.split_k = 1, c.group_m = p.group_m, c.workgroups = (int32_t)nblk;
+  c.from_attrs = (p.cfg_waves || p.cfg_split_k) ? 1 : 0;
+
+  // One tile row and too few column tiles to fill the GPU (decode-style shapes such as 32 x 4096 x 4096): the
+  // weights have to stream from HBM through all compute units, so K is cut into slices, one workgroup per
+  // (column tile, slice); partial sums go through the workspace and a small second kernel.  The slice count is the
+  // reference's KThreads (lib/gc/Analysis/MatmulConfigAnalysis.cpp:149-166); a caller's wish replaces the default.
   if (ES == 2 && fast_but_m && tiles_m == 1 && p.out_dt != DT_S32 && nbatch == 1) {
     const int n_cu = gcmi_num_cus();
     const int groups = (int)(p.K / KGROUP);
     int splits = (n_cu + tiles_n - 1) / tiles_n;
+    bool worth = tiles_n * 2 <= n_cu;
+    if (p.cfg_split_k > 0)
+      splits = p.cfg_split_k, worth = true;
     splits = splits < groups ? splits : groups;
     if (want) {
-      if (splits > 1 && tiles_n * 2 <= n_cu)
+      if (splits > 1 && worth)
         *want = (int64_t)splits * p.M * p.N;
-      return 0;
+      if (!cfg)
+        return 0;
     }
     while (splits > 1 && (int64_t)splits * p.M * p.N > ws_cap)
       splits--;
-    if (splits > 1 && tiles_n * 2 <= n_cu) {
+    if (splits > 1 && worth) {
+      c.kernel = GK_SPLITK, c.kbytes = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::KB, c.stages = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::NST;
+      c.waves_m = 2, c.waves_n = 8 / G_FAST_WJ, c.wave_m = 128, c.wave_n = 32 * G_FAST_WJ;
+      c.mfma_m = c.mfma_n = 32, c.mfma_k = 32 / ES, c.split_k = splits, c.workgroups = tiles_n * splits;
+      if (cfg)
+        *cfg = c;
+      if (dry)
+        return 0;
       p.splits = splits;
       p.partial = ws;
       if constexpr (ES == 2) {
@@ -1682,14 +1702,20 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
       return hipGetLastError() == hipSuccess ? 0 : 5;
     }
   }
-  if (want)
+  // Whole tiles: 4 waves of 128 x 128 unless the caller asks for 8 waves of 128 x 64 (or the result is an f32 / s32
+  // tensor of 8-bit operands, which only the 8-wave kernel writes).  Anything else: the bounds-checked kernel.
+  const bool w4_can = fast && (ES == 2 || p.out_dt == DT_BF16);
+  const bool use_w4 = w4_can && p.cfg_waves != 8;
+  c.kernel = !fast ? GK_EDGE : (use_w4 ? GK_WAVES4 : GK_WAVES8);
+  c.kbytes = fast ? 64 : G_KBYTES, c.stages = fast ? 4 : 2;
+  c.waves_m = 2, c.waves_n = use_w4 ? 2 : 4, c.wave_m = 128, c.wave_n = use_w4 ? 128 : 64;
+  c.mfma_m = c.mfma_n = fast ? 16 : 32, c.mfma_k = (fast ? 64 : 32) / ES;
+  if (cfg)
+    *cfg = c;
+  if (dry)
     return 0;
-  if (p.group_m <= 0)
-    p.group_m = 4;
   dim3 grid((unsigned)nblk, (unsigned)nbatch), block(G_THREADS);
-  const char *w4_env = getenv("GCMI_GEMM_W4");
-  const int use_w4 = w4_env ? atoi(w4_env) : 1;
-  if (fast && use_w4 && (ES == 2 || p.out_dt == DT_BF16)) {
+  if (use_w4) {
     if constexpr (ES == 2) {
       if (p.trans_b) {
         hipLaunchKernelGGL((gemm_tile256_w4_kernel<ES, true>), grid, dim3(256), 0, stream, p);
@@ -1701,22 +1727,15 @@ template <int ES> static int launch_tile256(const GemmParams *pp, hipStream_t st
   }
   if constexpr (ES == 2) {
     if (p.trans_b) {
-      if (fast && G_FAST_MI16)
+      if (fast)
         hipLaunchKernelGGL((gemm_tile256_mi16_kernel<ES, true>), grid, dim3(512), 0, stream, p);
-      else if (fast)
-        hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, false, true>), grid, dim3(1024 / G_FAST_WJ), 0,
-                           stream, p);
       else
         hipLaunchKernelGGL((gemm_tile256_kernel<ES, true, true>), grid, block, 0, stream, p);
       return hipGetLastError() == hipSuccess ? 0 : 5;
     }
   }
-  if (fast && G_FAST_MI16) {
-    hipLaunchKernelGGL(gemm_tile256_mi16_kernel<ES>, grid, dim3(512), 0, stream, p);
-    return hipGetLastError() == hipSuccess ? 0 : 5;
-  }
   if (fast)
-    hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ>), grid, dim3(1024 / G_FAST_WJ), 0, stream, p);
+    hipLaunchKernelGGL(gemm_tile256_mi16_kernel<ES>, grid, dim3(512), 0, stream, p);
   else
     hipLaunchKernelGGL((gemm_tile256_kernel<ES, true>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 5;

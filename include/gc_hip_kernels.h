@@ -128,7 +128,46 @@ size_t gcmi_gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans
 int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int64_t M, int64_t N, int64_t K,
                       int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
                       int trans_b, const void *bias, int bias_dtype, int act, const void *residual, int64_t ldr,
-                      int residual_dtype, int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
+                      int residual_dtype, int out_dtype, void *workspace, size_t workspace_bytes,
+                      const int64_t *matmul_config, void *stream);
+
+/*
+ * The tile descriptor: what the launcher chooses for a GEMM call, the GPU's
+ * counterpart of the reference's MatmulConfig (include/gc/Analysis/
+ * MatmulConfigAnalysis.h:25-34; chosen there by a CPU cost model,
+ * lib/gc/Analysis/MatmulConfigAnalysis.cpp:435-552, here per shape, element
+ * type and layout).  `kernel`: 0 bounds-checked tile (any shape), 1 whole
+ * tiles with 8 waves of 128 x 64, 2 whole tiles with 4 waves of 128 x 128,
+ * 3 K slices over workgroups + second pass (one tile row), 4 weight-streaming
+ * kernel (a short A against [N,K] weights).
+ *
+ * matmul_config (may be NULL) is the reference's per-op override: the nine
+ * integers {MThreads, NThreads, KThreads, MBlock, NBlock, KBlock,
+ * innermostMBlock, innermostNBlock, innermostKBlock} of the op's attributes
+ * (readConfigFromAttrs, MatmulConfigAnalysis.cpp:368-404: all nine or none;
+ * validateConfig, :40-65).  On the GPU they steer: MBlock x NBlock = the
+ * workgroup tile (256 x 256 is built), innermostMBlock x innermostNBlock = the
+ * tile of one wave (128 x 128: 4 waves per workgroup; 128 x 64: 8 waves),
+ * KThreads = the number of K slices where the shape is sliced.  A config that
+ * is invalid or names a tile that is not built is ignored, like an invalid one
+ * in the reference; gcmi_gemm_tile_config_query says why in `note`.
+ * gcmi_gemm_bf16_ws and gcmi_gemm_int8_cfg take the same nine integers.
+ */
+typedef struct gcmi_gemm_tile_config {
+  int32_t kernel;
+  int32_t bm, bn;           /* workgroup tile */
+  int32_t kbytes;           /* bytes of K per LDS stage and row */
+  int32_t stages;           /* slots of the LDS ring */
+  int32_t waves_m, waves_n; /* waves of a workgroup */
+  int32_t wave_m, wave_n;   /* tile of one wave */
+  int32_t mfma_m, mfma_n, mfma_k;
+  int32_t split_k;          /* K slices; 1: none */
+  int32_t group_m;          /* tile rows an XCD walks before moving on */
+  int32_t workgroups;
+  int32_t from_attrs;       /* 1: matmul_config was applied */
+} gcmi_gemm_tile_config;
+int gcmi_gemm_tile_config_query(int a_dtype, int64_t M, int64_t N, int64_t K, int trans_b, int out_dtype,
+                                const int64_t *matmul_config, gcmi_gemm_tile_config *out, char *note, size_t note_len);
 
 /*
  * gcmi_gemm_bf16 / gcmi_gemm_bf16_nt (trans_b) for callers that cannot
@@ -166,6 +205,11 @@ int gcmi_gemm_bf16_noalloc(const void *A, const void *B, void *C, int64_t M, int
 int gcmi_gemm_int8(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                    int64_t ldb, int64_t ldc, const int32_t *colsum, int32_t zp_a, const float *scale,
                    const float *bias, int act, int out_dtype, void *stream);
+
+/* gcmi_gemm_int8 with the op's MatmulConfig attributes (see gcmi_gemm_tile_config_query; NULL: none). */
+int gcmi_gemm_int8_cfg(const void *A, int a_dtype, const void *W, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                       int64_t ldb, int64_t ldc, const int32_t *colsum, int32_t zp_a, const float *scale,
+                       const float *bias, int act, int out_dtype, const int64_t *matmul_config, void *stream);
 
 /* Column sums of an s8 weight [K,N] into s32 [N]: the weight-only constant of
  * the compensation term (legacy/core/src/ops/matmul_core.cpp:546-557). */

@@ -47,6 +47,12 @@ def wl(gc):
 
 
 @pytest.fixture(scope="session")
+def ga(gc):
+    import importlib
+    return importlib.import_module("graph_compiler_amd.graph_api")
+
+
+@pytest.fixture(scope="session")
 def dev(gc):
     import torch
     assert torch.cuda.is_available(), "GPU tests need a GPU"

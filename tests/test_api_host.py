@@ -48,7 +48,7 @@ def test_every_reference_fixture_parses_and_plans(ga, name):
 
 def _steps(plan):
     """The launch lines of a plan (the last line reports the arena size)."""
-    return [ln for ln in plan.splitlines() if not ln.startswith("arena:")]
+    return [ln for ln in plan.splitlines() if not ln.startswith(("arena:", "  tile:"))]
 
 
 def test_fusion_plan_of_reference_mlp(ga):

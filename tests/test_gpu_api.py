@@ -255,7 +255,7 @@ def test_transposed_b_weight_needs_no_copy(ga, orc, wl, dev):
                     "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [N, K])],
                     "outputs": [ga._t(2, "bf16", [M, N])]}], [0, 1], [2])
     st, plan = ga.explain(g)
-    assert st == 0 and [ln for ln in plan.splitlines() if not ln.startswith("arena")] == ["gemm_bf16: MatMul"]
+    assert st == 0 and [ln for ln in plan.splitlines() if not ln.startswith(("arena", "  tile:"))] == ["gemm_bf16: MatMul"]
     out = torch.zeros(M, N, dtype=torch.bfloat16)
     _run(ga, g, [(0, x), (1, W)], [(2, out)])
     ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(x), wl.bf16_bits(W.t().contiguous())))
@@ -511,3 +511,34 @@ def test_execute_from_two_host_threads_on_one_executable(ga, dev):
     assert not errs, errs
     exe.close()
     comp.close()
+
+
+def test_matmul_config_attributes_change_the_kernel_not_the_result(ga, gc, orc, wl, dev):
+    """The op's nine MatmulConfig attributes (lib/gc/Analysis/MatmulConfigAnalysis.cpp:368-422) pick 8 waves of
+    128 x 64 in place of 4 waves of 128 x 128 -- the same products in the same order, so the same bits -- and the
+    number of K slices of a short A (another summation order: equal to rounding)."""
+    names = gc.MATMUL_CONFIG_NAMES
+
+    def run(M, K, N, cfg):
+        op = {"kind": "MatMul", "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [K, N])], "outputs": [ga._t(2, "bf16", [M, N])]}
+        if cfg:
+            op["attrs"] = {k: {"type": "s64", "value": v} for k, v in zip(names, cfg)}
+        torch.manual_seed(M + N)
+        A = (torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev)
+        B = (torch.randn(K, N) * 0.1).to(torch.bfloat16).to(dev)
+        out = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+        _run(ga, ga._graph([op], [0, 1], [2]), [(0, A), (1, B)], [(2, out)])
+        return A, B, out
+
+    A, B, dflt = run(512, 1024, 768, None)
+    _, _, w8 = run(512, 1024, 768, [2, 3, 1, 256, 256, 64, 128, 64, 32])
+    assert torch.equal(dflt.view(torch.int16), w8.view(torch.int16))
+    ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A.cpu()), wl.bf16_bits(B.cpu())))
+    assert_close(ref, dflt.float().cpu().numpy(), 1e-2, "default tile")
+    A, B, s16 = run(32, 4096, 4096, None)
+    _, _, s4 = run(32, 4096, 4096, [1, 16, 4, 256, 256, 64, 128, 128, 32])
+    _, _, s1 = run(32, 4096, 4096, [1, 16, 1, 256, 256, 64, 128, 128, 32])
+    ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A.cpu()), wl.bf16_bits(B.cpu())))
+    for name, got in (("16 slices", s16), ("4 slices", s4), ("no slices", s1)):
+        assert_close(ref, got.float().cpu().numpy(), 1e-2, name)
+    assert not torch.equal(s16.view(torch.int16), s1.view(torch.int16))  # another summation order did run

@@ -22,7 +22,7 @@ def mm(gc):
 
 
 def _steps(plan):
-    return [ln for ln in plan.splitlines() if not ln.startswith(("arena:", "target hints"))]
+    return [ln for ln in plan.splitlines() if not ln.startswith(("arena:", "target hints", "  tile:"))]
 
 
 def test_mlp_pattern_fuses_bias_and_activation_into_the_gemm(ga, mm):
