@@ -40,6 +40,40 @@ void remember(const char *what) {
 
 extern "C" const char *dnnl_graph_compiler_last_error(void) { return g_last_error.c_str(); }
 
+// No exception crosses the C ABI.  The mapping of the reference (src/dnnl/dnnl_graph_compiler.cpp:190-226): bad
+// input -> invalid_graph (compile) / invalid_arguments (execute), unsupported -> unimplemented, bad_alloc ->
+// out_of_memory, anything else -> runtime_error.
+namespace {
+template <typename F> dnnl_status_t guarded(dnnl_status_t on_invalid_argument, F &&body) {
+  try {
+    body();
+    return dnnl_success;
+  } catch (const std::invalid_argument &e) {
+    remember(e.what());
+    return on_invalid_argument;
+  } catch (const std::logic_error &e) {
+    remember(e.what());
+    return dnnl_unimplemented;
+  } catch (const std::bad_alloc &) {
+    remember("out of memory");
+    return dnnl_out_of_memory;
+  } catch (const std::exception &e) {
+    remember(e.what());
+    return dnnl_runtime_error;
+  } catch (...) {
+    remember("unknown error");
+    return dnnl_runtime_error;
+  }
+}
+void copy_out(const std::string &d, char *buf, size_t len) {
+  if (buf && len) {
+    const size_t n = d.size() < len - 1 ? d.size() : len - 1;
+    memcpy(buf, d.data(), n);
+    buf[n] = 0;
+  }
+}
+} // namespace
+
 extern "C" const dnnl_graph_compiler_version *dnnl_graph_compiler_get_version(void) {
   static const dnnl_graph_compiler_version ver = {
       {DNNL_GC_API_V_MAJOR, DNNL_GC_API_V_MINOR, DNNL_GC_API_V_PATCH, DNNL_GC_API_V_HASH}, // API version (oneDNN's)
@@ -68,25 +102,7 @@ extern "C" dnnl_status_t dnnl_graph_compiler_compile(const dnnl_graph_compiler *
                                                      const dnnl_graph_compiler_executable **exe) {
   if (!gc || !exe)
     return dnnl_invalid_arguments;
-  try {
-    *exe = new dnnl_graph_compiler_executable(graph_json);
-    return dnnl_success;
-  } catch (const std::invalid_argument &e) {
-    remember(e.what());
-    return dnnl_invalid_graph;
-  } catch (const std::logic_error &e) {
-    remember(e.what());
-    return dnnl_unimplemented;
-  } catch (const std::bad_alloc &) {
-    remember("out of memory");
-    return dnnl_out_of_memory;
-  } catch (const std::exception &e) {
-    remember(e.what());
-    return dnnl_runtime_error;
-  } catch (...) {
-    remember("unknown error");
-    return dnnl_runtime_error;
-  }
+  return guarded(dnnl_invalid_graph, [&] { *exe = new dnnl_graph_compiler_executable(graph_json); });
 }
 
 // The same for a module in MLIR's textual form (what the reference's gc-cpu-runner and benchgc's
@@ -95,25 +111,7 @@ extern "C" dnnl_status_t dnnl_graph_compiler_compile_mlir(const dnnl_graph_compi
                                                           const dnnl_graph_compiler_executable **exe) {
   if (!gc || !exe)
     return dnnl_invalid_arguments;
-  try {
-    *exe = new dnnl_graph_compiler_executable(gcapi::parse_mlir(module_text));
-    return dnnl_success;
-  } catch (const std::invalid_argument &e) {
-    remember(e.what());
-    return dnnl_invalid_graph;
-  } catch (const std::logic_error &e) {
-    remember(e.what());
-    return dnnl_unimplemented;
-  } catch (const std::bad_alloc &) {
-    remember("out of memory");
-    return dnnl_out_of_memory;
-  } catch (const std::exception &e) {
-    remember(e.what());
-    return dnnl_runtime_error;
-  } catch (...) {
-    remember("unknown error");
-    return dnnl_runtime_error;
-  }
+  return guarded(dnnl_invalid_graph, [&] { *exe = new dnnl_graph_compiler_executable(gcapi::parse_mlir(module_text)); });
 }
 
 extern "C" void dnnl_graph_compiler_destroy_executable(const dnnl_graph_compiler_executable *exe) { delete exe; }
@@ -123,20 +121,10 @@ extern "C" dnnl_status_t dnnl_graph_compiler_execute(const dnnl_graph_compiler_e
                                                      dnnl_graph_compiler_tensor *outputs) {
   if (!exe)
     return dnnl_invalid_arguments;
-  try {
-    // the executable keeps per-call pointer tables: one execute at a time per executable
-    const_cast<dnnl_graph_compiler_executable *>(exe)->impl.execute(inputs, outputs);
-    return dnnl_success;
-  } catch (const std::bad_alloc &) {
-    remember("out of memory");
-    return dnnl_out_of_memory;
-  } catch (const std::exception &e) {
-    remember(e.what());
-    return dnnl_runtime_error;
-  } catch (...) {
-    remember("unknown error");
-    return dnnl_runtime_error;
-  }
+  // like the reference's, this may be called from several threads; calls on one executable take turns inside.
+  // A missing tensor is a runtime error here, as there (the reference's execute maps every exception to it, :214-226)
+  return guarded(dnnl_runtime_error,
+                 [&] { const_cast<dnnl_graph_compiler_executable *>(exe)->impl.execute(inputs, outputs); });
 }
 
 extern "C" dnnl_status_t dnnl_graph_compiler_execute_async(const dnnl_graph_compiler_executable *exe,
@@ -144,129 +132,38 @@ extern "C" dnnl_status_t dnnl_graph_compiler_execute_async(const dnnl_graph_comp
                                                            dnnl_graph_compiler_tensor *outputs, void *stream) {
   if (!exe)
     return dnnl_invalid_arguments;
-  try {
+  return guarded(dnnl_invalid_arguments, [&] {
     const_cast<dnnl_graph_compiler_executable *>(exe)->impl.execute_async(inputs, outputs, (hipStream_t)stream);
-    return dnnl_success;
-  } catch (const std::invalid_argument &e) {
-    remember(e.what());
-    return dnnl_invalid_arguments;
-  } catch (const std::bad_alloc &) {
-    remember("out of memory");
-    return dnnl_out_of_memory;
-  } catch (const std::exception &e) {
-    remember(e.what());
-    return dnnl_runtime_error;
-  } catch (...) {
-    remember("unknown error");
-    return dnnl_runtime_error;
-  }
-}
-
-// Introspection for tests: the launch plan of a compiled partition, one line
-// per kernel, written into buf (truncated to len-1 characters).
-extern "C" __attribute__((visibility("default"))) size_t gc_executable_describe(const dnnl_graph_compiler_executable *exe,
-                                                                               char *buf, size_t len) {
-  if (!exe)
-    return 0;
-  std::string d = exe->impl.describe();
-  if (buf && len) {
-    size_t n = d.size() < len - 1 ? d.size() : len - 1;
-    memcpy(buf, d.data(), n);
-    buf[n] = 0;
-  }
-  return d.size();
+  });
 }
 
 // Parse, verify and plan a partition without touching the GPU; writes the
 // launch plan into buf and returns the status compile would have returned for
 // the host-side stages.
 extern "C" dnnl_status_t dnnl_graph_compiler_explain(const char *graph_json, char *buf, size_t len) {
-  try {
-    gcapi::Executable e(graph_json, true);
-    std::string d = e.describe();
-    if (buf && len) {
-      size_t n = d.size() < len - 1 ? d.size() : len - 1;
-      memcpy(buf, d.data(), n);
-      buf[n] = 0;
-    }
-    return dnnl_success;
-  } catch (const std::invalid_argument &e) {
-    remember(e.what());
-    return dnnl_invalid_graph;
-  } catch (const std::logic_error &e) {
-    remember(e.what());
-    return dnnl_unimplemented;
-  } catch (const std::bad_alloc &) {
-    return dnnl_out_of_memory;
-  } catch (const std::exception &e) {
-    remember(e.what());
-    return dnnl_runtime_error;
-  } catch (...) {
-    return dnnl_runtime_error;
-  }
+  return guarded(dnnl_invalid_graph, [&] { copy_out(gcapi::Executable(graph_json, true).describe(), buf, len); });
 }
 
 extern "C" dnnl_status_t dnnl_graph_compiler_explain_mlir(const char *module_text, char *buf, size_t len) {
-  try {
-    gcapi::Executable e(gcapi::parse_mlir(module_text), true);
-    std::string d = e.describe();
-    if (buf && len) {
-      size_t n = d.size() < len - 1 ? d.size() : len - 1;
-      memcpy(buf, d.data(), n);
-      buf[n] = 0;
-    }
-    return dnnl_success;
-  } catch (const std::invalid_argument &e) {
-    remember(e.what());
-    return dnnl_invalid_graph;
-  } catch (const std::logic_error &e) {
-    remember(e.what());
-    return dnnl_unimplemented;
-  } catch (const std::bad_alloc &) {
-    return dnnl_out_of_memory;
-  } catch (const std::exception &e) {
-    remember(e.what());
-    return dnnl_runtime_error;
-  } catch (...) {
-    return dnnl_runtime_error;
-  }
+  return guarded(dnnl_invalid_graph,
+                 [&] { copy_out(gcapi::Executable(gcapi::parse_mlir(module_text), true).describe(), buf, len); });
 }
 
 extern "C" dnnl_status_t dnnl_graph_compiler_generated_source_mlir(const char *module_text, const char *check_arch, char *buf,
                                                                    size_t len) {
-  try {
+  return guarded(dnnl_invalid_graph, [&] {
     gcapi::Executable e(gcapi::parse_mlir(module_text), true);
     const std::vector<gcjit::FusedKernelSource> ks = e.generated_kernels();
     std::string d;
     for (const auto &k : ks)
       d += k.source + "\n";
-    if (buf && len) {
-      size_t n = d.size() < len - 1 ? d.size() : len - 1;
-      memcpy(buf, d.data(), n);
-      buf[n] = 0;
-    }
+    copy_out(d, buf, len);
     if (check_arch && !ks.empty()) {
       const std::string log = gcjit::compile_only(ks, check_arch);
-      if (!log.empty()) {
-        remember(log.c_str());
-        return dnnl_runtime_error;
-      }
+      if (!log.empty())
+        throw std::runtime_error(log);
     }
-    return dnnl_success;
-  } catch (const std::invalid_argument &e) {
-    remember(e.what());
-    return dnnl_invalid_graph;
-  } catch (const std::logic_error &e) {
-    remember(e.what());
-    return dnnl_unimplemented;
-  } catch (const std::bad_alloc &) {
-    return dnnl_out_of_memory;
-  } catch (const std::exception &e) {
-    remember(e.what());
-    return dnnl_runtime_error;
-  } catch (...) {
-    return dnnl_runtime_error;
-  }
+  });
 }
 
 extern "C" long dnnl_graph_compiler_generated_kernel_launches(void) { return gcapi::Executable::generated_launches(); }
