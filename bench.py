@@ -107,10 +107,12 @@ def time_launches(torch, fn, nsets, steps, warmup):
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script with
 # --copy-calibration: a 1 GiB copy reads FETCH_SIZE = 524304 KiB (scale 2.0)
 # and WRITE_SIZE = 1048580 KiB (scale 1.0).
-TRAFFIC = {  # (bytes per launch, the committed profile they come from)
-    "gemm": (int((98541.8 * 2.0 + 32791.1) * 1024), "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
-    "int8": (int((144003.5 * 2.0 + 88175.4) * 1024), "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
-    "mha": (int((129697.3 * 2.0 + 65681.9) * 1024), "profiles/mha_fwd_fast_b4_h32_s2048_d128_every_block.md"),
+TRAFFIC = {  # (bytes per launch of the dominant kernel, the committed profile they come from)
+    "gemm": (235363595, "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
+    "int8": (384729793, "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
+    "chain": (685777635 + 575093617, "profiles/gemm_tile256_w4_bf16_mlp_chain.md"),  # both launches
+    "mha": (367382197, "profiles/mha_fwd_fast_b4_h32_s2048_d128_every_block.md"),
+    "mha_skip": (333763838, "profiles/mha_fwd_fast_b4_h32_s2048_d128.md"),
 }
 
 
@@ -291,7 +293,7 @@ def main():
         others["bf16_mlp_chain"] = {"workload": "x[4096x4096] -> W1[4096x11008]+ReLU -> W2[11008x4096]+bias, bf16",
                                     "value": round(ops / t["ms_per_step"] / 1e9, 2), "unit": "TFLOP/s", "dtype": "bf16",
                                     "ms_per_step": round(t["ms_per_step"], 5),
-                                    "roofline": roofline(ops, t["ms_per_step"], PEAK["bf16"]),
+                                    "roofline": roofline(ops, t["ms_per_step"], PEAK["bf16"], TRAFFIC["chain"]),
                                     "kernel_ms": {k: round(v, 5) for k, v in t.items()}}
         log("bf16 mlp chain: %.4f ms  %.1f TFLOP/s" % (t["ms_per_step"], ops / t["ms_per_step"] / 1e9))
         if not args.no_cpu:
@@ -336,7 +338,7 @@ def main():
                 "ms_per_step": round(t["ms_per_step"], 5),
                 "effective_value_dense_count": round(ops / t["ms_per_step"] / 1e9, 2),
                 "executed_ops": ops * frac_exec,
-                "roofline_executed_ops": roofline(ops * frac_exec, t["ms_per_step"], PEAK["bf16"]),
+                "roofline_executed_ops": roofline(ops * frac_exec, t["ms_per_step"], PEAK["bf16"], TRAFFIC["mha_skip"]),
                 "kernel_ms": {k: round(v, 5) for k, v in t.items()}}
             log("bf16 mha, masked blocks skipped: %.4f ms  %.1f TFLOP/s dense count, %.1f TFLOP/s executed" %
                 (t["ms_per_step"], ops / t["ms_per_step"] / 1e9, ops * frac_exec / t["ms_per_step"] / 1e9))
