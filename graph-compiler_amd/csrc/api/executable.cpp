@@ -203,13 +203,36 @@ void Executable::init(bool dry) {
   layout_arena();
   if (dry)
     return;
-  hip_check(hipMalloc((void **)&arena_, arena_bytes_), "hipMalloc(arena)");
-  hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
-  for (auto &s : slots_)
-    if (!s.init.empty())
-      hip_check(hipMemcpy(arena_ + s.offset, s.init.data(), s.init.size(), hipMemcpyHostToDevice), "upload constants");
-  ptr_.resize(slots_.size());
-  build_generated_kernels();
+  try { // a constructor that throws runs no destructor: what has been acquired is given back here
+    hip_check(hipMalloc((void **)&arena_, arena_bytes_), "hipMalloc(arena)");
+    hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
+    for (auto &s : slots_)
+      if (!s.init.empty())
+        hip_check(hipMemcpy(arena_ + s.offset, s.init.data(), s.init.size(), hipMemcpyHostToDevice), "upload constants");
+    ptr_.resize(slots_.size());
+    build_generated_kernels();
+  } catch (...) {
+    release();
+    throw;
+  }
+}
+
+void Executable::release() noexcept {
+  if (once_done_)
+    (void)hipEventDestroy(once_done_);
+  if (stream_)
+    (void)hipStreamDestroy(stream_);
+  if (arena_)
+    (void)hipFree(arena_);
+  if (staging_)
+    (void)hipFree(staging_);
+  once_done_ = nullptr, stream_ = nullptr, arena_ = nullptr, staging_ = nullptr;
+}
+
+char *Executable::staging() {
+  if (!staging_)
+    hip_check(hipMalloc((void **)&staging_, staging_bytes_ ? staging_bytes_ : 256), "hipMalloc(staging for host buffers)");
+  return staging_;
 }
 
 // Scratch of the steps whose kernels need some (partial sums of K-sliced GEMMs, mask tile classes of attention): a
@@ -254,11 +277,25 @@ void Executable::layout_arena() {
       if (s.out >= 0)
         pinned[s.out] = 1;
   }
-  for (int i = 0; i < n; i++)
-    if (slots_[i].is_input || slots_[i].is_output || !slots_[i].init.empty() || first[i] < 0)
+  // Graph inputs and outputs are the caller's buffers: a device pointer is used in place, and only a host buffer
+  // needs a device copy -- those copies live in a block of their own that the first such execute allocates.
+  // (An output that a once-only step computes stays in the arena: it is written once and copied out per call.)
+  size_t stage_off = 0;
+  for (int i = 0; i < n; i++) {
+    Slot &sl = slots_[i];
+    sl.staged = (sl.is_input || sl.is_output) && sl.init.empty() && !pinned[i];
+    if (sl.staged) {
+      sl.offset = stage_off;
+      stage_off += align256(sl.bytes);
+    } else if (sl.is_input || sl.is_output || !sl.init.empty() || first[i] < 0) {
       pinned[i] = 1;
+    }
+  }
+  staging_bytes_ = stage_off;
   size_t off = 0, naive = 0;
   for (int i = 0; i < n; i++) {
+    if (slots_[i].staged)
+      continue;
     naive += align256(slots_[i].bytes);
     if (pinned[i]) {
       slots_[i].offset = off;
@@ -268,7 +305,7 @@ void Executable::layout_arena() {
   const size_t temp_base = off;
   std::vector<int> order;
   for (int i = 0; i < n; i++)
-    if (!pinned[i])
+    if (!pinned[i] && !slots_[i].staged)
       order.push_back(i);
   std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return first[x] < first[y]; });
   std::vector<int> placed;
@@ -295,14 +332,7 @@ void Executable::layout_arena() {
   arena_bytes_no_reuse_ = naive ? naive : 256;
 }
 
-Executable::~Executable() {
-  if (once_done_)
-    (void)hipEventDestroy(once_done_);
-  if (stream_)
-    (void)hipStreamDestroy(stream_);
-  if (arena_)
-    (void)hipFree(arena_);
-}
+Executable::~Executable() { release(); }
 
 // ---------------------------------------------------------------------------
 void Executable::plan() {
@@ -1615,7 +1645,11 @@ void Executable::run(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_ten
     throw std::invalid_argument("Tensor not found");
   };
   for (size_t s = 0; s < slots_.size(); s++)
-    ptr_[s] = arena_ + slots_[s].offset;
+    ptr_[s] = slots_[s].staged ? nullptr : arena_ + slots_[s].offset;
+  auto staged_ptr = [&](int slot) -> void * {
+    const Slot &sl = slots_[(size_t)slot];
+    return sl.staged ? (void *)(staging() + sl.offset) : (void *)(arena_ + sl.offset);
+  };
 
   // inputs: device pointers are used in place, host buffers are staged
   for (size_t i = 0; i < g_.input_ids.size(); i++) {
@@ -1627,13 +1661,18 @@ void Executable::run(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_ten
     for (size_t s = 0; s < slots_.size(); s++)
       if (slots_[s].is_input && slots_[s].tensor_id == (long)id)
         slot = (int)s;
-    if (slot < 0 || !t->data)
+    if (slot < 0)
       continue;
+    if (!t->data) { // nothing to read: the kernels still get an address of the right size
+      ptr_[(size_t)slot] = staged_ptr(slot);
+      continue;
+    }
     if (is_device_pointer(t->data)) {
       ptr_[(size_t)slot] = t->data;
     } else {
       if (!wait)
         throw std::invalid_argument("execute_async: input " + std::to_string(id) + " is not a device pointer");
+      ptr_[(size_t)slot] = staged_ptr(slot);
       // a constant keeps its first contents: staged once
       const bool constant = g_.tensors.at(id).constant;
       if (const_staged_.size() < slots_.size())
@@ -1656,10 +1695,13 @@ void Executable::run(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_ten
     bool also_input = slots_[(size_t)slot].is_input;
     if (!wait && !is_device_pointer(t->data))
       throw std::invalid_argument("execute_async: output " + std::to_string(id) + " is not a device pointer");
-    if (is_device_pointer(t->data) && !also_input)
+    if (is_device_pointer(t->data) && !also_input && slots_[(size_t)slot].staged) {
       ptr_[(size_t)slot] = t->data;
-    else
+    } else {
+      if (!ptr_[(size_t)slot])
+        ptr_[(size_t)slot] = staged_ptr(slot);
       copy_back.emplace_back(t->data, slot);
+    }
   }
   if (step_done_.size() < steps_.size())
     step_done_.resize(steps_.size(), 0);
@@ -1725,7 +1767,8 @@ std::string Executable::describe() const {
       os << " " << h.first << "=" << h.second;
     os << "\n";
   }
-  os << "arena: " << arena_bytes_ << " bytes (" << arena_bytes_no_reuse_ << " with one region per buffer)\n";
+  os << "arena: " << arena_bytes_ << " bytes (" << arena_bytes_no_reuse_ << " with one region per buffer); staging for host buffers: "
+     << staging_bytes_ << " bytes, allocated by the first execute that passes one\n";
   return os.str();
 }
 

@@ -87,7 +87,8 @@ struct Step {
 
 struct Slot {
   size_t bytes = 0;
-  size_t offset = 0;   // into the arena
+  size_t offset = 0;   // into the arena, or into the staging block when `staged`
+  bool staged = false; // a graph input / output that the caller's device pointer replaces: no arena space (executable.cpp, layout_arena)
   long tensor_id = -1; // graph tensor it holds, -1 for temporaries / constants
   bool is_input = false, is_output = false;
   std::vector<char> init; // constant contents uploaded at compile time
@@ -131,6 +132,12 @@ private:
   char *arena_ = nullptr;
   size_t arena_bytes_ = 0;
   size_t arena_bytes_no_reuse_ = 0; // what one region per slot would take
+  // device copies of the caller's HOST buffers (graph inputs and outputs): one block, allocated by the first
+  // execute that passes a host pointer -- a caller that keeps its tensors on the device never pays for it
+  char *staging_ = nullptr;
+  size_t staging_bytes_ = 0;
+  char *staging();
+  void release() noexcept;
   hipStream_t stream_ = nullptr;
   std::unordered_map<int, bool> colsum_valid_; // ColSum results of constant weights are computed once
   std::vector<char> step_done_;                // per step: a `once` step has run

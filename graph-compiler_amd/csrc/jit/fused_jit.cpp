@@ -4,6 +4,7 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
+#include <deque>
 #include <map>
 #include <mutex>
 
@@ -57,11 +58,30 @@ bool compile(const std::string &src, const std::string &arch, std::vector<char> 
 }
 
 std::mutex g_mu;
-// "<device>|<source>" -> module.  Never destroyed: its modules would be unloaded during static destruction, when the
-// HIP runtime may already be gone.
-std::map<std::string, std::shared_ptr<Module>> &cache() {
-  static auto *c = new std::map<std::string, std::shared_ptr<Module>>();
+// "<device>|<source>" -> module.  The map holds weak references: a module is unloaded when the last executable
+// that uses it goes away and it has dropped out of the short list of recently built ones (kept so that compiling
+// the same partition again right after destroying it does not cost another run of the compiler).  Neither
+// container is ever destroyed: modules must not be unloaded during static destruction, when the HIP runtime may
+// already be gone.
+constexpr size_t kRecentModules = 32;
+std::map<std::string, std::weak_ptr<Module>> &cache() {
+  static auto *c = new std::map<std::string, std::weak_ptr<Module>>();
   return *c;
+}
+std::deque<std::shared_ptr<Module>> &recent() {
+  static auto *r = new std::deque<std::shared_ptr<Module>>();
+  return *r;
+}
+void remember(const std::shared_ptr<Module> &m) { // g_mu held
+  auto &r = recent();
+  for (auto it = r.begin(); it != r.end(); ++it)
+    if (*it == m) {
+      r.erase(it);
+      break;
+    }
+  r.push_back(m);
+  while (r.size() > kRecentModules)
+    r.pop_front();
 }
 
 } // namespace
@@ -93,8 +113,13 @@ std::shared_ptr<Module> Module::build(const std::vector<FusedKernelSource> &kern
   const std::string src = full_source(kernels), key = std::to_string(dev) + "|" + src;
   std::lock_guard<std::mutex> lock(g_mu);
   auto it = cache().find(key);
-  if (it != cache().end())
-    return it->second;
+  if (it != cache().end()) {
+    if (auto alive = it->second.lock()) {
+      remember(alive);
+      return alive;
+    }
+    cache().erase(it);
+  }
   std::vector<char> code;
   if (!compile(src, prop.gcnArchName, code, error))
     return nullptr;
@@ -104,7 +129,10 @@ std::shared_ptr<Module> Module::build(const std::vector<FusedKernelSource> &kern
     error = "hipModuleLoadData failed";
     return nullptr;
   }
+  for (auto e = cache().begin(); e != cache().end();) // entries whose module is gone
+    e = e->second.expired() ? cache().erase(e) : std::next(e);
   cache()[key] = m;
+  remember(m);
   return m;
 }
 

@@ -164,12 +164,15 @@ def test_arena_shares_memory_between_temporaries_with_disjoint_lifetimes(ga):
                     "outputs": [ga._t(10 + i, "bf16", [M, M])]})
     st, plan = ga.explain(ga._graph(ops, [0, 1, 2, 3, 4], [13]))
     assert st == 0, plan
-    m = re.search(r"arena: (\d+) bytes \((\d+) with one region per buffer\)", plan)
+    m = re.search(r"arena: (\d+) bytes \((\d+) with one region per buffer\); staging for host buffers: (\d+) bytes", plan)
     assert m, plan
-    shared, naive = int(m.group(1)), int(m.group(2))
+    shared, naive, staging = int(m.group(1)), int(m.group(2)), int(m.group(3))
     one = M * M * 2
-    assert naive == 9 * one          # 5 inputs + 3 temporaries + 1 output
-    assert shared == 8 * one         # t3 reuses t1's region
+    assert naive == 3 * one          # the 3 temporaries
+    assert shared == 2 * one         # t3 reuses t1's region
+    # the 5 inputs and the output are the caller's buffers: device copies exist only for host pointers, in a block
+    # of their own that the first such execute allocates
+    assert staging == 6 * one
 
 
 def test_k_sliced_matmuls_get_scratch_of_their_own_in_the_arena(ga, gc):
@@ -183,10 +186,11 @@ def test_k_sliced_matmuls_get_scratch_of_their_own_in_the_arena(ga, gc):
             "outputs": [ga._t(11, "bf16", [M, K])]}]
     st, plan = ga.explain(ga._graph(ops, [0, 1, 2], [11]))
     assert st == 0, plan
-    m = re.search(r"arena: (\d+) bytes \((\d+) with one region per buffer\)", plan)
-    shared, naive = int(m.group(1)), int(m.group(2))
+    m = re.search(r"arena: (\d+) bytes \((\d+) with one region per buffer\); staging for host buffers: (\d+) bytes", plan)
+    shared, naive, staging = int(m.group(1)), int(m.group(2)), int(m.group(3))
     ws = gc.lib().gcmi_gemm_bf16_workspace_bytes(M, N, K, 0)
     assert ws >= 2 * M * N * 4      # at least two slices of f32 partial sums
-    tensors = 2 * M * K * 2 + 2 * K * N * 2 + M * N * 2
-    assert naive == tensors + 2 * ws
-    assert shared == tensors + ws   # the second step's scratch takes the place of the first's
+    hidden = M * N * 2
+    assert naive == hidden + 2 * ws
+    assert shared == hidden + ws    # the second step's scratch takes the place of the first's
+    assert staging == 2 * M * K * 2 + 2 * K * N * 2   # A, both weights, the result
