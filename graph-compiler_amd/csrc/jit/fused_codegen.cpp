@@ -1,5 +1,6 @@
 // HIP source for one fused point-wise group (see fused_jit.h).  The code follows, statement by statement, what
 // fused_pointwise_kernel / fused_rowsum_kernel (kernels/eltwise.hip) do for the same parameter block.
+#include <cstdlib>
 #include <cstdio>
 #include <cstring>
 #include <sstream>
