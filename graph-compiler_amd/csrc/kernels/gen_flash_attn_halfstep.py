@@ -29,7 +29,9 @@ Wait states kept by construction (the assembler does not add them inside an asm 
   LDS data        -> MFMA       s_waitcnt lgkmcnt(n), counted here
   vector ALU      -> MFMA read  at least two instructions in between
   exp2            -> its reader at least one instruction in between
-  MFMA result     -> vector ALU read   at least four MFMAs (128 cycles) in between (the maximum of `next`)
+  MFMA result     -> vector ALU read   at least four MFMAs (128 cycles) in between (the maximum of `next`); after
+                                       the last MFMA of the statement 11 wait states, for whatever the compiler
+                                       places behind it
 """
 import os
 import sys
@@ -123,10 +125,18 @@ def gen(cur, nxt):
             read_v((slot - 2) // 4, (slot - 2) % 4)
         for ins in take(per_slot[slot]):
             emit(ins)
-        if slot >= 11:
+        if 11 <= slot <= 13:
             for ins in mx[:2]:
                 emit(ins)
             del mx[:2]
+    # After the last MFMA: the rest of the maximum, then enough wait states that ANY instruction the compiler puts
+    # behind this statement may touch the accumulators (it does not know that MFMAs wrote them: an 8-pass MFMA's
+    # result needs 11 wait states before a vector instruction reads or overwrites it).  These issue while the last
+    # MFMA still holds the matrix pipe, so they cost nothing.
+    for ins in mx:
+        emit(ins)
+    del mx[:]
+    emit("s_nop 7")
     assert not q and not mx, (q, mx)
     if OPTS:
         def keep(ins):
