@@ -98,16 +98,20 @@ int ws_acquire(size_t bytes, hipStream_t stream, LibraryWorkspace **out, void **
     w.mu.unlock();
     return fail(ST_RUNTIME, "workspace: hipEventCreate failed");
   }
-  if (w.used && w.last != stream && hipStreamWaitEvent(stream, w.done, 0) != hipSuccess) {
-    w.mu.unlock();
-    return fail(ST_RUNTIME, "workspace: hipStreamWaitEvent failed");
+  // A caller on another stream than the last user's waits for everything that stream has been given so far (the
+  // marker is recorded now, behind the last user's kernels: nothing is recorded per call, so a single-stream caller
+  // pays for no event).  A stream that no longer exists: wait for the device.
+  if (w.used && w.last != stream) {
+    if (hipEventRecord(w.done, w.last) != hipSuccess || hipStreamWaitEvent(stream, w.done, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      (void)hipDeviceSynchronize();
+    }
   }
   *out = &w, *ptr = w.ptr;
   return ST_OK;
 }
 void ws_release(LibraryWorkspace *w, hipStream_t stream) {
-  if (hipEventRecord(w->done, stream) == hipSuccess)
-    w->used = true, w->last = stream;
+  w->used = true, w->last = stream;
   w->mu.unlock();
 }
 } // namespace
