@@ -111,8 +111,8 @@ TRAFFIC = {  # (bytes per launch of the dominant kernel, the committed profile t
     "gemm": (235363595, "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
     "int8": (384729793, "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
     "chain": (685777635 + 575093617, "profiles/gemm_tile256_w4_bf16_mlp_chain.md"),  # both launches
-    "mha": (367382197, "profiles/mha_fwd_fast_b4_h32_s2048_d128_every_block.md"),
-    "mha_skip": (333763838, "profiles/mha_fwd_fast_b4_h32_s2048_d128.md"),
+    "mha": (366467595, "profiles/mha_fwd_fast_b4_h32_s2048_d128_every_block.md"),
+    "mha_skip": (335089174, "profiles/mha_fwd_fast_b4_h32_s2048_d128.md"),
 }
 
 
