@@ -404,6 +404,29 @@ def main():
                                           "ms_per_step": round(t["ms_per_step"], 5),
                                           "value": round(2.0 * 128 * 512 * 256 / t["ms_per_step"] / 1e9, 4), "unit": "TFLOP/s"}
 
+    # ---------------- the microkernel ABI (dnnl_brgemm_*, device pointers) at the size the reference's nest calls it with
+    if want("brgemm"):
+        import ctypes as C
+        L = gc.lib()
+        legs = {}
+        for name, dtA, dtB, es, Kk in (("f32", 3, 3, 4, 32), ("bf16_vnni2", 2, 2, 2, 32), ("u8s8_vnni4", 6, 5, 1, 64)):
+            Mb = Nb = 32
+            num = 16
+            Ab = torch.randint(0, 120, (num * Mb * Kk * es,), dtype=torch.uint8, device=dev)
+            Bb = torch.randint(0, 120, (num * Kk * Nb * es,), dtype=torch.uint8, device=dev)
+            Cb = torch.zeros(Mb * Nb, dtype=torch.int32, device=dev)
+            h = L.dnnl_brgemm_dispatch(Mb, Nb, Kk, Kk, Nb, Nb, Mb * Kk, Kk * Nb, 0.0, dtA, dtB)
+            a, b, c = C.c_void_p(Ab.data_ptr()), C.c_void_p(Bb.data_ptr()), C.c_void_p(Cb.data_ptr())
+            t = time_launches(torch, lambda i: L.dnnl_brgemm_execute(h, a, 0, b, 0, c, 0, num), 1, K, W)
+            legs[name] = {"M": Mb, "N": Nb, "K": Kk, "num": num, "us_per_call": round(t["ms_per_step"] * 1e3, 2),
+                          "GFLOP/s": round(2.0 * Mb * Nb * Kk * num / t["ms_per_step"] / 1e6, 1)}
+        others["brgemm_microkernel_abi"] = {
+            "workload": "one dnnl_brgemm_execute per step: 32x32 C tile, batch of 16 K blocks (the call the reference's "
+                        "deep-tile nest makes per innermost tile); launch bound by construction -- the GPU path of the "
+                        "nest is the whole-problem kernel above, this ABI exists for callers that bind the microkernel",
+            "legs": legs}
+        log("brgemm microkernel: %s" % json.dumps(legs))
+
     # ---------------- the vendor libraries on the same shapes, same process, same timing code (context only)
     if not args.no_vendor and not only:
         import torch.nn.functional as F

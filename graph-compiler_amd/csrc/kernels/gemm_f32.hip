@@ -13,8 +13,13 @@
 //   8bit: b at i*stride_b + (k - k%4)*LDB + 4n + k%4      (VNNI-4)
 // (lib/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmNaive.cpp:46-140).
 // Microkernel calls are small (typically 32x32x32 with a batch of 8-16); one
-// thread per C element, batch-major then k ascending as the reference sums.
+// thread per C element, operands staged through LDS, batch-major then k ascending as the reference sums, and
+// every product and every sum rounded on its own (no fused multiply-add: the
+// reference's loop is plain C++ built for baseline x86-64, which has none), so
+// f32 results equal the reference's bit for bit; bf16 products are exact in f32
+// and integer sums are exact anyway.
 #include "common.hpp"
+#include <type_traits>
 #include "gemm_params.h"
 
 namespace gcmi {
@@ -116,42 +121,136 @@ struct BrgemmParams {
   int32_t num, beta_zero, dtA, dtB;
 };
 
+// One workgroup = one 16 x 16 tile of C, one thread per element.  The terms of an element's sum keep the reference's
+// order (batch-major, k ascending, each product and each sum rounded on its own), so the only freedom is where the
+// operands come from: the workgroup stages BRG_CH terms' worth of its 16 rows of A and 16 columns of B in LDS as
+// widened values (f32, or s32 for the 8-bit types), both with the terms contiguous so that four terms come out of
+// one 16-byte read per operand -- and the loads of the next chunk are in flight in registers while this chunk is
+// summed.  A chunk is a run of whole batches when K is small (the usual 32 x 32 x 32 call) or a slice of one batch's
+// K.  K tails of the packed layouts are never read and never added (adding a zero would turn a -0 sum into +0).
+// A single wave issues a vector instruction only every 8-9 cycles on this GPU, so the chain of num*K dependent sums
+// is the floor; everything else is kept short: element offsets are worked out once, a chunk adds two scalars.
+static constexpr int BRG_CH = 128, BRG_PITCH = BRG_CH + 4, BRG_PER = 16 * BRG_CH / 256;
+
+template <typename ACC, int V> // V: the k elements packed beside each other in B (1 f32, 2 bf16, 4 8-bit)
 __global__ __launch_bounds__(256) void brgemm_kernel(BrgemmParams p) {
-  const int64_t n = (int64_t)blockIdx.x * 16 + (threadIdx.x & 15);
-  const int64_t m = (int64_t)blockIdx.y * 16 + (threadIdx.x >> 4);
-  if (m >= p.M || n >= p.N)
-    return;
-  if (p.dtA == DT_F32) {
-    const float *a = (const float *)p.A, *b = (const float *)p.B;
-    float *c = (float *)p.C + m * p.LDC + n;
-    float s = p.beta_zero ? 0.0f : *c;
-    for (int i = 0; i < p.num; i++)
-      for (int64_t k = 0; k < p.K; k++)
-        s += a[i * p.stride_a + m * p.LDA + k] * b[i * p.stride_b + k * p.LDB + n];
-    *c = s;
-  } else if (p.dtA == DT_BF16) {
-    const uint16_t *a = (const uint16_t *)p.A, *b = (const uint16_t *)p.B;
-    float *c = (float *)p.C + m * p.LDC + n;
-    float s = p.beta_zero ? 0.0f : *c;
-    for (int i = 0; i < p.num; i++)
-      for (int64_t k = 0; k < p.K; k++)
-        s += bf16_bits_to_f32(a[i * p.stride_a + m * p.LDA + k]) *
-             bf16_bits_to_f32(b[i * p.stride_b + (k & ~(int64_t)1) * p.LDB + 2 * n + (k & 1)]);
-    *c = s;
-  } else {
-    const uint8_t *a = (const uint8_t *)p.A, *b = (const uint8_t *)p.B;
-    int32_t *c = (int32_t *)p.C + m * p.LDC + n;
-    int32_t s = p.beta_zero ? 0 : *c;
-    for (int i = 0; i < p.num; i++)
-      for (int64_t k = 0; k < p.K; k++) {
-        uint8_t ar = a[i * p.stride_a + m * p.LDA + k];
-        uint8_t br = b[i * p.stride_b + (k & ~(int64_t)3) * p.LDB + 4 * n + (k & 3)];
-        int av = p.dtA == DT_S8 ? (int)(int8_t)ar : (int)ar;
-        int bv = p.dtB == DT_S8 ? (int)(int8_t)br : (int)br;
-        s += av * bv;
-      }
-    *c = s;
+#pragma clang fp contract(off) // a product and the sum it goes into are rounded separately, as the reference's are
+  __shared__ __attribute__((aligned(16))) ACC As[16][BRG_PITCH]; // [row of the tile][term of the chunk]
+  __shared__ __attribute__((aligned(16))) ACC Bs[16][BRG_PITCH]; // [column of the tile][term of the chunk]
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int64_t n0 = (int64_t)blockIdx.x * 16, m0 = (int64_t)blockIdx.y * 16;
+  // chunk geometry: kc terms of K per batch and chunk, nb batches per chunk; chunks run batch group by batch group
+  // and, inside one, K slice by K slice
+  const int kc = p.K < BRG_CH ? (int)p.K : BRG_CH;
+  const int nb = p.K < BRG_CH ? BRG_CH / (kc > 0 ? kc : 1) : 1;
+  const int64_t kchunks = p.K > 0 ? (p.K + kc - 1) / kc : 0;
+  const int64_t nchunks = ((p.num + nb - 1) / nb) * kchunks;
+  const bool a_signed = p.dtA == DT_S8, b_signed = p.dtB == DT_S8;
+
+  // Loads keep the raw element (a register each); widening waits until the value goes to LDS, one chunk later, so
+  // that nothing between a load and the sums of the current chunk needs the loaded value.
+  typedef typename std::conditional<V == 1, float, uint32_t>::type RAW;
+  auto load = [&](const void *base, int64_t idx) -> RAW {
+    if constexpr (V == 1)
+      return ((const float *)base)[idx];
+    else if constexpr (V == 2)
+      return ((const uint16_t *)base)[idx];
+    else
+      return ((const uint8_t *)base)[idx];
+  };
+  auto widen = [&](RAW v, bool is_signed) -> ACC {
+    if constexpr (V == 1)
+      return v;
+    else if constexpr (V == 2)
+      return __uint_as_float(v << 16);
+    else
+      return is_signed ? (int)(v ^ 0x80u) - 0x80 : (int)v;
+  };
+  // Slot e of a chunk.  A: (row, term), terms along consecutive threads.  B: (term group, column, k within the
+  // group), the order B lies in memory.  Term t of a chunk = (batch t / kc, k t % kc) relative to the chunk's first
+  // batch and first k (a multiple of V, so the packed position of k does not depend on the chunk).
+  int64_t a_off[BRG_PER], b_off[BRG_PER];
+  int a_bat[BRG_PER], a_k[BRG_PER], b_bat[BRG_PER], b_k[BRG_PER];
+#pragma unroll
+  for (int e = 0; e < BRG_PER; e++) {
+    const int idx = threadIdx.x + 256 * e;
+    const int ta = idx % BRG_CH, tb = (idx / (16 * V)) * V + idx % V;
+    const int kd = kc > 0 ? kc : 1;
+    const int64_t m = m0 + idx / BRG_CH, n = n0 + (idx % (16 * V)) / V;
+    a_bat[e] = (ta < nb * kc && m < p.M) ? ta / kd : 1 << 30, a_k[e] = ta % kd; // 1 << 30: never a valid batch
+    b_bat[e] = (tb < nb * kc && n < p.N) ? tb / kd : 1 << 30, b_k[e] = tb % kd;
+    a_off[e] = (int64_t)(ta / kd) * p.stride_a + m * p.LDA + a_k[e];
+    b_off[e] = (int64_t)(tb / kd) * p.stride_b + (int64_t)(b_k[e] - b_k[e] % V) * p.LDB + V * n + b_k[e] % V;
   }
+  RAW ra[BRG_PER], rb[BRG_PER];
+  auto fetch = [&](int64_t b0, int64_t k0) {
+    const int64_t a_chunk = b0 * p.stride_a + k0, b_chunk = b0 * p.stride_b + k0 * p.LDB;
+    const int64_t bats = p.num - b0, ks = p.K - k0; // batches and k left from here
+#pragma unroll
+    for (int e = 0; e < BRG_PER; e++) {
+      ra[e] = (a_bat[e] < bats && a_k[e] < ks) ? load(p.A, a_off[e] + a_chunk) : RAW(0);
+      rb[e] = (b_bat[e] < bats && b_k[e] < ks) ? load(p.B, b_off[e] + b_chunk) : RAW(0);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int e = 0; e < BRG_PER; e++) {
+      const int idx = threadIdx.x + 256 * e;
+      As[idx / BRG_CH][idx % BRG_CH] = widen(ra[e], a_signed);
+      Bs[(idx % (16 * V)) / V][(idx / (16 * V)) * V + idx % V] = widen(rb[e], b_signed);
+    }
+  };
+  auto term = [](ACC s, ACC a, ACC b) -> ACC {
+    if constexpr (V == 4)
+      return __mul24(a, b) + s; // 8-bit values: one 24-bit multiply-add, exact
+    else
+      return s + a * b;
+  };
+  const int64_t m = m0 + ty, n = n0 + tx;
+  const bool mine = m < p.M && n < p.N;
+  ACC *c = (ACC *)p.C + m * p.LDC + n;
+  ACC s = (p.beta_zero || !mine) ? ACC(0) : *c;
+  int64_t b0 = 0, k0 = 0, b0n = 0, k0n = 0; // this chunk's first batch and k, and the next chunk's
+  auto advance = [&]() {
+    k0n += kc;
+    if (k0n >= p.K)
+      k0n = 0, b0n += nb;
+  };
+  if (nchunks > 0) {
+    fetch(0, 0);
+    advance();
+  }
+  typedef ACC acc4 __attribute__((ext_vector_type(4)));
+  for (int64_t ch = 0; ch < nchunks; ch++) {
+    stash();
+    __syncthreads();
+    if (ch + 1 < nchunks)
+      fetch(b0n, k0n);
+    const int nbat = (int)((p.num - b0) < nb ? (p.num - b0) : nb);
+    const int klen = (int)((p.K - k0) < kc ? (p.K - k0) : kc);
+    for (int bi = 0; bi < nbat; bi++) {
+      const int t0 = bi * kc;
+      int k = 0;
+      if ((kc & 3) == 0) { // every batch of the chunk starts on a 16-byte boundary
+#pragma unroll 2
+        for (; k + 4 <= klen; k += 4) {
+          const acc4 a = *reinterpret_cast<const acc4 *>(&As[ty][t0 + k]);
+          const acc4 b = *reinterpret_cast<const acc4 *>(&Bs[tx][t0 + k]);
+          s = term(s, a.x, b.x);
+          s = term(s, a.y, b.y);
+          s = term(s, a.z, b.z);
+          s = term(s, a.w, b.w);
+        }
+      }
+      for (; k < klen; k++)
+        s = term(s, As[ty][t0 + k], Bs[tx][t0 + k]);
+    }
+    __syncthreads();
+    b0 = b0n, k0 = k0n;
+    advance();
+  }
+  if (mine)
+    *c = s;
 }
 
 } // namespace gcmi
@@ -187,6 +286,13 @@ extern "C" int gcmi_launch_brgemm(const void *A, const void *B, void *C, int64_t
     return 0;
   BrgemmParams p{A, B, C, M, N, K, LDA, LDB, LDC, stride_a, stride_b, num, beta_zero, dtA, dtB};
   dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16)), block(256);
-  hipLaunchKernelGGL(brgemm_kernel, grid, block, 0, stream, p);
+  if (grid.y > 65535)
+    return 2;
+  if (dtA == DT_F32)
+    hipLaunchKernelGGL((brgemm_kernel<float, 1>), grid, block, 0, stream, p);
+  else if (dtA == DT_BF16)
+    hipLaunchKernelGGL((brgemm_kernel<float, 2>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((brgemm_kernel<int32_t, 4>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 5;
 }
