@@ -391,7 +391,7 @@ void Executable::plan() {
       const LTensor &q = T(mm.in[0]), &k = T(mm.in[1]);
       size_t r = q.shape.size();
       bool ok = mm.in.size() == 2 && !ta && tb && q.dt == DT::bf16 && k.dt == DT::bf16 && r >= 3 &&
-                k.shape.size() == r && q.shape[r - 1] == 128 &&
+                k.shape.size() == r && (q.shape[r - 1] == 128 || q.shape[r - 1] == 64) &&
                 std::equal(q.shape.begin(), q.shape.end() - 2, k.shape.begin());
       size_t cur = mm.out[0];
       std::vector<size_t> chain{i};
@@ -446,7 +446,7 @@ void Executable::plan() {
             const LTensor &v = T(c.in[1]);
             bool fin = c.in.size() == 2 && c.in[0] == cur && !c.attr_bool("transpose_a", false) &&
                        !c.attr_bool("transpose_b", false) && v.dt == DT::bf16 && v.shape.size() == r &&
-                       v.shape[r - 1] == 128 && v.shape[r - 2] == Sk &&
+                       v.shape[r - 1] == q.shape[r - 1] && v.shape[r - 2] == Sk &&
                        std::equal(q.shape.begin(), q.shape.end() - 2, v.shape.begin()) && T(c.out[0]).dt == DT::bf16;
             if (!fin) {
               ok = false;
@@ -490,7 +490,7 @@ void Executable::plan() {
           s.note = "attention: MatMul+scale+mask+SoftMax+MatMul fused (" + std::to_string(chain.size()) + " ops)";
           s.a = slot_for(mm.in[0]), s.b = slot_for(mm.in[1]), s.c = slot_for(pv.in[1]), s.out = slot_for(pv.out[0]);
           s.mask = mask_slot, s.mask_ld = mask_ld;
-          s.BH = prod(q.shape, 0, r - 2), s.Sq = Sq, s.Sk = Sk, s.D = 128;
+          s.BH = prod(q.shape, 0, r - 2), s.Sq = Sq, s.Sk = Sk, s.D = q.shape[r - 1];
           s.scale = 1.0f;
           if (scale_t >= 0 && T((size_t)scale_t).has_splat) {
             const float x = (float)T((size_t)scale_t).splat;

@@ -510,8 +510,8 @@ int mha_any(const void *Q, const void *K, const void *V, const float *mask, int6
             size_t ws_bytes) {
   if (BH < 0 || Sq < 0 || Sk < 0)
     return fail(ST_INVALID, "mha_fwd: negative size");
-  if (D != 128)
-    return fail(ST_UNIMPL, "mha_fwd: head_dim %lld (only 128 is built)", (long long)D);
+  if (D != 128 && D != 64)
+    return fail(ST_UNIMPL, "mha_fwd: head_dim %lld (128 and 64 are built)", (long long)D);
   if (BH == 0 || Sq == 0)
     return ST_OK;
   if (Sk == 0)

@@ -231,7 +231,7 @@ int gcmi_gemm_f32_batched(const float *A, const float *B, float *C, int64_t batc
                           int trans_a, int trans_b, const float *bias, int act, void *stream);
 
 /*
- * Fused multi-head attention forward, bf16, head_dim 128:
+ * Fused multi-head attention forward, bf16, head_dim D = 128 or 64 (any other: status unimplemented):
  *   O = softmax(Q K^T * scale + mask) V,  softmax over keys in f32.
  * Takes over the composition batch_matmul_transpose_b -> mul -> add -> softmax
  * -> batch_matmul (lib/gc/Transforms/DecomposeAggregatedOps.cpp:24-38;

@@ -43,7 +43,7 @@ def test_validation_errors_need_no_gpu(gc):
     assert b"null" in L.gcmi_last_error()
     assert L.gcmi_gemm_bf16(None, None, None, -1, 4, 4, 4, 4, 4, None, 2, 0, 2, None) == 2
     assert L.gcmi_gemm_bf16(None, None, None, 0, 4, 4, 4, 4, 4, None, 2, 0, 2, None) == 0  # empty: nothing to do
-    assert L.gcmi_mha_fwd_bf16(None, None, None, None, 0, None, 1, 8, 8, 64, 1.0, None) == 3  # head_dim 64 not built
+    assert L.gcmi_mha_fwd_bf16(None, None, None, None, 0, None, 1, 8, 8, 96, 1.0, None) == 3  # head_dim 96 not built
     assert L.gcmi_gemm_int8(None, 3, None, None, 4, 4, 4, 4, 4, 4, None, 0, None, None, 0, 4, None) == 2
     assert L.dnnl_brgemm_dispatch(4, 4, 4, 4, 4, 4, 16, 16, 0.0, 3, 2) == -1  # f32 x bf16 is not a pair
     h = L.dnnl_brgemm_dispatch(4, 4, 4, 4, 4, 4, 16, 16, 0.0, 3, 3)

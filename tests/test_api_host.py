@@ -68,8 +68,9 @@ def test_fusion_plans_of_benchmark_partitions(ga):
     assert _steps(ga.explain(ga.mlp_chain_json(256, 256, 512))[1]) == ["gemm_bf16: MatMul+act", "gemm_bf16: MatMul+bias"]
     assert ga.explain(ga.mha_json(2, 2, 128, 128, 128))[1].startswith("attention:")
     assert ga.explain(ga.mha_json(2, 2, 128, 128, 128, with_mask=False, scale_op="Divide"))[1].startswith("attention:")
-    # head_dim 64 has no fused kernel: falls back to per-op kernels, still a valid plan
-    unfused = ga.explain(ga.mha_json(1, 2, 64, 64, 64))[1]
+    assert ga.explain(ga.mha_json(1, 2, 64, 64, 64))[1].startswith("attention:")
+    # head_dim 32 has no fused kernel: falls back to per-op kernels, still a valid plan
+    unfused = ga.explain(ga.mha_json(1, 2, 64, 64, 32))[1]
     assert "softmax: SoftMax" in unfused and "attention" not in unfused
 
 

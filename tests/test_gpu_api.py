@@ -190,21 +190,16 @@ def test_mlp_chain_partition(ga, orc, wl, dev):
 
 @pytest.mark.parametrize("D,with_mask,scale_op", [(128, True, "Multiply"), (128, False, "Divide"), (64, True, "Multiply")])
 def test_attention_partition(ga, orc, wl, dev, D, with_mask, scale_op):
-    """head_dim 128 runs the fused kernel; 64 falls back to per-op kernels with
-    the same results (softmax weights are a bf16 tensor in both)."""
+    """head dims 128 and 64 both run the fused kernel (softmax weights rounded to bf16, as the graph's tensor is)."""
     B, H, S = 1, 2, 128
     Q, K, V, mask, scale = wl.bf16_mha(B, H, S, D)
     sval = np.array([scale if scale_op == "Multiply" else 1.0 / scale], np.float32)
     out = torch.zeros(B, H, S, D, dtype=torch.bfloat16)
     ins = [(0, Q), (1, K), (2, sval)] + ([(3, mask)] if with_mask else []) + [(4, V)]
     _run(ga, ga.mha_json(B, H, S, S, D, with_mask, scale_op), ins, [(9, out)])
-    if D == 128:
-        ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q), wl.bf16_bits(K), wl.bf16_bits(V),
-                                           mask.numpy() if with_mask else None, scale))
-    else:
-        Sm = Q.float() @ K.float().transpose(-1, -2) * scale + (mask if with_mask else 0)
-        P = torch.softmax(Sm, -1).to(torch.bfloat16).float()
-        ref = (P @ V.float()).to(torch.bfloat16).float().numpy()
+    assert "attention" in ga.explain(ga.mha_json(B, H, S, S, D, with_mask, scale_op))[1]
+    ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q), wl.bf16_bits(K), wl.bf16_bits(V),
+                                       mask.numpy() if with_mask else None, scale))
     Sd = Q.double() @ K.double().transpose(-1, -2) * scale + (mask.double() if with_mask else 0)
     mag = (torch.softmax(Sd, -1) @ V.double().abs()).numpy()
     assert_close(ref, out.float().numpy(), 1e-2, "attention partition", mag=mag)
@@ -370,14 +365,14 @@ def test_execute_async_on_the_callers_stream(ga, dev):
 
 @pytest.mark.parametrize("seed", range(16))
 def test_random_attention_partitions_against_torch(ga, dev, seed):
-    """Attention graphs with random sizes (also ones the fused kernel's fast path does not take), head dims 128 and
-    64, the scale as Multiply or Divide, and masks that are absent, shared ([Sq,Sk] / [1,1,Sq,Sk]: fused kernel) or
-    per batch ([B,1,Sq,Sk]: the matcher declines and the ops run one by one): all against torch with P rounded to
-    bf16 as in the graph."""
+    """Attention graphs with random sizes (also ones the fused kernel's fast path does not take), head dims 128, 64
+    (fused) and 32 (no fused kernel: the ops run one by one), the scale as Multiply or Divide, and masks that are
+    absent, shared ([Sq,Sk] / [1,1,Sq,Sk]: fused kernel) or per batch ([B,1,Sq,Sk]: the matcher declines and the ops
+    run one by one): all against torch with P rounded to bf16 as in the graph."""
     rng = np.random.default_rng(7000 + seed)
     B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
     Sq, Sk = int(rng.choice([64, 128, 200, 256])), int(rng.choice([64, 128, 192, 200]))
-    D = 128 if seed % 4 else 64
+    D = [32, 128, 64, 128][seed % 4]
     scale_op = "Multiply" if rng.random() < 0.5 else "Divide"
     mask_kind = ["none", "2d", "4d_shared", "per_batch"][int(rng.integers(4))]
     s = [B, H, Sq, Sk]
@@ -399,7 +394,7 @@ def test_random_attention_partitions_against_torch(ga, dev, seed):
     st, plan = ga.explain(g)
     assert st == 0, plan
     fused = plan.startswith("attention") or "\nattention" in plan
-    assert fused == (D == 128 and not (mask_kind == "per_batch" and B > 1)), plan
+    assert fused == (D in (128, 64) and not (mask_kind == "per_batch" and B > 1)), plan
     torch.manual_seed(seed)
     Q = torch.randn(B, H, Sq, D).to(torch.bfloat16)
     K = torch.randn(B, H, Sk, D).to(torch.bfloat16)

@@ -38,9 +38,9 @@ def _mask(kind, Sq, Sk):
     return torch.randn(Sq, Sk) * 2
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("B,H,Sq,Sk,kind", CASES)
-def test_mha_matches_oracle(gc, orc, wl, dev, B, H, Sq, Sk, kind):
-    D = 128
+def test_mha_matches_oracle(gc, orc, wl, dev, B, H, Sq, Sk, kind, D):
     torch.manual_seed(0)
     Q = torch.randn(B, H, Sq, D).to(torch.bfloat16)
     torch.manual_seed(1)
@@ -53,7 +53,13 @@ def test_mha_matches_oracle(gc, orc, wl, dev, B, H, Sq, Sk, kind):
                                        None if mask is None else mask.numpy(), scale))
     out = gc.mha_fwd_bf16(Q.to(dev), K.to(dev), V.to(dev), None if mask is None else mask.to(dev), scale)
     torch.cuda.synchronize()
-    assert_close(ref, out.float().cpu().numpy(), 1e-2, "mha %s" % kind, mag=_pv_mag(Q, K, V, mask, scale))
+    assert_close(ref, out.float().cpu().numpy(), 1e-2, "mha %s D=%d" % (kind, D), mag=_pv_mag(Q, K, V, mask, scale))
+
+
+def test_head_dims_not_built_are_refused(gc, dev):
+    Q = torch.zeros(1, 1, 64, 96, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(Exception, match="head_dim 96"):
+        gc.mha_fwd_bf16(Q, Q, Q)
 
 
 def test_fully_masked_rows_are_nan_like_the_reference_softmax(gc, orc, wl, dev):
