@@ -1202,7 +1202,8 @@ static constexpr int W4_DUMP_WAVE_BYTES = 128 * W4_DUMP_PITCH; // 34816 per wave
 
 // Four results of one row: c = the raw accumulators of columns n .. n+3 of row m.  HAS_BIAS / HAS_RES are
 // compile-time so that the eight rows of an unrolled group are straight-line code (their LDS reads go out together).
-template <int ES, int ACT, int OUT, bool HAS_BIAS, bool HAS_RES, typename acc4_t>
+// NAN_FREE: the caller has shown that no result of this row can be a NaN, so the bf16 conversions need no fix-up.
+template <int ES, int ACT, int OUT, bool HAS_BIAS, bool HAS_RES, bool NAN_FREE = false, typename acc4_t>
 __device__ __forceinline__ void w4_epilogue_row(const GemmParams &p, const acc4_t &c, int64_t m, int64_t n,
                                                 const f32x4_t &bias4, const f32x4_t &scale4, const i32x4_t &cs4) {
   char *Cb = reinterpret_cast<char *>(p.C);
@@ -1299,7 +1300,7 @@ __device__ __forceinline__ void w4_epilogue_row(const GemmParams &p, const acc4_
         x[e] = x[e] + res4[e];
       rnd();
     }
-    const float any_nan = (x[0] + x[1]) + (x[2] + x[3]);
+    const float any_nan = NAN_FREE ? 0.0f : (x[0] + x[1]) + (x[2] + x[3]);
     if (__builtin_expect(any_nan != any_nan, 0)) {
       if (x[0] != x[0]) p0 = (p0 & 0xffff0000u) | 0x7FC0u;
       if (x[1] != x[1]) p0 = (p0 & 0x0000ffffu) | 0x7FC00000u;
@@ -1329,6 +1330,9 @@ __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, 
     cs4 = *reinterpret_cast<const i32x4_t *>(colp + 512 + col);
   }
   const bool has_bias = ES == 2 && p.bias != nullptr, has_res = ES == 2 && p.residual != nullptr;
+  const bool bias_finite = fabsf((bias4[0] + bias4[1]) + (bias4[2] + bias4[3])) < __builtin_inff() || // the usual case
+                           (fabsf(bias4[0]) < __builtin_inff() && fabsf(bias4[1]) < __builtin_inff() &&
+                            fabsf(bias4[2]) < __builtin_inff() && fabsf(bias4[3]) < __builtin_inff());
   constexpr int U = 8; // rows in flight per lane
 #pragma unroll 1
   for (int i0 = 0; i0 < 32; i0 += U) {
@@ -1337,10 +1341,25 @@ __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, 
     for (int u = 0; u < U; u++)
       c[u] = *reinterpret_cast<const acc4_t *>(dump + ((i0 + u) * 4 + rr) * W4_DUMP_PITCH + cc * 16);
     auto rows = [&](auto hb, auto hr) {
+      constexpr bool HB = decltype(hb)::value, HR = decltype(hr)::value;
+      // bf16 results of finite accumulators and finite biases through nothing but an add and a ReLU are no NaNs:
+      // one sum over the group's 32 accumulators (a NaN or an infinity among them makes it non-finite) replaces
+      // the check of every row
+      if constexpr (ES == 2 && OUT == DT_BF16 && !HR && (ACT == ACT_NONE || ACT == ACT_RELU)) {
+        float t = 0.0f;
+#pragma unroll
+        for (int u = 0; u < U; u++)
+          t += ((float)c[u][0] + (float)c[u][1]) + ((float)c[u][2] + (float)c[u][3]);
+        if (__builtin_expect(bias_finite && fabsf(t) < __builtin_inff(), 1)) {
+#pragma unroll
+          for (int u = 0; u < U; u++)
+            w4_epilogue_row<ES, ACT, OUT, HB, HR, true>(p, c[u], m0 + wm * 128 + (i0 + u) * 4 + rr, n, bias4, scale4, cs4);
+          return;
+        }
+      }
 #pragma unroll
       for (int u = 0; u < U; u++)
-        w4_epilogue_row<ES, ACT, OUT, decltype(hb)::value, decltype(hr)::value>(
-            p, c[u], m0 + wm * 128 + (i0 + u) * 4 + rr, n, bias4, scale4, cs4);
+        w4_epilogue_row<ES, ACT, OUT, HB, HR>(p, c[u], m0 + wm * 128 + (i0 + u) * 4 + rr, n, bias4, scale4, cs4);
     };
     typedef std::integral_constant<bool, true> T;
     typedef std::integral_constant<bool, false> F;
