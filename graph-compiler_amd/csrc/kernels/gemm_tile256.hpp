@@ -1227,7 +1227,7 @@ __device__ __forceinline__ void w4_epilogue_row(const GemmParams &p, const acc4_
     }
     // v_cvt_pk_bf16_f32 rounds to nearest even but keeps a NaN's sign and payload; a NaN among the four (their
     // sum is one; so is the sum of opposite infinities) sends them through the scalar rule: NaN -> 0x7FC0
-    const float any_nan = (x[0] + x[1]) + (x[2] + x[3]);
+    const float any_nan = NAN_FREE ? 0.0f : (x[0] + x[1]) + (x[2] + x[3]);
     if (__builtin_expect(any_nan != any_nan, 0)) {
       p0 = f32_to_bf16_bits(x[0]) | ((uint32_t)f32_to_bf16_bits(x[1]) << 16);
       p1 = f32_to_bf16_bits(x[2]) | ((uint32_t)f32_to_bf16_bits(x[3]) << 16);
@@ -1333,6 +1333,12 @@ __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, 
   const bool bias_finite = fabsf((bias4[0] + bias4[1]) + (bias4[2] + bias4[3])) < __builtin_inff() || // the usual case
                            (fabsf(bias4[0]) < __builtin_inff() && fabsf(bias4[1]) < __builtin_inff() &&
                             fabsf(bias4[2]) < __builtin_inff() && fabsf(bias4[3]) < __builtin_inff());
+  bool cols_tame = true;
+  if constexpr (ES == 1) {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      cols_tame = cols_tame && fabsf(scale4[e]) < 0x1p90f && fabsf(bias4[e]) < 0x1p120f;
+  }
   constexpr int U = 8; // rows in flight per lane
 #pragma unroll 1
   for (int i0 = 0; i0 < 32; i0 += U) {
@@ -1364,7 +1370,15 @@ __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, 
     typedef std::integral_constant<bool, true> T;
     typedef std::integral_constant<bool, false> F;
     if constexpr (ES == 1) {
-      rows(F{}, F{});
+      // |acc| < 2^31: with scales below 2^90 and biases below 2^120 in magnitude the dequantised value is finite, and
+      // so is every activation of it: no NaN to look for
+      if (__builtin_expect(cols_tame, 1)) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+          w4_epilogue_row<ES, ACT, OUT, false, false, true>(p, c[u], m0 + wm * 128 + (i0 + u) * 4 + rr, n, bias4, scale4, cs4);
+      } else {
+        rows(F{}, F{});
+      }
     } else {
       if (has_bias) {
         if (has_res)
