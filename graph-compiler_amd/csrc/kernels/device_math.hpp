@@ -44,8 +44,13 @@ __device__ __forceinline__ float erf_rational(float x) {
   q = fmaf(q, x2, -1.68282697438203e-03f);
   q = fmaf(q, x2, -7.37332916720468e-03f);
   q = fmaf(q, x2, -1.42647390514189e-02f);
-  const float r = __builtin_amdgcn_fmed3f((p * xc) * __builtin_amdgcn_rcpf(q), -1.0f, 1.0f);
-  return fabsf(x) >= 3.95f ? copysignf(1.0f, x) : r;
+  // |x| >= 3.95 must give exactly +-1 (the quotient there is 1 - 2 ulp).  Written as arithmetic, not as a choice
+  // between the quotient and +-1: adding xc = +-3.95 to the quotient of such a lane and clamping gives +-1, adding
+  // 0 * xc leaves every other lane's quotient as it is, signed zeros included.  (With a conditional expression the
+  // compiler branches around the polynomials per element: six scalar instructions each, and the chains of the
+  // elements of a row no longer interleave.)
+  const float sat = fabsf(x) >= 3.95f ? 1.0f : 0.0f;
+  return __builtin_amdgcn_fmed3f(fmaf(sat, xc, (p * xc) * __builtin_amdgcn_rcpf(q)), -1.0f, 1.0f);
 }
 
 // Activation in f32.  Operation order follows the reference graphs:
