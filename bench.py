@@ -108,11 +108,11 @@ def time_launches(torch, fn, nsets, steps, warmup):
 # --copy-calibration: a 1 GiB copy reads FETCH_SIZE = 524304 KiB (scale 2.0)
 # and WRITE_SIZE = 1048580 KiB (scale 1.0).
 TRAFFIC = {  # (bytes per launch of the dominant kernel, the committed profile they come from)
-    "gemm": (235363595, "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
-    "int8": (384729793, "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
-    "chain": (685777635 + 575093617, "profiles/gemm_tile256_w4_bf16_mlp_chain.md"),  # both launches
-    "mha": (366467595, "profiles/mha_fwd_fast_b4_h32_s2048_d128_every_block.md"),
-    "mha_skip": (335089174, "profiles/mha_fwd_fast_b4_h32_s2048_d128.md"),
+    "gemm": (235375279, "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
+    "int8": (384724261, "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
+    "chain": (684052143 + 575105079, "profiles/gemm_tile256_w4_bf16_mlp_chain.md"),  # both launches
+    "mha": (369234364, "profiles/mha_fwd_fast_b4_h32_s2048_d128_every_block.md"),
+    "mha_skip": (306034939, "profiles/mha_fwd_fast_b4_h32_s2048_d128.md"),
 }
 
 
