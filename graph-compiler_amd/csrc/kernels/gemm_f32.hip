@@ -128,7 +128,7 @@ struct BrgemmParams {
 // one 16-byte read per operand -- and the loads of the next chunk are in flight in registers while this chunk is
 // summed.  A chunk is a run of whole batches when K is small (the usual 32 x 32 x 32 call) or a slice of one batch's
 // K.  K tails of the packed layouts are never read and never added (adding a zero would turn a -0 sum into +0).
-// A single wave issues a vector instruction only every 8-9 cycles on this GPU, so the chain of num*K dependent sums
+// A wave issues a vector instruction that needs its predecessor's result only every 8-9 cycles, so the chain of num*K dependent sums
 // is the floor; everything else is kept short: element offsets are worked out once, a chunk adds two scalars.
 static constexpr int BRG_CH = 128, BRG_PITCH = BRG_CH + 4, BRG_PER = 16 * BRG_CH / 256;
 

@@ -6,8 +6,9 @@ One half step = 16 MFMAs of one wave: the 8 S MFMAs of the NEXT 32 keys (K fragm
 registers) and the 8 PV MFMAs of the CURRENT 32 keys, whose 16 scores per lane become weights on the vector ALU on
 the way (fma, exp2, row sum, pack to bf16) -- plus the maximum of the next half's scores.
 
-Why by hand: a wave of this GPU issues a vector instruction only every 8 cycles or so (two waves on a SIMD: about 6
-each), while an MFMA 32x32x16 holds the matrix pipe for 32.  Up to four vector instructions after each MFMA are
+Why by hand: in this instruction mix (most vector instructions use a result from one or two places back) a wave
+issues a vector instruction only every 8 cycles or so (two waves on a SIMD: about 6 each; independent instructions go
+at one per 4), while an MFMA 32x32x16 holds the matrix pipe for 32.  Up to four vector instructions after each MFMA are
 free; a phase of vector work alone, as the compiler arranges the softmax, leaves the matrix pipe idle for its whole
 length.  So every MFMA here is followed by at most four vector instructions and two LDS reads, and nothing else.
 
