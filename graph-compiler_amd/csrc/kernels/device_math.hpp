@@ -51,6 +51,15 @@ __device__ __forceinline__ float erf_rational(float x) {
   return __builtin_amdgcn_fmed3f((p * xc) * __builtin_amdgcn_rcpf(q), -1.0f, 1.0f);
 }
 
+// tanh for the GELU below, where it is added to 1: 1 - 2 / (e^(2|t|) + 1) with the sign of t, absolute error about
+// 2e-7 (relative accuracy near 0 is not kept: the math library's tanhf keeps it with a polynomial branch per element,
+// which costs the epilogues what the conditional in erf did).  Infinite and NaN arguments come out as +-1 and NaN.
+__device__ __forceinline__ float tanh_by_exp(float t) {
+  const float e = __builtin_amdgcn_exp2f(fabsf(t) * 2.885390081777927f); // 2 log2 e
+  const float r = fmaf(__builtin_amdgcn_rcpf(e + 1.0f), -2.0f, 1.0f);
+  return copysignf(r, t);
+}
+
 // Activation in f32.  Operation order follows the reference graphs:
 // ReLU   = max(x, 0), NaN propagates (lib/gc/Transforms/OneDNNGraphToLinalg.cpp:355-358)
 // GELU   = ((erf(x*c)+1)*x)*0.5, c = 0x3f3504f3 (legacy/core/src/ops/gelu.cpp:110-131)
@@ -66,7 +75,7 @@ __device__ __forceinline__ float apply_act(float x, int act) {
   }
   case ACT_GELU_TANH: {
     float t = (((x * x) * 0.044715f + 1.0f) * x) * 0.79788458f;
-    return (x * (tanhf(t) + 1.0f)) * 0.5f;
+    return (x * (tanh_by_exp(t) + 1.0f)) * 0.5f;
   }
   case ACT_SIGMOID:
     return 1.0f / (1.0f + expf(-x));

@@ -252,6 +252,18 @@ def test_gelu_erf_epilogue_absolute_accuracy(gc, dev):
     assert (out[xd < -5.84] == 0).all() and (out[xd > 5.84] == xd[xd > 5.84]).all()
 
 
+def test_gelu_tanh_epilogue_absolute_accuracy(gc, dev):
+    """The tanh form of GELU (legacy/core/src/ops/gelu.cpp:78-108) over a dense grid of x against float64: the
+    epilogue's tanh is 1 - 2 / (e^(2|t|) + 1), absolute error about 2e-7."""
+    x = torch.linspace(-10, 10, 200001, dtype=torch.float32).reshape(-1, 1)
+    one = torch.ones(1, 1, dtype=torch.float32)
+    out = gc.gemm_f32(x.to(dev), one.to(dev), act="gelu_tanh").cpu().numpy().astype(np.float64).ravel()
+    xd = x.numpy().astype(np.float64).ravel()
+    ref = 0.5 * xd * (1 + np.tanh(0.79788458 * xd * (1 + 0.044715 * xd * xd)))
+    assert np.abs(out - ref).max() <= 4e-6  # 0.5 * 10 * 2e-7 + f32 rounding of the argument and the product
+    assert (out[xd > 6] == xd[xd > 6]).all() and (out[xd < -6] == 0).all()
+
+
 @pytest.mark.parametrize("M,N,K,act,with_bias,out_f32", [(32, 4096, 4096, None, False, False), (1, 4096, 4096, "relu", True, False),
                                                          (100, 11008, 4096, "gelu_erf", True, False),
                                                          (32, 4096, 11008, None, True, True), (256, 2048, 1024, "sigmoid", False, False),
