@@ -1203,9 +1203,13 @@ static constexpr int W4_DUMP_WAVE_BYTES = 128 * W4_DUMP_PITCH; // 34816 per wave
 // Four results of one row: c = the raw accumulators of columns n .. n+3 of row m.  HAS_BIAS / HAS_RES are
 // compile-time so that the eight rows of an unrolled group are straight-line code (their LDS reads go out together).
 // NAN_FREE: the caller has shown that no result of this row can be a NaN, so the bf16 conversions need no fix-up.
-template <int ES, int ACT, int OUT, bool HAS_BIAS, bool HAS_RES, bool NAN_FREE = false, typename acc4_t>
+// MASKED (a tile that sticks out of C): row_ok says whether row m exists; nothing of a missing row is read or stored.
+template <int ES, int ACT, int OUT, bool HAS_BIAS, bool HAS_RES, bool MASKED, bool NAN_FREE = false, typename acc4_t>
 __device__ __forceinline__ void w4_epilogue_row(const GemmParams &p, const acc4_t &c, int64_t m, int64_t n,
-                                                const f32x4_t &bias4, const f32x4_t &scale4, const i32x4_t &cs4) {
+                                                const f32x4_t &bias4, const f32x4_t &scale4, const i32x4_t &cs4,
+                                                bool row_ok = true) {
+  if (MASKED && !row_ok)
+    return;
   char *Cb = reinterpret_cast<char *>(p.C);
   float x[4];
   uint32_t p0 = 0, p1 = 0; // bf16 results, two per register
@@ -1314,14 +1318,18 @@ __device__ __forceinline__ void w4_epilogue_row(const GemmParams &p, const acc4_
 }
 
 // One half (64 columns) of the wave tile.  OUT = DT_BF16 / DT_F32 / DT_S32.
-template <int ES, int ACT, int OUT>
+// MASKED: rows_in / cols_in of the tile's 256 x 256 lie inside C (cols_in is a multiple of 4).
+template <int ES, int ACT, int OUT, bool MASKED>
 __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, int64_t m0, int64_t n0, int wm, int wn,
-                                                 int lane, const char *dump, const float *colp) {
+                                                 int lane, const char *dump, const float *colp, int rows_in, int cols_in) {
   typedef typename std::conditional<ES == 2, float, int>::type acc_e;
   typedef acc_e acc4_t __attribute__((ext_vector_type(4)));
   const int rr = lane >> 4, cc = lane & 15;
   const int col = wn * 128 + half * 64 + 4 * cc; // this lane's four columns inside the workgroup tile
   const int64_t n = n0 + col;
+  if (MASKED && col >= cols_in)
+    return;
+  const int row0 = wm * 128 + rr; // + 4 * (i0 + u)
   const f32x4_t bias4 = *reinterpret_cast<const f32x4_t *>(colp + col); // -0.0 where there is no bias
   f32x4_t scale4 = {1.f, 1.f, 1.f, 1.f};
   i32x4_t cs4 = {0, 0, 0, 0}; // comp * colsum
@@ -1359,13 +1367,15 @@ __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, 
         if (__builtin_expect(bias_finite && fabsf(t) < __builtin_inff(), 1)) {
 #pragma unroll
           for (int u = 0; u < U; u++)
-            w4_epilogue_row<ES, ACT, OUT, HB, HR, true>(p, c[u], m0 + wm * 128 + (i0 + u) * 4 + rr, n, bias4, scale4, cs4);
+            w4_epilogue_row<ES, ACT, OUT, HB, HR, MASKED, true>(p, c[u], m0 + row0 + (i0 + u) * 4, n, bias4, scale4, cs4,
+                                                                row0 + (i0 + u) * 4 < rows_in);
           return;
         }
       }
 #pragma unroll
       for (int u = 0; u < U; u++)
-        w4_epilogue_row<ES, ACT, OUT, HB, HR>(p, c[u], m0 + wm * 128 + (i0 + u) * 4 + rr, n, bias4, scale4, cs4);
+        w4_epilogue_row<ES, ACT, OUT, HB, HR, MASKED>(p, c[u], m0 + row0 + (i0 + u) * 4, n, bias4, scale4, cs4,
+                                                      row0 + (i0 + u) * 4 < rows_in);
     };
     typedef std::integral_constant<bool, true> T;
     typedef std::integral_constant<bool, false> F;
@@ -1375,7 +1385,8 @@ __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, 
       if (__builtin_expect(cols_tame, 1)) {
 #pragma unroll
         for (int u = 0; u < U; u++)
-          w4_epilogue_row<ES, ACT, OUT, false, false, true>(p, c[u], m0 + wm * 128 + (i0 + u) * 4 + rr, n, bias4, scale4, cs4);
+          w4_epilogue_row<ES, ACT, OUT, false, false, MASKED, true>(p, c[u], m0 + row0 + (i0 + u) * 4, n, bias4, scale4, cs4,
+                                                                    row0 + (i0 + u) * 4 < rows_in);
       } else {
         rows(F{}, F{});
       }
@@ -1396,12 +1407,13 @@ __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, 
 }
 
 // kind = act + 8 * (0: bf16, 1: f32, 2: s32)
-template <int ES>
+template <int ES, bool MASKED>
 __device__ __forceinline__ void w4_epilogue_half_any(const GemmParams &p, int kind, int half, int64_t m0, int64_t n0,
-                                                     int wm, int wn, int lane, const char *dump, const float *colp) {
+                                                     int wm, int wn, int lane, const char *dump, const float *colp,
+                                                     int rows_in, int cols_in) {
 #define GCMI_W4_CASE(ACT, OUT, K)                                                                                     \
   case (int)ACT + 8 * K:                                                                                              \
-    w4_epilogue_half<ES, ACT, OUT>(p, half, m0, n0, wm, wn, lane, dump, colp);                                        \
+    w4_epilogue_half<ES, ACT, OUT, MASKED>(p, half, m0, n0, wm, wn, lane, dump, colp, rows_in, cols_in);              \
     break;
   switch (kind) {
     GCMI_W4_CASE(ACT_RELU, DT_BF16, 0)
@@ -1415,7 +1427,7 @@ __device__ __forceinline__ void w4_epilogue_half_any(const GemmParams &p, int ki
     GCMI_W4_CASE(ACT_SIGMOID, DT_F32, 1)
     GCMI_W4_CASE(ACT_NONE, DT_S32, 2)
   default:
-    w4_epilogue_half<ES, ACT_NONE, DT_BF16>(p, half, m0, n0, wm, wn, lane, dump, colp);
+    w4_epilogue_half<ES, ACT_NONE, DT_BF16, MASKED>(p, half, m0, n0, wm, wn, lane, dump, colp, rows_in, cols_in);
     break;
   }
 #undef GCMI_W4_CASE
@@ -1440,7 +1452,7 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gem
   const int wm = wave >> 1, wn = wave & 1;
   const int r16 = lane & 15, g16 = lane >> 4;
 
-  const int tiles_m = (int)(p.M / G_BM), tiles_n = (int)(p.N / G_BN);
+  const int tiles_m = (int)((p.M + G_BM - 1) / G_BM), tiles_n = (int)((p.N + G_BN - 1) / G_BN); // edge tiles stick out
   int tm, tn;
   tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
   // integer division runs on the vector unit; the operand addresses below must be in scalar registers
@@ -1456,16 +1468,19 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gem
       p.residual = reinterpret_cast<const char *>(p.residual) + bz * p.c_bs * (p.residual_dt == DT_BF16 ? 2 : 4);
   }
 
-  // per-lane source offsets of the wave's DMA instructions, as in gemm_tile256_fast_kernel
+  // per-lane source offsets of the wave's DMA instructions, as in gemm_tile256_fast_kernel.  An edge tile's rows past
+  // M and columns past N are fetched from the last row / the last 16-byte chunk inside (N is a multiple of the
+  // chunk's columns): their products land in accumulators that the epilogue never stores.
+  const int rows_in = (int)min((int64_t)G_BM, p.M - m0), cols_in = (int)min((int64_t)G_BN, p.N - n0);
   i32x4_t a_off, b_off;
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int row = (wave * 4 + i) * FG::A_ROWS_PER_DMA + lane / FG::A_CPR;
     const int c = (lane % FG::A_CPR) ^ FG::a_swz(row);
-    a_off[i] = (int)(row * lda_b + c * 16);
+    a_off[i] = (int)(min(row, rows_in - 1) * lda_b + c * 16);
     const int krow = (wave * 4 + i) * FG::B_ROWS_PER_DMA + lane / FG::B_CPR;
-    const int cb = (lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW);
-    b_off[i] = TB ? (int)(row * ldb_b + c * 16) : (int)(krow * ldb_b + cb * 16);
+    const int cb = min((lane % FG::B_CPR) ^ ((krow % FG::RG) * FG::CW), cols_in * ES / 16 - 1);
+    b_off[i] = TB ? (int)(min(row, cols_in - 1) * ldb_b + c * 16) : (int)(krow * ldb_b + cb * 16);
   }
   // fragment addresses as in gemm_tile256_mi16_kernel: A tile `it` = rows wm*128 + 16*it .., B tile `jt` = columns
   // wn*128 + 16*jt ..; slots 2 and 3 through a second base (an instruction's offset field has 16 bits)
@@ -1496,14 +1511,16 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gem
   // column parameters of this tile (see gemm_tile256_fast_kernel): 256 threads, one column each
   float cp_bias = -0.0f, cp_scale = 1.0f;
   int cp_cs = 0;
-  if (p.bias)
-    cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n0 + tid])
-                                   : reinterpret_cast<const float *>(p.bias)[n0 + tid];
-  if (ES == 1) {
-    if (p.scale)
-      cp_scale = p.scale[n0 + tid];
-    if (p.colsum)
-      cp_cs = p.comp * p.colsum[n0 + tid];
+  if (tid < cols_in) {
+    if (p.bias)
+      cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n0 + tid])
+                                     : reinterpret_cast<const float *>(p.bias)[n0 + tid];
+    if (ES == 1) {
+      if (p.scale)
+        cp_scale = p.scale[n0 + tid];
+      if (p.colsum)
+        cp_cs = p.comp * p.colsum[n0 + tid];
+    }
   }
 
   uint64_t a_ptr = (uint64_t)(reinterpret_cast<const char *>(p.A) + m0 * lda_b);
@@ -1543,10 +1560,19 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gem
   const int out_kind = p.out_dt == DT_BF16 ? 0 : ((ES == 1 && p.out_dt == DT_S32) ? 2 : 1);
   const int kind = (out_kind == 2 ? (int)ACT_NONE : p.act) + 8 * out_kind;
   const char *dump = smem + wave * W4_DUMP_WAVE_BYTES;
-  w4_epilogue_half_any<ES>(p, kind, 0, m0, n0, wm, wn, lane, dump, colp);
+  // a tile that sticks out of C takes the same code with every row and lane tested against the edge
+  const int rows_c = (int)min((int64_t)G_BM, p.M - m0), cols_c = (int)min((int64_t)G_BN, p.N - n0);
+  const bool edge_tile = rows_c < G_BM || cols_c < G_BN; // the same for the whole workgroup
+  if (edge_tile)
+    w4_epilogue_half_any<ES, true>(p, kind, 0, m0, n0, wm, wn, lane, dump, colp, rows_c, cols_c);
+  else
+    w4_epilogue_half_any<ES, false>(p, kind, 0, m0, n0, wm, wn, lane, dump, colp, G_BM, G_BN);
   // the right half: the accumulators of column tiles 4-7 are still where the main loop left them
   asm volatile(GCMI_W4_ASM_DUMP_HI : : "{v26}"(dump_ld) : "memory");
-  w4_epilogue_half_any<ES>(p, kind, 1, m0, n0, wm, wn, lane, dump, colp);
+  if (edge_tile)
+    w4_epilogue_half_any<ES, true>(p, kind, 1, m0, n0, wm, wn, lane, dump, colp, rows_c, cols_c);
+  else
+    w4_epilogue_half_any<ES, false>(p, kind, 1, m0, n0, wm, wn, lane, dump, colp, G_BM, G_BN);
 #ifdef GCMI_W4_TIMING
   const long long wall_issued = wall_clock64();
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1669,9 +1695,10 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
   const int res_es = p.residual_dt == DT_BF16 ? 2 : 4;
   // the kernels for whole tiles read four residual elements with one load
   const bool res_vec = !p.residual || (al16(p.residual) && (p.ldr * res_es) % 16 == 0);
-  const bool fast_but_m = p.N % G_BN == 0 && p.K % KGROUP == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) && res_vec &&
-                          (p.lda * ES) % 16 == 0 && (p.ldb * ES) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
-                          p.lda * ES * G_BM < (int64_t)1 << 31 && p.ldb * ES * (p.trans_b ? G_BN : BK) < (int64_t)1 << 31;
+  const bool aligned = p.K % KGROUP == 0 && p.K > 0 && al16(p.A) && al16(p.B) && al16(p.C) && res_vec &&
+                       (p.lda * ES) % 16 == 0 && (p.ldb * ES) % 16 == 0 && (p.ldc * out_es) % 16 == 0 &&
+                       p.lda * ES * G_BM < (int64_t)1 << 31 && p.ldb * ES * (p.trans_b ? G_BN : BK) < (int64_t)1 << 31;
+  const bool fast_but_m = aligned && p.N % G_BN == 0;
   if (p.trans_b && ES != 2)
     return 3;
   if (p.residual && (ES != 2 || (p.residual_dt != DT_BF16 && p.residual_dt != DT_F32) || p.out_dt == DT_S32))
@@ -1687,6 +1714,11 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
   else if (!((p.a_bs * ES) % 16 == 0 && (p.b_bs * ES) % 16 == 0 && (p.c_bs * out_es) % 16 == 0 &&
              (!p.residual || (p.c_bs * res_es) % 16 == 0)))
     fast = false; // every batch's operands must keep the alignment the fast path loads with
+  // Any M, N a whole number of 16-byte chunks: the 4-wave kernel still takes it; its edge tiles clamp their loads
+  // and store what lies inside C.
+  const bool ragged = !fast && aligned && p.N % (16 / ES) == 0 && (p.M % G_BM != 0 || p.N % G_BN != 0) &&
+                      (nbatch == 1 || ((p.a_bs * ES) % 16 == 0 && (p.b_bs * ES) % 16 == 0 && (p.c_bs * out_es) % 16 == 0 &&
+                                       (!p.residual || (p.c_bs * res_es) % 16 == 0)));
   if (p.group_m <= 0)
     p.group_m = 4;
   GemmTileConfig c{};
@@ -1736,13 +1768,15 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
     }
   }
   // Whole tiles: 4 waves of 128 x 128 unless the caller asks for 8 waves of 128 x 64 (or the result is an f32 / s32
-  // tensor of 8-bit operands, which only the 8-wave kernel writes).  Anything else: the bounds-checked kernel.
-  const bool w4_can = fast && (ES == 2 || p.out_dt == DT_BF16);
-  const bool use_w4 = w4_can && p.cfg_waves != 8;
-  c.kernel = !fast ? GK_EDGE : (use_w4 ? GK_WAVES4 : GK_WAVES8);
-  c.kbytes = fast ? 64 : G_KBYTES, c.stages = fast ? 4 : 2;
+  // tensor of 8-bit operands, which only the 8-wave kernel writes).  Tiles that stick out of C (`ragged`): the 4-wave
+  // kernel.  Anything else (a K tail, unaligned rows): the bounds-checked kernel.
+  const bool w4_can = (fast || ragged) && (ES == 2 || p.out_dt == DT_BF16);
+  const bool use_w4 = w4_can && (p.cfg_waves != 8 || !fast);
+  const bool tiled = fast || use_w4; // one of the kernels with the LDS ring
+  c.kernel = !tiled ? GK_EDGE : (use_w4 ? GK_WAVES4 : GK_WAVES8);
+  c.kbytes = tiled ? 64 : G_KBYTES, c.stages = tiled ? 4 : 2;
   c.waves_m = 2, c.waves_n = use_w4 ? 2 : 4, c.wave_m = 128, c.wave_n = use_w4 ? 128 : 64;
-  c.mfma_m = c.mfma_n = fast ? 16 : 32, c.mfma_k = (fast ? 64 : 32) / ES;
+  c.mfma_m = c.mfma_n = tiled ? 16 : 32, c.mfma_k = (tiled ? 64 : 32) / ES;
   if (cfg)
     *cfg = c;
   if (dry)

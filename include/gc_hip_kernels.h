@@ -137,7 +137,8 @@ int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int6
  * MatmulConfigAnalysis.h:25-34; chosen there by a CPU cost model,
  * lib/gc/Analysis/MatmulConfigAnalysis.cpp:435-552, here per shape, element
  * type and layout).  `kernel`: 0 bounds-checked tile (any shape), 1 whole
- * tiles with 8 waves of 128 x 64, 2 whole tiles with 4 waves of 128 x 128,
+ * tiles with 8 waves of 128 x 64, 2 tiles with 4 waves of 128 x 128 (any M,
+ * N a multiple of 16 bytes of columns: edge tiles store what lies inside C),
  * 3 K slices over workgroups + second pass (one tile row), 4 weight-streaming
  * kernel (a short A against [N,K] weights).
  *

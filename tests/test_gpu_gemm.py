@@ -252,6 +252,76 @@ def test_gelu_erf_epilogue_absolute_accuracy(gc, dev):
     assert (out[xd < -5.84] == 0).all() and (out[xd > 5.84] == xd[xd > 5.84]).all()
 
 
+@pytest.mark.parametrize("M,N", [(300, 264), (520, 256), (512, 520), (1000, 1000)])
+@pytest.mark.parametrize("variant", ["plain", "bias_gelu_f32", "bias_relu_residual", "nt"])
+def test_bf16_edge_tiles_of_the_four_wave_kernel(gc, orc, wl, dev, M, N, variant):
+    """M any, N a multiple of 8, K a multiple of 128: the whole-tile kernel takes the shape, its tiles on the lower
+    and right edges clamp their loads and store what lies inside C.  Every element equals, bit for bit, the element
+    of the same GEMM padded to whole tiles (same kernel, same sums), and the result matches the oracle."""
+    K = 384
+    c, _ = gc.tile_config(M, N, K, trans_b=(variant == "nt"), out_dtype=gc.F32 if variant == "bias_gelu_f32" else gc.BF16)
+    assert c.kernel == 2 and c.workgroups == -(-M // 256) * -(-N // 256)
+    Mp, Np = -(-M // 256) * 256, -(-N // 256) * 256
+    torch.manual_seed(0)
+    Ap = (torch.randn(Mp, K) * 0.5).to(torch.bfloat16)
+    torch.manual_seed(1)
+    Bp = (torch.randn(K, Np) * 0.5).to(torch.bfloat16)
+    torch.manual_seed(2)
+    biasp = torch.randn(Np).to(torch.bfloat16)
+    torch.manual_seed(3)
+    resp = torch.randn(Mp, Np).to(torch.bfloat16)
+    A, B, bias, res = Ap[:M].contiguous(), Bp[:, :N].contiguous(), biasp[:N].contiguous(), resp[:M, :N].contiguous()
+    d = lambda t: t.to(dev)
+    guard = torch.full((M + 2, N), 7.0, dtype=torch.float32 if variant == "bias_gelu_f32" else torch.bfloat16, device=dev)
+    out = guard[1:M + 1]
+    if variant == "plain":
+        gc.gemm_bf16(d(A), d(B), out=out)
+        full = gc.gemm_bf16(d(Ap), d(Bp))
+        ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B)))
+    elif variant == "bias_gelu_f32":
+        gc.gemm_bf16(d(A), d(B), d(bias), "gelu_erf", out_dtype=gc.F32, out=out)
+        full = gc.gemm_bf16(d(Ap), d(Bp), d(biasp), "gelu_erf", out_dtype=gc.F32)
+        ref = None
+    elif variant == "bias_relu_residual":
+        gc.gemm_bf16_residual(d(A), d(B), d(res), bias=d(bias), act="relu", out=out)
+        full = gc.gemm_bf16_residual(d(Ap), d(Bp), d(resp), bias=d(biasp), act="relu")
+        ref = None
+    else:
+        Bt, Btp = B.t().contiguous(), Bp.t().contiguous()
+        gc.gemm_bf16_nt(d(A), d(Bt), out=out)
+        full = gc.gemm_bf16_nt(d(Ap), d(Btp))
+        ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B)))
+    torch.cuda.synchronize()
+    assert (guard[0] == 7).all() and (guard[M + 1] == 7).all()  # nothing written outside C
+    bits = torch.int32 if out.dtype == torch.float32 else torch.int16
+    assert (out.view(bits) == full[:M, :N].contiguous().view(bits)).all()
+    if ref is not None:
+        assert_close(ref, out.float().cpu().numpy(), 1e-2, "bf16 edge tiles %dx%d %s" % (M, N, variant))
+
+
+@pytest.mark.parametrize("M,N", [(300, 272), (520, 768), (256, 528)])
+def test_int8_edge_tiles_of_the_four_wave_kernel(gc, orc, dev, M, N):
+    """The same for u8 x s8 with dequantisation, bias and GELU to bf16 (N a multiple of 16, K of 256)."""
+    K = 512
+    c, _ = gc.tile_config(M, N, K, a_dtype=gc.U8)
+    assert c.kernel == 2
+    torch.manual_seed(0)
+    A = torch.randint(0, 256, (M, K), dtype=torch.int32).to(torch.uint8)
+    torch.manual_seed(1)
+    W = torch.randint(-127, 128, (K, N), dtype=torch.int32).to(torch.int8)
+    torch.manual_seed(2)
+    sc = torch.rand(N) * 0.009 + 0.001
+    torch.manual_seed(3)
+    bs = torch.randn(N)
+    _, y = orc.int8_layer(A.numpy(), W.numpy(), sc.numpy(), bs.numpy(), 128, "gelu_erf")
+    Wd = W.to(dev)
+    guard = torch.full((M + 2, N), 7.0, dtype=torch.bfloat16, device=dev)
+    gc.gemm_int8(A.to(dev), Wd, gc.colsum_s8(Wd), 128, sc.to(dev), bs.to(dev), "gelu_erf", gc.BF16, out=guard[1:M + 1])
+    torch.cuda.synchronize()
+    assert (guard[0] == 7).all() and (guard[M + 1] == 7).all()
+    assert_close(orc.bf16_to_f32(y), guard[1:M + 1].float().cpu().numpy(), 1e-2, "int8 edge tiles")
+
+
 def test_gelu_tanh_epilogue_absolute_accuracy(gc, dev):
     """The tanh form of GELU (legacy/core/src/ops/gelu.cpp:78-108) over a dense grid of x against float64: the
     epilogue's tanh is 1 - 2 / (e^(2|t|) + 1), absolute error about 2e-7."""
