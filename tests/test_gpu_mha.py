@@ -22,7 +22,11 @@ def _pv_mag(Q, K, V, mask, scale):
 CASES = [(1, 2, 128, 128, "causal"), (1, 1, 256, 192, "none"), (2, 2, 100, 77, "causal"), (1, 2, 384, 384, "neg1e9"),
          (1, 1, 1, 1, "none"), (1, 3, 130, 64, "random"), (1, 1, 64, 300, "neg30000"),
          # the pipelined loop's ends: one key block (no steady state), two, an odd count with general mask tiles
-         (1, 2, 128, 64, "causal"), (1, 2, 256, 64, "random"), (1, 1, 128, 320, "random"), (1, 2, 128, 128, "none")]
+         (1, 2, 128, 64, "causal"), (1, 2, 256, 64, "random"), (1, 1, 128, 320, "random"), (1, 2, 128, 128, "none"),
+         # row and key counts off the tile sizes on the pipelined kernel: the last workgroup / key block overlaps its
+         # predecessor (duplicate keys masked out); general, constant and absent masks, one and several blocks
+         (1, 2, 200, 200, "causal"), (1, 2, 130, 68, "random"), (2, 2, 300, 1000, "causal"), (1, 1, 257, 321, "none"),
+         (1, 2, 129, 127 + 1, "neg1e9"), (1, 1, 1000, 100, "random"), (1, 2, 1111, 1112, "causal")]
 
 
 def _mask(kind, Sq, Sk):
