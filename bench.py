@@ -394,6 +394,33 @@ def main():
                                                   "(weight-streaming kernel); two launches each (partial sums, then reduction + "
                                                   "epilogue); algorithmic bytes = A + W + C once", "shapes": dec}
 
+    # ---------------- the same kernels on shapes off their tile sizes (parity cases elsewhere; here: no cliff)
+    if want("ragged"):
+        rag = {}
+        Mr, Nr, Kr = 4000, 4000, 4096
+        Ar = (torch.randn(Mr, Kr) * 0.1).to(torch.bfloat16).to(dev)
+        Br = (torch.randn(Kr, Nr) * 0.1).to(torch.bfloat16).to(dev)
+        Cr = torch.empty(Mr, Nr, dtype=torch.bfloat16, device=dev)
+        t = time_launches(torch, lambda i: gc.gemm_bf16(Ar, Br, out=Cr), 1, max(20, K // 2), W)
+        rag["bf16_gemm_4000x4000x4096"] = {"ms_per_step": round(t["ms_per_step"], 5),
+                                           "value": round(2.0 * Mr * Nr * Kr / t["ms_per_step"] / 1e9, 1), "unit": "TFLOP/s"}
+        del Ar, Br, Cr
+        for name, S, D in (("bf16_mha_b4_h32_s2000_d128_causal", 2000, 128), ("bf16_mha_b4_h32_s2048_d64_causal", 2048, 64)):
+            Q, Kk, V, mask, scale = wl.bf16_mha(4, 32, S, D)
+            Qd, Kd, Vd, md = Q.to(dev), Kk.to(dev), V.to(dev), mask.to(dev)
+            Od = torch.empty_like(Qd)
+            t = time_launches(torch, lambda i: gc.mha_fwd_bf16(Qd, Kd, Vd, md, scale, out=Od), 1, max(10, K // 4), 5)
+            rag[name] = {"ms_per_step": round(t["ms_per_step"], 5),
+                         "value": round(4.0 * 4 * 32 * S * S * D / t["ms_per_step"] / 1e9, 1),
+                         "unit": "TFLOP/s (dense count, masked blocks skipped)"}
+            del Qd, Kd, Vd, md, Od
+        others["shapes_off_the_tile_sizes"] = {
+            "workload": "M and N of a GEMM not multiples of 256 (edge tiles of the whole-tile kernel), a sequence length "
+                        "that is not a multiple of 128 / 64 (overlapping last windows on the pipelined attention kernel), "
+                        "head dim 64 (general attention kernel with mask tile classes)", "cases": rag}
+        log("off the tile sizes: %s" % json.dumps(rag))
+        torch.cuda.empty_cache()
+
     # ---------------- f32 plumbing case (configs[0])
     if want("f32"):
         A, B, bias = wl.f32_matmul_bias_relu()
