@@ -417,7 +417,7 @@ def main():
         others["shapes_off_the_tile_sizes"] = {
             "workload": "M and N of a GEMM not multiples of 256 (edge tiles of the whole-tile kernel), a sequence length "
                         "that is not a multiple of 128 / 64 (overlapping last windows on the pipelined attention kernel), "
-                        "head dim 64 (general attention kernel with mask tile classes)", "cases": rag}
+                        "head dim 64 (the pipelined attention kernel's second instantiation)", "cases": rag}
         log("off the tile sizes: %s" % json.dumps(rag))
         torch.cuda.empty_cache()
 

@@ -26,6 +26,10 @@ Fixed registers (the kernel binds its variables to them with register constraint
   %[koff]     immediate: byte offset of the K half tile (stage * 32768 + half * 8192)
   %[voff]     immediate: byte offset of the V half tile (stage * 32768 + 16384 + half * 8192)
 
+Head dim 64 (the second pair of macros): 4 d slices and 2 d tiles, i.e. 4 S + 4 PV MFMAs for the same vector work;
+O^T in v[0:31], Q fragments in v[96:111], K addresses in v[128:131], V addresses in v[136:137], V rows 128 bytes
+apart.  That half step is bound by the vector ALU: its first four slots carry ten vector instructions each.
+
 Wait states kept by construction (the assembler does not add them inside an asm statement):
   LDS data        -> MFMA       s_waitcnt lgkmcnt(n), counted here
   vector ALU      -> MFMA read  at least two instructions in between
@@ -41,20 +45,24 @@ OPTS = set(filter(None, os.environ.get("GCMI_FA_OPTS", "").split(",")))  # exper
 O, SA, SB, QF, KA, VA, L, NM, MRAW, ONES, KF, VF, TMP = 0, 64, 80, 96, 128, 136, 140, 141, 142, 143, 144, 176, 208
 
 
-def gen(cur, nxt):
+def gen(cur, nxt, D=128):
+    """D = 128: 16 MFMAs (8 S, 8 PV) per half step.  D = 64: 4 d slices and 2 d tiles, i.e. 8 MFMAs for the same vector
+    work -- that variant is bound by the vector ALU, and its slots take eight vector instructions each."""
     out = []
     emit = out.append
     lds = []  # LDS reads in issue order (names)
+    NDS, NDT, ROWB = D // 16, D // 32, 2 * D
+    N_MFMA = NDS + 2 * NDT  # MFMAs of the half step
 
     def read_k(ds):
         r = KF + 4 * ds
         emit("ds_read_b128 v[%d:%d], v%d offset:%%[koff]" % (r, r + 3, KA + ds))
         lds.append("k%d" % ds)
 
-    def read_v(ch, dt):
+    def read_v(ch, dt):  # chunk ch = 16 keys = 16 rows of the V tile; the second read is 8 rows further
         r = VF + 16 * ch + 4 * dt
-        emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%%[voff]+%d" % (r, r + 1, VA + dt, ch * 4096))
-        emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%%[voff]+%d" % (r + 2, r + 3, VA + dt, ch * 4096 + 2048))
+        emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%%[voff]+%d" % (r, r + 1, VA + dt, ch * 16 * ROWB))
+        emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%%[voff]+%d" % (r + 2, r + 3, VA + dt, ch * 16 * ROWB + 8 * ROWB))
         lds.append("v%d%d_lo" % (ch, dt))
         lds.append("v%d%d" % (ch, dt))
 
@@ -100,33 +108,41 @@ def gen(cur, nxt):
         del q[:n]
         return got
 
-    # preamble: K fragments 6 deep; the first scores' weights fill the wait for them
-    for ds in range(6):
+    # preamble: K fragments 6 deep (all 4 at D = 64); the first scores' weights fill the wait for them
+    k_ahead = min(6, NDS)
+    for ds in range(k_ahead):
         read_k(ds)
     for ins in take(11):  # the first four scores
         emit(ins)
-    per_slot = [4] * 12 + [0] * 4
-    for slot in range(16):
-        if slot < 8:
+    if D == 128:
+        per_slot = [4] * 12 + [0] * 4
+        v_reads = {slot: ((slot - 2) // 4, (slot - 2) % 4) for slot in range(2, 10)}
+        max_slots = (11, 12, 13)
+    else:  # the packed weights of chunk a are due before slot 4, those of chunk b before slot 6: all done in slot 4
+        per_slot = [10] * 4 + [6] + [0] * 3
+        v_reads = {0: (0, 0), 1: (0, 1), 2: (1, 0), 3: (1, 1)}
+        max_slots = (5, 6, 7)
+    for slot in range(N_MFMA):
+        if slot < NDS:
             ds = slot
             wait_for("k%d" % ds)
             s = "v[%d:%d]" % (nxt, nxt + 15)
             emit("v_mfma_f32_32x32x16_bf16 %s, v[%d:%d], v[%d:%d], %s" % (s, KF + 4 * ds, KF + 4 * ds + 3, QF + 4 * ds,
                                                                       QF + 4 * ds + 3, "0" if ds == 0 else s))
         else:
-            ch, dt = (slot - 8) // 4, (slot - 8) % 4
+            ch, dt = (slot - NDS) // NDT, (slot - NDS) % NDT
             wait_for("v%d%d" % (ch, dt))
             acc = "v[%d:%d]" % (O + 16 * dt, O + 16 * dt + 15)
             pw = cur + 8 * ch
             emit("v_mfma_f32_32x32x16_bf16 %s, v[%d:%d], v[%d:%d], %s" % (acc, VF + 16 * ch + 4 * dt, VF + 16 * ch + 4 * dt + 3, pw,
                                                                       pw + 3, acc))
-        if slot < 2:
-            read_k(6 + slot)
-        elif slot < 10:
-            read_v((slot - 2) // 4, (slot - 2) % 4)
+        if k_ahead + slot < NDS:
+            read_k(k_ahead + slot)
+        elif slot in v_reads:
+            read_v(*v_reads[slot])
         for ins in take(per_slot[slot]):
             emit(ins)
-        if 11 <= slot <= 13:
+        if slot in max_slots:
             for ins in mx[:2]:
                 emit(ins)
             del mx[:2]
@@ -187,10 +203,11 @@ def main():
     path = sys.argv[1]
     with open(path, "w") as f:
         f.write("// generated by gen_flash_attn_halfstep.py -- do not edit\n")
-        for name, cur, nxt in (("CUR_B", SB, SA), ("CUR_A", SA, SB)):
-            f.write("#define GCMI_FA_HALF_%s \\\n" % name)
-            f.write(" \\\n".join('  "%s\\n"' % ln for ln in gen(cur, nxt)))
-            f.write("\n\n")
+        for D, tag in ((128, "FA"), (64, "FA64")):
+            for name, cur, nxt in (("CUR_B", SB, SA), ("CUR_A", SA, SB)):
+                f.write("#define GCMI_%s_HALF_%s \\\n" % (tag, name))
+                f.write(" \\\n".join('  "%s\\n"' % ln for ln in gen(cur, nxt, D)))
+                f.write("\n\n")
         f.write("#define GCMI_FA_HALF_CLOBBERS %s\n" % ", ".join('"v%d"' % r for r in range(KF, TMP + 1)))
 
 

@@ -100,14 +100,17 @@ def test_mha_full_size_heads_and_invariants(gc, orc, wl, dev):
     assert (ones.float() - 1).abs().max().item() <= 2 ** -7
 
 
-@pytest.mark.parametrize("Sq,Sk,kind", [(512, 512, "causal"), (384, 640, "causal"), (256, 256, "neg1e9"), (300, 200, "random")])
-def test_skipping_masked_blocks_changes_no_bit(gc, dev, Sq, Sk, kind):
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("Sq,Sk,kind", [(512, 512, "causal"), (384, 640, "causal"), (256, 256, "neg1e9"), (300, 200, "random"),
+                                        (1000, 1000, "causal"), (200, 1100, "causal")])
+def test_skipping_masked_blocks_changes_no_bit(gc, dev, Sq, Sk, kind, D):
     """Key blocks whose mask tile is -inf for a whole query block carry softmax
-    weight exactly 0: leaving them out must give the same bits as visiting them."""
+    weight exactly 0: leaving them out must give the same bits as visiting them (both head dims of the pipelined
+    kernel, also with row and key counts off the tile sizes)."""
     torch.manual_seed(4)
-    Q = torch.randn(1, 8, Sq, 128).to(torch.bfloat16).to(dev)
-    K = torch.randn(1, 8, Sk, 128).to(torch.bfloat16).to(dev)
-    V = torch.randn(1, 8, Sk, 128).to(torch.bfloat16).to(dev)
+    Q = torch.randn(1, 8, Sq, D).to(torch.bfloat16).to(dev)
+    K = torch.randn(1, 8, Sk, D).to(torch.bfloat16).to(dev)
+    V = torch.randn(1, 8, Sk, D).to(torch.bfloat16).to(dev)
     mask = _mask(kind, Sq, Sk).to(dev)
     a = gc.mha_fwd_bf16(Q, K, V, mask, 0.088, skip_masked=True)
     b = gc.mha_fwd_bf16(Q, K, V, mask, 0.088, skip_masked=False)
@@ -139,6 +142,23 @@ def test_band_mask_over_many_key_blocks(gc, orc, wl, dev, skip):
                                            wl.bf16_bits(V[:, h:h + 1]), mask.numpy(), scale))
         assert_close(ref, out[:, h:h + 1].float().cpu().numpy(), 1e-2, "band mask head %d" % h,
                      mag=_pv_mag(Q[:, h:h + 1], K[:, h:h + 1], V[:, h:h + 1], mask, scale))
+
+
+@pytest.mark.parametrize("kind", ["causal", "none"])
+def test_head_dim_64_at_benchmark_size(gc, orc, wl, dev, kind):
+    """B4 H32 S2048 at head dim 64 on the pipelined kernel: three heads against the oracle."""
+    B, H, S, D = 4, 32, 2048, 64
+    Q, K, V, mask, scale = wl.bf16_mha(B, H, S, D)
+    if kind == "none":
+        mask = None
+    out = gc.mha_fwd_bf16(Q.to(dev), K.to(dev), V.to(dev), None if mask is None else mask.to(dev), scale)
+    torch.cuda.synchronize()
+    for (b, h) in [(0, 0), (2, 13), (3, 31)]:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = orc.bf16_to_f32(orc.mha_bf16(wl.bf16_bits(Q[sl]), wl.bf16_bits(K[sl]), wl.bf16_bits(V[sl]),
+                                           None if mask is None else mask.numpy(), scale))
+        assert_close(ref, out[sl].float().cpu().numpy(), 1e-2, "D=64 head (%d,%d) %s" % (b, h, kind),
+                     mag=_pv_mag(Q[sl], K[sl], V[sl], mask, scale))
 
 
 def test_negative_scale_takes_the_general_kernel(gc, orc, wl, dev):
