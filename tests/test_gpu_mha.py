@@ -26,7 +26,9 @@ CASES = [(1, 2, 128, 128, "causal"), (1, 1, 256, 192, "none"), (2, 2, 100, 77, "
          # row and key counts off the tile sizes on the pipelined kernel: the last workgroup / key block overlaps its
          # predecessor (duplicate keys masked out); general, constant and absent masks, one and several blocks
          (1, 2, 200, 200, "causal"), (1, 2, 130, 68, "random"), (2, 2, 300, 1000, "causal"), (1, 1, 257, 321, "none"),
-         (1, 2, 129, 127 + 1, "neg1e9"), (1, 1, 1000, 100, "random"), (1, 2, 1111, 1112, "causal")]
+         (1, 2, 129, 127 + 1, "neg1e9"), (1, 1, 1000, 100, "random"), (1, 2, 1111, 1112, "causal"),
+         # odd key counts with a mask: its rows start at any 4-byte aligned address
+         (1, 2, 131, 129, "random"), (1, 1, 1001, 1001, "causal"), (2, 2, 257, 70, "neg30000")]
 
 
 def _mask(kind, Sq, Sk):
