@@ -1,4 +1,5 @@
-// f32 GEMM (exact f32 FMA, no reduced-precision matrix path) and the
+// f32 GEMM (f32 multiply-add throughout: vector FMAs, or the f32 matrix
+// instruction on whole tiles; no reduced precision) and the
 // batch-reduce microkernel with the reference's operand layouts.
 //
 // gemm_f32_kernel: C[M,N] = act(beta*C + A.B + bias), arbitrary element strides
@@ -111,6 +112,88 @@ template <int BT> __global__ __launch_bounds__(256) void gemm_f32_kernel(F32Gemm
         x = x + p.bias[n];
       p.C[m * p.ldc + n] = apply_act(x, p.act);
     }
+  }
+}
+
+// The same GEMM on the matrix cores for whole 128 x 128 tiles of row-major operands: v_mfma_f32_32x32x2_f32 multiplies
+// and adds in f32 (no reduced precision), 256 flop per clock and compute unit against 128 for the vector ALU's FMA.
+// 256 threads = 4 waves as 2 x 2, a wave owns 64 x 64 = four 32 x 32 tiles (64 accumulator registers); 16-deep K
+// slices through LDS, the next slice prefetched into registers.  A is stored k-major in LDS ([k][m]) so that a
+// fragment read (lane = row, k = lane / 32) is one conflict-free ds_read_b32 per tile, B as it lies in memory.
+__global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(F32GemmParams p) {
+  constexpr int BT = 128, BK = 16;
+  __shared__ float As[BK][BT + 4];
+  __shared__ float Bs[BK][BT + 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, lh = lane >> 5;
+  const int64_t m0 = (int64_t)blockIdx.y * BT, n0 = (int64_t)blockIdx.x * BT;
+  p.A += (int64_t)blockIdx.z * p.a_bs, p.B += (int64_t)blockIdx.z * p.b_bs, p.C += (int64_t)blockIdx.z * p.c_bs;
+  // slice loads, 16 bytes per thread and operand piece: A 128 rows x 16 k = 512 float4 (two per thread: row = idx / 4,
+  // k = 4 * (idx % 4)), B 16 k x 128 n = 512 float4 (k = idx / 32, n = 4 * (idx % 32))
+  f32x4_t ra[2], rb[2];
+  auto fetch = [&](int64_t k0) {
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+      const int idx = tid + 256 * e;
+      ra[e] = *reinterpret_cast<const f32x4_t *>(p.A + (m0 + idx / 4) * p.a_rs + k0 + 4 * (idx % 4));
+      rb[e] = *reinterpret_cast<const f32x4_t *>(p.B + (k0 + idx / 32) * p.b_rs + n0 + 4 * (idx % 32));
+    }
+  };
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        acc[i][j][r] = 0.0f;
+  fetch(0);
+  for (int64_t k0 = 0; k0 < p.K; k0 += BK) {
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+      const int idx = tid + 256 * e;
+#pragma unroll
+      for (int c = 0; c < 4; c++)
+        As[4 * (idx % 4) + c][idx / 4] = ra[e][c];
+      *reinterpret_cast<f32x4_t *>(&Bs[idx / 32][4 * (idx % 32)]) = rb[e];
+    }
+    __syncthreads();
+    if (k0 + BK < p.K)
+      fetch(k0 + BK);
+#pragma unroll
+    for (int ks = 0; ks < BK; ks += 2) { // k ascending per output element
+      float a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+        a[i] = As[ks + lh][wm * 64 + i * 32 + l32];
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+        b[j] = Bs[ks + lh][wn * 64 + j * 32 + l32];
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  // lane (l32, lh) holds column l32 and rows 8 * (r / 4) + 4 * lh + r % 4 of every tile: 32 lanes write 128 bytes
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int64_t n = n0 + wn * 64 + j * 32 + l32;
+    const float bias = p.bias ? p.bias[n] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int64_t m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+        float x = acc[i][j][r];
+        if (p.beta != 0.0f)
+          x = x + p.C[m * p.ldc + n];
+        if (p.bias)
+          x = x + bias;
+        p.C[m * p.ldc + n] = apply_act(x, p.act);
+      }
   }
 }
 
@@ -265,6 +348,15 @@ extern "C" int gcmi_launch_gemm_f32(const F32GemmParams *pp, hipStream_t stream)
   const int64_t nbatch = p.batch > 1 ? p.batch : 1;
   if (nbatch > 65535)
     return 2;
+  // whole 128 x 128 tiles of row-major operands with 16-byte aligned rows, and enough of them: the matrix cores
+  auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  if (p.a_cs == 1 && p.b_cs == 1 && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 16 == 0 && p.K > 0 && p.a_rs % 4 == 0 &&
+      p.b_rs % 4 == 0 && al16(p.A) && al16(p.B) && (nbatch == 1 || (p.a_bs % 4 == 0 && p.b_bs % 4 == 0)) &&
+      (p.M / 128) * (p.N / 128) * nbatch >= 64 && p.M / 128 <= 65535) {
+    dim3 grid((unsigned)(p.N / 128), (unsigned)(p.M / 128), (unsigned)nbatch);
+    hipLaunchKernelGGL(gemm_f32_mfma_kernel, grid, dim3(256), 0, stream, p);
+    return hipGetLastError() == hipSuccess ? 0 : 5;
+  }
   auto tiles = [&](int bt) { return ((p.N + bt - 1) / bt) * ((p.M + bt - 1) / bt) * nbatch; };
   const int bt = tiles(64) >= 256 ? 64 : tiles(32) >= 256 ? 32 : 16;
   dim3 grid((unsigned)((p.N + bt - 1) / bt), (unsigned)((p.M + bt - 1) / bt), (unsigned)nbatch), block(256);

@@ -209,7 +209,9 @@ def test_int8_full_size_exact_checksums_and_rows(gc, orc, wl, dev):
 
 
 @pytest.mark.parametrize("M,N,K,ta,tb", [(128, 256, 512, False, False), (512, 64, 128, True, False),
-                                         (70, 33, 45, False, True), (65, 67, 19, True, True), (1, 1, 1, False, False)])
+                                         (70, 33, 45, False, True), (65, 67, 19, True, True), (1, 1, 1, False, False),
+                                         # 64 or more whole 128 x 128 tiles of row-major operands: the f32 matrix instruction
+                                         (1024, 1024, 256, False, False), (1536, 768, 80, False, False)])
 def test_f32_gemm_bias_relu(gc, orc, dev, M, N, K, ta, tb):
     torch.manual_seed(0)
     A = torch.rand((K, M) if ta else (M, K)) * 2 - 1
