@@ -729,10 +729,11 @@ __global__ __launch_bounds__(1024 / WJ, 1) void gemm_tile256_fast_kernel(GemmPar
 
   const int tiles_m = (int)((p.M + G_BM - 1) / G_BM), tiles_n = (int)(p.N / G_BN);
   int tm, tn, slice = 0;
-  if (SPLIT) { // one tile row: tile = column block, K slice = blockIdx / tiles
-    tm = 0;
-    tn = (int)blockIdx.x % tiles_n;
-    slice = (int)blockIdx.x / tiles_n;
+  if (SPLIT) { // the tiles of one K slice are neighbours in the grid; K slice = blockIdx / tiles
+    const int tiles = tiles_m * tiles_n, tile = (int)blockIdx.x % tiles;
+    tm = tile / tiles_n;
+    tn = tile % tiles_n;
+    slice = (int)blockIdx.x / tiles;
   } else {
     tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
   }
@@ -1675,6 +1676,16 @@ static void launch_splitk_reduce(const GemmParams &p, hipStream_t stream) {
 // Host-side launch of the 256x256 tile kernels for one element size.
 // want != null: nothing is launched; *want receives the floats of workspace this call would use if it had them.
 // cfg != null: receives what was (or would be) chosen.
+// constants of the slice-count choice (microseconds; the whole-K tile kernel must lose by this margin)
+#ifndef GCMI_SPLIT_T1_FIXED
+#define GCMI_SPLIT_T1_FIXED 8.0
+#endif
+#ifndef GCMI_SPLIT_W4_FIXED
+#define GCMI_SPLIT_W4_FIXED 10.0
+#endif
+#ifndef GCMI_SPLIT_MARGIN
+#define GCMI_SPLIT_MARGIN 0.9
+#endif
 template <int ES>
 static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *want = nullptr, GemmTileConfig *cfg = nullptr) {
   GemmParams p = *pp;
@@ -1725,30 +1736,66 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
   c.bm = G_BM, c.bn = G_BN, c.split_k = 1, c.group_m = p.group_m, c.workgroups = (int32_t)nblk;
   c.from_attrs = (p.cfg_waves || p.cfg_split_k) ? 1 : 0;
 
-  // One tile row and too few column tiles to fill the GPU (decode-style shapes such as 32 x 4096 x 4096): the
-  // weights have to stream from HBM through all compute units, so K is cut into slices, one workgroup per
-  // (column tile, slice); partial sums go through the workspace and a small second kernel.  The slice count is the
-  // reference's KThreads (lib/gc/Analysis/MatmulConfigAnalysis.cpp:149-166); a caller's wish replaces the default.
-  if (ES == 2 && fast_but_m && tiles_m == 1 && p.out_dt != DT_S32 && nbatch == 1) {
+  // Too few tiles to fill the GPU (decode-style shapes such as 32 x 4096 x 4096, where the weights have to stream
+  // from HBM through all compute units, and deep products such as 1024 x 1024 x 8192): K is cut into slices, one
+  // workgroup per (tile, slice); partial sums go through the workspace and a small second kernel.  The slice count
+  // plays the part of the reference's KThreads (lib/gc/Analysis/MatmulConfigAnalysis.cpp:149-166): here the count
+  // that makes the sum of a workgroup's share of K and the traffic of the partial sums smallest; a caller's wish
+  // replaces the default.
+  if (ES == 2 && fast_but_m && (nblk * 2 <= gcmi_num_cus() || p.cfg_split_k > 1) && p.out_dt != DT_S32 && nbatch == 1) {
     const int n_cu = gcmi_num_cus();
     const int groups = (int)(p.K / KGROUP);
-    int splits = (n_cu + tiles_n - 1) / tiles_n;
-    bool worth = tiles_n * 2 <= n_cu;
-    if (p.cfg_split_k > 0)
-      splits = p.cfg_split_k, worth = true;
+    const int tiles = (int)nblk;
+    int splits = 1;
+    // Rows of A fill at most half a tile: the kernel that skips the empty 32-row blocks of its tile, any slice count.
+    // Taller: the 4-wave kernel, run as a strided batch over equal K slices with f32 results (one slice = one batch).
+    bool by_w4 = p.M > 128;
+    if (p.cfg_split_k > 0) {
+      splits = p.cfg_split_k < groups ? p.cfg_split_k : groups;
+      by_w4 = by_w4 && groups % splits == 0;
+    } else {
+      // Microseconds, fitted to measurements: a workgroup's ring groups of K (128 elements each), the partial sums'
+      // way through memory (8 bytes each, about 1.7 us per slice and 2^20 outputs), and what a launch costs
+      // besides.  Slices never exceed one workgroup per compute unit.
+      const double mn = (double)p.M * (double)p.N / 1048576.0;
+      const int smax = n_cu / tiles < groups ? n_cu / tiles : groups;
+      double best = GCMI_SPLIT_T1_FIXED + 1.94 * groups;
+      if (by_w4) {
+        best *= GCMI_SPLIT_MARGIN;
+        for (int s = 2; s <= smax; s++)
+          if (groups % s == 0) {
+            const double t = GCMI_SPLIT_W4_FIXED + 1.94 * (groups / s) + 1.7 * s * mn;
+            if (t < best)
+              best = t, splits = s;
+          }
+      } else {
+        const double per_group = 1.35 + 0.65 * (double)((p.M + 31) / 32 - 1) / 3.0;
+        for (int s = 2; s <= smax; s++) {
+          const double t = 7.0 + per_group * ((groups + s - 1) / s) + 1.7 * s * mn;
+          if (t < best)
+            best = t, splits = s;
+        }
+      }
+    }
     splits = splits < groups ? splits : groups;
     if (want) {
-      if (splits > 1 && worth)
+      if (splits > 1)
         *want = (int64_t)splits * p.M * p.N;
       if (!cfg)
         return 0;
     }
-    while (splits > 1 && (int64_t)splits * p.M * p.N > ws_cap)
+    while (splits > 1 && ((int64_t)splits * p.M * p.N > ws_cap || (by_w4 && groups % splits != 0)))
       splits--;
-    if (splits > 1 && worth) {
-      c.kernel = GK_SPLITK, c.kbytes = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::KB, c.stages = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::NST;
-      c.waves_m = 2, c.waves_n = 8 / G_FAST_WJ, c.wave_m = 128, c.wave_n = 32 * G_FAST_WJ;
-      c.mfma_m = c.mfma_n = 32, c.mfma_k = 32 / ES, c.split_k = splits, c.workgroups = tiles_n * splits;
+    if (splits > 1) {
+      c.kernel = GK_SPLITK, c.split_k = splits, c.workgroups = tiles * splits;
+      if (by_w4) {
+        c.kbytes = 64, c.stages = 4, c.waves_m = 2, c.waves_n = 2, c.wave_m = 128, c.wave_n = 128;
+        c.mfma_m = c.mfma_n = 16, c.mfma_k = 64 / ES;
+      } else {
+        c.kbytes = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::KB, c.stages = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::NST;
+        c.waves_m = 2, c.waves_n = 8 / G_FAST_WJ, c.wave_m = 128, c.wave_n = 32 * G_FAST_WJ;
+        c.mfma_m = c.mfma_n = 32, c.mfma_k = 32 / ES;
+      }
       if (cfg)
         *cfg = c;
       if (dry)
@@ -1756,11 +1803,22 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
       p.splits = splits;
       p.partial = ws;
       if constexpr (ES == 2) {
-        if (p.trans_b)
+        if (by_w4) {
+          GemmParams q = p;
+          q.K = p.K / splits, q.batch = splits;
+          q.a_bs = q.K, q.b_bs = p.trans_b ? q.K : q.K * p.ldb, q.c_bs = p.M * p.N;
+          q.C = ws, q.ldc = p.N, q.out_dt = DT_F32;
+          q.bias = nullptr, q.act = ACT_NONE, q.residual = nullptr, q.partial = nullptr, q.splits = 0;
+          const dim3 grid((unsigned)tiles, (unsigned)splits);
+          if (p.trans_b)
+            hipLaunchKernelGGL((gemm_tile256_w4_kernel<ES, true>), grid, dim3(256), 0, stream, q);
+          else
+            hipLaunchKernelGGL(gemm_tile256_w4_kernel<ES>, grid, dim3(256), 0, stream, q);
+        } else if (p.trans_b)
           hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true, true>),
-                             dim3((unsigned)(tiles_n * splits)), dim3(1024 / G_FAST_WJ), 0, stream, p);
+                             dim3((unsigned)(tiles * splits)), dim3(1024 / G_FAST_WJ), 0, stream, p);
         else
-          hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true>), dim3((unsigned)(tiles_n * splits)),
+          hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true>), dim3((unsigned)(tiles * splits)),
                              dim3(1024 / G_FAST_WJ), 0, stream, p);
       }
       launch_splitk_reduce(p, stream);

@@ -6,7 +6,8 @@
  * asynchronous on `stream`.
  *
  * Scratch memory.  Two kinds of call need device memory beyond their operands:
- * K-sliced GEMMs (a short A against wide weights: f32 partial sums) and masked
+ * K-sliced GEMMs (too few 256 x 256 tiles for the GPU, e.g. a short A against
+ * wide weights or 1024 x 1024 x 8192: f32 partial sums) and masked
  * attention (one byte per mask tile).  Each entry point says where it comes
  * from:
  *   - plain entry points (gcmi_gemm_bf16, gcmi_mha_fwd_bf16, ...): a workspace
@@ -139,7 +140,8 @@ int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int6
  * type and layout).  `kernel`: 0 bounds-checked tile (any shape), 1 whole
  * tiles with 8 waves of 128 x 64, 2 tiles with 4 waves of 128 x 128 (any M,
  * N a multiple of 16 bytes of columns: edge tiles store what lies inside C),
- * 3 K slices over workgroups + second pass (one tile row), 4 weight-streaming
+ * 3 K slices over workgroups + second pass (tiles on less than half of the
+ * compute units), 4 weight-streaming
  * kernel (a short A against [N,K] weights).
  *
  * matmul_config (may be NULL) is the reference's per-op override: the nine

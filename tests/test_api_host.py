@@ -157,7 +157,7 @@ def test_arena_shares_memory_between_temporaries_with_disjoint_lifetimes(ga):
     allocations by lifetime ticks, lib/gc/Transforms/MergeAllocTickBased.cpp).  The plan reports both sizes."""
     import json
     import re
-    M = 512  # two tile rows: these matmuls are not K-sliced and need no scratch
+    M = 4096  # 256 tiles each: these matmuls are not K-sliced and need no scratch
     ops = []
     for i in range(4):
         src = 0 if i == 0 else 10 + i - 1

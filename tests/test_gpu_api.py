@@ -525,9 +525,11 @@ def test_matmul_config_attributes_change_the_kernel_not_the_result(ga, gc, orc, 
         _run(ga, ga._graph([op], [0, 1], [2]), [(0, A), (1, B)], [(2, out)])
         return A, B, out
 
-    A, B, dflt = run(512, 1024, 768, None)
+    A, B, dflt = run(512, 1024, 768, None)  # six tiles: the default cuts K into slices
+    _, _, w4 = run(512, 1024, 768, [2, 3, 1, 256, 256, 64, 128, 128, 32])
     _, _, w8 = run(512, 1024, 768, [2, 3, 1, 256, 256, 64, 128, 64, 32])
-    assert torch.equal(dflt.view(torch.int16), w8.view(torch.int16))
+    assert torch.equal(w4.view(torch.int16), w8.view(torch.int16))
+    assert (dflt.float() - w4.float()).abs().max().item() <= 0.0625
     ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A.cpu()), wl.bf16_bits(B.cpu())))
     assert_close(ref, dflt.float().cpu().numpy(), 1e-2, "default tile")
     A, B, s16 = run(32, 4096, 4096, None)

@@ -367,6 +367,77 @@ def test_short_a_takes_split_k(gc, orc, wl, dev, M, N, K, act, with_bias, out_f3
     assert torch.equal(out, again)  # fixed summation order: reruns agree bit for bit
 
 
+def _gemm_ws(gc, A, B, trans_b, out, slices=None, bias=None, act=None, ws=None):
+    """gcmi_gemm_bf16_ws with a caller's workspace; slices: the KThreads of a full MatmulConfig attribute set."""
+    import ctypes as C
+    M, K = A.shape
+    N = B.shape[0] if trans_b else B.shape[1]
+    cfg = None if slices is None else (C.c_int64 * 9)(1, 1, slices, 256, 256, 64, 128, 128, 32)
+    st = gc.lib().gcmi_gemm_bf16_ws(A.data_ptr(), B.data_ptr(), out.data_ptr(), 1, M, N, K, K, B.shape[1], N, 0, 0, 0, int(trans_b),
+                                    None if bias is None else bias.data_ptr(), gc.BF16, gc.ACT[act], None, 0, 0,
+                                    gc.F32 if out.dtype == torch.float32 else gc.BF16,
+                                    None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel() * ws.element_size(), cfg,
+                                    C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert st == 0, gc.lib().gcmi_last_error().decode()
+
+
+@pytest.mark.parametrize("M,N,K,act,with_bias,out_f32", [(512, 512, 4096, "relu", True, False), (300, 1024, 2048, "gelu_erf", True, False),
+                                                         (640, 768, 3072, None, True, True), (1024, 1024, 2048, None, False, False),
+                                                         (257, 2048, 1024, "sigmoid", False, False)])
+def test_few_tiles_and_a_deep_k_take_k_slices(gc, orc, wl, dev, M, N, K, act, with_bias, out_f32):
+    """Several tile rows but too few tiles for the GPU: equal K slices run as a strided batch of the 4-wave kernel
+    into f32 partial sums, the second kernel adds them and applies the epilogue.  Same rounding points as one pass."""
+    c, _ = gc.tile_config(M, N, K, out_dtype=gc.F32 if out_f32 else gc.BF16)
+    assert c.kernel == 3 and c.split_k > 1 and K // 128 % c.split_k == 0 and c.workgroups <= 256, (c.kernel, c.split_k, c.workgroups)
+    torch.manual_seed(M + N)
+    A = (torch.randn(M, K) * 0.5).to(torch.bfloat16)
+    torch.manual_seed(K)
+    B = (torch.randn(K, N) * 0.05).to(torch.bfloat16)
+    torch.manual_seed(3)
+    bias = torch.randn(N).to(torch.bfloat16) if with_bias else None
+    for trans_b in (False, True):
+        Bd = B.t().contiguous().to(dev) if trans_b else B.to(dev)
+        f = gc.gemm_bf16_nt if trans_b else gc.gemm_bf16
+        out = f(A.to(dev), Bd, None if bias is None else bias.to(dev), act, out_dtype=gc.F32 if out_f32 else gc.BF16)
+        again = f(A.to(dev), Bd, None if bias is None else bias.to(dev), act, out_dtype=gc.F32 if out_f32 else gc.BF16)
+        torch.cuda.synchronize()
+        assert torch.equal(out, again)  # fixed summation order: reruns agree bit for bit
+        if out_f32:
+            ref = A.float().double() @ B.float().double()
+            if bias is not None:
+                ref = ref + bias.double()
+            assert_close(ref.float().numpy(), out.cpu().numpy(), 1e-4, "k slices f32 out")
+        else:
+            ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B), None if bias is None else wl.bf16_bits(bias), act))
+            mm = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B)))
+            assert_close(ref, out.float().cpu().numpy(), 2e-2 if (with_bias or act) else 1e-2, "k slices", mag=mm)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_k_slices_exact_on_integers_for_any_slice_count(gc, dev, trans_b):
+    """Small integers make every partial sum exact, so each slice count must give the bits of the f32 product: the
+    default, even counts (the 4-wave kernel as a batch), counts that do not divide K's ring groups (the kernel with
+    slices of unequal length, here on two and three tile rows, the last one short), one slice (no second pass), a
+    workspace too small for the count asked for (fewer slices), and none at all."""
+    torch.manual_seed(11)
+    for M, N, K in [(512, 512, 2048), (600, 768, 1536), (257, 1024, 1024)]:
+        A = torch.randint(-3, 4, (M, K), device=dev).to(torch.bfloat16)
+        B = torch.randint(-3, 4, (K, N), device=dev).to(torch.bfloat16)
+        want = A.float() @ B.float()
+        Bd = B.t().contiguous() if trans_b else B
+        ws = torch.empty(16 * M * N, dtype=torch.float32, device=dev)
+        for slices, w in [(None, ws), (1, ws), (2, ws), (3, ws), (4, ws), (5, ws), (7, ws), (8, ws), (4, ws[:2 * M * N + 5]), (4, None)]:
+            out = torch.full((M, N), 7.0, dtype=torch.float32, device=dev)
+            _gemm_ws(gc, A, Bd, trans_b, out, slices, ws=w)
+            torch.cuda.synchronize()
+            assert torch.equal(out, want), (M, N, K, slices, None if w is None else w.numel())
+        bias = torch.randint(-4, 5, (N,), device=dev).to(torch.bfloat16)
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        _gemm_ws(gc, A, Bd, trans_b, out, 3, bias=bias, act="relu", ws=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(out, torch.relu((want.to(torch.bfloat16).float() + bias.float()).to(torch.bfloat16)))  # rounded after each op
+
+
 NT_SHAPES = [(256, 256, 128), (512, 768, 256), (300, 200, 100), (257, 511, 129), (1, 7, 5), (33, 1, 64), (128, 256, 8),
              (32, 4096, 4096), (1, 1024, 2048), (32, 11008, 4096), (64, 512, 2048), (33, 1024, 1024), (17, 2048, 512),
              (32, 4096, 11008), (65, 1024, 1024), (32, 1056, 1088), (32, 8192, 1024), (64, 8192, 512)]

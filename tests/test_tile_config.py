@@ -74,12 +74,12 @@ def test_explain_prints_the_descriptor_and_the_override(ga, gc):
 def test_mlir_attribute_dictionary_is_read(ga):
     attrs = "{MThreads = 4 : i32, NThreads = 2 : i32,  KThreads = 1 : i32, MBlock = 256 : i32, NBlock = 256 : i32, " \
             "KBlock = 256 : i32,innermostMBlock = 128 : i32, innermostNBlock = 64 : i32,  innermostKBlock = 32 : i32 }"
-    mod = """func.func @entry(%a: tensor<512x512xbf16>, %b: tensor<512x512xbf16>) -> tensor<512x512xbf16> {
+    mod = """func.func @entry(%a: tensor<4096x4096xbf16>, %b: tensor<4096x4096xbf16>) -> tensor<4096x4096xbf16> {
   %c0 = arith.constant 0.0 : bf16
-  %e = tensor.empty() : tensor<512x512xbf16>
-  %z = linalg.fill ins(%c0 : bf16) outs(%e : tensor<512x512xbf16>) -> tensor<512x512xbf16>
-  %r = linalg.matmul """ + attrs + """ ins(%a, %b : tensor<512x512xbf16>, tensor<512x512xbf16>) outs(%z : tensor<512x512xbf16>) -> tensor<512x512xbf16>
-  return %r : tensor<512x512xbf16>
+  %e = tensor.empty() : tensor<4096x4096xbf16>
+  %z = linalg.fill ins(%c0 : bf16) outs(%e : tensor<4096x4096xbf16>) -> tensor<4096x4096xbf16>
+  %r = linalg.matmul """ + attrs + """ ins(%a, %b : tensor<4096x4096xbf16>, tensor<4096x4096xbf16>) outs(%z : tensor<4096x4096xbf16>) -> tensor<4096x4096xbf16>
+  return %r : tensor<4096x4096xbf16>
 }"""
     st, plan = ga.explain_mlir(mod)
     assert st == 0 and "8 waves" in plan and "[MatmulConfig attributes applied]" in plan, plan
