@@ -213,7 +213,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32,decode,api,block,norm")
+    ap.add_argument("--only", default="", help="comma list of: gemm,int8,chain,mha,f32,decode,api,block,norm,brgemm,ragged,few_tiles")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the 4096^3 GEMM the CPU baseline computes")
     ap.add_argument("--mha-mode", default="both", choices=["both", "skip", "every"],
                     help="attention: time the default entry point (masked key blocks skipped), the every-block mode, or both")
@@ -407,18 +407,37 @@ def main():
         del Ar, Br, Cr
         for name, S, D in (("bf16_mha_b4_h32_s2000_d128_causal", 2000, 128), ("bf16_mha_b4_h32_s2048_d64_causal", 2048, 64)):
             Q, Kk, V, mask, scale = wl.bf16_mha(4, 32, S, D)
-            Qd, Kd, Vd, md = Q.to(dev), Kk.to(dev), V.to(dev), mask.to(dev)
+            Qd, Kkd, Vd, md = Q.to(dev), Kk.to(dev), V.to(dev), mask.to(dev)
             Od = torch.empty_like(Qd)
-            t = time_launches(torch, lambda i: gc.mha_fwd_bf16(Qd, Kd, Vd, md, scale, out=Od), 1, max(10, K // 4), 5)
+            t = time_launches(torch, lambda i: gc.mha_fwd_bf16(Qd, Kkd, Vd, md, scale, out=Od), 1, max(10, K // 4), 5)
             rag[name] = {"ms_per_step": round(t["ms_per_step"], 5),
                          "value": round(4.0 * 4 * 32 * S * S * D / t["ms_per_step"] / 1e9, 1),
                          "unit": "TFLOP/s (dense count, masked blocks skipped)"}
-            del Qd, Kd, Vd, md, Od
+            del Qd, Kkd, Vd, md, Od
         others["shapes_off_the_tile_sizes"] = {
             "workload": "M and N of a GEMM not multiples of 256 (edge tiles of the whole-tile kernel), a sequence length "
                         "that is not a multiple of 128 / 64 (overlapping last windows on the pipelined attention kernel), "
                         "head dim 64 (the pipelined attention kernel's second instantiation)", "cases": rag}
         log("off the tile sizes: %s" % json.dumps(rag))
+        torch.cuda.empty_cache()
+
+    # ---------------- bf16 GEMMs whose 256 x 256 tiles would not fill the GPU: 128 x 128 tiles and / or K slices
+    if want("few_tiles"):
+        few = {}
+        for Mf, Nf, Kf in ((2048, 2048, 2048), (1024, 4096, 4096), (512, 4096, 4096), (1024, 1024, 8192), (2048, 4096, 4096)):
+            Af = (torch.randn(Mf, Kf) * 0.1).to(torch.bfloat16).to(dev)
+            Bf = (torch.randn(Kf, Nf) * 0.1).to(torch.bfloat16).to(dev)
+            Cf = torch.empty(Mf, Nf, dtype=torch.bfloat16, device=dev)
+            t = time_launches(torch, lambda i: gc.gemm_bf16(Af, Bf, out=Cf), 1, max(20, K // 2), W)
+            cfgf, _ = gc.tile_config(Mf, Nf, Kf)
+            few["%dx%dx%d" % (Mf, Nf, Kf)] = {"ms_per_step": round(t["ms_per_step"], 5),
+                                              "value": round(2.0 * Mf * Nf * Kf / t["ms_per_step"] / 1e9, 1), "unit": "TFLOP/s",
+                                              "tile": int(cfgf.bm), "k_slices": int(cfgf.split_k), "workgroups": int(cfgf.workgroups)}
+            del Af, Bf, Cf
+        others["bf16_gemm_few_tiles"] = {
+            "workload": "bf16 GEMMs of 16 to 128 tiles of 256 x 256 (one compute unit works 1.9 us per tile and 128 of K): the "
+                        "launcher gives them to more workgroups by 128 x 128 tiles, equal K slices, or both", "cases": few}
+        log("few tiles: %s" % json.dumps(few))
         torch.cuda.empty_cache()
 
     # ---------------- f32 plumbing case (configs[0])

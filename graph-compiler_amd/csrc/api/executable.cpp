@@ -1737,7 +1737,8 @@ std::string Executable::describe() const {
   static const char *names[] = {"gemm_f32", "gemm_bf16", "gemm_int8", "colsum", "attention", "eltwise", "reduce", "softmax"};
   std::ostringstream os;
   static const char *kernels[] = {"bounds-checked tile", "whole tiles, 8 waves", "whole tiles, 4 waves (one per SIMD)",
-                                  "K slices + second pass", "weight streaming (+ second pass)"};
+                                  "K slices + second pass", "weight streaming (+ second pass)",
+                                  "small tiles, 4 waves, two workgroups per compute unit"};
   for (auto &s : steps_) {
     os << (s.kind == Step::Fused ? (s.sum_ins >= 0 ? "reduce" : "fused") : names[(int)s.kind]) << ": " << s.note << "\n";
     if ((s.kind == Step::GemmBf16 && s.batch <= 1 && !s.ta) || s.kind == Step::GemmInt8) {

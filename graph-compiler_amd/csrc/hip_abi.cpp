@@ -163,8 +163,20 @@ bool apply_matmul_config(const int64_t *c, int64_t M, int64_t N, int64_t K, Gemm
     *why = "invalid (fewer K blocks than KThreads)";
     return false;
   }
+  if (MBlock == 128 && NBlock == 128) { // the small tile: 4 waves of 64 x 64, no K slices
+    if (iM != 64 || iN != 64) {
+      *why = "not built (a wave's tile of the 128 x 128 workgroup tile is 64 x 64)";
+      return false;
+    }
+    if (KThreads != 1) {
+      *why = "not built (the 128 x 128 workgroup tile takes no K slices)";
+      return false;
+    }
+    p.cfg_tile = 128;
+    return true;
+  }
   if (MBlock != 256 || NBlock != 256) {
-    *why = "not built (the workgroup tile is 256 x 256)";
+    *why = "not built (the workgroup tile is 256 x 256 or 128 x 128)";
     return false;
   }
   if (iM != 128 || (iN != 128 && iN != 64)) {
@@ -172,6 +184,7 @@ bool apply_matmul_config(const int64_t *c, int64_t M, int64_t N, int64_t K, Gemm
     return false;
   }
   (void)M, (void)N;
+  p.cfg_tile = 256;
   p.cfg_waves = iN == 128 ? 4 : 8;
   p.cfg_split_k = (int32_t)(KThreads > 1024 ? 1024 : KThreads);
   return true;

@@ -38,6 +38,7 @@ struct GemmParams {
   // wishes of the caller (the op's MatmulConfig attributes, translated): 0 = the launcher's own choice
   int32_t cfg_waves;    // 4 or 8 waves per workgroup on whole tiles
   int32_t cfg_split_k;  // number of K slices (1: none) where the shape can be sliced
+  int32_t cfg_tile;     // 128: the 128 x 128 tile kernel where the shape allows it; 256: never that kernel
 };
 
 // What the launcher decides for one GEMM call: the GPU's counterpart of the reference's MatmulConfig
@@ -60,8 +61,9 @@ enum GemmKernel : int32_t {
   GK_EDGE = 0,    // bounds-checked 256x256 tile, 8 waves, 32x32 MFMAs: any shape and alignment
   GK_WAVES8 = 1,  // whole tiles, 8 waves of 128 x 64, 16x16 MFMAs
   GK_WAVES4 = 2,  // whole tiles, 4 waves of 128 x 128 (one per SIMD), 16x16 MFMAs, hand-placed main loop
-  GK_SPLITK = 3,  // one tile row: K slices over workgroups + second pass
+  GK_SPLITK = 3,  // too few tiles for the GPU: K slices over workgroups + second pass
   GK_STREAM = 4,  // a short A against [N,K] weights: weight-streaming kernel (+ second pass)
+  GK_TILE128 = 5, // 128 x 128 tiles, 4 waves of 64 x 64, two workgroups per compute unit: problems of few 256 x 256 tiles
 };
 
 struct F32GemmParams {

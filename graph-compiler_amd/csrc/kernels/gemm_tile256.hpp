@@ -1320,17 +1320,19 @@ __device__ __forceinline__ void w4_epilogue_row(const GemmParams &p, const acc4_
 
 // One half (64 columns) of the wave tile.  OUT = DT_BF16 / DT_F32 / DT_S32.
 // MASKED: rows_in / cols_in of the tile's 256 x 256 lie inside C (cols_in is a multiple of 4).
-template <int ES, int ACT, int OUT, bool MASKED>
+// WR x WC: the wave's tile (128 x 128 in the 256 x 256 kernel, 64 x 64 in the 128 x 128 one); rows_in / cols_in count
+// from the workgroup tile's corner whatever its size.
+template <int ES, int ACT, int OUT, bool MASKED, int WR = 128, int WC = 128>
 __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, int64_t m0, int64_t n0, int wm, int wn,
                                                  int lane, const char *dump, const float *colp, int rows_in, int cols_in) {
   typedef typename std::conditional<ES == 2, float, int>::type acc_e;
   typedef acc_e acc4_t __attribute__((ext_vector_type(4)));
   const int rr = lane >> 4, cc = lane & 15;
-  const int col = wn * 128 + half * 64 + 4 * cc; // this lane's four columns inside the workgroup tile
+  const int col = wn * WC + half * 64 + 4 * cc; // this lane's four columns inside the workgroup tile
   const int64_t n = n0 + col;
   if (MASKED && col >= cols_in)
     return;
-  const int row0 = wm * 128 + rr; // + 4 * (i0 + u)
+  const int row0 = wm * WR + rr; // + 4 * (i0 + u)
   const f32x4_t bias4 = *reinterpret_cast<const f32x4_t *>(colp + col); // -0.0 where there is no bias
   f32x4_t scale4 = {1.f, 1.f, 1.f, 1.f};
   i32x4_t cs4 = {0, 0, 0, 0}; // comp * colsum
@@ -1350,7 +1352,7 @@ __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, 
   }
   constexpr int U = 8; // rows in flight per lane
 #pragma unroll 1
-  for (int i0 = 0; i0 < 32; i0 += U) {
+  for (int i0 = 0; i0 < WR / 4; i0 += U) {
     acc4_t c[U];
 #pragma unroll
     for (int u = 0; u < U; u++)
@@ -1408,13 +1410,13 @@ __device__ __forceinline__ void w4_epilogue_half(const GemmParams &p, int half, 
 }
 
 // kind = act + 8 * (0: bf16, 1: f32, 2: s32)
-template <int ES, bool MASKED>
+template <int ES, bool MASKED, int WR = 128, int WC = 128>
 __device__ __forceinline__ void w4_epilogue_half_any(const GemmParams &p, int kind, int half, int64_t m0, int64_t n0,
                                                      int wm, int wn, int lane, const char *dump, const float *colp,
                                                      int rows_in, int cols_in) {
 #define GCMI_W4_CASE(ACT, OUT, K)                                                                                     \
   case (int)ACT + 8 * K:                                                                                              \
-    w4_epilogue_half<ES, ACT, OUT, MASKED>(p, half, m0, n0, wm, wn, lane, dump, colp, rows_in, cols_in);              \
+    w4_epilogue_half<ES, ACT, OUT, MASKED, WR, WC>(p, half, m0, n0, wm, wn, lane, dump, colp, rows_in, cols_in);      \
     break;
   switch (kind) {
     GCMI_W4_CASE(ACT_RELU, DT_BF16, 0)
@@ -1428,7 +1430,7 @@ __device__ __forceinline__ void w4_epilogue_half_any(const GemmParams &p, int ki
     GCMI_W4_CASE(ACT_SIGMOID, DT_F32, 1)
     GCMI_W4_CASE(ACT_NONE, DT_S32, 2)
   default:
-    w4_epilogue_half<ES, ACT_NONE, DT_BF16, MASKED>(p, half, m0, n0, wm, wn, lane, dump, colp, rows_in, cols_in);
+    w4_epilogue_half<ES, ACT_NONE, DT_BF16, MASKED, WR, WC>(p, half, m0, n0, wm, wn, lane, dump, colp, rows_in, cols_in);
     break;
   }
 #undef GCMI_W4_CASE
@@ -1585,6 +1587,209 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gem
 #endif
 }
 
+// ---------------------------------------------------------------------------
+// 128 x 128 tiles for bf16 problems whose 256 x 256 tiles would leave most of the GPU idle (a 256 x 256 tile keeps
+// one compute unit busy for 1.9 us per 128 elements of K whatever else the GPU does).  4 waves as 2 x 2, each owning
+// 64 x 64 as 4 x 4 tiles of 16 x 16 (v_mfma_f32_16x16x32_bf16, 64 accumulator registers), two workgroups per compute
+// unit so that one computes while the other waits at its barrier.  Ring of 4 stages of 32 elements of K (A 8 KiB +
+// B 8 KiB each), filled by global_load_lds_dwordx4 with the swizzles of the 256 x 256 kernels (A rows of 64 bytes:
+// chunk ^ (row / 4 % 4); B rows of 256 bytes read through the transposing LDS load: chunk ^ 4 * (k % 4)).  A stage
+// computes k-block s from registers while the fragments of block s+1 are read and block s+3 is requested; one
+// barrier per stage.  Rows past M and columns past N (N a multiple of 8) are fetched from the last row / chunk
+// inside and never stored.  The epilogue is the 4-wave kernel's: accumulators through a wave-private LDS region,
+// then rows of four columns per lane.
+static constexpr int T128_B = 128, T128_KB = 64, T128_NST = 4;
+static constexpr int T128_A_BYTES = T128_B * T128_KB, T128_STAGE_BYTES = 2 * T128_A_BYTES;
+static constexpr int T128_DUMP_WAVE_BYTES = 64 * W4_DUMP_PITCH; // 17408 per wave
+static constexpr int T128_SMEM_BYTES = 4 * T128_DUMP_WAVE_BYTES + T128_B * 4;
+static_assert(T128_NST * T128_STAGE_BYTES <= 4 * T128_DUMP_WAVE_BYTES, "the ring overlaps the column parameters");
+
+template <bool TB = false> __global__ __launch_bounds__(256, 2) void gemm_tile128_kernel(GemmParams p) {
+  constexpr int ES = 2, KB = T128_KB, BK = KB / ES, NST = T128_NST, A_BYTES = T128_A_BYTES, STAGE = T128_STAGE_BYTES;
+  constexpr int RG = 4, CW = 4, B_ROW_BYTES = T128_B * ES, B_CPR = B_ROW_BYTES / 16;
+  __shared__ __align__(1024) char smem[T128_SMEM_BYTES];
+  float *colp = reinterpret_cast<float *>(smem + 4 * T128_DUMP_WAVE_BYTES);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int r16 = lane & 15, g16 = lane >> 4;
+
+  const int tiles_m = (int)((p.M + T128_B - 1) / T128_B), tiles_n = (int)((p.N + T128_B - 1) / T128_B);
+  int tm, tn;
+  tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, p.group_m, tm, tn);
+  tm = __builtin_amdgcn_readfirstlane(tm), tn = __builtin_amdgcn_readfirstlane(tn);
+  const int64_t m0 = (int64_t)tm * T128_B, n0 = (int64_t)tn * T128_B;
+  const int64_t lda_b = p.lda * ES, ldb_b = p.ldb * ES;
+  {
+    const int64_t bz = blockIdx.y; // strided batch
+    p.A = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * ES;
+    p.B = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * ES;
+    p.C = reinterpret_cast<char *>(p.C) + bz * p.c_bs * (p.out_dt == DT_BF16 ? 2 : 4);
+    if (p.residual)
+      p.residual = reinterpret_cast<const char *>(p.residual) + bz * p.c_bs * (p.residual_dt == DT_BF16 ? 2 : 4);
+  }
+  const int rows_in = (int)min((int64_t)T128_B, p.M - m0), cols_in = (int)min((int64_t)T128_B, p.N - n0);
+
+  // this wave's two DMA instructions per operand and stage: 1 KiB each = 16 rows of A (or of B stored [N,K]), 4 k-rows of B
+  uint32_t a_src[2], b_src[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int d = wave * 2 + i;
+    const int row = d * 16 + lane / 4;
+    const int c = (lane % 4) ^ ((row >> 2) & 3);
+    a_src[i] = (uint32_t)(min(row, rows_in - 1) * lda_b + c * 16);
+    const int krow = d * 4 + lane / B_CPR;
+    const int cb = min((lane % B_CPR) ^ ((krow % RG) * CW), cols_in * ES / 16 - 1);
+    b_src[i] = TB ? (uint32_t)(min(row, cols_in - 1) * ldb_b + c * 16) : (uint32_t)(krow * ldb_b + cb * 16);
+  }
+  auto issue = [&](char *__restrict__ stage, const char *a_base, const char *b_base) {
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(a_base + a_src[i]),
+                                       (GCMI_LDS void *)(stage + (wave * 2 + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(b_base + b_src[i]),
+                                       (GCMI_LDS void *)(stage + A_BYTES + (wave * 2 + i) * 1024), 16, 0, 0);
+  };
+  // fragment reads as in gemm_tile256_mi16_kernel: A tile `it` = rows wm*64 + 16*it .., B tile `jt` = columns wn*64 + 16*jt ..
+  const int row_a = wm * 64 + r16;
+  const uint32_t a_ld = (uint32_t)(row_a * KB + ((g16 ^ ((row_a >> 2) & 3)) << 4));
+  uint32_t b_ld[4];
+  {
+    const int kk = r16 >> 2, cc = r16 & 3;
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++) {
+      const int chunk = (wn * 4 + jt) * 2 + (cc >> 1);
+      b_ld[jt] = (uint32_t)(A_BYTES + (2 * RG * g16 + kk) * B_ROW_BYTES + ((chunk ^ (kk * CW)) << 4) + (cc & 1) * 8);
+      if (TB) {
+        const int row_b = wn * 64 + jt * 16 + r16;
+        b_ld[jt] = (uint32_t)(A_BYTES + row_b * KB + ((g16 ^ ((row_b >> 2) & 3)) << 4));
+      }
+    }
+  }
+  auto load_frags = [&](const char *__restrict__ st, uint4(&a)[4], uint4(&b)[4]) {
+#pragma unroll
+    for (int it = 0; it < 4; it++)
+      a[it] = *reinterpret_cast<const uint4 *>(st + a_ld + it * (16 * KB));
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++) {
+      if constexpr (TB) {
+        b[jt] = *reinterpret_cast<const uint4 *>(st + b_ld[jt]);
+      } else {
+        const uint2 lo = MfmaOp<ES>::tr_read(st + b_ld[jt]);
+        const uint2 hi = MfmaOp<ES>::tr_read(st + b_ld[jt] + RG * B_ROW_BYTES);
+        b[jt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+    }
+  };
+  f32x4_t acc[4][4]; // [jt][it]: rows 16*it + lane%16, columns 16*jt + 4*(lane/16) .. +3 (B fragment as first operand)
+#pragma unroll
+  for (int jt = 0; jt < 4; jt++)
+#pragma unroll
+    for (int it = 0; it < 4; it++)
+      acc[jt][it] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  auto mfma_all = [&](const uint4(&a)[4], const uint4(&b)[4]) {
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++)
+#pragma unroll
+      for (int it = 0; it < 4; it++)
+        acc[jt][it] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b[jt]),
+                                                              __builtin_bit_cast(bf16x8_t, a[it]), acc[jt][it], 0, 0, 0);
+  };
+
+  const int64_t b_step = TB ? (int64_t)KB : (int64_t)BK * ldb_b;
+  const int KT = (int)(p.K / BK); // a positive multiple of NST (checked by the launcher)
+  const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b;
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + (TB ? n0 * ldb_b : n0 * ES);
+
+  float cp_bias = -0.0f; // an absent bias adds nothing, not even to -0.0
+  if (tid < cols_in && p.bias)
+    cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n0 + tid])
+                                   : reinterpret_cast<const float *>(p.bias)[n0 + tid];
+#pragma unroll
+  for (int d = 0; d < NST - 1; d++)
+    issue(smem + d * STAGE, a_ptr + d * KB, b_ptr + d * b_step);
+  if (tid < T128_B)
+    colp[tid] = cp_bias;
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NST - 2) * 4) : "memory");
+  __builtin_amdgcn_s_barrier();
+  uint4 fa0[4], fb0[4], fa1[4], fb1[4];
+  load_frags(smem, fa0, fb0);
+
+  // One stage: k-block kt is in the `cur` registers.  Request block kt+NST-1 into the slot block kt-1 was read from
+  // (every wave's reads of it had returned before it passed the previous barrier); wait for this wave's share of
+  // block kt+1 and for its own LDS reads; barrier: block kt+1 is visible; read its fragments under the MFMAs of kt.
+  auto stage = [&](auto has_fill, auto has_next, auto behindc, const char *__restrict__ nxt, char *__restrict__ fill,
+                   const char *a_fill, const char *b_fill, uint4(&ca)[4], uint4(&cb)[4], uint4(&na)[4], uint4(&nb)[4]) {
+    constexpr bool HAS_FILL = decltype(has_fill)::value, HAS_NEXT = decltype(has_next)::value;
+    constexpr int BEHIND = decltype(behindc)::value;
+    if constexpr (HAS_FILL)
+      issue(fill, a_fill, b_fill);
+    if constexpr (HAS_NEXT) {
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(BEHIND * 4) : "memory");
+      __builtin_amdgcn_s_barrier();
+      load_frags(nxt, na, nb);
+    }
+    mfma_all(ca, cb);
+    // MFMA, two LDS reads, MFMA, two LDS reads ... then the remaining MFMAs
+    if constexpr (HAS_NEXT) {
+      constexpr int N_DS = TB ? 8 : 12;
+      static_for<0, 16>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        constexpr int left = N_DS - 2 * i;
+        if constexpr (left > 0)
+          __builtin_amdgcn_sched_group_barrier(0x100, left < 2 ? left : 2, 0);
+      });
+    }
+  };
+  typedef std::integral_constant<bool, true> T;
+  typedef std::integral_constant<bool, false> F;
+  int kt0 = 0;
+  for (; kt0 + 2 * NST <= KT; kt0 += NST) {
+    static_for<0, NST>([&](auto sc) {
+      constexpr int st = decltype(sc)::value;
+      constexpr int nxt = (st + 1) % NST, fill = (st + NST - 1) % NST;
+      const int kf = kt0 + st + NST - 1;
+      if constexpr (st % 2 == 0)
+        stage(T{}, T{}, std::integral_constant<int, NST - 2>{}, smem + nxt * STAGE, smem + fill * STAGE, a_ptr + (int64_t)kf * KB,
+              b_ptr + kf * b_step, fa0, fb0, fa1, fb1);
+      else
+        stage(T{}, T{}, std::integral_constant<int, NST - 2>{}, smem + nxt * STAGE, smem + fill * STAGE, a_ptr + (int64_t)kf * KB,
+              b_ptr + kf * b_step, fa1, fb1, fa0, fb0);
+    });
+  }
+  static_for<0, NST>([&](auto sc) { // last group: only its first stage requests a block; the ring drains
+    constexpr int st = decltype(sc)::value;
+    constexpr int nxt = (st + 1) % NST, fill = (st + NST - 1) % NST;
+    constexpr int behind = NST - 2 - st > 0 ? NST - 2 - st : 0;
+    const int kf = kt0 + st + NST - 1;
+    if constexpr (st % 2 == 0)
+      stage(std::integral_constant<bool, st == 0>{}, std::integral_constant<bool, (st < NST - 1)>{}, std::integral_constant<int, behind>{},
+            smem + nxt * STAGE, smem + fill * STAGE, a_ptr + (int64_t)kf * KB, b_ptr + kf * b_step, fa0, fb0, fa1, fb1);
+    else
+      stage(std::integral_constant<bool, st == 0>{}, std::integral_constant<bool, (st < NST - 1)>{}, std::integral_constant<int, behind>{},
+            smem + nxt * STAGE, smem + fill * STAGE, a_ptr + (int64_t)kf * KB, b_ptr + kf * b_step, fa1, fb1, fa0, fb0);
+  });
+
+  // the accumulator regions lie over the ring: every wave's reads of the last block must have returned
+  __syncthreads();
+  char *dump = smem + wave * T128_DUMP_WAVE_BYTES;
+#pragma unroll
+  for (int jt = 0; jt < 4; jt++)
+#pragma unroll
+    for (int it = 0; it < 4; it++)
+      *reinterpret_cast<f32x4_t *>(dump + (it * 16 + r16) * W4_DUMP_PITCH + (jt * 16 + 4 * g16) * 4) = acc[jt][it];
+  const int kind = p.act + 8 * (p.out_dt == DT_BF16 ? 0 : 1);
+  if (rows_in < T128_B || cols_in < T128_B)
+    w4_epilogue_half_any<ES, true, 64, 64>(p, kind, 0, m0, n0, wm, wn, lane, dump, colp, rows_in, cols_in);
+  else
+    w4_epilogue_half_any<ES, false, 64, 64>(p, kind, 0, m0, n0, wm, wn, lane, dump, colp, T128_B, T128_B);
+}
+
 // Second pass of split-K: out = epilogue(sum over slices of the f32 partials), slices added in ascending
 // order (deterministic), the same rounding points as the fused epilogue.  One thread per 4 columns; the
 // loads of eight slices are in flight together.
@@ -1676,16 +1881,32 @@ static void launch_splitk_reduce(const GemmParams &p, hipStream_t stream) {
 // Host-side launch of the 256x256 tile kernels for one element size.
 // want != null: nothing is launched; *want receives the floats of workspace this call would use if it had them.
 // cfg != null: receives what was (or would be) chosen.
-// constants of the slice-count choice (microseconds; the whole-K tile kernel must lose by this margin)
-#ifndef GCMI_SPLIT_T1_FIXED
-#define GCMI_SPLIT_T1_FIXED 8.0
-#endif
-#ifndef GCMI_SPLIT_W4_FIXED
-#define GCMI_SPLIT_W4_FIXED 10.0
-#endif
-#ifndef GCMI_SPLIT_MARGIN
-#define GCMI_SPLIT_MARGIN 0.9
-#endif
+// Estimates behind the choice of tile and K slices for bf16 problems that do not fill the GPU with 256 x 256 tiles,
+// in microseconds, fitted to graph-replayed timings on a 256-CU board (load = workgroups / compute units).  One ring
+// group = 128 elements of K.  The rates grow with the load because the board lowers its clock as more of it works.
+static inline double gcmi_us_per_group_256(double load) { // one workgroup per compute unit
+  if (load <= 0.25)
+    return 1.94;
+  if (load <= 0.5)
+    return 1.94 + 0.16 * (load - 0.25) / 0.25;
+  if (load <= 1.0)
+    return 2.1 + 0.65 * (load - 0.5) / 0.5;
+  return 2.75;
+}
+static inline double gcmi_us_per_group_128(double load) { // up to two workgroups per compute unit
+  if (load <= 0.25)
+    return 0.85;
+  if (load <= 1.0)
+    return 0.85 + 0.27 * (load - 0.25) / 0.75;
+  if (load <= 2.0)
+    return 1.12 + 1.05 * (load - 1.0);
+  return 2.17;
+}
+static constexpr double GCMI_US_FIXED_256 = 8.0, GCMI_US_FIXED_128 = 3.7; // launch, ring fill, epilogue
+static constexpr double GCMI_US_SECOND_PASS = 3.0;     // the second kernel of a K-sliced product
+static constexpr double GCMI_US_PER_SLICE_MOUT = 1.7;  // partial sums written and read back, per slice and 2^20 outputs
+static constexpr double GCMI_ONE_PASS_MARGIN = 0.9;    // slices must win by this factor
+enum GemmPlan { PLAN_TILE256 = 0, PLAN_TILE128, PLAN_SLICES_SHORT_A, PLAN_SLICES_TILE256, PLAN_SLICES_TILE128 };
 template <int ES>
 static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *want = nullptr, GemmTileConfig *cfg = nullptr) {
   GemmParams p = *pp;
@@ -1734,96 +1955,142 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
     p.group_m = 4;
   GemmTileConfig c{};
   c.bm = G_BM, c.bn = G_BN, c.split_k = 1, c.group_m = p.group_m, c.workgroups = (int32_t)nblk;
-  c.from_attrs = (p.cfg_waves || p.cfg_split_k) ? 1 : 0;
+  c.from_attrs = (p.cfg_waves || p.cfg_split_k || p.cfg_tile == 256) ? 1 : 0;
 
-  // Too few tiles to fill the GPU (decode-style shapes such as 32 x 4096 x 4096, where the weights have to stream
-  // from HBM through all compute units, and deep products such as 1024 x 1024 x 8192): K is cut into slices, one
-  // workgroup per (tile, slice); partial sums go through the workspace and a small second kernel.  The slice count
-  // plays the part of the reference's KThreads (lib/gc/Analysis/MatmulConfigAnalysis.cpp:149-166): here the count
-  // that makes the sum of a workgroup's share of K and the traffic of the partial sums smallest; a caller's wish
-  // replaces the default.
-  if (ES == 2 && fast_but_m && (nblk * 2 <= gcmi_num_cus() || p.cfg_split_k > 1) && p.out_dt != DT_S32 && nbatch == 1) {
-    const int n_cu = gcmi_num_cus();
-    const int groups = (int)(p.K / KGROUP);
-    const int tiles = (int)nblk;
-    int splits = 1;
-    // Rows of A fill at most half a tile: the kernel that skips the empty 32-row blocks of its tile, any slice count.
-    // Taller: the 4-wave kernel, run as a strided batch over equal K slices with f32 results (one slice = one batch).
-    bool by_w4 = p.M > 128;
-    if (p.cfg_split_k > 0) {
+  // What runs.  bf16 problems that fill the GPU with 256 x 256 tiles take those; smaller ones are given to more
+  // workgroups, either by 128 x 128 tiles (two workgroups per compute unit: four times the workgroups), or by cutting
+  // K into slices (one workgroup per tile and slice; f32 partial sums through the workspace and a small second
+  // kernel; the slice count plays the part of the reference's KThreads, lib/gc/Analysis/MatmulConfigAnalysis.cpp:149-166),
+  // or both; the estimates above decide.  A short A (M <= 128: decode-style shapes such as 32 x 4096 x 4096, whose
+  // weights have to stream from HBM through all compute units) keeps the kernel that skips the empty 32-row blocks
+  // of its tile and takes slices of unequal length; taller problems are sliced evenly and run the tile kernels as a
+  // strided batch: batch = K slice, results f32 with c_bs = M * N.  A caller's MatmulConfig replaces the choice.
+  const bool batch_ok = nbatch == 1 || ((p.a_bs * ES) % 16 == 0 && (p.b_bs * ES) % 16 == 0 && (p.c_bs * out_es) % 16 == 0 &&
+                                        (!p.residual || (p.c_bs * res_es) % 16 == 0));
+  const bool t128_can = ES == 2 && aligned && p.N % (16 / ES) == 0 && p.out_dt != DT_S32 && batch_ok;
+  const bool slices_can = ES == 2 && fast_but_m && p.out_dt != DT_S32 && nbatch == 1; // the 256-wide kernels: whole column tiles
+  const int64_t nblk128 = ((p.M + 127) / 128) * ((p.N + 127) / 128);
+  const int n_cu = gcmi_num_cus();
+  const int groups = (int)(p.K / KGROUP);
+  int plan = PLAN_TILE256, splits = 1;
+  if (p.cfg_tile == 128) {
+    if (t128_can && nblk128 <= 0x7fffffff)
+      plan = PLAN_TILE128, c.from_attrs = 1;
+  } else if (p.cfg_tile == 256) {
+    if (slices_can && p.cfg_split_k > 1) {
       splits = p.cfg_split_k < groups ? p.cfg_split_k : groups;
-      by_w4 = by_w4 && groups % splits == 0;
-    } else {
-      // Microseconds, fitted to measurements: a workgroup's ring groups of K (128 elements each), the partial sums'
-      // way through memory (8 bytes each, about 1.7 us per slice and 2^20 outputs), and what a launch costs
-      // besides.  Slices never exceed one workgroup per compute unit.
-      const double mn = (double)p.M * (double)p.N / 1048576.0;
-      const int smax = n_cu / tiles < groups ? n_cu / tiles : groups;
-      double best = GCMI_SPLIT_T1_FIXED + 1.94 * groups;
-      if (by_w4) {
-        best *= GCMI_SPLIT_MARGIN;
-        for (int s = 2; s <= smax; s++)
-          if (groups % s == 0) {
-            const double t = GCMI_SPLIT_W4_FIXED + 1.94 * (groups / s) + 1.7 * s * mn;
-            if (t < best)
-              best = t, splits = s;
-          }
-      } else {
-        const double per_group = 1.35 + 0.65 * (double)((p.M + 31) / 32 - 1) / 3.0;
-        for (int s = 2; s <= smax; s++) {
-          const double t = 7.0 + per_group * ((groups + s - 1) / s) + 1.7 * s * mn;
+      plan = p.M > 128 && groups % splits == 0 ? PLAN_SLICES_TILE256 : PLAN_SLICES_SHORT_A;
+    }
+  } else if (ES == 2 && aligned && nblk * nbatch < n_cu) {
+    const double mn = (double)p.M * (double)p.N / 1048576.0;
+    const double w256 = (double)(nblk * nbatch) / n_cu, w128 = (double)(nblk128 * nbatch) / n_cu;
+    double best = GCMI_US_FIXED_256 + gcmi_us_per_group_256(w256) * groups; // one pass, less than one round
+    if (p.M > 128 && t128_can) {
+      const double t = GCMI_US_FIXED_128 + gcmi_us_per_group_128(w128) * groups * (double)((nblk128 * nbatch + 2 * n_cu - 1) / (2 * n_cu));
+      if (t < best)
+        best = t, plan = PLAN_TILE128;
+    }
+    best *= GCMI_ONE_PASS_MARGIN;
+    if (nbatch == 1 && p.M > 128) {
+      for (int s = 2; s <= groups; s++) {
+        if (groups % s != 0)
+          continue;
+        const double through_memory = GCMI_US_SECOND_PASS + GCMI_US_PER_SLICE_MOUT * s * mn;
+        if (slices_can && nblk * s <= n_cu) {
+          const double t = GCMI_US_FIXED_256 + gcmi_us_per_group_256(w256 * s) * (groups / s) + through_memory;
           if (t < best)
-            best = t, splits = s;
+            best = t, plan = PLAN_SLICES_TILE256, splits = s;
+        }
+        if (t128_can && nblk128 * s <= 2 * n_cu) {
+          const double t = GCMI_US_FIXED_128 + gcmi_us_per_group_128(w128 * s) * (groups / s) + through_memory;
+          if (t < best)
+            best = t, plan = PLAN_SLICES_TILE128, splits = s;
         }
       }
+    } else if (nbatch == 1 && slices_can && nblk * 2 <= n_cu) { // a short A: 1.35 (32 rows) to 2 us (128) per group
+      const double per_group = 1.35 + 0.65 * (double)((p.M + 31) / 32 - 1) / 3.0;
+      const int smax = n_cu / (int)nblk < groups ? n_cu / (int)nblk : groups;
+      for (int s = 2; s <= smax; s++) {
+        const double t = 7.0 + per_group * ((groups + s - 1) / s) + GCMI_US_PER_SLICE_MOUT * s * mn;
+        if (t < best)
+          best = t, plan = PLAN_SLICES_SHORT_A, splits = s;
+      }
     }
-    splits = splits < groups ? splits : groups;
-    if (want) {
-      if (splits > 1)
-        *want = (int64_t)splits * p.M * p.N;
-      if (!cfg)
-        return 0;
-    }
-    while (splits > 1 && ((int64_t)splits * p.M * p.N > ws_cap || (by_w4 && groups % splits != 0)))
+  }
+  if (splits > 1) {
+    if (want)
+      *want = (int64_t)splits * p.M * p.N;
+    // less workspace than that: fewer slices, or none
+    while (splits > 1 && ((int64_t)splits * p.M * p.N > ws_cap || (plan != PLAN_SLICES_SHORT_A && groups % splits != 0)))
       splits--;
-    if (splits > 1) {
-      c.kernel = GK_SPLITK, c.split_k = splits, c.workgroups = tiles * splits;
-      if (by_w4) {
-        c.kbytes = 64, c.stages = 4, c.waves_m = 2, c.waves_n = 2, c.wave_m = 128, c.wave_n = 128;
-        c.mfma_m = c.mfma_n = 16, c.mfma_k = 64 / ES;
-      } else {
-        c.kbytes = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::KB, c.stages = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::NST;
-        c.waves_m = 2, c.waves_n = 8 / G_FAST_WJ, c.wave_m = 128, c.wave_n = 32 * G_FAST_WJ;
-        c.mfma_m = c.mfma_n = 32, c.mfma_k = 32 / ES;
-      }
-      if (cfg)
-        *cfg = c;
-      if (dry)
-        return 0;
-      p.splits = splits;
-      p.partial = ws;
-      if constexpr (ES == 2) {
-        if (by_w4) {
-          GemmParams q = p;
-          q.K = p.K / splits, q.batch = splits;
-          q.a_bs = q.K, q.b_bs = p.trans_b ? q.K : q.K * p.ldb, q.c_bs = p.M * p.N;
-          q.C = ws, q.ldc = p.N, q.out_dt = DT_F32;
-          q.bias = nullptr, q.act = ACT_NONE, q.residual = nullptr, q.partial = nullptr, q.splits = 0;
-          const dim3 grid((unsigned)tiles, (unsigned)splits);
-          if (p.trans_b)
-            hipLaunchKernelGGL((gemm_tile256_w4_kernel<ES, true>), grid, dim3(256), 0, stream, q);
-          else
-            hipLaunchKernelGGL(gemm_tile256_w4_kernel<ES>, grid, dim3(256), 0, stream, q);
-        } else if (p.trans_b)
-          hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true, true>),
-                             dim3((unsigned)(tiles * splits)), dim3(1024 / G_FAST_WJ), 0, stream, p);
-        else
-          hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true>), dim3((unsigned)(tiles * splits)),
-                             dim3(1024 / G_FAST_WJ), 0, stream, p);
-      }
-      launch_splitk_reduce(p, stream);
-      return hipGetLastError() == hipSuccess ? 0 : 5;
+    if (splits == 1)
+      plan = plan == PLAN_SLICES_TILE128 ? PLAN_TILE128 : PLAN_TILE256;
+  }
+  if (want && !cfg)
+    return 0;
+  if (splits > 1) {
+    const bool by128 = plan == PLAN_SLICES_TILE128, by256 = plan == PLAN_SLICES_TILE256;
+    const int tiles = (int)(by128 ? nblk128 : nblk);
+    c.kernel = GK_SPLITK, c.split_k = splits, c.workgroups = tiles * splits;
+    if (by128) {
+      c.bm = c.bn = 128, c.kbytes = T128_KB, c.stages = T128_NST;
+      c.waves_m = c.waves_n = 2, c.wave_m = c.wave_n = 64, c.mfma_m = c.mfma_n = 16, c.mfma_k = 32;
+    } else if (by256) {
+      c.kbytes = 64, c.stages = 4, c.waves_m = 2, c.waves_n = 2, c.wave_m = 128, c.wave_n = 128;
+      c.mfma_m = c.mfma_n = 16, c.mfma_k = 64 / ES;
+    } else {
+      c.kbytes = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::KB, c.stages = FastGemm<ES, G_FAST_KS, G_FAST_WJ, true>::NST;
+      c.waves_m = 2, c.waves_n = 8 / G_FAST_WJ, c.wave_m = 128, c.wave_n = 32 * G_FAST_WJ;
+      c.mfma_m = c.mfma_n = 32, c.mfma_k = 32 / ES;
     }
+    if (cfg)
+      *cfg = c;
+    if (dry)
+      return 0;
+    p.splits = splits;
+    p.partial = ws;
+    if constexpr (ES == 2) {
+      if (by128 || by256) {
+        GemmParams q = p;
+        q.K = p.K / splits, q.batch = splits;
+        q.a_bs = q.K, q.b_bs = p.trans_b ? q.K : q.K * p.ldb, q.c_bs = p.M * p.N;
+        q.C = ws, q.ldc = p.N, q.out_dt = DT_F32;
+        q.bias = nullptr, q.act = ACT_NONE, q.residual = nullptr, q.partial = nullptr, q.splits = 0;
+        const dim3 grid((unsigned)tiles, (unsigned)splits);
+        if (by128 && p.trans_b)
+          hipLaunchKernelGGL(gemm_tile128_kernel<true>, grid, dim3(256), 0, stream, q);
+        else if (by128)
+          hipLaunchKernelGGL(gemm_tile128_kernel<false>, grid, dim3(256), 0, stream, q);
+        else if (p.trans_b)
+          hipLaunchKernelGGL((gemm_tile256_w4_kernel<ES, true>), grid, dim3(256), 0, stream, q);
+        else
+          hipLaunchKernelGGL(gemm_tile256_w4_kernel<ES>, grid, dim3(256), 0, stream, q);
+      } else if (p.trans_b)
+        hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true, true>),
+                           dim3((unsigned)(tiles * splits)), dim3(1024 / G_FAST_WJ), 0, stream, p);
+      else
+        hipLaunchKernelGGL((gemm_tile256_fast_kernel<ES, G_FAST_KS, G_FAST_WJ, true>), dim3((unsigned)(tiles * splits)),
+                           dim3(1024 / G_FAST_WJ), 0, stream, p);
+    }
+    launch_splitk_reduce(p, stream);
+    return hipGetLastError() == hipSuccess ? 0 : 5;
+  }
+  if (plan == PLAN_TILE128) {
+    c.kernel = GK_TILE128, c.bm = c.bn = 128, c.kbytes = T128_KB, c.stages = T128_NST;
+    c.waves_m = c.waves_n = 2, c.wave_m = c.wave_n = 64, c.mfma_m = c.mfma_n = 16, c.mfma_k = 32;
+    c.workgroups = (int32_t)nblk128;
+    if (cfg)
+      *cfg = c;
+    if (dry)
+      return 0;
+    if constexpr (ES == 2) {
+      const dim3 grid((unsigned)nblk128, (unsigned)nbatch);
+      if (p.trans_b)
+        hipLaunchKernelGGL(gemm_tile128_kernel<true>, grid, dim3(256), 0, stream, p);
+      else
+        hipLaunchKernelGGL(gemm_tile128_kernel<false>, grid, dim3(256), 0, stream, p);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : 5;
   }
   // Whole tiles: 4 waves of 128 x 128 unless the caller asks for 8 waves of 128 x 64 (or the result is an f32 / s32
   // tensor of 8-bit operands, which only the 8-wave kernel writes).  Tiles that stick out of C (`ragged`): the 4-wave

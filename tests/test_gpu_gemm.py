@@ -256,13 +256,18 @@ def test_gelu_erf_epilogue_absolute_accuracy(gc, dev):
 
 @pytest.mark.parametrize("M,N", [(300, 264), (520, 256), (512, 520), (1000, 1000)])
 @pytest.mark.parametrize("variant", ["plain", "bias_gelu_f32", "bias_relu_residual", "nt"])
-def test_bf16_edge_tiles_of_the_four_wave_kernel(gc, orc, wl, dev, M, N, variant):
-    """M any, N a multiple of 8, K a multiple of 128: the whole-tile kernel takes the shape, its tiles on the lower
-    and right edges clamp their loads and store what lies inside C.  Every element equals, bit for bit, the element
-    of the same GEMM padded to whole tiles (same kernel, same sums), and the result matches the oracle."""
+@pytest.mark.parametrize("tile", [256, 128])
+def test_bf16_edge_tiles_of_the_four_wave_kernels(gc, orc, wl, dev, M, N, variant, tile):
+    """M any, N a multiple of 8, K a multiple of 128: the 4-wave kernels (256 x 256 and 128 x 128 tiles, each asked for
+    by its MatmulConfig) take the shape; tiles on the lower and right edges clamp their loads and store what lies
+    inside C.  Every element equals, bit for bit, the element of the same GEMM padded to whole tiles (same kernel,
+    same sums), and the result matches the oracle."""
     K = 384
-    c, _ = gc.tile_config(M, N, K, trans_b=(variant == "nt"), out_dtype=gc.F32 if variant == "bias_gelu_f32" else gc.BF16)
-    assert c.kernel == 2 and c.workgroups == -(-M // 256) * -(-N // 256)
+    how = 1 if tile == 256 else "tile128"
+    cfg = [1, 1, 1, 256, 256, 64, 128, 128, 32] if tile == 256 else [1, 1, 1, 128, 128, 64, 64, 64, 32]
+    c, _ = gc.tile_config(M, N, K, trans_b=(variant == "nt"), out_dtype=gc.F32 if variant == "bias_gelu_f32" else gc.BF16,
+                          matmul_config=cfg)
+    assert c.kernel == (2 if tile == 256 else 5) and c.workgroups == -(-M // tile) * -(-N // tile) and c.from_attrs == 1
     Mp, Np = -(-M // 256) * 256, -(-N // 256) * 256
     torch.manual_seed(0)
     Ap = (torch.randn(Mp, K) * 0.5).to(torch.bfloat16)
@@ -274,24 +279,24 @@ def test_bf16_edge_tiles_of_the_four_wave_kernel(gc, orc, wl, dev, M, N, variant
     resp = torch.randn(Mp, Np).to(torch.bfloat16)
     A, B, bias, res = Ap[:M].contiguous(), Bp[:, :N].contiguous(), biasp[:N].contiguous(), resp[:M, :N].contiguous()
     d = lambda t: t.to(dev)
-    guard = torch.full((M + 2, N), 7.0, dtype=torch.float32 if variant == "bias_gelu_f32" else torch.bfloat16, device=dev)
+    odt = torch.float32 if variant == "bias_gelu_f32" else torch.bfloat16
+    guard = torch.full((M + 2, N), 7.0, dtype=odt, device=dev)
     out = guard[1:M + 1]
+    full = torch.empty((Mp, Np), dtype=odt, device=dev)
+    ref = None
     if variant == "plain":
-        gc.gemm_bf16(d(A), d(B), out=out)
-        full = gc.gemm_bf16(d(Ap), d(Bp))
+        _gemm_ws(gc, d(A), d(B), False, out, how)
+        _gemm_ws(gc, d(Ap), d(Bp), False, full, how)
         ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B)))
     elif variant == "bias_gelu_f32":
-        gc.gemm_bf16(d(A), d(B), d(bias), "gelu_erf", out_dtype=gc.F32, out=out)
-        full = gc.gemm_bf16(d(Ap), d(Bp), d(biasp), "gelu_erf", out_dtype=gc.F32)
-        ref = None
+        _gemm_ws(gc, d(A), d(B), False, out, how, bias=d(bias), act="gelu_erf")
+        _gemm_ws(gc, d(Ap), d(Bp), False, full, how, bias=d(biasp), act="gelu_erf")
     elif variant == "bias_relu_residual":
-        gc.gemm_bf16_residual(d(A), d(B), d(res), bias=d(bias), act="relu", out=out)
-        full = gc.gemm_bf16_residual(d(Ap), d(Bp), d(resp), bias=d(biasp), act="relu")
-        ref = None
+        _gemm_ws(gc, d(A), d(B), False, out, how, bias=d(bias), act="relu", residual=d(res))
+        _gemm_ws(gc, d(Ap), d(Bp), False, full, how, bias=d(biasp), act="relu", residual=d(resp))
     else:
-        Bt, Btp = B.t().contiguous(), Bp.t().contiguous()
-        gc.gemm_bf16_nt(d(A), d(Bt), out=out)
-        full = gc.gemm_bf16_nt(d(Ap), d(Btp))
+        _gemm_ws(gc, d(A), d(B.t().contiguous()), True, out, how)
+        _gemm_ws(gc, d(Ap), d(Bp.t().contiguous()), True, full, how)
         ref = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(A), wl.bf16_bits(B)))
     torch.cuda.synchronize()
     assert (guard[0] == 7).all() and (guard[M + 1] == 7).all()  # nothing written outside C
@@ -367,14 +372,19 @@ def test_short_a_takes_split_k(gc, orc, wl, dev, M, N, K, act, with_bias, out_f3
     assert torch.equal(out, again)  # fixed summation order: reruns agree bit for bit
 
 
-def _gemm_ws(gc, A, B, trans_b, out, slices=None, bias=None, act=None, ws=None):
-    """gcmi_gemm_bf16_ws with a caller's workspace; slices: the KThreads of a full MatmulConfig attribute set."""
+def _gemm_ws(gc, A, B, trans_b, out, slices=None, bias=None, act=None, ws=None, residual=None):
+    """gcmi_gemm_bf16_ws with a caller's workspace; slices: the KThreads of a full MatmulConfig attribute set with the
+    256 x 256 tile, or "tile128": the set that names the 128 x 128 tile."""
     import ctypes as C
     M, K = A.shape
     N = B.shape[0] if trans_b else B.shape[1]
-    cfg = None if slices is None else (C.c_int64 * 9)(1, 1, slices, 256, 256, 64, 128, 128, 32)
+    if slices == "tile128":
+        cfg = (C.c_int64 * 9)(1, 1, 1, 128, 128, 64, 64, 64, 32)
+    else:
+        cfg = None if slices is None else (C.c_int64 * 9)(1, 1, slices, 256, 256, 64, 128, 128, 32)
     st = gc.lib().gcmi_gemm_bf16_ws(A.data_ptr(), B.data_ptr(), out.data_ptr(), 1, M, N, K, K, B.shape[1], N, 0, 0, 0, int(trans_b),
-                                    None if bias is None else bias.data_ptr(), gc.BF16, gc.ACT[act], None, 0, 0,
+                                    None if bias is None else bias.data_ptr(), gc.BF16, gc.ACT[act],
+                                    None if residual is None else residual.data_ptr(), N, gc.BF16,
                                     gc.F32 if out.dtype == torch.float32 else gc.BF16,
                                     None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel() * ws.element_size(), cfg,
                                     C.c_void_p(torch.cuda.current_stream().cuda_stream))
@@ -385,10 +395,12 @@ def _gemm_ws(gc, A, B, trans_b, out, slices=None, bias=None, act=None, ws=None):
                                                          (640, 768, 3072, None, True, True), (1024, 1024, 2048, None, False, False),
                                                          (257, 2048, 1024, "sigmoid", False, False)])
 def test_few_tiles_and_a_deep_k_take_k_slices(gc, orc, wl, dev, M, N, K, act, with_bias, out_f32):
-    """Several tile rows but too few tiles for the GPU: equal K slices run as a strided batch of the 4-wave kernel
-    into f32 partial sums, the second kernel adds them and applies the epilogue.  Same rounding points as one pass."""
+    """Several tile rows but too few 256 x 256 tiles for the GPU: 128 x 128 tiles, and where K is deep, equal K slices
+    run as a strided batch of a tile kernel into f32 partial sums; the second kernel adds them and applies the
+    epilogue.  Same rounding points as one pass."""
     c, _ = gc.tile_config(M, N, K, out_dtype=gc.F32 if out_f32 else gc.BF16)
-    assert c.kernel == 3 and c.split_k > 1 and K // 128 % c.split_k == 0 and c.workgroups <= 256, (c.kernel, c.split_k, c.workgroups)
+    assert c.kernel in (3, 5) and c.workgroups <= 512, (c.kernel, c.split_k, c.workgroups)
+    assert (c.kernel == 3) == (c.split_k > 1) and K // 128 % c.split_k == 0
     torch.manual_seed(M + N)
     A = (torch.randn(M, K) * 0.5).to(torch.bfloat16)
     torch.manual_seed(K)
@@ -418,7 +430,7 @@ def test_k_slices_exact_on_integers_for_any_slice_count(gc, dev, trans_b):
     """Small integers make every partial sum exact, so each slice count must give the bits of the f32 product: the
     default, even counts (the 4-wave kernel as a batch), counts that do not divide K's ring groups (the kernel with
     slices of unequal length, here on two and three tile rows, the last one short), one slice (no second pass), a
-    workspace too small for the count asked for (fewer slices), and none at all."""
+    workspace too small for the count asked for or chosen (fewer slices), none at all, and the 128 x 128 tile by name."""
     torch.manual_seed(11)
     for M, N, K in [(512, 512, 2048), (600, 768, 1536), (257, 1024, 1024)]:
         A = torch.randint(-3, 4, (M, K), device=dev).to(torch.bfloat16)
@@ -426,7 +438,8 @@ def test_k_slices_exact_on_integers_for_any_slice_count(gc, dev, trans_b):
         want = A.float() @ B.float()
         Bd = B.t().contiguous() if trans_b else B
         ws = torch.empty(16 * M * N, dtype=torch.float32, device=dev)
-        for slices, w in [(None, ws), (1, ws), (2, ws), (3, ws), (4, ws), (5, ws), (7, ws), (8, ws), (4, ws[:2 * M * N + 5]), (4, None)]:
+        for slices, w in [(None, ws), (1, ws), (2, ws), (3, ws), (4, ws), (5, ws), (7, ws), (8, ws), (4, ws[:2 * M * N + 5]), (4, None),
+                          ("tile128", ws), (None, ws[:2 * M * N]), (None, None)]:
             out = torch.full((M, N), 7.0, dtype=torch.float32, device=dev)
             _gemm_ws(gc, A, Bd, trans_b, out, slices, ws=w)
             torch.cuda.synchronize()
