@@ -179,6 +179,12 @@ static int launch_skinny_nt(const GemmParams *pp, hipStream_t stream, int64_t *w
   // the weights must be worth streaming this way: with few of them the tile kernel's launch is as good
   if (p.N * p.K < (int64_t)1 << 20)
     return -1;
+  // Left to its own choice the launcher keeps this kernel for what it wins: up to 32 rows against up to 24 Mi
+  // weights (32 x 4096 x 4096: 13.2 us against 14 us for K slices of 128 x 128 tiles).  With more rows or wider
+  // weights the tile kernels are ahead (64 x 11008 x 4096: 41 us here, 26 us there).  A caller's slice count
+  // (its KThreads) still selects it for any shape it can run.
+  if (p.cfg_split_k <= 0 && (p.M > 32 || p.N * p.K > (int64_t)3 << 23))
+    return -1;
   const int mt = p.M <= 32 ? 1 : 2;
   const int n_cu = gcmi_num_cus(), nblocks = (int)(p.N / 32), steps = (int)(p.K / 64);
   // workgroup slices: whole rounds of one workgroup per compute unit (measured: 32 x 4096 x 4096 takes 20 us with

@@ -1597,7 +1597,7 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gem
 // computes k-block s from registers while the fragments of block s+1 are read and block s+3 is requested; one
 // barrier per stage.  Rows past M and columns past N (N a multiple of 8) are fetched from the last row / chunk
 // inside and never stored.  The epilogue is the 4-wave kernel's: accumulators through a wave-private LDS region,
-// then rows of four columns per lane.
+// then rows of four columns per lane.  blockIdx.y: the batch, or with GemmParams::splits the K slice.
 static constexpr int T128_B = 128, T128_KB = 64, T128_NST = 4;
 static constexpr int T128_A_BYTES = T128_B * T128_KB, T128_STAGE_BYTES = 2 * T128_A_BYTES;
 static constexpr int T128_DUMP_WAVE_BYTES = 64 * W4_DUMP_PITCH; // 17408 per wave
@@ -1622,7 +1622,18 @@ template <bool TB = false> __global__ __launch_bounds__(256, 2) void gemm_tile12
   tm = __builtin_amdgcn_readfirstlane(tm), tn = __builtin_amdgcn_readfirstlane(tn);
   const int64_t m0 = (int64_t)tm * T128_B, n0 = (int64_t)tn * T128_B;
   const int64_t lda_b = p.lda * ES, ldb_b = p.ldb * ES;
-  {
+  const int64_t b_step = TB ? (int64_t)KB : (int64_t)BK * ldb_b;
+  int KT = (int)(p.K / BK); // k-blocks: a positive multiple of NST (checked by the launcher)
+  int64_t k_first = 0;      // first k-block of this workgroup
+  if (p.splits > 1) {
+    // K slices: blockIdx.y is the slice, whole ring groups each (they differ by at most one group); its f32 sums go
+    // to the workspace as they are, the second kernel adds the slices and runs the epilogue
+    const int slice = blockIdx.y, groups = KT / NST;
+    const int g0 = (int)((int64_t)slice * groups / p.splits), g1 = (int)((int64_t)(slice + 1) * groups / p.splits);
+    k_first = (int64_t)g0 * NST, KT = (g1 - g0) * NST;
+    p.C = p.partial + (int64_t)slice * p.M * p.N, p.ldc = p.N, p.out_dt = DT_F32;
+    p.bias = nullptr, p.act = ACT_NONE, p.residual = nullptr;
+  } else {
     const int64_t bz = blockIdx.y; // strided batch
     p.A = reinterpret_cast<const char *>(p.A) + bz * p.a_bs * ES;
     p.B = reinterpret_cast<const char *>(p.B) + bz * p.b_bs * ES;
@@ -1700,10 +1711,8 @@ template <bool TB = false> __global__ __launch_bounds__(256, 2) void gemm_tile12
                                                               __builtin_bit_cast(bf16x8_t, a[it]), acc[jt][it], 0, 0, 0);
   };
 
-  const int64_t b_step = TB ? (int64_t)KB : (int64_t)BK * ldb_b;
-  const int KT = (int)(p.K / BK); // a positive multiple of NST (checked by the launcher)
-  const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b;
-  const char *b_ptr = reinterpret_cast<const char *>(p.B) + (TB ? n0 * ldb_b : n0 * ES);
+  const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b + k_first * KB;
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + (TB ? n0 * ldb_b : n0 * ES) + k_first * b_step;
 
   float cp_bias = -0.0f; // an absent bias adds nothing, not even to -0.0
   if (tid < cols_in && p.bias)
@@ -1898,8 +1907,8 @@ static inline double gcmi_us_per_group_128(double load) { // up to two workgroup
     return 0.85;
   if (load <= 1.0)
     return 0.85 + 0.27 * (load - 0.25) / 0.75;
-  if (load <= 2.0)
-    return 1.12 + 1.05 * (load - 1.0);
+  if (load <= 2.0) // as soon as some compute units hold two workgroups, those set the pace
+    return 1.9 + 0.27 * (load - 1.0);
   return 2.17;
 }
 static constexpr double GCMI_US_FIXED_256 = 8.0, GCMI_US_FIXED_128 = 3.7; // launch, ring fill, epilogue
@@ -1963,8 +1972,10 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
   // kernel; the slice count plays the part of the reference's KThreads, lib/gc/Analysis/MatmulConfigAnalysis.cpp:149-166),
   // or both; the estimates above decide.  A short A (M <= 128: decode-style shapes such as 32 x 4096 x 4096, whose
   // weights have to stream from HBM through all compute units) keeps the kernel that skips the empty 32-row blocks
-  // of its tile and takes slices of unequal length; taller problems are sliced evenly and run the tile kernels as a
-  // strided batch: batch = K slice, results f32 with c_bs = M * N.  A caller's MatmulConfig replaces the choice.
+  // of its tile and takes slices of unequal length, unless the 128 x 128 tiles are estimated faster (from 32 rows
+  // on they are).  The 128 x 128 kernel cuts K itself (blockIdx.y = slice, whole ring groups, lengths differing by at
+  // most one); the 256 x 256 kernel runs equal slices as a strided batch: batch = K slice, results f32 with
+  // c_bs = M * N.  A caller's MatmulConfig replaces the choice.
   const bool batch_ok = nbatch == 1 || ((p.a_bs * ES) % 16 == 0 && (p.b_bs * ES) % 16 == 0 && (p.c_bs * out_es) % 16 == 0 &&
                                         (!p.residual || (p.c_bs * res_es) % 16 == 0));
   const bool t128_can = ES == 2 && aligned && p.N % (16 / ES) == 0 && p.out_dt != DT_S32 && batch_ok;
@@ -1985,29 +1996,29 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
     const double mn = (double)p.M * (double)p.N / 1048576.0;
     const double w256 = (double)(nblk * nbatch) / n_cu, w128 = (double)(nblk128 * nbatch) / n_cu;
     double best = GCMI_US_FIXED_256 + gcmi_us_per_group_256(w256) * groups; // one pass, less than one round
-    if (p.M > 128 && t128_can) {
+    const bool small_tile = p.M >= 32 && t128_can; // shorter: most of a 128-row tile would be padding
+    if (small_tile) {
       const double t = GCMI_US_FIXED_128 + gcmi_us_per_group_128(w128) * groups * (double)((nblk128 * nbatch + 2 * n_cu - 1) / (2 * n_cu));
       if (t < best)
         best = t, plan = PLAN_TILE128;
     }
     best *= GCMI_ONE_PASS_MARGIN;
-    if (nbatch == 1 && p.M > 128) {
+    if (nbatch == 1 && (small_tile || p.M > 128)) {
       for (int s = 2; s <= groups; s++) {
-        if (groups % s != 0)
-          continue;
         const double through_memory = GCMI_US_SECOND_PASS + GCMI_US_PER_SLICE_MOUT * s * mn;
-        if (slices_can && nblk * s <= n_cu) {
+        if (slices_can && p.M > 128 && groups % s == 0 && nblk * s <= n_cu) {
           const double t = GCMI_US_FIXED_256 + gcmi_us_per_group_256(w256 * s) * (groups / s) + through_memory;
           if (t < best)
             best = t, plan = PLAN_SLICES_TILE256, splits = s;
         }
-        if (t128_can && nblk128 * s <= 2 * n_cu) {
-          const double t = GCMI_US_FIXED_128 + gcmi_us_per_group_128(w128 * s) * (groups / s) + through_memory;
+        if (small_tile && nblk128 * s <= 2 * n_cu) {
+          const double t = GCMI_US_FIXED_128 + gcmi_us_per_group_128(w128 * s) * ((groups + s - 1) / s) + through_memory;
           if (t < best)
             best = t, plan = PLAN_SLICES_TILE128, splits = s;
         }
       }
-    } else if (nbatch == 1 && slices_can && nblk * 2 <= n_cu) { // a short A: 1.35 (32 rows) to 2 us (128) per group
+    }
+    if (nbatch == 1 && p.M <= 128 && slices_can && nblk * 2 <= n_cu) { // a short A: 1.35 (32 rows) to 2 us (128) per group
       const double per_group = 1.35 + 0.65 * (double)((p.M + 31) / 32 - 1) / 3.0;
       const int smax = n_cu / (int)nblk < groups ? n_cu / (int)nblk : groups;
       for (int s = 2; s <= smax; s++) {
@@ -2021,7 +2032,7 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
     if (want)
       *want = (int64_t)splits * p.M * p.N;
     // less workspace than that: fewer slices, or none
-    while (splits > 1 && ((int64_t)splits * p.M * p.N > ws_cap || (plan != PLAN_SLICES_SHORT_A && groups % splits != 0)))
+    while (splits > 1 && ((int64_t)splits * p.M * p.N > ws_cap || (plan == PLAN_SLICES_TILE256 && groups % splits != 0)))
       splits--;
     if (splits == 1)
       plan = plan == PLAN_SLICES_TILE128 ? PLAN_TILE128 : PLAN_TILE256;
@@ -2050,18 +2061,20 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
     p.splits = splits;
     p.partial = ws;
     if constexpr (ES == 2) {
-      if (by128 || by256) {
+      if (by128) { // the kernel cuts K itself: blockIdx.y = slice
+        const dim3 grid((unsigned)tiles, (unsigned)splits);
+        if (p.trans_b)
+          hipLaunchKernelGGL(gemm_tile128_kernel<true>, grid, dim3(256), 0, stream, p);
+        else
+          hipLaunchKernelGGL(gemm_tile128_kernel<false>, grid, dim3(256), 0, stream, p);
+      } else if (by256) { // equal slices as a strided batch with f32 results
         GemmParams q = p;
         q.K = p.K / splits, q.batch = splits;
         q.a_bs = q.K, q.b_bs = p.trans_b ? q.K : q.K * p.ldb, q.c_bs = p.M * p.N;
         q.C = ws, q.ldc = p.N, q.out_dt = DT_F32;
         q.bias = nullptr, q.act = ACT_NONE, q.residual = nullptr, q.partial = nullptr, q.splits = 0;
         const dim3 grid((unsigned)tiles, (unsigned)splits);
-        if (by128 && p.trans_b)
-          hipLaunchKernelGGL(gemm_tile128_kernel<true>, grid, dim3(256), 0, stream, q);
-        else if (by128)
-          hipLaunchKernelGGL(gemm_tile128_kernel<false>, grid, dim3(256), 0, stream, q);
-        else if (p.trans_b)
+        if (p.trans_b)
           hipLaunchKernelGGL((gemm_tile256_w4_kernel<ES, true>), grid, dim3(256), 0, stream, q);
         else
           hipLaunchKernelGGL(gemm_tile256_w4_kernel<ES>, grid, dim3(256), 0, stream, q);

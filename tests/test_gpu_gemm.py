@@ -458,7 +458,7 @@ NT_SHAPES = [(256, 256, 128), (512, 768, 256), (300, 200, 100), (257, 511, 129),
 
 def _streams_weights(M, N, K):
     """Shapes the [N,K] entry point gives to the weight-streaming kernel (short A, enough weights)."""
-    return M <= 64 and N % 32 == 0 and K % 64 == 0 and K >= 256 and N * K >= 1 << 20
+    return M <= 32 and N % 32 == 0 and K % 64 == 0 and K >= 256 and 1 << 20 <= N * K <= 3 << 23
 
 
 @pytest.mark.parametrize("M,N,K", NT_SHAPES)
@@ -502,6 +502,16 @@ def test_bf16_gemm_streaming_kernel_exact_on_integers(gc, dev):
         out = gc.gemm_bf16_nt(A, Bt, out_dtype=gc.F32)
         torch.cuda.synchronize()
         assert torch.equal(out, A.float() @ Bt.float().t())
+        # left to itself the launcher keeps the streaming kernel for up to 32 rows; a slice count by name (KThreads)
+        # selects it for every shape it can run, the 64-row instantiation included
+        c, _ = gc.tile_config(M, N, K, trans_b=True, out_dtype=gc.F32, matmul_config=[1, 1, 16, 256, 256, 64, 128, 128, 32])
+        if K >= 1024:  # 16 slices need 16 K blocks of 64 (the reference's validity rule), else the set is ignored
+            assert c.kernel == 4, (M, N, K, c.kernel)
+        ws = torch.empty(16 * M * N, dtype=torch.float32, device=dev)
+        out2 = torch.full((M, N), 7.0, dtype=torch.float32, device=dev)
+        _gemm_ws(gc, A, Bt, True, out2, 16, ws=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(out2, out)
 
 
 def test_bf16_gemm_transposed_b_strided_rows(gc, dev):

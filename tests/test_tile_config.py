@@ -23,9 +23,24 @@ def test_defaults_per_shape(gc):
     c, _ = gc.tile_config(300, 200, 100)                                # ragged: bounds-checked tile
     assert c.kernel == 0
     c, _ = gc.tile_config(32, 4096, 4096)                               # one tile row: K slices fill the GPU
-    assert c.kernel == 3 and c.split_k == 16 and c.workgroups == 16 * 16
+    assert c.kernel == 3 and (c.bm, c.bn) == (128, 128) and c.split_k == 8 and c.workgroups == 32 * 8
+    c, _ = gc.tile_config(16, 4096, 4096)                               # fewer rows: the kernel that skips empty row blocks
+    assert c.kernel == 3 and (c.bm, c.bn) == (256, 256) and c.split_k == 16 and c.workgroups == 16 * 16
+    c, _ = gc.tile_config(2048, 2048, 2048)                             # 64 large tiles: small tiles instead
+    assert (c.kernel, c.bm, c.wave_m, c.wave_n, c.split_k, c.workgroups) == (5, 128, 64, 64, 1, 256)
+    c, _ = gc.tile_config(1024, 1024, 8192)                             # and a deep K: slices of small tiles
+    assert (c.kernel, c.bm, c.split_k, c.workgroups) == (3, 128, 4, 256)
     c, _ = gc.tile_config(32, 4096, 4096, trans_b=True)                 # [N,K] weights, short A: streamed
     assert c.kernel == 4 and c.split_k >= 4
+
+
+def test_attributes_name_the_small_tile(gc):
+    c, note = gc.tile_config(4096, 4096, 4096, matmul_config=_cfg(MBlock=128, NBlock=128, iM=64, iN=64))
+    assert (c.kernel, c.bm, c.bn, c.workgroups, c.from_attrs, note) == (5, 128, 128, 1024, 1, "")
+    c, note = gc.tile_config(4096, 4096, 4096, matmul_config=_cfg(MBlock=128, NBlock=128, iM=64, iN=64, KThreads=2))
+    assert c.from_attrs == 0 and c.kernel == 2 and "no K slices" in note
+    c, note = gc.tile_config(2048, 2048, 2048, matmul_config=_cfg())   # the large tile by name: no small tiles, no slices
+    assert (c.kernel, c.bm, c.split_k, c.from_attrs) == (2, 256, 1, 1)
 
 
 def test_all_nine_attributes_steer_waves_and_k_slices(gc):
