@@ -108,11 +108,11 @@ def time_launches(torch, fn, nsets, steps, warmup):
 # --copy-calibration: a 1 GiB copy reads FETCH_SIZE = 524304 KiB (scale 2.0)
 # and WRITE_SIZE = 1048580 KiB (scale 1.0).
 TRAFFIC = {  # (bytes per launch of the dominant kernel, the committed profile they come from)
-    "gemm": (235375279, "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
-    "int8": (384724261, "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
-    "chain": (684052143 + 575105079, "profiles/gemm_tile256_w4_bf16_mlp_chain.md"),  # both launches
-    "mha": (369234364, "profiles/mha_fwd_fast_b4_h32_s2048_d128_every_block.md"),
-    "mha_skip": (306034939, "profiles/mha_fwd_fast_b4_h32_s2048_d128.md"),
+    "gemm": (235417028, "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
+    "int8": (384764352, "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
+    "chain": (681050751 + 575140903, "profiles/gemm_tile256_w4_bf16_mlp_chain.md"),  # both launches
+    "mha": (362734179, "profiles/mha_fwd_fast_b4_h32_s2048_d128_every_block.md"),
+    "mha_skip": (330983112, "profiles/mha_fwd_fast_b4_h32_s2048_d128.md"),
 }
 
 
@@ -390,9 +390,11 @@ def main():
             dec["%dx%dx%d" % (Md, Nd, Kdd)] = entry
             del sets
             torch.cuda.empty_cache()
-        others["bf16_decode_gemm"] = {"workload": "A[32 x K] . W bf16 with W stored [K,N] (tile kernel over K slices) and [N,K] "
-                                                  "(weight-streaming kernel); two launches each (partial sums, then reduction + "
-                                                  "epilogue); algorithmic bytes = A + W + C once", "shapes": dec}
+        others["bf16_decode_gemm"] = {"workload": "A[32 x K] . W bf16 with W stored [K,N] and [N,K]: K slices over 128 x 128 tiles, "
+                                                  "over the 256-wide tile kernel that skips empty row blocks, or the weight-streaming "
+                                                  "kernel ([N,K], up to 24 Mi weights), as the launcher estimates; two launches each "
+                                                  "(partial sums, then reduction + epilogue); algorithmic bytes = A + W + C once",
+                                      "shapes": dec}
 
     # ---------------- the same kernels on shapes off their tile sizes (parity cases elsewhere; here: no cliff)
     if want("ragged"):

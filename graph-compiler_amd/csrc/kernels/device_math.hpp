@@ -23,32 +23,26 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) {
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
-// erf(x) as an odd rational P(x^2)*x / Q(x^2), fitted on |x| <= 3.95; absolute error below 5e-7.  The reference
-// evaluates erf with approximations of the same class (a table of degree-5 polynomials, or Abramowitz-Stegun 7.1.26
-// with absolute error 1.5e-7: legacy/core/src/compiler/ir/transform/cpu/target_specific_lower.cpp:1012-1130), so
-// nothing finer than that is pinned by it.
-// The argument is clamped to +-4.125 and the quotient to +-1.  Beyond the fitted range the quotient keeps rising:
-// between 3.95 and 4.05 it is within two units in the last place of 1 (erf itself is within 2.3e-8 of 1 there), and
-// from 4.05 on it is 1 or more for every float (all of [4.05, 4.3) checked on the GPU), so |x| >= 4.125 gives
-// exactly +-1 with no comparison: 19 vector instructions per element, no branch, and the four elements of a row
-// interleave.  (A conditional `|x| >= bound ? +-1 : quotient` makes the compiler branch around the polynomials per
-// element: six scalar instructions each, and the chains serialise.)
+// erf for the GELU below, where it is added to 1: for x >= 0, erf(x) = 1 - 2^(-x q(x)) with q a polynomial of degree 6
+// fitted to -log2(erfc(x)) / x on [0, 4.2] (weighted for the error of erf itself), odd in x; absolute error below
+// 2e-7 (relative accuracy near 0 is not kept).  The reference evaluates erf with approximations of the same class (a
+// table of degree-5 polynomials, or Abramowitz-Stegun 7.1.26 with absolute error 1.5e-7:
+// legacy/core/src/compiler/ir/transform/cpu/target_specific_lower.cpp:1012-1130), so nothing finer than that is
+// pinned by it.  |x| is clamped to 4.2, where 2^(-x q) < 2^-28 and the difference is exactly 1, so large arguments,
+// infinities included, give +-1 with no comparison; 14 issue slots per element (the exponential counts four), no
+// branch, and the four elements of a row interleave.  (An odd rational P(x^2) x / Q(x^2) of the same accuracy took 19;
+// a conditional `|x| >= bound ? +-1 : ...` makes the compiler branch around the polynomial per element: six scalar
+// instructions each, and the chains serialise.)
 __device__ __forceinline__ float erf_rational(float x) {
-  const float xc = __builtin_amdgcn_fmed3f(x, -4.125f, 4.125f);
-  const float x2 = xc * xc;
-  float p = -2.72614225801306e-10f;
-  p = fmaf(p, x2, 2.77068142495902e-08f);
-  p = fmaf(p, x2, -2.10102402082508e-06f);
-  p = fmaf(p, x2, -5.69250639462346e-05f);
-  p = fmaf(p, x2, -7.34990630326855e-04f);
-  p = fmaf(p, x2, -2.95459980854025e-03f);
-  p = fmaf(p, x2, -1.60960333262415e-02f);
-  float q = -1.45660718464996e-05f;
-  q = fmaf(q, x2, -2.13374055278905e-04f);
-  q = fmaf(q, x2, -1.68282697438203e-03f);
-  q = fmaf(q, x2, -7.37332916720468e-03f);
-  q = fmaf(q, x2, -1.42647390514189e-02f);
-  return __builtin_amdgcn_fmed3f((p * xc) * __builtin_amdgcn_rcpf(q), -1.0f, 1.0f);
+  const float a = fminf(fabsf(x), 4.2f);
+  float q = -1.0021075286203995e-04f;
+  q = fmaf(q, a, 4.615070065483451e-04f);
+  q = fmaf(q, a, 2.3023963440209627e-03f);
+  q = fmaf(q, a, -2.9452694579958916e-02f);
+  q = fmaf(q, a, 1.4896376430988312e-01f);
+  q = fmaf(q, a, 9.183286428451538e-01f);
+  q = fmaf(q, a, 1.6279137134552002f);
+  return copysignf(1.0f - __builtin_amdgcn_exp2f(-(q * a)), x);
 }
 
 // tanh for the GELU below, where it is added to 1: 1 - 2 / (e^(2|t|) + 1) with the sign of t, absolute error about
