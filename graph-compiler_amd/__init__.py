@@ -221,8 +221,8 @@ def colsum_s8(W):
     return out
 
 
-def gemm_int8(A, W, colsum=None, zp_a=0, scale=None, bias=None, act=None, out_dtype=S32, out=None):
-    """A [M,K] uint8 or int8, W [K,N] int8 cuda tensors."""
+def gemm_int8(A, W, colsum=None, zp_a=0, scale=None, bias=None, act=None, out_dtype=S32, out=None, matmul_config=None):
+    """A [M,K] uint8 or int8, W [K,N] int8 cuda tensors.  matmul_config: the nine MatmulConfig integers, or None."""
     import torch
     M, K = A.shape
     K2, N = W.shape
@@ -231,6 +231,12 @@ def gemm_int8(A, W, colsum=None, zp_a=0, scale=None, bias=None, act=None, out_dt
     odt = {S32: torch.int32, F32: torch.float32, BF16: torch.bfloat16}[out_dtype]
     if out is None:
         out = torch.empty((M, N), device=A.device, dtype=odt)
+    if matmul_config is not None:
+        arr = (C.c_int64 * 9)(*matmul_config)
+        check(lib().gcmi_gemm_int8_cfg(_ptr(A), adt, _ptr(W), _ptr(out), M, N, K, A.stride(0) if M > 1 else K,
+                                       W.stride(0) if K > 1 else N, out.stride(0) if M > 1 else N, _ptr(colsum), int(zp_a),
+                                       _ptr(scale), _ptr(bias), ACT[act], out_dtype, arr, _stream()), "gcmi_gemm_int8_cfg")
+        return out
     check(lib().gcmi_gemm_int8(_ptr(A), adt, _ptr(W), _ptr(out), M, N, K, A.stride(0) if M > 1 else K,
                                W.stride(0) if K > 1 else N, out.stride(0) if M > 1 else N, _ptr(colsum), int(zp_a),
                                _ptr(scale), _ptr(bias), ACT[act], out_dtype, _stream()), "gcmi_gemm_int8")
