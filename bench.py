@@ -436,9 +436,23 @@ def main():
                                               "value": round(2.0 * Mf * Nf * Kf / t["ms_per_step"] / 1e9, 1), "unit": "TFLOP/s",
                                               "tile": int(cfgf.bm), "k_slices": int(cfgf.split_k), "workgroups": int(cfgf.workgroups)}
             del Af, Bf, Cf
+        # the int8 layer at a quarter of its rows: 172 tiles of 256 x 256, or 688 of 128 x 128
+        Mi, Ni, Ki = 1024, 4096, 4096
+        Ai = torch.randint(0, 256, (Mi, Ki), dtype=torch.uint8, device=dev)
+        Wi = torch.randint(-127, 128, (Ki, Ni), dtype=torch.int8, device=dev)
+        csi = gc.colsum_s8(Wi)
+        sci, bii = (torch.rand(Ni, device=dev) * 0.009 + 0.001).float(), torch.randn(Ni, device=dev).float()
+        Oi = torch.empty(Mi, Ni, dtype=torch.bfloat16, device=dev)
+        t = time_launches(torch, lambda i: gc.gemm_int8(Ai, Wi, csi, 128, sci, bii, "gelu_erf", gc.BF16, out=Oi), 1, max(20, K // 2), W)
+        cfgf, _ = gc.tile_config(Mi, Ni, Ki, a_dtype=gc.U8)
+        few["int8_%dx%dx%d_dequant_bias_gelu" % (Mi, Ni, Ki)] = {
+            "ms_per_step": round(t["ms_per_step"], 5), "value": round(2.0 * Mi * Ni * Ki / t["ms_per_step"] / 1e9, 1), "unit": "TOP/s",
+            "tile": int(cfgf.bm), "k_slices": int(cfgf.split_k), "workgroups": int(cfgf.workgroups)}
+        del Ai, Wi, Oi
         others["bf16_gemm_few_tiles"] = {
             "workload": "bf16 GEMMs of 16 to 128 tiles of 256 x 256 (one compute unit works 1.9 us per tile and 128 of K): the "
-                        "launcher gives them to more workgroups by 128 x 128 tiles, equal K slices, or both", "cases": few}
+                        "launcher gives them to more workgroups by 128 x 128 tiles, K slices, or both; and one 8-bit layer "
+                        "of 64 such tiles (128 x 128 tiles)", "cases": few}
         log("few tiles: %s" % json.dumps(few))
         torch.cuda.empty_cache()
 

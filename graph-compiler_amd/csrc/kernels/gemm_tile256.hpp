@@ -1601,14 +1601,19 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gem
 static constexpr int T128_B = 128, T128_KB = 64, T128_NST = 4;
 static constexpr int T128_A_BYTES = T128_B * T128_KB, T128_STAGE_BYTES = 2 * T128_A_BYTES;
 static constexpr int T128_DUMP_WAVE_BYTES = 64 * W4_DUMP_PITCH; // 17408 per wave
-static constexpr int T128_SMEM_BYTES = 4 * T128_DUMP_WAVE_BYTES + T128_B * 4;
+static constexpr int T128_SMEM_BYTES = 4 * T128_DUMP_WAVE_BYTES + 3 * 256 * 4; // accumulator regions / ring, column parameters
 static_assert(T128_NST * T128_STAGE_BYTES <= 4 * T128_DUMP_WAVE_BYTES, "the ring overlaps the column parameters");
 
-template <bool TB = false> __global__ __launch_bounds__(256, 2) void gemm_tile128_kernel(GemmParams p) {
-  constexpr int ES = 2, KB = T128_KB, BK = KB / ES, NST = T128_NST, A_BYTES = T128_A_BYTES, STAGE = T128_STAGE_BYTES;
-  constexpr int RG = 4, CW = 4, B_ROW_BYTES = T128_B * ES, B_CPR = B_ROW_BYTES / 16;
+template <bool TB = false, int ES = 2> __global__ __launch_bounds__(256, 2) void gemm_tile128_kernel(GemmParams p) {
+  static_assert(!TB || ES == 2, "B stored [N,K]: bf16 only");
+  constexpr int KB = T128_KB, BK = KB / ES, NST = T128_NST, A_BYTES = T128_A_BYTES, STAGE = T128_STAGE_BYTES;
+  // a k-row of the B tile: 256 bytes of bf16 (4 k-rows per transposing read, chunk ^ 4 * (k % 4)) or 128 bytes of
+  // int8 (8 k-rows per read, chunk ^ 2 * (k % 8 / 2): the read of 8 k-rows x 16 columns touches every bank once)
+  constexpr int RG = ES == 2 ? 4 : 8, B_ROW_BYTES = T128_B * ES, B_CPR = B_ROW_BYTES / 16;
+  typedef typename std::conditional<ES == 2, f32x4_t, i32x4_t>::type acc4_t;
   __shared__ __align__(1024) char smem[T128_SMEM_BYTES];
-  float *colp = reinterpret_cast<float *>(smem + 4 * T128_DUMP_WAVE_BYTES);
+  float *colp = reinterpret_cast<float *>(smem + 4 * T128_DUMP_WAVE_BYTES); // [0..127] bias, [256..] scale, [512..] comp * colsum
+  auto b_swz = [](int krow) { return ES == 2 ? (krow % 4) * 4 : ((krow % 8) >> 1) * 2; };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1651,8 +1656,8 @@ template <bool TB = false> __global__ __launch_bounds__(256, 2) void gemm_tile12
     const int row = d * 16 + lane / 4;
     const int c = (lane % 4) ^ ((row >> 2) & 3);
     a_src[i] = (uint32_t)(min(row, rows_in - 1) * lda_b + c * 16);
-    const int krow = d * 4 + lane / B_CPR;
-    const int cb = min((lane % B_CPR) ^ ((krow % RG) * CW), cols_in * ES / 16 - 1);
+    const int krow = d * (1024 / B_ROW_BYTES) + lane / B_CPR;
+    const int cb = min((lane % B_CPR) ^ b_swz(krow), cols_in * ES / 16 - 1);
     b_src[i] = TB ? (uint32_t)(min(row, cols_in - 1) * ldb_b + c * 16) : (uint32_t)(krow * ldb_b + cb * 16);
   }
   auto issue = [&](char *__restrict__ stage, const char *a_base, const char *b_base) {
@@ -1670,11 +1675,14 @@ template <bool TB = false> __global__ __launch_bounds__(256, 2) void gemm_tile12
   const uint32_t a_ld = (uint32_t)(row_a * KB + ((g16 ^ ((row_a >> 2) & 3)) << 4));
   uint32_t b_ld[4];
   {
-    const int kk = r16 >> 2, cc = r16 & 3;
+    // the 16 lanes of a group hand the transposing read RG k-rows x 16 columns in 8-byte pieces (bf16: k row
+    // lane%16/4, 4 columns at lane%4; int8: k row lane%16/2, 8 columns at lane%2) and get back column lane%16
+    const int kk = ES == 2 ? (r16 >> 2) : (r16 >> 1), cc = ES == 2 ? (r16 & 3) : (r16 & 1);
 #pragma unroll
     for (int jt = 0; jt < 4; jt++) {
-      const int chunk = (wn * 4 + jt) * 2 + (cc >> 1);
-      b_ld[jt] = (uint32_t)(A_BYTES + (2 * RG * g16 + kk) * B_ROW_BYTES + ((chunk ^ (kk * CW)) << 4) + (cc & 1) * 8);
+      const int chunk = ES == 2 ? (wn * 4 + jt) * 2 + (cc >> 1) : (wn * 4 + jt);
+      const int sub = ES == 2 ? (cc & 1) * 8 : cc * 8;
+      b_ld[jt] = (uint32_t)(A_BYTES + (2 * RG * g16 + kk) * B_ROW_BYTES + ((chunk ^ b_swz(kk)) << 4) + sub);
       if (TB) {
         const int row_b = wn * 64 + jt * 16 + r16;
         b_ld[jt] = (uint32_t)(A_BYTES + row_b * KB + ((g16 ^ ((row_b >> 2) & 3)) << 4));
@@ -1696,33 +1704,61 @@ template <bool TB = false> __global__ __launch_bounds__(256, 2) void gemm_tile12
       }
     }
   };
-  f32x4_t acc[4][4]; // [jt][it]: rows 16*it + lane%16, columns 16*jt + 4*(lane/16) .. +3 (B fragment as first operand)
+  acc4_t acc[4][4]; // [jt][it]: rows 16*it + lane%16, columns 16*jt + 4*(lane/16) .. +3 (B fragment as first operand)
 #pragma unroll
   for (int jt = 0; jt < 4; jt++)
 #pragma unroll
     for (int it = 0; it < 4; it++)
-      acc[jt][it] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      acc[jt][it] = acc4_t{0, 0, 0, 0};
+  const uint32_t a_xor = p.a_xor;
   auto mfma_all = [&](const uint4(&a)[4], const uint4(&b)[4]) {
+    if constexpr (ES == 2) {
 #pragma unroll
-    for (int jt = 0; jt < 4; jt++)
+      for (int jt = 0; jt < 4; jt++)
 #pragma unroll
-      for (int it = 0; it < 4; it++)
-        acc[jt][it] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b[jt]),
-                                                              __builtin_bit_cast(bf16x8_t, a[it]), acc[jt][it], 0, 0, 0);
+        for (int it = 0; it < 4; it++)
+          acc[jt][it] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b[jt]),
+                                                                __builtin_bit_cast(bf16x8_t, a[it]), acc[jt][it], 0, 0, 0);
+    } else {
+      // row tile by row tile; its bytes are flipped (u8 activations: a - 128 as s8 == a ^ 0x80) just before its four
+      // MFMAs, a whole stage after they were read, so no flip waits for LDS
+#pragma unroll
+      for (int it = 0; it < 4; it++) {
+        const uint4 f = make_uint4(a[it].x ^ a_xor, a[it].y ^ a_xor, a[it].z ^ a_xor, a[it].w ^ a_xor);
+#pragma unroll
+        for (int jt = 0; jt < 4; jt++)
+          acc[jt][it] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4_t, b[jt]), __builtin_bit_cast(i32x4_t, f),
+                                                              acc[jt][it], 0, 0, 0);
+      }
+    }
   };
 
   const char *a_ptr = reinterpret_cast<const char *>(p.A) + m0 * lda_b + k_first * KB;
   const char *b_ptr = reinterpret_cast<const char *>(p.B) + (TB ? n0 * ldb_b : n0 * ES) + k_first * b_step;
 
-  float cp_bias = -0.0f; // an absent bias adds nothing, not even to -0.0
-  if (tid < cols_in && p.bias)
-    cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n0 + tid])
-                                   : reinterpret_cast<const float *>(p.bias)[n0 + tid];
+  float cp_bias = -0.0f, cp_scale = 1.0f; // an absent bias adds nothing, not even to -0.0
+  int cp_cs = 0;
+  if (tid < cols_in) {
+    if (p.bias)
+      cp_bias = p.bias_dt == DT_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t *>(p.bias)[n0 + tid])
+                                     : reinterpret_cast<const float *>(p.bias)[n0 + tid];
+    if (ES == 1) {
+      if (p.scale)
+        cp_scale = p.scale[n0 + tid];
+      if (p.colsum)
+        cp_cs = p.comp * p.colsum[n0 + tid];
+    }
+  }
 #pragma unroll
   for (int d = 0; d < NST - 1; d++)
     issue(smem + d * STAGE, a_ptr + d * KB, b_ptr + d * b_step);
-  if (tid < T128_B)
+  if (tid < T128_B) {
     colp[tid] = cp_bias;
+    if (ES == 1) {
+      colp[256 + tid] = cp_scale;
+      reinterpret_cast<int *>(colp)[512 + tid] = cp_cs;
+    }
+  }
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NST - 2) * 4) : "memory");
   __builtin_amdgcn_s_barrier();
   uint4 fa0[4], fb0[4], fa1[4], fb1[4];
@@ -1791,8 +1827,9 @@ template <bool TB = false> __global__ __launch_bounds__(256, 2) void gemm_tile12
   for (int jt = 0; jt < 4; jt++)
 #pragma unroll
     for (int it = 0; it < 4; it++)
-      *reinterpret_cast<f32x4_t *>(dump + (it * 16 + r16) * W4_DUMP_PITCH + (jt * 16 + 4 * g16) * 4) = acc[jt][it];
-  const int kind = p.act + 8 * (p.out_dt == DT_BF16 ? 0 : 1);
+      *reinterpret_cast<acc4_t *>(dump + (it * 16 + r16) * W4_DUMP_PITCH + (jt * 16 + 4 * g16) * 4) = acc[jt][it];
+  const int out_kind = p.out_dt == DT_BF16 ? 0 : ((ES == 1 && p.out_dt == DT_S32) ? 2 : 1);
+  const int kind = (out_kind == 2 ? (int)ACT_NONE : p.act) + 8 * out_kind;
   if (rows_in < T128_B || cols_in < T128_B)
     w4_epilogue_half_any<ES, true, 64, 64>(p, kind, 0, m0, n0, wm, wn, lane, dump, colp, rows_in, cols_in);
   else
@@ -1978,7 +2015,7 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
   // c_bs = M * N.  A caller's MatmulConfig replaces the choice.
   const bool batch_ok = nbatch == 1 || ((p.a_bs * ES) % 16 == 0 && (p.b_bs * ES) % 16 == 0 && (p.c_bs * out_es) % 16 == 0 &&
                                         (!p.residual || (p.c_bs * res_es) % 16 == 0));
-  const bool t128_can = ES == 2 && aligned && p.N % (16 / ES) == 0 && p.out_dt != DT_S32 && batch_ok;
+  const bool t128_can = aligned && p.N % (16 / ES) == 0 && (ES == 2 ? p.out_dt != DT_S32 : !p.trans_b) && batch_ok;
   const bool slices_can = ES == 2 && fast_but_m && p.out_dt != DT_S32 && nbatch == 1; // the 256-wide kernels: whole column tiles
   const int64_t nblk128 = ((p.M + 127) / 128) * ((p.N + 127) / 128);
   const int n_cu = gcmi_num_cus();
@@ -1992,7 +2029,7 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
       splits = p.cfg_split_k < groups ? p.cfg_split_k : groups;
       plan = p.M > 128 && groups % splits == 0 ? PLAN_SLICES_TILE256 : PLAN_SLICES_SHORT_A;
     }
-  } else if (ES == 2 && aligned && nblk * nbatch < n_cu) {
+  } else if (aligned && nblk * nbatch < n_cu) { // (8-bit operands: the small tile in one pass is the only alternative)
     const double mn = (double)p.M * (double)p.N / 1048576.0;
     const double w256 = (double)(nblk * nbatch) / n_cu, w128 = (double)(nblk128 * nbatch) / n_cu;
     double best = GCMI_US_FIXED_256 + gcmi_us_per_group_256(w256) * groups; // one pass, less than one round
@@ -2003,7 +2040,7 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
         best = t, plan = PLAN_TILE128;
     }
     best *= GCMI_ONE_PASS_MARGIN;
-    if (nbatch == 1 && (small_tile || p.M > 128)) {
+    if (ES == 2 && nbatch == 1 && (small_tile || p.M > 128)) {
       for (int s = 2; s <= groups; s++) {
         const double through_memory = GCMI_US_SECOND_PASS + GCMI_US_PER_SLICE_MOUT * s * mn;
         if (slices_can && p.M > 128 && groups % s == 0 && nblk * s <= n_cu) {
@@ -2090,18 +2127,18 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
   }
   if (plan == PLAN_TILE128) {
     c.kernel = GK_TILE128, c.bm = c.bn = 128, c.kbytes = T128_KB, c.stages = T128_NST;
-    c.waves_m = c.waves_n = 2, c.wave_m = c.wave_n = 64, c.mfma_m = c.mfma_n = 16, c.mfma_k = 32;
+    c.waves_m = c.waves_n = 2, c.wave_m = c.wave_n = 64, c.mfma_m = c.mfma_n = 16, c.mfma_k = 64 / ES;
     c.workgroups = (int32_t)nblk128;
     if (cfg)
       *cfg = c;
     if (dry)
       return 0;
-    if constexpr (ES == 2) {
-      const dim3 grid((unsigned)nblk128, (unsigned)nbatch);
-      if (p.trans_b)
-        hipLaunchKernelGGL(gemm_tile128_kernel<true>, grid, dim3(256), 0, stream, p);
-      else
-        hipLaunchKernelGGL(gemm_tile128_kernel<false>, grid, dim3(256), 0, stream, p);
+    const dim3 grid((unsigned)nblk128, (unsigned)nbatch);
+    if (p.trans_b) {
+      if constexpr (ES == 2)
+        hipLaunchKernelGGL((gemm_tile128_kernel<true, 2>), grid, dim3(256), 0, stream, p);
+    } else {
+      hipLaunchKernelGGL((gemm_tile128_kernel<false, ES>), grid, dim3(256), 0, stream, p);
     }
     return hipGetLastError() == hipSuccess ? 0 : 5;
   }

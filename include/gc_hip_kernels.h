@@ -143,7 +143,7 @@ int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int6
  * 3 K slices over workgroups + second pass (tiles on less than half of the
  * compute units), 4 weight-streaming
  * kernel (a short A against [N,K] weights), 5 tiles of 128 x 128 with 4 waves
- * of 64 x 64 (bf16 problems of few 256 x 256 tiles; with split_k > 1 kind 3 is
+ * of 64 x 64 (problems of few 256 x 256 tiles; with split_k > 1 kind 3 is
  * reported and bm = bn = 128 tells).
  *
  * matmul_config (may be NULL) is the reference's per-op override: the nine
@@ -151,7 +151,7 @@ int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int6
  * innermostMBlock, innermostNBlock, innermostKBlock} of the op's attributes
  * (readConfigFromAttrs, MatmulConfigAnalysis.cpp:368-404: all nine or none;
  * validateConfig, :40-65).  On the GPU they steer: MBlock x NBlock = the
- * workgroup tile (256 x 256, and for bf16 128 x 128, are built),
+ * workgroup tile (256 x 256 and 128 x 128 are built),
  * innermostMBlock x innermostNBlock = the tile of one wave (128 x 128: 4 waves
  * per workgroup; 128 x 64: 8 waves; 64 x 64 with the 128 x 128 tile), KThreads
  * = the number of K slices where the shape is sliced (1 with the 128 x 128 tile).  A config that

@@ -306,12 +306,15 @@ def test_bf16_edge_tiles_of_the_four_wave_kernels(gc, orc, wl, dev, M, N, varian
         assert_close(ref, out.float().cpu().numpy(), 1e-2, "bf16 edge tiles %dx%d %s" % (M, N, variant))
 
 
-@pytest.mark.parametrize("M,N", [(300, 272), (520, 768), (256, 528)])
-def test_int8_edge_tiles_of_the_four_wave_kernel(gc, orc, dev, M, N):
-    """The same for u8 x s8 with dequantisation, bias and GELU to bf16 (N a multiple of 16, K of 256)."""
+@pytest.mark.parametrize("M,N", [(300, 272), (520, 256), (512, 528), (1000, 1008)])
+@pytest.mark.parametrize("tile", [256, 128])
+def test_int8_edge_tiles_of_the_four_wave_kernels(gc, orc, dev, M, N, tile):
+    """The same for u8 x s8 with dequantisation, bias and GELU to bf16 (N a multiple of 16, K of 256), on the tile
+    each MatmulConfig names; the two tiles give the same bits (integer sums are exact, the epilogue is one code)."""
     K = 512
-    c, _ = gc.tile_config(M, N, K, a_dtype=gc.U8)
-    assert c.kernel == 2
+    cfg = [1, 1, 1, 256, 256, 64, 128, 128, 32] if tile == 256 else [1, 1, 1, 128, 128, 64, 64, 64, 32]
+    c, _ = gc.tile_config(M, N, K, a_dtype=gc.U8, matmul_config=cfg)
+    assert c.kernel == (2 if tile == 256 else 5) and c.workgroups == -(-M // tile) * -(-N // tile) and c.from_attrs == 1
     torch.manual_seed(0)
     A = torch.randint(0, 256, (M, K), dtype=torch.int32).to(torch.uint8)
     torch.manual_seed(1)
@@ -323,10 +326,37 @@ def test_int8_edge_tiles_of_the_four_wave_kernel(gc, orc, dev, M, N):
     _, y = orc.int8_layer(A.numpy(), W.numpy(), sc.numpy(), bs.numpy(), 128, "gelu_erf")
     Wd = W.to(dev)
     guard = torch.full((M + 2, N), 7.0, dtype=torch.bfloat16, device=dev)
-    gc.gemm_int8(A.to(dev), Wd, gc.colsum_s8(Wd), 128, sc.to(dev), bs.to(dev), "gelu_erf", gc.BF16, out=guard[1:M + 1])
+    gc.gemm_int8(A.to(dev), Wd, gc.colsum_s8(Wd), 128, sc.to(dev), bs.to(dev), "gelu_erf", gc.BF16, out=guard[1:M + 1], matmul_config=cfg)
+    other = gc.gemm_int8(A.to(dev), Wd, gc.colsum_s8(Wd), 128, sc.to(dev), bs.to(dev), "gelu_erf", gc.BF16)  # the launcher's choice
     torch.cuda.synchronize()
     assert (guard[0] == 7).all() and (guard[M + 1] == 7).all()
+    assert torch.equal(guard[1:M + 1].view(torch.int16), other.view(torch.int16))
     assert_close(orc.bf16_to_f32(y), guard[1:M + 1].float().cpu().numpy(), 1e-2, "int8 edge tiles")
+
+
+@pytest.mark.parametrize("a_signed", [False, True])
+def test_int8_few_tiles_take_the_small_tile(gc, dev, a_signed):
+    """8-bit problems under one round of 256 x 256 tiles run on 128 x 128 tiles: raw accumulators against the integer
+    product, and every output type bit for bit against the large tiles (asked for by name)."""
+    big = [1, 1, 1, 256, 256, 64, 128, 128, 32]
+    torch.manual_seed(5)
+    for M, N, K in [(128, 128, 256), (512, 384, 1024), (129, 16, 256), (1024, 2048, 1024)]:
+        c, _ = gc.tile_config(M, N, K, a_dtype=gc.S8 if a_signed else gc.U8)
+        assert (c.kernel, c.bm, c.bn) == (5, 128, 128), (M, N, K, c.kernel)
+        A = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=dev) if a_signed else torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev)
+        W = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev)
+        cs = gc.colsum_s8(W)
+        zp = 3 if a_signed else 128
+        scale = (torch.rand(N, device=dev) * 0.009 + 0.001).float()
+        bias = torch.randn(N, device=dev).float()
+        raw = gc.gemm_int8(A, W, cs, zp, out_dtype=gc.S32)
+        assert torch.equal(raw.cpu().to(torch.int64), A.cpu().to(torch.int64) @ W.cpu().to(torch.int64))
+        for odt, act, sc, bi in [(gc.BF16, "gelu_erf", scale, bias), (gc.F32, "relu", scale, bias), (gc.BF16, None, scale, None)]:
+            got = gc.gemm_int8(A, W, cs, zp, sc, bi, act, odt)
+            want = gc.gemm_int8(A, W, cs, zp, sc, bi, act, odt, matmul_config=big)
+            torch.cuda.synchronize()
+            v = torch.int16 if odt == gc.BF16 else torch.int32
+            assert torch.equal(want.view(v), got.view(v)), (M, N, K, odt, act)
 
 
 def test_gelu_tanh_epilogue_absolute_accuracy(gc, dev):
