@@ -30,6 +30,16 @@ def test_defaults_per_shape(gc):
     assert (c.kernel, c.bm, c.wave_m, c.wave_n, c.split_k, c.workgroups) == (5, 128, 64, 64, 1, 256)
     c, _ = gc.tile_config(1024, 1024, 8192)                             # and a deep K: slices of small tiles
     assert (c.kernel, c.bm, c.split_k, c.workgroups) == (3, 128, 4, 256)
+    c, _ = gc.tile_config(128, 4096, 11008)                             # 86 ring groups of K: slices of unequal length
+    assert (c.kernel, c.bm, c.split_k, c.workgroups) == (3, 128, 8, 256)
+    c, _ = gc.tile_config(2048, 11008, 4096)                            # 344 large tiles: more than a round, they stay
+    assert (c.kernel, c.bm, c.split_k, c.workgroups) == (2, 256, 1, 344)
+    c, _ = gc.tile_config(1024, 4096, 4096, a_dtype=gc.U8)              # 8-bit, 64 large tiles: small tiles, never K slices
+    assert (c.kernel, c.bm, c.mfma_k, c.split_k, c.workgroups) == (5, 128, 64, 1, 256)
+    c, _ = gc.tile_config(1024, 1024, 8192, a_dtype=gc.U8)
+    assert (c.kernel, c.bm, c.split_k) == (5, 128, 1)
+    c, _ = gc.tile_config(64, 4096, 4096, trans_b=True)                 # [N,K] weights, 64 rows: slices of small tiles
+    assert (c.kernel, c.bm, c.split_k) == (3, 128, 8)
     c, _ = gc.tile_config(32, 4096, 4096, trans_b=True)                 # [N,K] weights, short A: streamed
     assert c.kernel == 4 and c.split_k >= 4
 
