@@ -1905,10 +1905,64 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
   c.kbytes = tiled ? 64 : G_KBYTES, c.stages = tiled ? 4 : 2;
   c.waves_m = 2, c.waves_n = use_w4 ? 2 : 4, c.wave_m = 128, c.wave_n = use_w4 ? 128 : 64;
   c.mfma_m = c.mfma_n = tiled ? 16 : 32, c.mfma_k = (tiled ? 64 : 32) / ES;
+  // More than a round of whole tiles with a poorly filled last round: the tiles of the last round are a block of
+  // columns (or rows) of C; where 128 x 128 tiles are estimated to finish that block clearly sooner than the large
+  // ones (up to about 40 % of a round), it becomes a launch of its own behind the whole rounds.  Both kernels add
+  // the products of an element in the same order, so C has the same bits either way.
+  int64_t tail_cols = 0, tail_rows = 0;
+  if (use_w4 && fast && nbatch == 1 && p.cfg_tile == 0 && t128_can && nblk > n_cu && nblk % n_cu != 0) {
+    const int64_t tail = nblk % n_cu;
+    const double t256 = GCMI_US_FIXED_256 + gcmi_us_per_group_256((double)tail / n_cu) * groups;
+    const double t128 = GCMI_US_FIXED_128 + 2.0 + gcmi_us_per_group_128(4.0 * tail / n_cu) * groups * (double)((4 * tail + 2 * n_cu - 1) / (2 * n_cu));
+    if (t128 < GCMI_ONE_PASS_MARGIN * t256) {
+      if (tail % tiles_m == 0)
+        tail_cols = tail / tiles_m * G_BN;
+      else if (tail % tiles_n == 0)
+        tail_rows = tail / tiles_n * G_BM;
+    }
+  }
+  if (tail_cols || tail_rows)
+    c.workgroups = (int32_t)(nblk - nblk % n_cu + 4 * (nblk % n_cu));
   if (cfg)
     *cfg = c;
   if (dry)
     return 0;
+  if (tail_cols || tail_rows) {
+    GemmParams head = p, rest = p;
+    const int bias_es = p.bias_dt == DT_BF16 ? 2 : 4;
+    if (tail_cols) {
+      const int64_t n1 = p.N - tail_cols;
+      head.N = n1, rest.N = tail_cols;
+      rest.B = reinterpret_cast<const char *>(p.B) + (p.trans_b ? n1 * p.ldb : n1) * ES;
+      rest.C = reinterpret_cast<char *>(p.C) + n1 * out_es;
+      if (p.bias)
+        rest.bias = reinterpret_cast<const char *>(p.bias) + n1 * bias_es;
+      if (p.scale)
+        rest.scale = p.scale + n1;
+      if (p.colsum)
+        rest.colsum = p.colsum + n1;
+      if (p.residual)
+        rest.residual = reinterpret_cast<const char *>(p.residual) + n1 * res_es;
+    } else {
+      const int64_t m1 = p.M - tail_rows;
+      head.M = m1, rest.M = tail_rows;
+      rest.A = reinterpret_cast<const char *>(p.A) + m1 * p.lda * ES;
+      rest.C = reinterpret_cast<char *>(p.C) + m1 * p.ldc * out_es;
+      if (p.residual)
+        rest.residual = reinterpret_cast<const char *>(p.residual) + m1 * p.ldr * res_es;
+    }
+    const dim3 hgrid((unsigned)(nblk - nblk % n_cu)), tgrid((unsigned)(4 * (nblk % n_cu)));
+    if (p.trans_b) {
+      if constexpr (ES == 2) {
+        hipLaunchKernelGGL((gemm_tile256_w4_kernel<ES, true>), hgrid, dim3(256), 0, stream, head);
+        hipLaunchKernelGGL((gemm_tile128_kernel<true, 2>), tgrid, dim3(256), 0, stream, rest);
+      }
+    } else {
+      hipLaunchKernelGGL(gemm_tile256_w4_kernel<ES>, hgrid, dim3(256), 0, stream, head);
+      hipLaunchKernelGGL((gemm_tile128_kernel<false, ES>), tgrid, dim3(256), 0, stream, rest);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : 5;
+  }
   dim3 grid((unsigned)nblk, (unsigned)nbatch), block(G_THREADS);
   if (use_w4) {
     if constexpr (ES == 2) {

@@ -481,6 +481,54 @@ def test_k_slices_exact_on_integers_for_any_slice_count(gc, dev, trans_b):
         assert torch.equal(out, torch.relu((want.to(torch.bfloat16).float() + bias.float()).to(torch.bfloat16)))  # rounded after each op
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 5120, 512), (4352, 4096, 256), (8192, 4352, 256)])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_a_thin_last_round_runs_on_small_tiles(gc, dev, M, N, K, trans_b):
+    """Just over a round of 256 x 256 tiles (320, 272 and 544 of them on 256 compute units): the last round's block of
+    columns or rows is a second launch on 128 x 128 tiles.  Exact on integers, and bit for bit the single launch of
+    large tiles (asked for by name) with bias, GELU and a residual."""
+    big = [1, 1, 1, 256, 256, 64, 128, 128, 32]
+    tiles = (M // 256) * (N // 256)
+    c, _ = gc.tile_config(M, N, K, trans_b=trans_b)
+    assert c.kernel == 2 and c.workgroups == tiles - tiles % 256 + 4 * (tiles % 256), (c.kernel, c.workgroups)
+    c, _ = gc.tile_config(M, N, K, trans_b=trans_b, matmul_config=big)
+    assert c.kernel == 2 and c.workgroups == tiles
+    torch.manual_seed(M + N)
+    A = torch.randint(-3, 4, (M, K), device=dev).to(torch.bfloat16)
+    B = torch.randint(-3, 4, (K, N), device=dev).to(torch.bfloat16)
+    out = torch.full((M, N), 7.0, dtype=torch.float32, device=dev)
+    _gemm_ws(gc, A, B.t().contiguous() if trans_b else B, trans_b, out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, A.float() @ B.float())
+    A = (torch.randn(M, K, device=dev) * 0.5).to(torch.bfloat16)
+    B = (torch.randn(K, N, device=dev) * 0.5).to(torch.bfloat16)
+    Bd = B.t().contiguous() if trans_b else B
+    bias, res = torch.randn(N, device=dev).to(torch.bfloat16), torch.randn(M, N, device=dev).to(torch.bfloat16)
+    o1, o2 = torch.empty(M, N, dtype=torch.bfloat16, device=dev), torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    _gemm_ws(gc, A, Bd, trans_b, o1, bias=bias, act="gelu_erf", residual=res)
+    _gemm_ws(gc, A, Bd, trans_b, o2, 1, bias=bias, act="gelu_erf", residual=res)
+    torch.cuda.synchronize()
+    assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
+
+
+def test_a_thin_last_round_of_the_int8_layer(gc, dev):
+    big = [1, 1, 1, 256, 256, 64, 128, 128, 32]
+    M, N, K = 4096, 5120, 512
+    c, _ = gc.tile_config(M, N, K, a_dtype=gc.U8)
+    assert c.kernel == 2 and c.workgroups == 256 + 4 * 64
+    torch.manual_seed(9)
+    A = torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev)
+    W = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev)
+    cs = gc.colsum_s8(W)
+    scale, bias = (torch.rand(N, device=dev) * 0.009 + 0.001).float(), torch.randn(N, device=dev).float()
+    a = gc.gemm_int8(A, W, cs, 128, scale, bias, "gelu_erf", gc.BF16)
+    b = gc.gemm_int8(A, W, cs, 128, scale, bias, "gelu_erf", gc.BF16, matmul_config=big)
+    raw = gc.gemm_int8(A, W, cs, 128, out_dtype=gc.S32)  # s32 results: the 8-wave kernel, one launch
+    torch.cuda.synchronize()
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert torch.equal(raw.cpu().to(torch.int64), A.cpu().to(torch.int64) @ W.cpu().to(torch.int64))
+
+
 NT_SHAPES = [(256, 256, 128), (512, 768, 256), (300, 200, 100), (257, 511, 129), (1, 7, 5), (33, 1, 64), (128, 256, 8),
              (32, 4096, 4096), (1, 1024, 2048), (32, 11008, 4096), (64, 512, 2048), (33, 1024, 1024), (17, 2048, 512),
              (32, 4096, 11008), (65, 1024, 1024), (32, 1056, 1088), (32, 8192, 1024), (64, 8192, 512)]

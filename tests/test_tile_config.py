@@ -38,6 +38,10 @@ def test_defaults_per_shape(gc):
     assert (c.kernel, c.bm, c.mfma_k, c.split_k, c.workgroups) == (5, 128, 64, 1, 256)
     c, _ = gc.tile_config(1024, 1024, 8192, a_dtype=gc.U8)
     assert (c.kernel, c.bm, c.split_k) == (5, 128, 1)
+    c, _ = gc.tile_config(4096, 5120, 4096)                             # 320 large tiles: a round, and 64 tiles as 256 small ones
+    assert (c.kernel, c.bm, c.workgroups) == (2, 256, 256 + 4 * 64)
+    c, _ = gc.tile_config(4096, 11008, 4096)                            # 176 tiles in the last round: too many for that
+    assert (c.kernel, c.workgroups) == (2, 688)
     c, _ = gc.tile_config(64, 4096, 4096, trans_b=True)                 # [N,K] weights, 64 rows: slices of small tiles
     assert (c.kernel, c.bm, c.split_k) == (3, 128, 8)
     c, _ = gc.tile_config(32, 4096, 4096, trans_b=True)                 # [N,K] weights, short A: streamed
