@@ -426,7 +426,8 @@ def main():
     # ---------------- bf16 GEMMs whose 256 x 256 tiles would not fill the GPU: 128 x 128 tiles and / or K slices
     if want("few_tiles"):
         few = {}
-        for Mf, Nf, Kf in ((2048, 2048, 2048), (1024, 4096, 4096), (512, 4096, 4096), (1024, 1024, 8192), (2048, 4096, 4096)):
+        for Mf, Nf, Kf in ((2048, 2048, 2048), (1024, 4096, 4096), (512, 4096, 4096), (1024, 1024, 8192), (2048, 4096, 4096),
+                           (4096, 5120, 4096)):  # the last: 320 large tiles, a round and a thin one (run on small tiles)
             Af = (torch.randn(Mf, Kf) * 0.1).to(torch.bfloat16).to(dev)
             Bf = (torch.randn(Kf, Nf) * 0.1).to(torch.bfloat16).to(dev)
             Cf = torch.empty(Mf, Nf, dtype=torch.bfloat16, device=dev)
@@ -451,8 +452,9 @@ def main():
         del Ai, Wi, Oi
         others["bf16_gemm_few_tiles"] = {
             "workload": "bf16 GEMMs of 16 to 128 tiles of 256 x 256 (one compute unit works 1.9 us per tile and 128 of K): the "
-                        "launcher gives them to more workgroups by 128 x 128 tiles, K slices, or both; and one 8-bit layer "
-                        "of 64 such tiles (128 x 128 tiles)", "cases": few}
+                        "launcher gives them to more workgroups by 128 x 128 tiles, K slices, or both; one of 320 tiles (a "
+                        "full round on large tiles, the 64 left over on small ones); and one 8-bit layer of 64 large "
+                        "tiles (128 x 128 tiles)", "cases": few}
         log("few tiles: %s" % json.dumps(few))
         torch.cuda.empty_cache()
 
