@@ -21,7 +21,7 @@ ACT = {None: 0, "none": 0, "relu": 1, "gelu_erf": 2, "gelu_tanh": 3, "sigmoid": 
 # every symbol the public headers declare (checked by the CPU test-suite)
 EXPORTS = {
     "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_bf16_nt", "gcmi_gemm_bf16_batched", "gcmi_gemm_bf16_residual", "gcmi_gemm_f32_batched",
-                         "gcmi_gemm_bf16_ws", "gcmi_gemm_bf16_workspace_bytes", "gcmi_mha_fwd_bf16_ws", "gcmi_mha_fwd_workspace_bytes",
+                         "gcmi_gemm_bf16_ws", "gcmi_gemm_bf16_workspace_bytes", "gcmi_gemm_bf16_workspace_bytes_cfg", "gcmi_mha_fwd_bf16_ws", "gcmi_mha_fwd_workspace_bytes",
                          "gcmi_gemm_bf16_noalloc", "gcmi_noalloc_scratch_bytes", "gcmi_gemm_int8_cfg", "gcmi_gemm_tile_config_query",
                          "gcmi_gemm_int8", "gcmi_colsum_s8",
                          "gcmi_gemm_f32", "gcmi_mha_fwd_bf16", "gcmi_mha_fwd_bf16_opt"],
@@ -59,6 +59,8 @@ def lib():
     L.gcmi_gemm_bf16_residual.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, vp, ci, ci, vp, i64, ci, ci, vp]
     L.gcmi_gemm_bf16_workspace_bytes.restype = C.c_size_t
     L.gcmi_gemm_bf16_workspace_bytes.argtypes = [i64, i64, i64, ci]
+    L.gcmi_gemm_bf16_workspace_bytes_cfg.restype = C.c_size_t
+    L.gcmi_gemm_bf16_workspace_bytes_cfg.argtypes = [i64, i64, i64, ci, C.POINTER(C.c_int64)]
     L.gcmi_gemm_bf16_ws.restype = ci
     L.gcmi_gemm_bf16_ws.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, vp, ci, ci, vp, i64, ci, ci, vp, C.c_size_t, vp, vp]
     L.gcmi_gemm_int8_cfg.restype = ci

@@ -243,7 +243,7 @@ void Executable::plan_workspaces() {
   for (Step &s : steps_) {
     size_t bytes = 0;
     if (s.kind == Step::GemmBf16 && s.batch <= 1)
-      bytes = gcmi_gemm_bf16_workspace_bytes(s.M, s.N, s.K, s.tb ? 1 : 0);
+      bytes = gcmi_gemm_bf16_workspace_bytes_cfg(s.M, s.N, s.K, s.tb ? 1 : 0, s.mm_cfg.size() == 9 ? s.mm_cfg.data() : nullptr);
     else if (s.kind == Step::Mha && s.mask >= 0)
       bytes = gcmi_mha_fwd_workspace_bytes(s.Sq, s.Sk, s.D, 1);
     if (bytes)
@@ -1752,6 +1752,8 @@ std::string Executable::describe() const {
            << " B of K per stage x " << c.stages << " stages, waves " << c.waves_m << "x" << c.waves_n << " of " << c.wave_m << "x"
            << c.wave_n << ", mfma " << c.mfma_m << "x" << c.mfma_n << "x" << c.mfma_k << ", split_k " << c.split_k << ", "
            << c.workgroups << " workgroups";
+        if (c.split_k > 1) // the slot the partial sums of the slices were planned into
+          os << ", workspace " << (s.ws >= 0 ? slots_[(size_t)s.ws].bytes : 0) << " B";
         if (c.from_attrs)
           os << " [MatmulConfig attributes applied]";
         else if (why[0])

@@ -312,7 +312,8 @@ int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M
 }
 } // namespace
 
-extern "C" size_t gcmi_gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_b) {
+extern "C" size_t gcmi_gemm_bf16_workspace_bytes_cfg(int64_t M, int64_t N, int64_t K, int trans_b,
+                                                     const int64_t *matmul_config) {
   if (M <= 0 || N <= 0 || K <= 0)
     return 0;
   GemmParams p{};
@@ -320,8 +321,16 @@ extern "C" size_t gcmi_gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K
   p.A = p.B = (const void *)(uintptr_t)256, p.C = (void *)(uintptr_t)256;
   p.M = M, p.N = N, p.K = K, p.lda = K, p.ldb = trans_b ? K : N, p.ldc = N;
   p.bias_dt = GCMI_BF16, p.out_dt = GCMI_BF16, p.trans_b = trans_b ? 1 : 0, p.batch = 1;
+  if (matmul_config) { // the slices a caller's MatmulConfig names, exactly as gcmi_gemm_bf16_ws will apply it
+    const char *why;
+    (void)apply_matmul_config(matmul_config, M, N, K, p, &why);
+  }
   const int64_t want = gcmi_launch_gemm_bf16_workspace(&p);
   return want > 0 ? (size_t)want * 4 : 0;
+}
+
+extern "C" size_t gcmi_gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_b) {
+  return gcmi_gemm_bf16_workspace_bytes_cfg(M, N, K, trans_b, nullptr);
 }
 
 extern "C" int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int64_t M, int64_t N, int64_t K,

@@ -1895,10 +1895,11 @@ static int launch_tile256(const GemmParams *pp, hipStream_t stream, int64_t *wan
     }
     return hipGetLastError() == hipSuccess ? 0 : 5;
   }
-  // Whole tiles: 4 waves of 128 x 128 unless the caller asks for 8 waves of 128 x 64 (or the result is an f32 / s32
-  // tensor of 8-bit operands, which only the 8-wave kernel writes).  Tiles that stick out of C (`ragged`): the 4-wave
-  // kernel.  Anything else (a K tail, unaligned rows): the bounds-checked kernel.
-  const bool w4_can = (fast || ragged) && (ES == 2 || p.out_dt == DT_BF16);
+  // Whole tiles: 4 waves of 128 x 128 unless the caller asks for 8 waves of 128 x 64.  Results of 8-bit operands
+  // leave the 4-wave kernel as bf16, f32 or as the raw s32 accumulators (same main loop, the epilogue is a plain
+  // store).  Tiles that stick out of C (`ragged`): the 4-wave kernel.  Anything else (a K tail, unaligned rows): the
+  // bounds-checked kernel.
+  const bool w4_can = fast || ragged;
   const bool use_w4 = w4_can && (p.cfg_waves != 8 || !fast);
   const bool tiled = fast || use_w4; // one of the kernels with the LDS ring
   c.kernel = !tiled ? GK_EDGE : (use_w4 ? GK_WAVES4 : GK_WAVES8);

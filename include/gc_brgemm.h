@@ -15,7 +15,11 @@
  * dimensions and batch strides are in elements; dtypes are dnnl_data_type_t
  * values (bf16 2, f32 3, s8 5, u8 6).  With beta == 0 the LDC-strided M x N
  * block is overwritten (the behaviour of the reference's oneDNN back-end,
- * lib/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmOnednn.cpp:94-98).
+ * lib/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmOnednn.cpp:94-98).  The
+ * reference's naive fallback runtime differs when LDC > N: its beta == 0 clears
+ * the first M*N elements of C densely (BrgemmNaive.cpp:36-44), so rows past
+ * M*N/LDC are accumulated into and the padding in front of them is cleared; that
+ * is not reproduced here (tests/golden holds both results for such cases).
  *
  * Handles are small dense integers from a process-wide table that is never
  * freed; dispatch is thread safe and may run from static constructors.  An

@@ -126,6 +126,9 @@ int gcmi_gemm_bf16_residual(const void *A, const void *B, void *C, int64_t batch
  * allocates (lib/gc/Transforms/DeepTileContractionOp.cpp:988-996).
  */
 size_t gcmi_gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_b);
+/* The same for a call that passes `matmul_config` (nine MatmulConfig integers, or NULL): a KThreads that names more
+ * slices than the shape would get by default needs a workspace where the default needs none. */
+size_t gcmi_gemm_bf16_workspace_bytes_cfg(int64_t M, int64_t N, int64_t K, int trans_b, const int64_t *matmul_config);
 int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int64_t M, int64_t N, int64_t K,
                       int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
                       int trans_b, const void *bias, int bias_dtype, int act, const void *residual, int64_t ldr,

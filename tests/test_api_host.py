@@ -195,3 +195,25 @@ def test_k_sliced_matmuls_get_scratch_of_their_own_in_the_arena(ga, gc):
     assert naive == hidden + 2 * ws
     assert shared == hidden + ws    # the second step's scratch takes the place of the first's
     assert staging == 2 * M * K * 2 + 2 * K * N * 2   # A, both weights, the result
+
+
+@pytest.mark.parametrize("M,N,K,kthreads", [(4096, 4096, 4096, 4), (1024, 4096, 4096, 8)])
+def test_slices_named_by_a_matmul_config_get_their_workspace(ga, gc, M, N, K, kthreads):
+    """Shapes the launcher would not slice by default: a MatmulConfig whose KThreads names slices must get the
+    partial sums' slot planned (else the launch silently runs unsliced while the plan text says otherwise), and the
+    plan text, the tile descriptor and the workspace query must tell the same story."""
+    import ctypes as C
+    import re
+    nine = [1, 1, kthreads, 256, 256, 64, 128, 128, 32]
+    assert gc.lib().gcmi_gemm_bf16_workspace_bytes(M, N, K, 0) == 0
+    c, note = gc.tile_config(M, N, K, matmul_config=nine)
+    assert (c.kernel, c.split_k, c.from_attrs, note) == (3, kthreads, 1, "")
+    ws = gc.lib().gcmi_gemm_bf16_workspace_bytes_cfg(M, N, K, 0, (C.c_int64 * 9)(*nine))
+    assert ws == kthreads * M * N * 4
+    op = {"kind": "MatMul", "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [K, N])], "outputs": [ga._t(2, "bf16", [M, N])],
+          "attrs": {k: {"type": "s64", "value": v} for k, v in zip(gc.MATMUL_CONFIG_NAMES, nine)}}
+    st, plan = ga.explain(ga._graph([op], [0, 1], [2]))
+    assert st == 0, plan
+    assert re.search(r"split_k %d, \d+ workgroups, workspace %d B \[MatmulConfig attributes applied\]" % (kthreads, ws), plan), plan
+    arena = int(re.search(r"arena: (\d+) bytes", plan).group(1))
+    assert arena >= ws

@@ -184,15 +184,23 @@ def test_int8_layer_special_scales_and_biases(gc, orc, dev, act):
     assert_close(orc.bf16_to_f32(want[~special]), orc.bf16_to_f32(got[~special]), 1e-2, "finite part")
 
 
-def test_int8_full_size_exact_checksums_and_rows(gc, orc, wl, dev):
-    """BASELINE config 3 (4096 x 4096 x 11008).  Exactness of all 45M
-    accumulators through integer checksums (row sums and column sums of the
-    s32 result against int64 products of the operand sums), exact rows against
-    the oracle, and the fused epilogue against the oracle on those rows."""
+@pytest.mark.parametrize("a_signed", [False, True])
+def test_int8_full_size_exact_checksums_and_rows(gc, orc, wl, dev, a_signed):
+    """BASELINE config 3 (4096 x 4096 x 11008), on the kernel the benchmark times (4 waves of 128 x 128, asserted
+    through the tile descriptor): the raw s32 accumulators leave it through a plain store.  Exactness of all 45M
+    accumulators through integer checksums (row sums and column sums of the s32 result against int64 products of the
+    operand sums), exact rows against the oracle (lib/gc/ExecutionEngine/CPURuntime/Microkernel/BrgemmNaive.cpp:102-140
+    is what it restates), the 8-wave kernel's accumulators bit for bit, and the fused epilogue against the oracle on
+    those rows.  u8 activations (the config) and s8 activations (no byte flip, no zero-point term)."""
     A, W, scale, bias = wl.int8_mlp_layer()
+    zp = 128
+    if a_signed:
+        A, zp = (A.to(torch.int16) - 128).to(torch.int8), 0
+    c, _ = gc.tile_config(4096, 11008, 4096, a_dtype=gc.S8 if a_signed else gc.U8, out_dtype=gc.S32)
+    assert (c.kernel, c.waves_m * c.waves_n, c.wave_m, c.wave_n) == (2, 4, 128, 128)
     Ad, Wd = A.to(dev), W.to(dev)
     cs = gc.colsum_s8(Wd)
-    raw = gc.gemm_int8(Ad, Wd, cs, 0, None, None, None, gc.S32)
+    raw = gc.gemm_int8(Ad, Wd, cs, 0 if a_signed else 128, None, None, None, gc.S32)
     torch.cuda.synchronize()
     assert (cs.cpu() == W.to(torch.int64).sum(0)).all()
     raw64 = raw.to(torch.int64)
@@ -200,10 +208,25 @@ def test_int8_full_size_exact_checksums_and_rows(gc, orc, wl, dev):
     row_want = (A.to(torch.int64) @ W.to(torch.int64).sum(1, keepdim=True)).squeeze(1)   # A W 1
     assert (raw64.sum(0).cpu() == col_want).all()
     assert (raw64.sum(1).cpu() == row_want).all()
+    # a second, position-dependent checksum: a swap of two accumulators inside a row or a column would keep the plain
+    # sums; weights r_i = i + 1 and c_j = j + 1 catch it.  (r^T A) W c in int64.
+    r = torch.arange(1, 4097, dtype=torch.int64)
+    cw = torch.arange(1, 11009, dtype=torch.int64)
+    want_rc = ((r.unsqueeze(0) @ A.to(torch.int64)) @ (W.to(torch.int64) @ cw.unsqueeze(1))).item()
+    got_rc = int((raw64.cpu() * r.unsqueeze(1) * cw.unsqueeze(0)).sum().item())
+    assert got_rc == want_rc
     rows = [0, 255, 256, 1027, 2048, 3333, 4095] + list(range(61, 4096, 449))
-    acc, y = orc.int8_layer(A[rows].numpy(), W.numpy(), scale.numpy(), bias.numpy(), 128, "gelu_erf")
+    acc = orc.deep_tile_matmul(A[rows].numpy(), W.numpy(), orc.S8 if a_signed else orc.U8, orc.S8)
     assert (raw[rows].cpu().numpy() == acc).all()
-    out = gc.gemm_int8(Ad, Wd, cs, 128, scale.to(dev), bias.to(dev), "gelu_erf", gc.BF16)
+    eight = gc.gemm_int8(Ad, Wd, cs, 0 if a_signed else 128, None, None, None, gc.S32,
+                         matmul_config=[1, 1, 1, 256, 256, 64, 128, 64, 32])
+    torch.cuda.synchronize()
+    assert torch.equal(raw, eight)
+    del eight, raw64
+    if a_signed:
+        return
+    _, y = orc.int8_layer(A[rows].numpy(), W.numpy(), scale.numpy(), bias.numpy(), zp, "gelu_erf")
+    out = gc.gemm_int8(Ad, Wd, cs, zp, scale.to(dev), bias.to(dev), "gelu_erf", gc.BF16)
     torch.cuda.synchronize()
     assert_close(orc.bf16_to_f32(y), out[rows].float().cpu().numpy(), 1e-2, "int8 mlp rows")
 
@@ -243,12 +266,11 @@ def test_gelu_erf_epilogue_absolute_accuracy(gc, dev):
     (the reference's own erf is an approximation of that class): GELU over a
     dense grid of x, computed as a [M,1]x[1,1] matmul with the activation fused,
     against float64."""
-    from scipy.special import erf
     x = torch.linspace(-8, 8, 200001, dtype=torch.float32).reshape(-1, 1)
     one = torch.ones(1, 1, dtype=torch.float32)
     out = gc.gemm_f32(x.to(dev), one.to(dev), act="gelu_erf").cpu().numpy().astype(np.float64).ravel()
     xd = x.numpy().astype(np.float64).ravel()
-    ref = 0.5 * xd * (1 + erf(xd * 0.7071067811865476))
+    ref = 0.5 * xd * (1 + torch.special.erf(torch.from_numpy(xd) * 0.7071067811865476).numpy())  # float64
     assert np.abs(out - ref).max() <= 2e-6  # |x| <= 8: 0.5 * 8 * 2e-7 + f32 rounding
     # the argument of erf is clamped at 4.2 = 5.94 / sqrt 2, and from 3.9 on the result is exactly +-1, as libm's is
     assert (out[xd < -5.84] == 0).all() and (out[xd > 5.84] == xd[xd > 5.84]).all()
@@ -523,7 +545,9 @@ def test_a_thin_last_round_of_the_int8_layer(gc, dev):
     scale, bias = (torch.rand(N, device=dev) * 0.009 + 0.001).float(), torch.randn(N, device=dev).float()
     a = gc.gemm_int8(A, W, cs, 128, scale, bias, "gelu_erf", gc.BF16)
     b = gc.gemm_int8(A, W, cs, 128, scale, bias, "gelu_erf", gc.BF16, matmul_config=big)
-    raw = gc.gemm_int8(A, W, cs, 128, out_dtype=gc.S32)  # s32 results: the 8-wave kernel, one launch
+    raw = gc.gemm_int8(A, W, cs, 128, out_dtype=gc.S32)  # s32 results: the same two launches, plain stores
+    c, _ = gc.tile_config(M, N, K, a_dtype=gc.U8, out_dtype=gc.S32)
+    assert c.kernel == 2 and c.workgroups == 256 + 4 * 64
     torch.cuda.synchronize()
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     assert torch.equal(raw.cpu().to(torch.int64), A.cpu().to(torch.int64) @ W.cpu().to(torch.int64))

@@ -18,8 +18,12 @@ def test_defaults_per_shape(gc):
     assert note == ""
     c, _ = gc.tile_config(4096, 11008, 4096, a_dtype=gc.U8)             # config 3: 688 tiles
     assert (c.kernel, c.mfma_k, c.workgroups) == (2, 64, 688)
-    c, _ = gc.tile_config(4096, 11008, 4096, a_dtype=gc.U8, out_dtype=gc.S32)  # raw accumulators: the 8-wave kernel
-    assert (c.kernel, c.waves_m * c.waves_n, c.wave_n) == (1, 8, 64)
+    for odt in (gc.S32, gc.F32):                                        # raw accumulators / f32: the same 4-wave kernel
+        c, _ = gc.tile_config(4096, 11008, 4096, a_dtype=gc.U8, out_dtype=odt)
+        assert (c.kernel, c.waves_m * c.waves_n, c.wave_n, c.mfma_k, c.workgroups) == (2, 4, 128, 64, 688)
+    c, _ = gc.tile_config(4096, 11008, 4096, a_dtype=gc.U8, out_dtype=gc.S32,   # 8 waves of 128 x 64 by name
+                          matmul_config=_cfg(iN=64))
+    assert (c.kernel, c.waves_m * c.waves_n, c.wave_n, c.from_attrs) == (1, 8, 64, 1)
     c, _ = gc.tile_config(300, 200, 100)                                # ragged: bounds-checked tile
     assert c.kernel == 0
     c, _ = gc.tile_config(32, 4096, 4096)                               # one tile row: K slices fill the GPU
