@@ -1437,7 +1437,6 @@ __device__ __forceinline__ void w4_epilogue_half_any(const GemmParams &p, int ki
 }
 
 template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gemm_tile256_w4_kernel(GemmParams p) {
-  static_assert(!TB || ES == 2, "B stored [N,K]: bf16 only");
   typedef FastGemm<ES, 2, 4, false, TB> FG; // 4 waves: 4 DMA instructions per operand, wave and stage
   static_assert(FG::NST == 4 && FG::NDMA == 4 && FG::STAGE_BYTES == 32768 && FG::A_BYTES == 16384, "the assembly's ring");
 #ifdef GCMI_W4_TIMING
@@ -1544,7 +1543,9 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gem
 #ifdef GCMI_W4_TIMING // measurement builds: core clock cycles and 100 MHz ticks spent in the main loop
   const long long tick0 = clock64(), wall0 = wall_clock64();
 #endif
-  if constexpr (ES == 1)
+  if constexpr (ES == 1 && TB)
+    asm volatile(GCMI_W4_ASM_I8_TB GCMI_W4_OPERANDS);
+  else if constexpr (ES == 1)
     asm volatile(GCMI_W4_ASM_I8 GCMI_W4_OPERANDS);
   else if constexpr (TB)
     asm volatile(GCMI_W4_ASM_BF16_TB GCMI_W4_OPERANDS);

@@ -205,7 +205,7 @@ def main():
     path = sys.argv[1]
     with open(path, "w") as f:
         f.write("// generated by gen_gemm_w4_mainloop.py -- do not edit\n")
-        for name, es, tb in (("BF16", 2, False), ("BF16_TB", 2, True), ("I8", 1, False)):
+        for name, es, tb in (("BF16", 2, False), ("BF16_TB", 2, True), ("I8", 1, False), ("I8_TB", 1, True)):
             lines = gen(es, tb)
             f.write("#define GCMI_W4_ASM_%s \\\n" % name)
             f.write(" \\\n".join('  "%s\\n"' % ln for ln in lines))

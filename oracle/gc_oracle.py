@@ -72,6 +72,12 @@ def _load():
     lib.gco_mha_bf16.argtypes = [vp, vp, vp, vp, f32, i64, i64, i64, i64, vp]
     lib.gco_compare_p2p.restype = i64
     lib.gco_compare_p2p.argtypes = [vp, vp, i64, f32, vp]
+    lib.gco_compare_norm.restype = ci
+    lib.gco_compare_norm.argtypes = [vp, vp, i64, f32, vp]
+    lib.gco_compare_norm_rows.restype = i64
+    lib.gco_compare_norm_rows.argtypes = [vp, vp, i64, i64, f32, vp]
+    lib.gco_mha_f64.restype = ci
+    lib.gco_mha_f64.argtypes = [vp, vp, vp, vp, C.c_double, i64, i64, i64, i64, ci, vp]
     lib.gco_num_threads.restype = ci
     return lib
 
@@ -340,6 +346,45 @@ def compare_p2p(ref, res, thr):
     md = C.c_float(0)
     bad = lib().gco_compare_p2p(_p(ref), _p(res), ref.size, float(thr), C.byref(md))
     return int(bad), float(md.value)
+
+
+def compare_norm(ref, res, thr):
+    """benchgc norm rule (test/benchgc/src/benchgc/arg/compare.py:41-57).  Returns (passed, l2)."""
+    ref = _c(ref, np.float32).ravel()
+    res = _c(res, np.float32).ravel()
+    assert ref.size == res.size
+    v = C.c_float(0)
+    ok = lib().gco_compare_norm(_p(ref), _p(res), ref.size, float(thr), C.byref(v))
+    return bool(ok), float(v.value)
+
+
+def compare_norm_rows(ref, res, thr):
+    """The norm rule per row of the last dim.  Returns (n_failing_rows, l2 per row)."""
+    ref = _c(ref, np.float32)
+    res = _c(res, np.float32)
+    assert ref.shape == res.shape
+    cols = ref.shape[-1]
+    rows = ref.size // cols
+    l2 = np.empty(rows, np.float32)
+    bad = lib().gco_compare_norm_rows(_p(ref), _p(res), rows, cols, float(thr), _p(l2))
+    return int(bad), l2
+
+
+def mha_f64(Q16, K16, V16, mask, scale, round_p):
+    """The attention composition in float64 (error attribution).  round_p: round the softmax weights to bf16 where the
+    reference graph does.  Q,K,V: uint16 [B,H,S,D]; returns float64 [B,H,Sq,D], not rounded."""
+    Q16 = _c(Q16, np.uint16)
+    K16 = _c(K16, np.uint16)
+    V16 = _c(V16, np.uint16)
+    Bn, H, Sq, D = Q16.shape
+    Sk = K16.shape[2]
+    out = np.empty((Bn, H, Sq, D), np.float64)
+    m = None if mask is None else _c(mask, np.float32)
+    rc = lib().gco_mha_f64(_p(Q16), _p(K16), _p(V16), None if m is None else _p(m), float(scale),
+                           Bn * H, Sq, Sk, D, 1 if round_p else 0, _p(out))
+    if rc:
+        raise MemoryError
+    return out
 
 
 def num_threads():

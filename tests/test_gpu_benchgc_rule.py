@@ -100,6 +100,44 @@ def test_config2_strict_failures_are_cancellations(gc, orc, wl, dev):
     assert bad.sum() <= 0.01 * bad.size
 
 
+def test_config3_strict_failures_are_gelu_tail_or_cancellations(gc, orc, wl, dev):
+    """int8 MLP layer at full size (4096 x 4096 x 11008, dequantise + bias + GELU to bf16): 48 rows against the
+    oracle under the strict rule at 1e-2, and under the harness's norm rule per row.  The accumulators are exact
+    (tests/test_gpu_gemm.py), so whatever differs comes from the epilogue: the GPU forms acc * scale + bias as one
+    fused multiply-add and evaluates erf by its own polynomial (absolute error 1.5e-7).  A strict failure must
+    therefore be one of: (a) a pre-activation value x in the negative GELU tail, where gelu(x) = x/2 * (erf + 1) is a
+    difference of nearly equal numbers in the reference's own f32 arithmetic as well -- (erf + 1) < 2e-5 from
+    x < -4.2 on, so 1.5e-7 is more than 1e-2 of it, and past x = -4.7 |gelu| < 1e-5 falls under the rule's absolute
+    branch and passes --, or (b) a cancellation of acc * scale against the bias."""
+    A, W, scale, bias = wl.int8_mlp_layer()
+    Ad, Wd = A.to(dev), W.to(dev)
+    cs = gc.colsum_s8(Wd)
+    out = gc.gemm_int8(Ad, Wd, cs, 128, scale.to(dev), bias.to(dev), "gelu_erf", gc.BF16)
+    torch.cuda.synchronize()
+    rows = sorted(set(list(range(0, 4096, 256)) + list(range(255, 4096, 256)) + list(range(97, 4096, 331))))[:48]
+    acc, y = orc.int8_layer(A[rows].numpy(), W.numpy(), scale.numpy(), bias.numpy(), 128, "gelu_erf")
+    ref = orc.bf16_to_f32(y)
+    res = out[rows].float().cpu().numpy()
+    bad = strict_failures(orc, ref, res, 1e-2)
+    prod = (acc.astype(np.float64) - 128.0 * W.to(torch.int64).sum(0).numpy()[None, :]) * scale.double().numpy()[None, :]
+    x = prod + bias.double().numpy()[None, :]                   # the pre-activation value, exact
+    tail = (x < -4.0) & (x > -5.0)
+    cancel = np.abs(x) < CANCEL_FRACTION * (np.abs(prod) + np.abs(bias.double().numpy())[None, :])
+    n = int(bad.sum())
+    print("\nconfig 3: strict rule fails on %d of %d elements (%d in the GELU tail -5 < x < -4, %d cancellations of "
+          "acc*scale + bias); elements in that tail window: %d" % (n, bad.size, int((bad & tail).sum()),
+                                                                   int((bad & cancel & ~tail).sum()), int(tail.sum())))
+    assert (tail | cancel)[bad].all(), x[bad & ~(tail | cancel)][:8]
+    assert n <= 1e-3 * bad.size
+    # elsewhere the two agree to a bf16 step, and nearly always bit for bit
+    differ = ref != res
+    assert differ.mean() < 1e-3
+    # the harness's norm rule (test/benchgc/src/benchgc/arg/compare.py:41-57), per sampled row
+    nbad, l2 = orc.compare_norm_rows(ref, res, 1e-4)
+    print("config 3: per-row norm of the difference: max %.2e, median %.2e" % (float(l2.max()), float(np.median(l2))))
+    assert nbad == 0
+
+
 def test_config4_full_size_and_strict_failures(gc, orc, wl, dev):
     """bf16 MLP chain at full size (4096 x 4096 x 11008 -> 4096): sampled rows of both layers against
     the oracle's chain, column checksums of both layers over all rows in f64, and the strict-rule count."""

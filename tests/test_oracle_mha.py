@@ -78,3 +78,28 @@ def test_fully_masked_row_is_nan(orc):
     mask[2, :] = -np.inf
     out = orc.bf16_to_f32(orc.mha_bf16(_bits(Q), _bits(K), _bits(V), mask, 0.1))
     assert np.isnan(out[0, 0, 2]).all() and not np.isnan(out[0, 0, [0, 1, 3]]).any()
+
+
+def test_mha_f64_is_the_torch_composition_and_its_rounded_form_is_the_oracle(orc):
+    """gco_mha_f64 without rounding equals the float64 torch composition to 1e-12; with the softmax weights rounded
+    at the reference's point it reproduces gco_mha_bf16 once its result is rounded to bf16 (the f32 sums of the
+    oracle differ from f64 by far less than a bf16 step: a handful of ties may fall the other way)."""
+    Q, K, V = _inputs(1, 2, 96, 80, 128, seed=11)
+    scale = 1 / np.sqrt(128)
+    for mask in (None, torch.triu(torch.full((96, 80), float("-inf")), diagonal=1), torch.randn(96, 80)):
+        m = None if mask is None else mask.numpy()
+        exact = orc.mha_f64(_bits(Q), _bits(K), _bits(V), m, scale, False)
+        assert np.abs(exact - _torch_ref(Q, K, V, mask, scale)).max() < 1e-12
+        rounded = orc.mha_f64(_bits(Q), _bits(K), _bits(V), m, scale, True)
+        got = orc.mha_bf16(_bits(Q), _bits(K), _bits(V), m, scale)
+        want = orc.f32_to_bf16(rounded.astype(np.float32))
+        differ = (got != want)
+        assert differ.mean() < 5e-3
+        S = Q.double() @ K.double().transpose(-1, -2) * scale + (0 if mask is None else mask.double())
+        mag = (torch.softmax(S, -1) @ V.double().abs()).numpy()
+        # where they differ: one bf16 step of the value, plus (a weight at a rounding tie that falls the other way in
+        # f32 moves its whole row) one step of a weight times the terms' magnitude
+        gap = np.abs(orc.bf16_to_f32(got).astype(np.float64) - orc.bf16_to_f32(want))
+        assert (gap[differ] <= 2.0 ** -7 * np.abs(rounded[differ]) + 2.0 ** -8 * mag[differ]).all()
+        # the rounding of P is what separates the two f64 forms: a few 2^-9 of the terms' magnitude
+        assert (np.abs(rounded - exact) <= 2.0 ** -8 * mag).all() and np.abs(rounded - exact).max() > 0

@@ -104,3 +104,37 @@ def test_compare_p2p_rule(orc):
     assert bad == 1  # only the -inf vs +inf pair fails; 1e-6 -> absolute rule
     bad, _ = orc.compare_p2p(ref[:2], res[:2], 1e-3)
     assert bad == 1  # 0.5% relative error on the first element
+
+
+def test_compare_norm_rule(orc):
+    """test/benchgc/src/benchgc/arg/compare.py:41-57: sqrt(sum (ref-res)^2 / sum ref^2) < thr, strictly; an empty
+    tensor passes.  Hand-computed: ref (3, 4), res (3, 4.5): sqrt(0.25 / 25) = 0.1."""
+    ok, v = orc.compare_norm(np.array([3.0, 4.0], np.float32), np.array([3.0, 4.5], np.float32), 0.11)
+    assert ok and abs(v - 0.1) < 1e-7
+    ok, v = orc.compare_norm(np.array([3.0, 4.0], np.float32), np.array([3.0, 4.5], np.float32), np.float32(v))
+    assert not ok                                   # equal to the threshold: '<' fails
+    ok, v = orc.compare_norm(np.array([1.0, -2.0], np.float32), np.array([1.0, -2.0], np.float32), 1e-30)
+    assert ok and v == 0.0
+    ok, _ = orc.compare_norm(np.array([1.0, -2.0], np.float32), np.array([1.0, -2.0], np.float32), 0.0)
+    assert not ok                                   # 0 < 0 is false
+    assert orc.compare_norm(np.zeros(0, np.float32), np.zeros(0, np.float32), 0.0) == (True, 0.0)
+    ok, v = orc.compare_norm(np.array([1.0, 2.0], np.float32), np.array([1.0, np.nan], np.float32), 1.0)
+    assert not ok and np.isnan(v)
+    # a sign error or a swapped pair is a large norm, unlike under a loose per-element tolerance
+    ref = np.arange(1, 9, dtype=np.float32)
+    swapped = ref.copy()
+    swapped[[0, 1]] = swapped[[1, 0]]
+    assert abs(orc.compare_norm(ref, swapped, 1.0)[1] - np.sqrt(2.0 / 204.0)) < 1e-7
+    # per row: rows are judged one by one
+    ref2 = np.array([[3.0, 4.0], [1.0, 0.0], [0.0, 0.0]], np.float32)
+    res2 = np.array([[3.0, 4.5], [1.0, 0.0], [0.0, 0.0]], np.float32)
+    bad, l2 = orc.compare_norm_rows(ref2, res2, 0.05)
+    assert bad == 2 and abs(l2[0] - 0.1) < 1e-7 and l2[1] == 0.0 and np.isnan(l2[2])  # 0/0: not a pass
+    # against torch in float32, the arithmetic the harness itself uses
+    import torch
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal(10000).astype(np.float32)
+    b = (a + 1e-3 * rng.standard_normal(10000)).astype(np.float32)
+    ta, tb = torch.from_numpy(a), torch.from_numpy(b)
+    want = torch.sqrt(torch.square(ta - tb).sum() / torch.square(ta).sum()).item()
+    assert abs(orc.compare_norm(a, b, 1.0)[1] - want) <= 1e-6 * want
