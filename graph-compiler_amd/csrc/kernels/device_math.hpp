@@ -45,6 +45,26 @@ __device__ __forceinline__ float erf_rational(float x) {
   return copysignf(1.0f - __builtin_amdgcn_exp2f(-(q * a)), x);
 }
 
+// GELU (erf form) of a FINITE x whose result is stored as bf16: x Phi(x) with Phi(-|x|) = erfc(t) / 2 = 2^(-t q(t) - 1),
+// t = |x| / sqrt 2, q of degree 4 fitted to -log2(erfc(t)) / t on [0, 4.2]:
+//   x < 0:  x Phi(x) = x e          x >= 0:  x (1 - e) = x - x e          (e = 2^(-t q(t) - 1))
+// both as max(x, -0) - |x e|.  Relative error of the result below 2^-11.9 wherever |gelu| > 1e-5 (absolute error below
+// 1.1e-9 elsewhere): a quarter of the last place of a bf16 -- about 4 % of the results in |x| < 6 round to the
+// neighbouring bf16 value of the exactly rounded one, none differs by more.  q has positive derivative for all t >= 0, so no clamp is
+// needed: for |x| > 13 the power underflows to 0 and the result is x or -0 exactly, as with the reference's
+// saturated erf (legacy/core/src/ops/gelu.cpp:110-131 gives (erf + 1) * x * 0.5 = -0 there).  13 issue slots (the
+// exponential counts four) against 19 for erf_rational + 1, * x, * 0.5.  Not for infinite or NaN x (inf * 0).
+__device__ __forceinline__ float gelu_erf_bf16_result(float x) {
+  const float t = fabsf(x) * 0.70710678f;
+  float q = 1.4229814987629652e-03f;
+  q = fmaf(q, t, -2.0445456728339195e-02f);
+  q = fmaf(q, t, 1.293562352657318e-01f);
+  q = fmaf(q, t, 9.348235130310059e-01f);
+  q = fmaf(q, t, 1.6235692501068115f);
+  const float g = x * __builtin_amdgcn_exp2f(fmaf(-t, q, -1.0f));
+  return fmaxf(x, -0.0f) - fabsf(g);
+}
+
 // tanh for the GELU below, where it is added to 1: 1 - 2 / (e^(2|t|) + 1) with the sign of t, absolute error about
 // 2e-7 (relative accuracy near 0 is not kept: the math library's tanhf keeps it with a polynomial branch per element,
 // which costs the epilogues what the conditional in erf did).  Infinite and NaN arguments come out as +-1 and NaN.

@@ -1189,6 +1189,9 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(512, 1) void gem
 // compiler's allocator does not hold 64 accumulator tiles and three fragment sets without copies and spills);
 // set-up and epilogue are the C++ below.
 #include "gemm_w4_mainloop.inc"
+#if defined(GCMI_W4_EXPERIMENT_OPTS) && !defined(GCMI_W4_ALLOW_EXPERIMENT)
+#error "gemm_w4_mainloop.inc was generated with experiment switches (some give wrong products): regenerate it without GCMI_W4_EXPERIMENT"
+#endif
 
 // Epilogue of gemm_tile256_w4_kernel.  The main loop's assembly ends by writing the raw accumulators of column
 // tiles 0-3 (the left 64 columns of the wave's 128 x 128) to a wave-private LDS region, 128 rows of 256 bytes at a
@@ -1224,8 +1227,15 @@ __device__ __forceinline__ void w4_epilogue_row(const GemmParams &p, const acc4_
       return;
     }
 #pragma unroll
-    for (int e = 0; e < 4; e++)
-      x[e] = act_const<ACT>(fmaf((float)ci[e], scale4[e], bias4[e])); // an absent bias is -0.0: the product itself
+    for (int e = 0; e < 4; e++) {
+      const float v = fmaf((float)ci[e], scale4[e], bias4[e]); // an absent bias is -0.0: the product itself
+#ifndef GCMI_GELU_BF16_PRECISE // (measurement builds define it to time the f32-grade erf in this place)
+      if constexpr (OUT == DT_BF16 && NAN_FREE && ACT == ACT_GELU_ERF)
+        x[e] = gelu_erf_bf16_result(v); // v is finite here and the result is rounded to bf16 below
+      else
+#endif
+        x[e] = act_const<ACT>(v);
+    }
     if constexpr (OUT == DT_F32) {
       *reinterpret_cast<f32x4_t *>(Cb + (m * p.ldc + n) * 4) = f32x4_t{x[0], x[1], x[2], x[3]};
       return;

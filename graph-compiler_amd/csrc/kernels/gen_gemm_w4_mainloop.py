@@ -36,9 +36,17 @@ After the last stage the accumulators of column tiles 0-3 go to LDS for the epil
 Measured on MI355X, bf16 4096^3 (clock counters in the kernel): the loop issues MFMAs 93-94 % of its cycles; what
 is left of the time is the clock the board settles at under this power draw (1.6-1.7 GHz; 2.3 GHz with MFMAs only).
 
-Experiments (environment variable GCMI_W4_OPTS, comma separated):
+8-bit operands with u8 activations: the A fragments of block s+1 are flipped to s8 (v_xor with 0x80808080) during
+stage s, one register per MFMA from the 24th MFMA on.  The A tiles are read first, and LDS returns data in order, so
+each tile's four flips sit behind a partial wait (s_waitcnt lgkmcnt(n), n = the reads issued after that tile's) that
+has long been satisfied; a full wait in front of the flips (all 24 reads, the last of them just issued) stalled every
+stage: 12 % more cycles than a loop without flips, now 4 %.
+
+Experiments (measurement builds only: honoured when GCMI_W4_EXPERIMENT=1 is set as well, and then the output carries
+a macro that the library's sources refuse; environment variable GCMI_W4_OPTS, comma separated):
   nodma nobar nolds noxor   leave out the DMA requests / barriers / fragment reads / byte flips (wrong products)
-  dmaburst rdburst xor1     other placements of the requests, the reads and the flips (correct products)
+  dmaburst rdburst          other placements of the requests and the reads (correct products)
+  xorlate xor1 xor0=N       the flips behind a full wait over the last 16 MFMAs / the last 32; first flip at MFMA N
 """
 import os
 import sys
@@ -48,7 +56,7 @@ DUMP_PITCH = 272  # W4_DUMP_PITCH of gemm_tile256.hpp
 A_BYTES = 16384
 AF = [32, 64]
 BF = [96, 128]
-OPTS = set(filter(None, os.environ.get("GCMI_W4_OPTS", "").split(",")))
+OPTS = set(filter(None, os.environ.get("GCMI_W4_OPTS", "").split(","))) if os.environ.get("GCMI_W4_EXPERIMENT") == "1" else set()
 
 
 def gen(es, tb):
@@ -87,6 +95,13 @@ def gen(es, tb):
         """the fragment reads of one k-block in the order its MFMAs want them"""
         if "nolds" in OPTS:
             return []
+        if es == 1:  # the eight A tiles first: they are the ones the byte flips wait for
+            rd = []
+            for it in range(8):
+                rd += read_a(slot, it, par)
+            for jt in range(8):
+                rd += read_b(slot, jt, par)
+            return rd
         rd = read_b(slot, 0, par)
         for it in range(8):
             rd += read_a(slot, it, par)
@@ -127,7 +142,20 @@ def gen(es, tb):
                 extras[pos + k * rstep].append(ins)
             if es == 1 and "noxor" not in OPTS:
                 # u8 activations: flip the A tiles of the next block once they are here, each long before its first use
-                if "xor1" in OPTS:  # one register per MFMA over the second half of the stage
+                if "xorlate" not in OPTS and "xor1" not in OPTS:
+                    # LDS returns data in order: tile `it` has arrived once at most the reads issued
+                    # after it are outstanding.  Flip tile by tile, four registers behind one partial wait each,
+                    # one register per MFMA, starting XOR0 MFMAs into the stage.
+                    xor0 = int(next((o[5:] for o in OPTS if o.startswith('xor0=')), 24))
+                    x = xor_tiles(par ^ 1)
+                    for it in range(8):
+                        at = xor0 + 4 * it
+                        issued = sum(1 for k in range(len(rd)) if pos + k * rstep <= at)  # reads issued up to here
+                        dmas = min(8, at // step + 1) if fill else 0  # requests issued up to here, should they count
+                        extras[at].append("s_waitcnt lgkmcnt(%d)" % max(0, min(15, issued - (it + 1) - dmas)))
+                        for r in range(4):
+                            extras[at + r].append(x[4 * it + r])
+                elif "xor1" in OPTS:  # one register per MFMA over the second half of the stage
                     extras[31].append("s_waitcnt lgkmcnt(%d)" % (len(rd) - 9 if "rdburst" in OPTS else 0))
                     for k, ins in enumerate(xor_tiles(par ^ 1)):
                         extras[32 + k].append(ins)
@@ -189,6 +217,8 @@ def gen(es, tb):
     return out
 
 
+
+
 def dump(half):
     """Accumulators of column tiles 4*half .. 4*half+3 to the wave's LDS region as a 128 x 64 row-major block: tile
     (jt, it) holds rows 16*it.. and columns 16*(jt%4)..; v26 = the lane's address for tile (0, 0)."""
@@ -205,6 +235,8 @@ def main():
     path = sys.argv[1]
     with open(path, "w") as f:
         f.write("// generated by gen_gemm_w4_mainloop.py -- do not edit\n")
+        if OPTS:  # a measurement build: the library's sources refuse this text
+            f.write('#define GCMI_W4_EXPERIMENT_OPTS "%s"\n' % ",".join(sorted(OPTS)))
         for name, es, tb in (("BF16", 2, False), ("BF16_TB", 2, True), ("I8", 1, False), ("I8_TB", 1, True)):
             lines = gen(es, tb)
             f.write("#define GCMI_W4_ASM_%s \\\n" % name)

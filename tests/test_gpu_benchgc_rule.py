@@ -104,11 +104,14 @@ def test_config3_strict_failures_are_gelu_tail_or_cancellations(gc, orc, wl, dev
     """int8 MLP layer at full size (4096 x 4096 x 11008, dequantise + bias + GELU to bf16): 48 rows against the
     oracle under the strict rule at 1e-2, and under the harness's norm rule per row.  The accumulators are exact
     (tests/test_gpu_gemm.py), so whatever differs comes from the epilogue: the GPU forms acc * scale + bias as one
-    fused multiply-add and evaluates erf by its own polynomial (absolute error 1.5e-7).  A strict failure must
-    therefore be one of: (a) a pre-activation value x in the negative GELU tail, where gelu(x) = x/2 * (erf + 1) is a
-    difference of nearly equal numbers in the reference's own f32 arithmetic as well -- (erf + 1) < 2e-5 from
-    x < -4.2 on, so 1.5e-7 is more than 1e-2 of it, and past x = -4.7 |gelu| < 1e-5 falls under the rule's absolute
-    branch and passes --, or (b) a cancellation of acc * scale against the bias."""
+    fused multiply-add and evaluates GELU for a bf16 result as x * Phi(x) with Phi(-|x|) = 2^(-t q(t) - 1) (relative
+    error below 2^-11.9 of the value, tail included).  A strict failure could only be (a) a pre-activation value x in
+    the negative GELU tail, where the REFERENCE's gelu(x) = x/2 * (erf + 1) is a difference of nearly equal f32 numbers
+    -- (erf + 1) < 2e-5 from x < -4.2 on; past x = -4.7 |gelu| < 1e-5 falls under the rule's absolute branch --, or
+    (b) a cancellation of acc * scale against the bias.  (With the f32-grade erf this kernel used before, whose error
+    is absolute, 6 of these 495,360 elements failed, all in that tail; with the relative form: none.)  Where the
+    reference's erf has saturated (x < -5.5) it returns -0 and the GPU the tiny negative value GELU really has there
+    (-5.9e-9 at x = -6, underflowing to -0 below x = -13): different bits, both zero to any tolerance."""
     A, W, scale, bias = wl.int8_mlp_layer()
     Ad, Wd = A.to(dev), W.to(dev)
     cs = gc.colsum_s8(Wd)
@@ -129,9 +132,10 @@ def test_config3_strict_failures_are_gelu_tail_or_cancellations(gc, orc, wl, dev
                                                                    int((bad & cancel & ~tail).sum()), int(tail.sum())))
     assert (tail | cancel)[bad].all(), x[bad & ~(tail | cancel)][:8]
     assert n <= 1e-3 * bad.size
-    # elsewhere the two agree to a bf16 step, and nearly always bit for bit
-    differ = ref != res
+    # elsewhere the two agree to a bf16 step, and nearly always bit for bit (leaving out the saturated tail, see above)
+    differ = (ref != res) & ((np.abs(ref) > 1e-7) | (np.abs(res) > 1e-7))
     assert differ.mean() < 1e-3
+    assert (np.abs(ref - res)[differ] <= 2.0 ** -7 * np.abs(ref)[differ]).all()
     # the harness's norm rule (test/benchgc/src/benchgc/arg/compare.py:41-57), per sampled row
     nbad, l2 = orc.compare_norm_rows(ref, res, 1e-4)
     print("config 3: per-row norm of the difference: max %.2e, median %.2e" % (float(l2.max()), float(np.median(l2))))

@@ -276,6 +276,47 @@ def test_gelu_erf_epilogue_absolute_accuracy(gc, dev):
     assert (out[xd < -5.84] == 0).all() and (out[xd > 5.84] == xd[xd > 5.84]).all()
 
 
+def test_gelu_of_the_int8_layer_with_bf16_result(gc, orc, dev):
+    """The 8-bit tile kernels evaluate GELU for a bf16 result with a shorter polynomial (relative error below 2^-11.9
+    of the value, a quarter of a bf16's last place; the f32-result path keeps the 1.5e-7 form).  A one-hot weight and
+    per-column scales and biases put x = (a - 128) * scale + bias on a dense grid over [-9, 9]: every result against
+    the float64 GELU -- within half a bf16 step of it plus that 2^-11.9 --, against the oracle at the stated 1e-2, and
+    the share of results that are not the exactly rounded value."""
+    M = N = K = 256
+    A = torch.zeros(M, K, dtype=torch.uint8)
+    A[:, 0] = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    W = torch.zeros(K, N, dtype=torch.int8)
+    W[0, :] = 1
+    scale = ((torch.arange(N, dtype=torch.float32) % 64 + 1) / 64 * 0.0625)          # up to 8 / 128 per count
+    bias = ((torch.arange(N, dtype=torch.float32) // 64) - 1.5) * 0.37 + torch.arange(N, dtype=torch.float32) * 1e-3
+    Wd = W.to(dev)
+    out = gc.gemm_int8(A.to(dev), Wd, gc.colsum_s8(Wd), 128, scale.to(dev), bias.to(dev), "gelu_erf", gc.BF16)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy().astype(np.float64)
+    # the pre-activation value as the kernel forms it: one fused multiply-add, rounded to f32 once
+    x = torch.addcmul(bias[None, :].double(), (A[:, :1].to(torch.float64) - 128), scale[None, :].double()).float().double()
+    exact = (0.5 * x * (1 + torch.special.erf(x * 0.7071067811865476))).numpy()
+    assert x.min() < -8 and x.max() > 8
+    bits = np.abs(exact).astype(np.float32).view(np.uint32)
+    step = (((bits >> 23) << 23).view(np.float32)).astype(np.float64) * 2.0 ** -7      # a bf16 step at |exact|
+    assert (np.abs(got - exact) <= 0.5 * step + 2.0 ** -11.9 * np.abs(exact) + 1.2e-9).all()
+    rounded = orc.bf16_to_f32(orc.f32_to_bf16(exact.astype(np.float32))).astype(np.float64)
+    share = float((got != rounded).mean())
+    assert share < 0.06, share
+    _, y = orc.int8_layer(A.numpy(), W.numpy(), scale.numpy(), bias.numpy(), 128, "gelu_erf")
+    assert_close(orc.bf16_to_f32(y), got, 1e-2, "int8 layer, GELU grid")
+    # large |x|: x itself, or -0, as the reference's saturated erf gives
+    big = torch.tensor([[255, 0]], dtype=torch.uint8).repeat(256, 128)
+    Wb = torch.zeros(K, N, dtype=torch.int8)
+    Wb[0, :] = 127
+    Wb[1, :] = -127
+    Wbd = Wb.to(dev)
+    o2 = gc.gemm_int8(big.to(dev), Wbd, gc.colsum_s8(Wbd), 128, torch.full((N,), 0.01).to(dev), None, "gelu_erf", gc.BF16)
+    torch.cuda.synchronize()
+    _, y2 = orc.int8_layer(big.numpy(), Wb.numpy(), np.full(N, 0.01, np.float32), None, 128, "gelu_erf")
+    assert (o2.view(torch.int16).cpu().numpy().view(np.uint16) == np.asarray(y2).reshape(M, N)).all()
+
+
 @pytest.mark.parametrize("M,N", [(300, 264), (520, 256), (512, 520), (1000, 1000)])
 @pytest.mark.parametrize("variant", ["plain", "bias_gelu_f32", "bias_relu_residual", "nt"])
 @pytest.mark.parametrize("tile", [256, 128])
