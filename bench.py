@@ -503,6 +503,19 @@ def main():
         vend["torch_mm_bf16_4096"] = {"ms_per_step": round(t["ms_per_step"], 5),
                                       "value": round(flops / t["ms_per_step"] / 1e9, 1), "unit": "TFLOP/s"}
         del sets
+        # the vendor library's s8 x s8 -> s32 GEMM at the int8 layer's shape: raw accumulators only (no zero point, no
+        # dequantise / bias / GELU, and 4 bytes per result written instead of 2) -- a same-box yardstick for the main
+        # loop, not the same work
+        try:
+            Ai = torch.randint(-128, 128, (4096, 4096), dtype=torch.int8, device=dev)
+            Wi = torch.randint(-127, 128, (4096, 11008), dtype=torch.int8, device=dev)
+            t = time_launches(torch, lambda i: torch._int_mm(Ai, Wi), 1, max(10, K // 2), 5)
+            vend["torch_int_mm_s8s8s32_4096x11008x4096"] = {
+                "ms_per_step": round(t["ms_per_step"], 5), "value": round(2.0 * 4096 * 4096 * 11008 / t["ms_per_step"] / 1e9, 1),
+                "unit": "TOP/s"}
+            del Ai, Wi
+        except Exception as e:
+            vend["torch_int_mm_s8s8s32_4096x11008x4096"] = {"error": str(e)[:120]}
         Q, Kk, V, mask, scale = wl.bf16_mha(seed=0)
         Qv, Kv, Vv = Q.to(dev), Kk.to(dev), V.to(dev)
         mops = 4.0 * 4 * 32 * 2048 * 2048 * 128
@@ -753,7 +766,29 @@ def main():
         "kernel_ms": {k: round(v, 5) for k, v in res.items()} if res else None,
         "others": others,
     }
-    print(json.dumps(line), flush=True)
+    # The whole record (workload descriptions, per-launch event timings of every entry) goes to stderr; the line on
+    # stdout is the same record without the prose and the per-launch sub-dicts, so that it stays a few KB.
+    log("full record: " + json.dumps(line))
+
+    def compact(v, depth=0):
+        if isinstance(v, dict):
+            return {k: compact(x, depth + 1) for k, x in v.items()
+                    if not (depth >= 1 and k in ("workload", "kernel_ms", "note", "sample", "traffic_source"))}
+        return v
+
+    short = dict(line)
+    short["others"] = compact(others, 1)
+    print(json.dumps(short, separators=(",", ":")), flush=True)
+    # the three other named configurations once more, last on stderr
+    for key, name in (("int8_mlp_layer", "C3 int8 layer"), ("bf16_mlp_chain", "C4 bf16 mlp chain"),
+                      ("bf16_mha", "C5 attention, every key block")):
+        e = others.get(key)
+        if e and "roofline" in e:
+            log("%s: %.4f ms, %.1f %s, frac %.4f of the dense MFMA peak" %
+                (name, e["ms_per_step"], e["value"], e["unit"].split(" ")[0], e["roofline"]["frac"]))
+    if res:
+        log("C2 bf16 gemm 4096^3: %.4f ms, %.1f TFLOP/s, frac %.4f of the dense MFMA peak" %
+            (res["ms_per_step"], flops / res["ms_per_step"] / 1e9, flops / res["ms_per_step"] / 1e9 / PEAK["bf16"]))
 
 
 if __name__ == "__main__":

@@ -69,29 +69,54 @@ struct LibraryWorkspace {
   hipEvent_t done = nullptr;
   hipStream_t last = nullptr;
   bool used = false;
+  // Blocks that were outgrown.  They are kept until the process ends: a kernel enqueued earlier (or a HIP graph
+  // captured from an earlier call through an entry point that did not refuse capture) may still name them.
+  std::vector<void *> retired;
 };
 LibraryWorkspace g_ws[64];
 
+// hipStreamPerThread is one handle value for a different stream in every thread, and the legacy null stream
+// synchronises with others by rules of its own: a comparison of handles says nothing about them.
+bool same_stream_for_sure(hipStream_t a, hipStream_t b) {
+  return a == b && a != nullptr && a != hipStreamPerThread && a != hipStreamLegacy;
+}
+
 // Takes the device's buffer (at least `bytes`) for one call on `stream`; the lock is held until release().
 int ws_acquire(size_t bytes, hipStream_t stream, LibraryWorkspace **out, void **ptr) {
+  // Under stream capture nothing here is legal (allocation, device-wide waits), and a captured graph would keep the
+  // address of a buffer that later calls share: such callers bring their own workspace.
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+    (void)hipGetLastError();
+    cap = hipStreamCaptureStatusNone;
+  }
+  if (cap != hipStreamCaptureStatusNone)
+    return fail(ST_INVALID, "this call needs scratch memory and its stream is being captured: use the entry point that takes "
+                            "a workspace (gcmi_gemm_bf16_ws / gcmi_mha_fwd_bf16_ws) or gcmi_gemm_bf16_noalloc");
+  // the buffer of the device the stream belongs to (the current device for the null and per-thread streams)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
     return fail(ST_RUNTIME, "workspace: no current device");
+  if (stream != nullptr && stream != hipStreamPerThread && stream != hipStreamLegacy) {
+    hipDevice_t sdev = 0;
+    if (hipStreamGetDevice(stream, &sdev) == hipSuccess && (int)sdev >= 0 && (int)sdev < 64)
+      dev = (int)sdev;
+    else
+      (void)hipGetLastError();
+  }
   LibraryWorkspace &w = g_ws[dev];
   w.mu.lock();
   if (w.cap < bytes) {
-    if (w.ptr) { // kernels of earlier calls may still read it
-      (void)hipDeviceSynchronize();
-      (void)hipFree(w.ptr);
-      w.ptr = nullptr, w.cap = 0, w.used = false;
-    }
     const size_t want = bytes < ((size_t)8 << 20) ? ((size_t)8 << 20) : bytes;
-    if (hipMalloc(&w.ptr, want) != hipSuccess) {
-      w.ptr = nullptr;
+    void *fresh = nullptr;
+    if (hipMalloc(&fresh, want) != hipSuccess) {
       w.mu.unlock();
       return fail(1, "workspace: hipMalloc of %zu bytes failed", want);
     }
-    w.cap = want;
+    if (w.ptr)
+      w.retired.push_back(w.ptr); // never freed: see above
+    w.ptr = fresh, w.cap = want;
+    // the new block has no earlier user, but the order between callers is kept as it was (w.used, w.last)
   }
   if (!w.done && hipEventCreateWithFlags(&w.done, hipEventDisableTiming) != hipSuccess) {
     w.done = nullptr;
@@ -101,7 +126,7 @@ int ws_acquire(size_t bytes, hipStream_t stream, LibraryWorkspace **out, void **
   // A caller on another stream than the last user's waits for everything that stream has been given so far (the
   // marker is recorded now, behind the last user's kernels: nothing is recorded per call, so a single-stream caller
   // pays for no event).  A stream that no longer exists: wait for the device.
-  if (w.used && w.last != stream) {
+  if (w.used && !same_stream_for_sure(w.last, stream)) {
     if (hipEventRecord(w.done, w.last) != hipSuccess || hipStreamWaitEvent(stream, w.done, 0) != hipSuccess) {
       (void)hipGetLastError();
       (void)hipDeviceSynchronize();

@@ -135,7 +135,9 @@ def test_config3_strict_failures_are_gelu_tail_or_cancellations(gc, orc, wl, dev
     # elsewhere the two agree to a bf16 step, and nearly always bit for bit (leaving out the saturated tail, see above)
     differ = (ref != res) & ((np.abs(ref) > 1e-7) | (np.abs(res) > 1e-7))
     assert differ.mean() < 1e-3
-    assert (np.abs(ref - res)[differ] <= 2.0 ** -7 * np.abs(ref)[differ]).all()
+    # one bf16 step where GELU is not in its far tail; there (|gelu| < 1e-4, where the reference's own f32 (erf + 1)
+    # has few correct digits left) an absolute 1e-6
+    assert (np.abs(ref - res)[differ] <= np.where(np.abs(ref)[differ] > 1e-4, 2.0 ** -7 * np.abs(ref)[differ], 1e-6)).all()
     # the harness's norm rule (test/benchgc/src/benchgc/arg/compare.py:41-57), per sampled row
     nbad, l2 = orc.compare_norm_rows(ref, res, 1e-4)
     print("config 3: per-row norm of the difference: max %.2e, median %.2e" % (float(l2.max()), float(np.median(l2))))

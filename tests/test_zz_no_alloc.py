@@ -64,3 +64,51 @@ def test_noalloc_rejects_what_does_not_fit_the_static_scratch(gc, dev):
     assert st == 2 and "static" in msg and "bytes of scratch" in msg, (st, msg)
     torch.cuda.synchronize()
     assert gc.gemm_bf16(A, B).abs().max().item() == 0  # the allocating entry point takes the same call
+
+
+def test_noalloc_allocates_nothing_and_can_be_captured(gc, dev):
+    """The property the entry point is named for: device memory in use does not change over K-sliced calls (the
+    allocating entry point would grow the library's workspace on a fresh shape), and a call recorded into a HIP graph
+    replays to the eager result (several replays with eager work in between: the graph names the static array, whose
+    address never changes).  The allocating entry point refuses a capturing stream with a message that names the
+    alternatives."""
+    M, N, K = 128, 8192, 4096     # K-sliced, 16 MiB of partial sums: beyond the library workspace's first size
+    assert gc.lib().gcmi_gemm_bf16_workspace_bytes(M, N, K, 0) > 8 << 20
+    torch.manual_seed(3)
+    A = (torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev)
+    B = (torch.randn(K, N) * 0.05).to(torch.bfloat16).to(dev)
+    got = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        assert _noalloc(gc, A, B, False, None, None, got) == 0, gc.lib().gcmi_last_error().decode()
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    eager = got.clone()
+    side = torch.cuda.Stream()
+    out_g = torch.zeros_like(got)
+    with torch.cuda.stream(side):
+        assert _noalloc(gc, A, B, False, None, None, out_g) == 0  # once outside the graph on this stream
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        g.capture_begin()
+        rc = _noalloc(gc, A, B, False, None, None, out_g)
+        # the allocating entry point on the capturing stream: refused, nothing recorded
+        s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc_alloc = gc.lib().gcmi_gemm_bf16(A.data_ptr(), B.data_ptr(), out_g.data_ptr(), M, N, K, K, N, N, None, gc.BF16, 0,
+                                           gc.BF16, s)
+        msg = gc.lib().gcmi_last_error().decode()
+        g.capture_end()
+    side.synchronize()
+    assert rc == 0
+    assert rc_alloc == 2 and "captured" in msg and "gcmi_gemm_bf16_ws" in msg, (rc_alloc, msg)
+    for rep in range(3):
+        out_g.zero_()
+        # eager work of the program's own between the replays, through the same static scratch
+        small = torch.empty(32, 2048, dtype=torch.bfloat16, device=dev)
+        assert _noalloc(gc, A[:32, :1024].contiguous(), B[:1024, :2048].contiguous(), False, None, None, small) == 0
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g.view(torch.int16), eager.view(torch.int16)), rep
