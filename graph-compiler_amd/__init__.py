@@ -21,7 +21,7 @@ ACT = {None: 0, "none": 0, "relu": 1, "gelu_erf": 2, "gelu_tanh": 3, "sigmoid": 
 # every symbol the public headers declare (checked by the CPU test-suite)
 EXPORTS = {
     "gc_hip_kernels.h": ["gcmi_init", "gcmi_last_error", "gcmi_gemm_bf16", "gcmi_gemm_bf16_nt", "gcmi_gemm_bf16_batched", "gcmi_gemm_bf16_residual", "gcmi_gemm_f32_batched",
-                         "gcmi_gemm_bf16_ws", "gcmi_gemm_bf16_workspace_bytes", "gcmi_gemm_bf16_workspace_bytes_cfg", "gcmi_mha_fwd_bf16_ws", "gcmi_mha_fwd_workspace_bytes",
+                         "gcmi_gemm_bf16_ws", "gcmi_gemm_bf16_workspace_bytes", "gcmi_gemm_bf16_workspace_bytes_cfg", "gcmi_mha_fwd_bf16_ws", "gcmi_mha_fwd_workspace_bytes", "gcmi_mha_classify_mask",
                          "gcmi_gemm_bf16_noalloc", "gcmi_noalloc_scratch_bytes", "gcmi_gemm_int8_cfg", "gcmi_gemm_tile_config_query",
                          "gcmi_gemm_int8", "gcmi_colsum_s8",
                          "gcmi_gemm_f32", "gcmi_mha_fwd_bf16", "gcmi_mha_fwd_bf16_opt"],
@@ -71,6 +71,8 @@ def lib():
     L.gcmi_mha_fwd_workspace_bytes.argtypes = [i64, i64, i64, ci]
     L.gcmi_mha_fwd_bf16_ws.restype = ci
     L.gcmi_mha_fwd_bf16_ws.argtypes = [vp, vp, vp, vp, i64, vp, i64, i64, i64, i64, f32, ci, vp, C.c_size_t, vp]
+    L.gcmi_mha_classify_mask.restype = ci
+    L.gcmi_mha_classify_mask.argtypes = [vp, i64, i64, i64, i64, vp, C.c_size_t, vp]
     L.gcmi_gemm_bf16_noalloc.restype = ci
     L.gcmi_gemm_bf16_noalloc.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp, ci, ci, ci, vp]
     L.gcmi_noalloc_scratch_bytes.restype = C.c_size_t
@@ -277,4 +279,33 @@ def mha_fwd_bf16(Q, K, V, mask=None, scale=None, out=None, skip_masked=True):
     mld = 0 if mask is None else mask.stride(0)
     check(lib().gcmi_mha_fwd_bf16_opt(_ptr(Q), _ptr(K), _ptr(V), _ptr(mask), mld, _ptr(out), Bn * H, Sq, Sk, D,
                                       float(scale), int(bool(skip_masked)), _stream()), "gcmi_mha_fwd_bf16")
+    return out
+
+
+def mha_mask_classes(mask, Sq, Sk, D):
+    """The tile classes of a mask that stays the same between calls: one classification pass into a workspace the
+    caller keeps (None: this shape uses no classes).  Pass it to mha_fwd_bf16_classified."""
+    import torch
+    n = lib().gcmi_mha_fwd_workspace_bytes(Sq, Sk, D, 1)
+    if n == 0:
+        return None
+    ws = torch.empty(n, dtype=torch.uint8, device=mask.device)
+    check(lib().gcmi_mha_classify_mask(_ptr(mask), mask.stride(0), Sq, Sk, D, _ptr(ws), n, _stream()), "gcmi_mha_classify_mask")
+    return ws
+
+
+def mha_fwd_bf16_classified(Q, K, V, mask, classes, scale=None, out=None, skip_masked=True):
+    """mha_fwd_bf16 for a mask whose classes were prepared by mha_mask_classes (no classification pass per call)."""
+    import torch
+    Bn, H, Sq, D = Q.shape
+    Sk = K.shape[2]
+    assert Q.is_contiguous() and K.is_contiguous() and V.is_contiguous()
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    if out is None:
+        out = torch.empty_like(Q)
+    flags = (1 if skip_masked else 0) | (2 if classes is not None else 0)
+    check(lib().gcmi_mha_fwd_bf16_ws(_ptr(Q), _ptr(K), _ptr(V), _ptr(mask), mask.stride(0), _ptr(out), Bn * H, Sq, Sk, D,
+                                     float(scale), flags, _ptr(classes), 0 if classes is None else classes.numel(), _stream()),
+          "gcmi_mha_fwd_bf16_ws")
     return out

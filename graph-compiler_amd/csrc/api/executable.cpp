@@ -244,7 +244,7 @@ void Executable::plan_workspaces() {
     size_t bytes = 0;
     if (s.kind == Step::GemmBf16 && s.batch <= 1)
       bytes = gcmi_gemm_bf16_workspace_bytes_cfg(s.M, s.N, s.K, s.tb ? 1 : 0, s.mm_cfg.size() == 9 ? s.mm_cfg.data() : nullptr);
-    else if (s.kind == Step::Mha && s.mask >= 0)
+    else if (s.kind == Step::Mha && s.mask >= 0 && s.ws < 0)
       bytes = gcmi_mha_fwd_workspace_bytes(s.Sq, s.Sk, s.D, 1);
     if (bytes)
       s.ws = new_slot(bytes);
@@ -478,7 +478,8 @@ void Executable::plan() {
             if (mt.dt != DT::f32) { // the kernel adds an f32 mask
               int f = new_slot((size_t)mt.numel() * 4);
               Step cp;
-              cp.kind = Step::Elt, cp.note = "mask -> f32", cp.op = gcmi::ELT_COPY, cp.a = mask_slot, cp.out = f;
+              cp.kind = Step::Elt, cp.note = mt.constant ? "mask -> f32, once: the mask is constant" : "mask -> f32";
+              cp.once = mt.constant, cp.op = gcmi::ELT_COPY, cp.a = mask_slot, cp.out = f;
               cp.a_dt = dt_dnnl(mt.dt), cp.out_dt = GCMI_F32;
               cp.dims = {mt.numel()}, cp.sa = {1};
               v.push_back(cp);
@@ -491,6 +492,19 @@ void Executable::plan() {
           s.a = slot_for(mm.in[0]), s.b = slot_for(mm.in[1]), s.c = slot_for(pv.in[1]), s.out = slot_for(pv.out[0]);
           s.mask = mask_slot, s.mask_ld = mask_ld;
           s.BH = prod(q.shape, 0, r - 2), s.Sq = Sq, s.Sk = Sk, s.D = q.shape[r - 1];
+          if (mask_t >= 0 && T((size_t)mask_t).constant) {
+            // A constant mask is classified once per executable (its tiles: all 0, all -inf, general), like the column
+            // sums of constant weights: the reference's constant-tensor cache (src/dnnl/JsonParser.cpp:295-299).
+            const size_t bytes = gcmi_mha_fwd_workspace_bytes(Sq, Sk, s.D, 1);
+            if (bytes) {
+              Step cl;
+              cl.kind = Step::MhaClassify, cl.note = "mask tile classes, once: the mask is constant", cl.once = true;
+              cl.a = mask_slot, cl.mask_ld = mask_ld, cl.Sq = Sq, cl.Sk = Sk, cl.D = s.D;
+              cl.out = new_slot(bytes);
+              v.push_back(cl);
+              s.ws = cl.out, s.classes_valid = true;
+            }
+          }
           s.scale = 1.0f;
           if (scale_t >= 0 && T((size_t)scale_t).has_splat) {
             const float x = (float)T((size_t)scale_t).splat;
@@ -1518,10 +1532,16 @@ void Executable::launch(const Step &s) {
       scale = s.scale_div ? 1.0f / v : v;
     }
     gc_check(gcmi_mha_fwd_bf16_ws(P(s.a), P(s.b), P(s.c), (const float *)P(s.mask), s.mask_ld, P(s.out), s.BH, s.Sq, s.Sk,
-                                  s.D, scale, 1, P(s.ws), s.ws >= 0 ? slots_[(size_t)s.ws].bytes : 0, stream_),
+                                  s.D, scale, GCMI_MHA_SKIP_MASKED | (s.classes_valid ? GCMI_MHA_CLASSES_VALID : 0), P(s.ws),
+                                  s.ws >= 0 ? slots_[(size_t)s.ws].bytes : 0, stream_),
              "attention");
     break;
   }
+  case Step::MhaClassify:
+    gc_check(gcmi_mha_classify_mask((const float *)P(s.a), s.mask_ld, s.Sq, s.Sk, s.D, P(s.out), slots_[(size_t)s.out].bytes,
+                                    stream_),
+             "mask tile classes");
+    break;
   case Step::Elt: {
     gcmi::EltParams p{};
     p.a = P(s.a), p.b = P(s.b), p.out = P(s.out);
@@ -1734,7 +1754,8 @@ void Executable::run(dnnl_graph_compiler_tensor *inputs, dnnl_graph_compiler_ten
 }
 
 std::string Executable::describe() const {
-  static const char *names[] = {"gemm_f32", "gemm_bf16", "gemm_int8", "colsum", "attention", "eltwise", "reduce", "softmax"};
+  static const char *names[] = {"gemm_f32", "gemm_bf16", "gemm_int8", "colsum", "attention", "eltwise", "reduce", "softmax",
+                                "fused", "attention mask"};
   std::ostringstream os;
   static const char *kernels[] = {"bounds-checked tile", "whole tiles, 8 waves", "whole tiles, 4 waves (one per SIMD)",
                                   "K slices + second pass", "weight streaming (+ second pass)",

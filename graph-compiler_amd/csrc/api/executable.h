@@ -29,7 +29,7 @@
 namespace gcapi {
 
 struct Step {
-  enum Kind { GemmF32, GemmBf16, GemmInt8, ColSum, Mha, Elt, Reduce, Softmax, Fused } kind;
+  enum Kind { GemmF32, GemmBf16, GemmInt8, ColSum, Mha, Elt, Reduce, Softmax, Fused, MhaClassify } kind;
   std::string note; // what was fused, for introspection
   bool once = false; // depends on constant tensors only: runs in the first execute, its result is kept
   // operands are arena slot indices (-1 = none)
@@ -49,6 +49,7 @@ struct Step {
   float scale = 1.0f;
   int scale_slot = -1;   // 1-element tensor holding the scale (or its reciprocal)
   bool scale_div = false;
+  bool classes_valid = false; // `ws` holds the mask's tile classes, prepared by a once-only MhaClassify step
   // generic kernels: parameter blocks are filled at plan time with slot ids
   // resolved to pointers at execute time
   std::vector<int64_t> dims, sa, sb;

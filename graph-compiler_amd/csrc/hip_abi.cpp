@@ -541,6 +541,27 @@ extern "C" int gcmi_mha_fwd_bf16_ws(const void *Q, const void *K, const void *V,
                  workspace_bytes);
 }
 
+extern "C" int gcmi_mha_classify_mask(const float *mask, int64_t mask_ld, int64_t Sq, int64_t Sk, int64_t D, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+  if (!mask || Sq <= 0 || Sk <= 0 || Sq > 0x7fffffff || Sk > 0x7fffffff)
+    return fail(ST_INVALID, "mha_classify_mask: bad arguments");
+  if (mask_ld < Sk)
+    return fail(ST_INVALID, "mha_classify_mask: mask_ld < Sk");
+  MhaParams p{};
+  // aligned stand-ins for the operands the pass does not touch
+  p.Q = p.K = p.V = (const void *)(uintptr_t)256, p.O = (void *)(uintptr_t)256;
+  p.mask = mask, p.mask_ld = mask_ld, p.BH = 1, p.Sq = (int)Sq, p.Sk = (int)Sk, p.D = (int)D, p.scale = 1.0f;
+  p.classes_mode = 2;
+  const int64_t want = gcmi_launch_mha_workspace(&p);
+  if (want <= 0)
+    return ST_OK; // this shape has no mask classes: nothing to prepare
+  if (!workspace || (int64_t)workspace_bytes < want)
+    return fail(ST_INVALID, "mha_classify_mask: the workspace holds %zu bytes, %lld are needed (gcmi_mha_fwd_workspace_bytes)",
+                workspace_bytes, (long long)want);
+  p.tile_class = (uint8_t *)workspace, p.tile_class_cap = (int64_t)workspace_bytes;
+  return launched(gcmi_launch_mha_fwd(&p, (hipStream_t)stream), "mha_classify_mask");
+}
+
 extern "C" size_t gcmi_mha_fwd_workspace_bytes(int64_t Sq, int64_t Sk, int64_t D, int has_mask) {
   if (!has_mask || Sq <= 0 || Sk <= 0 || Sq > 0x7fffffff || Sk > 0x7fffffff)
     return 0;
@@ -572,7 +593,11 @@ int mha_any(const void *Q, const void *K, const void *V, const float *mask, int6
   MhaParams p{};
   p.Q = Q, p.K = K, p.V = V, p.O = O, p.mask = mask, p.mask_ld = mask_ld;
   p.BH = (int)BH, p.Sq = (int)Sq, p.Sk = (int)Sk, p.D = (int)D, p.scale = scale;
-  p.skip_masked = skip_masked ? 1 : 0;
+  p.skip_masked = (skip_masked & 1) ? 1 : 0;
+  // bit 1 (GCMI_MHA_CLASSES_VALID): the caller's workspace holds this mask's classes already
+  p.classes_mode = (skip_masked & 2) ? 1 : 0;
+  if ((skip_masked & 2) && (ws_from != Ws::Caller || !ws))
+    return fail(ST_INVALID, "mha_fwd: GCMI_MHA_CLASSES_VALID needs the workspace that gcmi_mha_classify_mask filled");
   // the classes of the mask's tiles (constant 0, constant -inf, general) go through a small workspace
   const int64_t want = gcmi_launch_mha_workspace(&p);
   LibraryWorkspace *lw = nullptr;

@@ -92,6 +92,9 @@ struct MhaParams {
   uint8_t *tile_class;
   int64_t tile_class_cap;
   int32_t skip_masked; // 1: tiles whose mask is all -inf are not computed (the result is the same)
+  // 1: tile_class already holds the classes of this mask (an earlier call's classification pass for the same mask,
+  // shape and buffer): the pass is not launched again.  2: launch the pass only, no attention kernel.
+  int32_t classes_mode;
 };
 
 } // namespace gcmi

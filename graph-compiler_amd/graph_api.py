@@ -263,9 +263,10 @@ def mlp_chain_json(M, K, H):
          "outputs": [_t(6, "bf16", [M, K])]}], [0, 1, 4, 5], [6])
 
 
-def mha_json(B, H, Sq, Sk, D, with_mask=True, scale_op="Multiply"):
+def mha_json(B, H, Sq, Sk, D, with_mask=True, scale_op="Multiply", mask_constant=False):
     """MatMul(Q,K^T) -> Multiply(scale) -> Add(mask) -> SoftMax -> MatMul(P,V).
-    ids: 0 Q, 1 K, 2 scale f32[1], 3 mask f32[Sq,Sk], 4 V -> 9."""
+    ids: 0 Q, 1 K, 2 scale f32[1], 3 mask f32[Sq,Sk], 4 V -> 9.  mask_constant: the mask is a constant of the
+    partition (property_type "constant"): its contents are taken from the first execute."""
     s = [B, H, Sq, Sk]
     ops = [{"kind": "MatMul", "attrs": {"transpose_b": {"type": "bool", "value": 1}},
             "inputs": [_t(0, "bf16", [B, H, Sq, D]), _t(1, "bf16", [B, H, Sk, D])], "outputs": [_t(5, "f32", s)]},
@@ -273,7 +274,8 @@ def mha_json(B, H, Sq, Sk, D, with_mask=True, scale_op="Multiply"):
     cur = 6
     ins = [0, 1, 2]
     if with_mask:
-        ops.append({"kind": "Add", "inputs": [_t(6, "f32", s), _t(3, "f32", [Sq, Sk])], "outputs": [_t(7, "f32", s)]})
+        mk = {"property_type": "constant"} if mask_constant else {}
+        ops.append({"kind": "Add", "inputs": [_t(6, "f32", s), _t(3, "f32", [Sq, Sk], **mk)], "outputs": [_t(7, "f32", s)]})
         cur = 7
         ins.append(3)
     ops.append({"kind": "SoftMax", "attrs": {"axis": {"type": "s64", "value": -1}},

@@ -273,8 +273,20 @@ int gcmi_mha_fwd_bf16_opt(const void *Q, const void *K, const void *V, const flo
  * keys) mask tile, gcmi_mha_fwd_workspace_bytes in all (0: the shape has no
  * use for one).  With NULL or too small a workspace every tile is read from
  * the mask and nothing is skipped; the result is the same.
+ *
+ * A mask that does not change between calls (a constant of the partition, the
+ * counterpart of the reference's constant-tensor cache, src/dnnl/JsonParser.cpp:
+ * 295-299) need not be classified by every call: gcmi_mha_classify_mask runs the
+ * pass alone into `workspace`, and calls that pass skip_masked |
+ * GCMI_MHA_CLASSES_VALID with the same mask, mask_ld, Sq, Sk, D and workspace
+ * launch the attention kernel only.  The caller vouches that the mask's contents
+ * are still what was classified; the result is otherwise undefined.
  */
+#define GCMI_MHA_SKIP_MASKED 1
+#define GCMI_MHA_CLASSES_VALID 2
 size_t gcmi_mha_fwd_workspace_bytes(int64_t Sq, int64_t Sk, int64_t D, int has_mask);
+int gcmi_mha_classify_mask(const float *mask, int64_t mask_ld, int64_t Sq, int64_t Sk, int64_t D, void *workspace,
+                           size_t workspace_bytes, void *stream);
 int gcmi_mha_fwd_bf16_ws(const void *Q, const void *K, const void *V, const float *mask, int64_t mask_ld, void *O,
                          int64_t BH, int64_t Sq, int64_t Sk, int64_t D, float scale, int skip_masked, void *workspace,
                          size_t workspace_bytes, void *stream);

@@ -217,3 +217,14 @@ def test_slices_named_by_a_matmul_config_get_their_workspace(ga, gc, M, N, K, kt
     assert re.search(r"split_k %d, \d+ workgroups, workspace %d B \[MatmulConfig attributes applied\]" % (kthreads, ws), plan), plan
     arena = int(re.search(r"arena: (\d+) bytes", plan).group(1))
     assert arena >= ws
+
+
+def test_a_constant_attention_mask_is_classified_once(ga):
+    """The tile classes of a mask that is a constant of the partition are a once-only step with a slot of its own
+    (kept for the executable's lifetime); a variable mask is classified by every call into the step's scratch."""
+    st, plan = ga.explain(ga.mha_json(2, 4, 512, 512, 128, True, "Multiply", mask_constant=True))
+    assert st == 0 and "attention mask: mask tile classes, once: the mask is constant" in plan and "attention:" in plan, plan
+    st, plan2 = ga.explain(ga.mha_json(2, 4, 512, 512, 128, True, "Multiply"))
+    assert st == 0 and "once" not in plan2 and "attention:" in plan2, plan2
+    st, plan3 = ga.explain(ga.mha_json(1, 1, 16, 16, 128, True, "Multiply", mask_constant=True))   # too small for classes
+    assert st == 0 and "once" not in plan3, plan3

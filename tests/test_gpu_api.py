@@ -188,6 +188,41 @@ def test_mlp_chain_partition(ga, orc, wl, dev):
     assert_close(orc.bf16_to_f32(y), out.float().numpy(), 2e-2, "mlp chain partition", mag=mm)
 
 
+@pytest.mark.parametrize("D", [128, 64])
+def test_attention_with_a_constant_mask_classifies_it_once(ga, gc, wl, dev, D):
+    """A mask with property_type "constant": its tile classes are prepared in the first execute and kept.  Two
+    executes (other Q the second time) give the bits of the partition whose mask is a variable, and of the raw entry
+    points with and without prepared classes."""
+    B, H, S = 1, 4, 512
+    Q, K, V, mask, scale = wl.bf16_mha(B, H, S, D)
+    sval = np.array([scale], np.float32)
+    Qd, Kd, Vd, md = Q.to(dev), K.to(dev), V.to(dev), mask.to(dev)
+    outs = {}
+    for const in (True, False):
+        comp = ga.Compiler()
+        st, exe = comp.compile(ga.mha_json(B, H, S, S, D, True, "Multiply", mask_constant=const))
+        assert st == 0
+        res = []
+        for rep in range(2):
+            q = Qd if rep == 0 else Qd.flip(2).contiguous()
+            o = torch.zeros(B, H, S, D, dtype=torch.bfloat16, device=dev)
+            assert exe.execute([(0, q), (1, Kd), (2, torch.from_numpy(sval).to(dev)), (3, md), (4, Vd)], [(9, o)]) == 0
+            res.append(o.clone())
+        outs[const] = res
+        exe.close()
+        comp.close()
+    for rep in range(2):
+        assert torch.equal(outs[True][rep].view(torch.int16), outs[False][rep].view(torch.int16))
+    cls = gc.mha_mask_classes(md, S, S, D)
+    assert cls is not None
+    for skip in (True, False):
+        a = gc.mha_fwd_bf16_classified(Qd, Kd, Vd, md, cls, scale, skip_masked=skip)
+        b = gc.mha_fwd_bf16(Qd, Kd, Vd, md, scale, skip_masked=skip)
+        torch.cuda.synchronize()
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert torch.equal(outs[True][0].view(torch.int16), a.view(torch.int16))
+
+
 @pytest.mark.parametrize("D,with_mask,scale_op", [(128, True, "Multiply"), (128, False, "Divide"), (64, True, "Multiply")])
 def test_attention_partition(ga, orc, wl, dev, D, with_mask, scale_op):
     """head dims 128 and 64 both run the fused kernel (softmax weights rounded to bf16, as the graph's tensor is)."""
