@@ -14,10 +14,12 @@ the same run and reported under "others" (--only picks some of them).  One JSON
 line goes to stdout; progress goes to stderr.
 
 Time basis: `value`, `ms_per_step` and `roofline.achieved` all come from ONE
-clock: the timed region of K back-to-back launches, bracketed by a HIP event
-pair on the stream the kernels are launched on (torch's current stream) and by
-the wall clock around the same region; the larger of the two, divided by K, is
-the step time.  A second pass brackets every launch with its own event pair;
+clock: the timed region of K back-to-back launches between two
+synchronizations, bracketed by a HIP event pair on the stream the kernels are
+launched on (torch's current stream); that time divided by K is the step time.
+The wall clock around the same region is reported beside it
+(`kernel_ms.wall_ms_per_step`: it adds the host's wake-up from the final
+synchronize, 20-30 us per region).  A second pass brackets every launch with its own event pair;
 those figures are reported under `kernel_ms` only (they include the event
 pair's own overhead and isolate launches from each other).  `roofline.traffic`
 is not measured in this run: it is the HBM-side byte count of the committed
@@ -35,6 +37,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+SETTLE_MIN_S, SETTLE_MAX_S = 0.3, 2.0  # untimed load in front of every timed region, see time_launches
 PEAK = {"bf16": 2500.0, "int8": 5000.0, "f32": 157.3}  # dense MFMA, TFLOP/s | TOP/s
 HBM_PEAK_GBS = 8000.0
 
@@ -55,18 +58,22 @@ def load_package():
 
 def time_launches(torch, fn, nsets, steps, warmup):
     """fn(i) launches one step on buffer set i.  Two passes of `steps` launches:
-    the first is bracketed by one event pair and the wall clock (ms_per_step:
-    the basis of `value` AND of the roofline figure); the second brackets every
+    the first is bracketed by one event pair (ms_per_step: the basis of `value`
+    AND of the roofline figure) and by the wall clock; the second brackets every
     launch with its own event pair (kernel_ms_*: extra keys, not used for any
     headline figure).
 
     Before the `warmup` steps the board is brought to its working clocks: an
-    idle MI355X raises them over the first tens of milliseconds of load (the
-    first 100 launches of the 4096^3 GEMM run 15-20 % slower than the 300th),
-    so groups of 50 untimed launches run until two groups in a row agree to
-    1 % (at most 16 groups); `settle_launches` says how many that took."""
-    settle, prev = 0, None
-    for _ in range(16):
+    idle MI355X raises them under load, most of the way within tens of
+    milliseconds (the first 100 launches of the 4096^3 GEMM run 15-20 % slower
+    than the 300th) and the last 3-5 % over a few hundred (20 timed launches
+    right after 300 untimed ones: 97-101 us; the same 20 after 0.3 s of load:
+    the 94 us that 2000 timed launches average).  So groups of 50 untimed
+    launches run for at least SETTLE_MIN_S seconds and until three groups in a
+    row agree to 0.5 % (at most SETTLE_MAX_S); `settle_launches` says how many
+    that took."""
+    settle, times, t_begin = 0, [], time.perf_counter()
+    while True:
         g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         g0.record()
         for i in range(50):
@@ -74,10 +81,11 @@ def time_launches(torch, fn, nsets, steps, warmup):
         g1.record()
         torch.cuda.synchronize()
         settle += 50
-        cur = g0.elapsed_time(g1)
-        if prev is not None and abs(cur - prev) <= 0.01 * prev:
+        times.append(g0.elapsed_time(g1))
+        loaded = time.perf_counter() - t_begin
+        steady = len(times) >= 3 and max(times[-3:]) <= 1.005 * min(times[-3:])
+        if (steady and loaded >= SETTLE_MIN_S) or loaded >= SETTLE_MAX_S:
             break
-        prev = cur
     for i in range(warmup):
         fn(i % nsets)
     torch.cuda.synchronize()
@@ -98,7 +106,10 @@ def time_launches(torch, fn, nsets, steps, warmup):
         stops[i].record()
     torch.cuda.synchronize()
     per = sorted(s.elapsed_time(e) for s, e in zip(starts, stops))
-    return {"ms_per_step": max(region_ms, wall_ms) / steps, "wall_ms_per_step": wall_ms / steps,
+    # The step time is the device's: the HIP-event pair around the K launches on the stream they run on.  The wall
+    # clock around the same region (kept beside it) adds the host's wake-up from the final synchronize, 20-30 us per
+    # region whatever its length: 1 % of 20 steps of the headline GEMM, nothing of 2000.
+    return {"ms_per_step": region_ms / steps, "wall_ms_per_step": wall_ms / steps,
             "event_ms_per_step": region_ms / steps, "settle_launches": settle,
             "kernel_ms_mean": sum(per) / len(per), "kernel_ms_min": per[0], "kernel_ms_median": per[len(per) // 2]}
 

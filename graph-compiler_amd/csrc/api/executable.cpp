@@ -527,7 +527,7 @@ void Executable::plan() {
     // ---------------- quantised: Dequantize(A) , Dequantize(W) -> MatMul -> [bias] -> [act] -> [cast]
     bool int8 = false;
     size_t dq_a = 0, dq_w = 0;
-    if (!ta && !tb && producer.count(mm.in[0]) && producer.count(mm.in[1]) && T(mm.out[0]).dt == DT::f32) {
+    if (!ta && producer.count(mm.in[0]) && producer.count(mm.in[1]) && T(mm.out[0]).dt == DT::f32) {
       dq_a = producer[mm.in[0]], dq_w = producer[mm.in[1]];
       const Op &da = g_.ops[dq_a], &dw = g_.ops[dq_w];
       if (da.kind == "Dequantize" && dw.kind == "Dequantize" && single_use(mm.in[0]) && single_use(mm.in[1])) {
@@ -541,7 +541,7 @@ void Executable::plan() {
         if (axw < 0)
           axw += (int64_t)qw.shape.size();
         int8 = sa.size() == 1 && qw.dt == DT::s8 && qw.shape.size() == 2 && qa.shape.size() >= 2 && zw0 &&
-               (sw.size() == 1 || axw == 1) && is_dense(qa) && is_dense(qw);
+               (sw.size() == 1 || axw == (tb ? 0 : 1)) && is_dense(qa) && is_dense(qw); // scales per output channel
       }
     }
 
@@ -614,7 +614,21 @@ void Executable::plan() {
       int32_t zpA = 0;
       if (da.attrs.count("zps") && !da.attrs.at("zps").ia.empty())
         zpA = (int32_t)da.attrs.at("zps").ia[0];
-      int64_t K = qw.shape[0], N = qw.shape[1], M = qa.numel() / K;
+      // weights stored [N,K] (transpose_b, the layout of torch.nn.Linear): the 8-bit tile kernels read [K,N], so a
+      // transposed copy is made -- once per executable when the weights are a constant, the reference's pre-packing
+      // of constant weights (docs/CPU_pipeline_overview.md:58); measured on the 4-wave kernel, reading [N,K] tiles
+      // in place is no faster than [K,N]
+      int64_t K = tb ? qw.shape[1] : qw.shape[0], N = tb ? qw.shape[0] : qw.shape[1], M = qa.numel() / K;
+      int w_slot = slot_for(dw.in[0]);
+      if (tb) {
+        Step cp;
+        cp.kind = Step::Elt, cp.op = gcmi::ELT_COPY, cp.once = qw.constant;
+        cp.note = qw.constant ? "transpose copy of W [N,K] -> [K,N], once: W is constant" : "transpose copy of W [N,K] -> [K,N]";
+        cp.a = w_slot, cp.out = new_slot((size_t)K * N);
+        cp.a_dt = cp.out_dt = GCMI_S8, cp.dims = {K, N}, cp.sa = {1, K};
+        v.push_back(cp);
+        w_slot = cp.out;
+      }
       // output_scales = data_scales (x) weight_scales
       // (legacy/core/src/compiler/ir/graph/transform/quantization/graph_reschedule.cpp:220-235)
       std::vector<float> sc((size_t)N);
@@ -624,13 +638,13 @@ void Executable::plan() {
       int cs_slot = new_slot((size_t)N * 4);
       Step cs;
       cs.kind = Step::ColSum, cs.note = qw.constant ? "colsum(W), once: W is constant" : "colsum(W)";
-      cs.a = slot_for(dw.in[0]), cs.out = cs_slot, cs.K = K, cs.N = N, cs.lda = N;
+      cs.a = w_slot, cs.out = cs_slot, cs.K = K, cs.N = N, cs.lda = N;
       cs.op = qw.constant ? 1 : 0;
       v.push_back(cs);
       Step s;
       s.kind = Step::GemmInt8;
       s.note = "Dequantize x2 + MatMul" + fused + (T(cur).dt == DT::bf16 ? "+cast" : "") + " fused";
-      s.a = slot_for(da.in[0]), s.b = slot_for(dw.in[0]), s.out = slot_for(cur);
+      s.a = slot_for(da.in[0]), s.b = w_slot, s.out = slot_for(cur);
       s.M = M, s.N = N, s.K = K, s.lda = K, s.ldb = N, s.ldc = N;
       s.a_dt = dt_dnnl(qa.dt), s.zp = zpA, s.aux = cs_slot, s.scales_slot = sc_slot;
       s.bias = bias_t >= 0 ? slot_for((size_t)bias_t) : -1;

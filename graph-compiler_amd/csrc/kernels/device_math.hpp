@@ -52,16 +52,18 @@ __device__ __forceinline__ float erf_rational(float x) {
 // 1.1e-9 elsewhere): a quarter of the last place of a bf16 -- about 4 % of the results in |x| < 6 round to the
 // neighbouring bf16 value of the exactly rounded one, none differs by more.  q has positive derivative for all t >= 0, so no clamp is
 // needed: for |x| > 13 the power underflows to 0 and the result is x or -0 exactly, as with the reference's
-// saturated erf (legacy/core/src/ops/gelu.cpp:110-131 gives (erf + 1) * x * 0.5 = -0 there).  13 issue slots (the
+// saturated erf (legacy/core/src/ops/gelu.cpp:110-131 gives (erf + 1) * x * 0.5 = -0 there).  12 issue slots (the
 // exponential counts four) against 19 for erf_rational + 1, * x, * 0.5.  Not for infinite or NaN x (inf * 0).
 __device__ __forceinline__ float gelu_erf_bf16_result(float x) {
-  const float t = fabsf(x) * 0.70710678f;
-  float q = 1.4229814987629652e-03f;
-  q = fmaf(q, t, -2.0445456728339195e-02f);
-  q = fmaf(q, t, 1.293562352657318e-01f);
-  q = fmaf(q, t, 9.348235130310059e-01f);
-  q = fmaf(q, t, 1.6235692501068115f);
-  const float g = x * __builtin_amdgcn_exp2f(fmaf(-t, q, -1.0f));
+  // q(t) t with t = |x| / sqrt 2 written as a polynomial in |x| (the factors of 1 / sqrt 2 are in the coefficients;
+  // |x| is an operand modifier, not an instruction)
+  const float a = fabsf(x);
+  float q = 2.5154993636533618e-04f;
+  q = fmaf(q, a, -5.1113637164235115e-03f);
+  q = fmaf(q, a, 4.5734334737062454e-02f);
+  q = fmaf(q, a, 4.6741172671318054e-01f);
+  q = fmaf(q, a, 1.1480368375778198f);
+  const float g = x * __builtin_amdgcn_exp2f(fmaf(-a, q, -1.0f));
   return fmaxf(x, -0.0f) - fabsf(g);
 }
 

@@ -229,21 +229,25 @@ def gemm_json(M, K, N, dtype="bf16"):
                     "outputs": [_t(2, dtype, [M, N])]}], [0, 1], [2])
 
 
-def int8_mlp_json(M, K, N, scale_a, zp_a, scales_w, out_dtype="bf16", act="GELU"):
+def int8_mlp_json(M, K, N, scale_a, zp_a, scales_w, out_dtype="bf16", act="GELU", weights_nk=False, weights_constant=True):
     """Dequantize(u8 A) , Dequantize(s8 W, per channel) -> MatMul(+bias f32) -> GELU -> Typecast.
-    ids: 0 A u8, 1 W s8, 2 bias f32 -> 7 (or 6 when out_dtype is f32)."""
+    ids: 0 A u8, 1 W s8, 2 bias f32 -> 7 (or 6 when out_dtype is f32).  weights_nk: W is stored [N,K] and the MatMul
+    has transpose_b (the layout of torch.nn.Linear)."""
+    wshape = [N, K] if weights_nk else [K, N]
+    wprop = {"property_type": "constant"} if weights_constant else {}
     ops = [
         {"kind": "Dequantize", "attrs": {"qtype": {"type": "string", "value": "per_tensor"},
                                          "scales": {"type": "f32[]", "value": [float(scale_a)]},
                                          "zps": {"type": "s64[]", "value": [int(zp_a)]}},
          "inputs": [_t(0, "u8", [M, K])], "outputs": [_t(3, "f32", [M, K])]},
         {"kind": "Dequantize", "attrs": {"qtype": {"type": "string", "value": "per_channel"},
-                                         "axis": {"type": "s64", "value": 1},
+                                         "axis": {"type": "s64", "value": 0 if weights_nk else 1},
                                          "scales": {"type": "f32[]", "value": [float(s) for s in scales_w]},
                                          "zps": {"type": "s64[]", "value": [0] * len(scales_w)}},
-         "inputs": [_t(1, "s8", [K, N], property_type="constant")], "outputs": [_t(4, "f32", [K, N])]},
-        {"kind": "MatMul", "inputs": [_t(3, "f32", [M, K]), _t(4, "f32", [K, N]), _t(2, "f32", [N])],
-         "outputs": [_t(5, "f32", [M, N])]}]
+         "inputs": [_t(1, "s8", wshape, **wprop)], "outputs": [_t(4, "f32", wshape)]},
+        dict({"kind": "MatMul", "inputs": [_t(3, "f32", [M, K]), _t(4, "f32", wshape), _t(2, "f32", [N])],
+              "outputs": [_t(5, "f32", [M, N])]},
+             **({"attrs": {"transpose_b": {"type": "bool", "value": 1}}} if weights_nk else {}))]
     last = 5
     if act:
         ops.append({"kind": act, "inputs": [_t(5, "f32", [M, N])], "outputs": [_t(6, "f32", [M, N])]})

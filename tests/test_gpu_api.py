@@ -178,6 +178,36 @@ def test_int8_partition_through_the_api_with_device_tensors(ga, gc, orc, wl, dev
     c.close()
 
 
+@pytest.mark.parametrize("constant", [True, False])
+def test_int8_partition_with_weights_stored_nk(ga, orc, wl, dev, constant):
+    """transpose_b on the quantised MatMul (weights [N,K], per-channel scales along axis 0): the fused 8-bit GEMM
+    runs on a transposed copy that is made once when the weights are a constant; the bits are those of the [K,N]
+    partition."""
+    M, K, N = 512, 256, 768
+    A, W, scale, bias = wl.int8_mlp_layer(M, K, N)
+    sA = 0.02
+    js_kn, oid = ga.int8_mlp_json(M, K, N, sA, 128, scale.tolist())
+    js_nk, oid2 = ga.int8_mlp_json(M, K, N, sA, 128, scale.tolist(), weights_nk=True, weights_constant=constant)
+    st, plan = ga.explain(js_nk)
+    assert st == 0 and "Dequantize x2 + MatMul" in plan and "transpose copy of W" in plan, plan
+    assert ("once" in plan.split("transpose copy of W")[1].splitlines()[0]) == constant
+    want = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    _run(ga, js_kn, [(0, A.to(dev)), (1, W.to(dev)), (2, bias.to(dev))], [(oid, want)])
+    Wt = W.t().contiguous().to(dev)
+    c = ga.Compiler()
+    st, exe = c.compile(js_nk)
+    assert st == 0
+    for rep in range(2):
+        a = A if rep == 0 else A.flip(0).contiguous()
+        got = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+        assert exe.execute([(0, a.to(dev)), (1, Wt), (2, bias.to(dev))], [(oid2, got)]) == 0
+        torch.cuda.synchronize()
+        ref = want if rep == 0 else want.flip(0)
+        assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), rep
+    exe.close()
+    c.close()
+
+
 def test_mlp_chain_partition(ga, orc, wl, dev):
     M, K, H = 512, 512, 1280
     x, W1, W2, b2 = wl.bf16_mlp_chain(M, K, H)
