@@ -1447,6 +1447,10 @@ __device__ __forceinline__ void w4_epilogue_half_any(const GemmParams &p, int ki
 }
 
 template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gemm_tile256_w4_kernel(GemmParams p) {
+  // B stored [N,K]: bf16 only.  (The same loop for 8-bit operands -- plain 16-byte fragment reads in place of the
+  // transposing ones -- was measured against [K,N] on one board and is no faster: 166.9-168.9 against 167.2-168.6 us
+  // for the 4096 x 4096 x 11008 layer; an 8-bit weight stored [N,K] is copied once instead.)
+  static_assert(!TB || ES == 2, "B stored [N,K]: bf16 only");
   typedef FastGemm<ES, 2, 4, false, TB> FG; // 4 waves: 4 DMA instructions per operand, wave and stage
   static_assert(FG::NST == 4 && FG::NDMA == 4 && FG::STAGE_BYTES == 32768 && FG::A_BYTES == 16384, "the assembly's ring");
 #ifdef GCMI_W4_TIMING
@@ -1553,9 +1557,7 @@ template <int ES, bool TB = false> __global__ __launch_bounds__(256, 1) void gem
 #ifdef GCMI_W4_TIMING // measurement builds: core clock cycles and 100 MHz ticks spent in the main loop
   const long long tick0 = clock64(), wall0 = wall_clock64();
 #endif
-  if constexpr (ES == 1 && TB)
-    asm volatile(GCMI_W4_ASM_I8_TB GCMI_W4_OPERANDS);
-  else if constexpr (ES == 1)
+  if constexpr (ES == 1)
     asm volatile(GCMI_W4_ASM_I8 GCMI_W4_OPERANDS);
   else if constexpr (TB)
     asm volatile(GCMI_W4_ASM_BF16_TB GCMI_W4_OPERANDS);

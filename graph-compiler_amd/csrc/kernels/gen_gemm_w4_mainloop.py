@@ -237,7 +237,7 @@ def main():
         f.write("// generated by gen_gemm_w4_mainloop.py -- do not edit\n")
         if OPTS:  # a measurement build: the library's sources refuse this text
             f.write('#define GCMI_W4_EXPERIMENT_OPTS "%s"\n' % ",".join(sorted(OPTS)))
-        for name, es, tb in (("BF16", 2, False), ("BF16_TB", 2, True), ("I8", 1, False), ("I8_TB", 1, True)):
+        for name, es, tb in (("BF16", 2, False), ("BF16_TB", 2, True), ("I8", 1, False)):
             lines = gen(es, tb)
             f.write("#define GCMI_W4_ASM_%s \\\n" % name)
             f.write(" \\\n".join('  "%s\\n"' % ln for ln in lines))
