@@ -314,6 +314,16 @@ int gemm_bf16_any(bool trans_b, const void *A, const void *B, void *C, int64_t M
     return launched(gcmi_launch_gemm_bf16(&p, (hipStream_t)stream), "gemm_bf16");
   }
   if (ws_from == Ws::Static) {
+    // the static array is per device and its address is the current device's: a stream of another device would be
+    // handed the wrong GPU's address
+    if (stream != nullptr && (hipStream_t)stream != hipStreamPerThread && (hipStream_t)stream != hipStreamLegacy) {
+      int cur = -1;
+      hipDevice_t sdev = -1;
+      if (hipGetDevice(&cur) == hipSuccess && hipStreamGetDevice((hipStream_t)stream, &sdev) == hipSuccess && (int)sdev != cur)
+        return fail(ST_INVALID, "gemm_bf16_noalloc: the stream belongs to device %d, the current device is %d; make the "
+                                "stream's device current (hipSetDevice) before the call", (int)sdev, cur);
+      (void)hipGetLastError();
+    }
     void *sp = nullptr;
     size_t sb = 0;
     if (gcmi_noalloc_scratch(&sp, &sb) != 0)
