@@ -45,6 +45,9 @@ stage: 12 % more cycles than a loop without flips, now 4 %.
 Experiments (measurement builds only: honoured when GCMI_W4_EXPERIMENT=1 is set as well, and then the output carries
 a macro that the library's sources refuse; environment variable GCMI_W4_OPTS, comma separated):
   nodma nobar nolds noxor   leave out the DMA requests / barriers / fragment reads / byte flips (wrong products)
+  nodma_a nodma_b           leave out the A tile's / the B tile's requests only (wrong products)
+  nolds_a nolds_b           leave out the A / the B fragment reads only ([K,N] bf16: wrong products)
+  copypar                   (with nolds) block 0's fragments in both register sets, so that every MFMA has real operands
   dmaburst rdburst          other placements of the requests and the reads (correct products)
   xorlate xor1 xor0=N       the flips behind a full wait over the last 16 MFMAs / the last 32; first flip at MFMA N
 """
@@ -107,6 +110,10 @@ def gen(es, tb):
             rd += read_a(slot, it, par)
         for jt in range(1, 8):
             rd += read_b(slot, jt, par)
+        if "nolds_a" in OPTS:
+            rd = [r for r in rd if not r.startswith("ds_read_b128")]
+        if "nolds_b" in OPTS:
+            rd = [r for r in rd if r.startswith("ds_read_b128")]
         return rd
 
     def xor_tiles(par):
@@ -128,6 +135,8 @@ def gen(es, tb):
             d = [dma(slot, i) for i in range(8)]
             pre.append(d[0][0])
             for i in range(8):
+                if ("nodma_a" in OPTS and i < 4) or ("nodma_b" in OPTS and i >= 4):
+                    continue
                 extras[i * step].append(d[i][1])
                 if i < 7:
                     extras[i * step + step - 1].append(d[i + 1][0])
@@ -194,7 +203,17 @@ def gen(es, tb):
         emit("v_accvgpr_write_b32 a%d, 0" % r)
     emit("s_waitcnt vmcnt(24) lgkmcnt(0)")
     emit("s_barrier")
-    out.extend(all_reads(0, 0))
+    if "copypar" in OPTS:  # (with nolds) both register sets hold block 0: every stage multiplies real data
+        saved = set(OPTS)
+        OPTS.discard("nolds"), OPTS.discard("nolds_a"), OPTS.discard("nolds_b")
+        out.extend(all_reads(0, 0))
+        OPTS.update(saved)
+        emit("s_waitcnt lgkmcnt(0)")
+        for k in range(32):
+            emit("v_mov_b32 v%d, v%d" % (AF[1] + k, AF[0] + k))
+            emit("v_mov_b32 v%d, v%d" % (BF[1] + k, BF[0] + k))
+    else:
+        out.extend(all_reads(0, 0))
     if es == 1:
         emit("s_waitcnt lgkmcnt(0)")
         out.extend(xor_tiles(0))
