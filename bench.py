@@ -119,9 +119,9 @@ def time_launches(torch, fn, nsets, steps, warmup):
 # --copy-calibration: a 1 GiB copy reads FETCH_SIZE = 524304 KiB (scale 2.0)
 # and WRITE_SIZE = 1048580 KiB (scale 1.0).
 TRAFFIC = {  # (bytes per launch of the dominant kernel, the committed profile they come from)
-    "gemm": (235417028, "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
-    "int8": (384764352, "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
-    "chain": (681050751 + 575140903, "profiles/gemm_tile256_w4_bf16_mlp_chain.md"),  # both launches
+    "gemm": (235414490, "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
+    "int8": (384693096, "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
+    "chain": (684027008 + 575145347, "profiles/gemm_tile256_w4_bf16_mlp_chain.md"),  # both launches
     "mha": (362734179, "profiles/mha_fwd_fast_b4_h32_s2048_d128_every_block.md"),
     "mha_skip": (330983112, "profiles/mha_fwd_fast_b4_h32_s2048_d128.md"),
 }
