@@ -1,9 +1,14 @@
-// bf16 x bf16 -> f32 GEMMs: the 256x256 MFMA tile kernels (gemm_tile256.hpp) and the streaming kernel for a short
-// A against [N,K] weights (gemm_skinny.hpp).
+// bf16 x bf16 -> f32 GEMMs: the 256x256 MFMA tile kernels (gemm_tile256.hpp) and the streaming kernels for a short
+// A against [N,K] weights (gemm_rows32.hpp: up to 32 rows; gemm_skinny.hpp: up to 64 rows where a caller's slice
+// count asks for it, and the shapes the former does not take).
+#include "gemm_rows32.hpp"
 #include "gemm_skinny.hpp"
 
 extern "C" int gcmi_launch_gemm_bf16(const gcmi::GemmParams *p, hipStream_t stream) {
-  const int rc = gcmi::launch_skinny_nt(p, stream);
+  int rc = gcmi::launch_rows32(p, stream);
+  if (rc >= 0)
+    return rc;
+  rc = gcmi::launch_skinny_nt(p, stream);
   if (rc >= 0)
     return rc;
   return gcmi::launch_tile256<2>(p, stream);
@@ -12,6 +17,8 @@ extern "C" int gcmi_launch_gemm_bf16(const gcmi::GemmParams *p, hipStream_t stre
 // floats of workspace (GemmParams::partial) the launch above would use for this call: 0 when K is not sliced
 extern "C" int64_t gcmi_launch_gemm_bf16_workspace(const gcmi::GemmParams *p) {
   int64_t want = 0;
+  if (gcmi::launch_rows32(p, nullptr, &want) >= 0)
+    return want;
   if (gcmi::launch_skinny_nt(p, nullptr, &want) >= 0)
     return want;
   gcmi::launch_tile256<2>(p, nullptr, &want);
@@ -20,6 +27,8 @@ extern "C" int64_t gcmi_launch_gemm_bf16_workspace(const gcmi::GemmParams *p) {
 
 // what the launch above would choose (nothing is launched)
 extern "C" int gcmi_launch_gemm_bf16_config(const gcmi::GemmParams *p, gcmi::GemmTileConfig *cfg) {
+  if (gcmi::launch_rows32(p, (hipStream_t)-1, nullptr, cfg) >= 0)
+    return 0;
   if (gcmi::launch_skinny_nt(p, (hipStream_t)-1, nullptr, cfg) >= 0)
     return 0;
   return gcmi::launch_tile256<2>(p, (hipStream_t)-1, nullptr, cfg);

@@ -600,8 +600,10 @@ NT_SHAPES = [(256, 256, 128), (512, 768, 256), (300, 200, 100), (257, 511, 129),
 
 
 def _streams_weights(M, N, K):
-    """Shapes the [N,K] entry point gives to the weight-streaming kernel (short A, enough weights)."""
-    return M <= 32 and N % 32 == 0 and K % 64 == 0 and K >= 256 and 1 << 20 <= N * K <= 3 << 23
+    """Shapes the [N,K] entry point gives to one of the weight-streaming kernels (short A, enough weights): the
+    8-wave kernel with the LDS ring, or the one that loads fragments straight into registers."""
+    ring = M <= 32 and N % 4 == 0 and N >= 512 and K % 128 == 0 and K >= 512 and N * K >= 1 << 22
+    return ring or (M <= 32 and N % 32 == 0 and K % 64 == 0 and K >= 256 and 1 << 20 <= N * K <= 3 << 23)
 
 
 @pytest.mark.parametrize("M,N,K", NT_SHAPES)
@@ -655,6 +657,63 @@ def test_bf16_gemm_streaming_kernel_exact_on_integers(gc, dev):
         _gemm_ws(gc, A, Bt, True, out2, 16, ws=ws)
         torch.cuda.synchronize()
         assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("M", [1, 7, 16, 32])
+@pytest.mark.parametrize("N,K", [(4096, 1024), (4100, 4096), (520, 11008), (11008, 4096), (12352, 640)])
+def test_short_a_streaming_kernel_exact_on_integers(gc, dev, M, N, K):
+    """Up to 32 rows against [N,K] weights: 8-wave workgroups on panels of 64 columns (the last one 4 or 8 columns
+    wide here), K in one piece where the panels fill the GPU and in slices with the second pass where they do not,
+    slice lengths that differ (86 and 5 stages), rows past M.  Small integers: every sum is exact in f32, whatever
+    the order.  The caller's slice count and a call without workspace (one slice, epilogue in the kernel) agree."""
+    c, _ = gc.tile_config(M, N, K, trans_b=True, out_dtype=gc.F32)
+    assert (c.kernel, c.bm, c.bn, c.waves_m * c.waves_n) == (4, 32, 64, 4) and c.workgroups == -(-N // 64) * c.split_k
+    assert c.split_k == (1 if N > 10000 else min(K // 512, (256 + -(-N // 64) // 2) // -(-N // 64)))
+    torch.manual_seed(M + N + K)
+    A = torch.randint(-3, 4, (M, K), device=dev).to(torch.bfloat16)
+    Bt = torch.randint(-3, 4, (N, K), device=dev).to(torch.bfloat16)
+    want = A.float() @ Bt.float().t()
+    guard = torch.full((M + 2, N), 7.0, dtype=torch.float32, device=dev)
+    out = guard[1:M + 1]
+    gc.gemm_bf16_nt(A, Bt, out_dtype=gc.F32, out=out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    assert bool((guard[0] == 7.0).all()) and bool((guard[M + 1] == 7.0).all())
+    one = torch.full((M, N), 7.0, dtype=torch.float32, device=dev)
+    _gemm_ws(gc, A, Bt, True, one)  # no workspace: K in one piece
+    ws = torch.empty(3 * M * N, dtype=torch.float32, device=dev)
+    three = torch.full((M, N), 7.0, dtype=torch.float32, device=dev)
+    _gemm_ws(gc, A, Bt, True, three, 3, ws=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(one, want) and torch.equal(three, want)
+
+
+@pytest.mark.parametrize("M,N,K", [(32, 4096, 4096), (9, 11008, 4096), (32, 4096, 11008), (20, 1032, 4096)])
+def test_short_a_streaming_kernel_rounding_points(gc, dev, M, N, K):
+    """N(0,1) data through bias, GELU and a residual, bf16 and f32 results: against the same sums in float64 rounded
+    at the reference's points (after the matmul and after each op for bf16 results), to one bf16 step of the larger of
+    the value and the rounded intermediate; sliced and unsliced agree to the same bound."""
+    torch.manual_seed(N + K)
+    A = (torch.randn(M, K, device=dev) * 0.5).to(torch.bfloat16)
+    Bt = (torch.randn(N, K, device=dev) * 0.05).to(torch.bfloat16)
+    bias, res = torch.randn(N, device=dev).to(torch.bfloat16), torch.randn(M, N, device=dev).to(torch.bfloat16)
+    acc = A.double() @ Bt.double().t()
+    r = lambda t: t.to(torch.bfloat16).double()  # noqa: E731
+    gelu = lambda t: 0.5 * t * (1.0 + torch.special.erf(t / 2.0 ** 0.5))  # noqa: E731
+    want16 = r(r(gelu(r(r(acc) + bias.double()))) + res.double())
+    want32 = gelu(acc + bias.double()) + res.double()
+    o16 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    o32 = torch.empty(M, N, dtype=torch.float32, device=dev)
+    _gemm_ws(gc, A, Bt, True, o16, bias=bias, act="gelu_erf", residual=res)
+    _gemm_ws(gc, A, Bt, True, o32, bias=bias, act="gelu_erf", residual=res)
+    ws = torch.empty(4 * M * N, dtype=torch.float32, device=dev)
+    s16 = torch.empty_like(o16)
+    _gemm_ws(gc, A, Bt, True, s16, 4, bias=bias, act="gelu_erf", residual=res, ws=ws)
+    torch.cuda.synchronize()
+    mag = torch.maximum(acc.abs(), torch.maximum(want16.abs(), res.double().abs())) + 1.0
+    assert float(((o16.double() - want16).abs() / mag).max()) < 2.0 ** -7
+    assert float(((s16.double() - want16).abs() / mag).max()) < 2.0 ** -7
+    assert float(((o32.double() - want32).abs() / mag).max()) < 1e-5
 
 
 def test_bf16_gemm_transposed_b_strided_rows(gc, dev):
