@@ -711,6 +711,8 @@ def test_short_a_streaming_kernel_rounding_points(gc, dev, M, N, K):
     _gemm_ws(gc, A, Bt, True, s16, 4, bias=bias, act="gelu_erf", residual=res, ws=ws)
     torch.cuda.synchronize()
     mag = torch.maximum(acc.abs(), torch.maximum(want16.abs(), res.double().abs())) + 1.0
+    # a bias given as f32 holds the same values: the same bits come out
+    assert torch.equal(gc.gemm_bf16_nt(A, Bt, bias.float(), "relu", gc.F32), gc.gemm_bf16_nt(A, Bt, bias, "relu", gc.F32))
     assert float(((o16.double() - want16).abs() / mag).max()) < 2.0 ** -7
     assert float(((s16.double() - want16).abs() / mag).max()) < 2.0 ** -7
     assert float(((o32.double() - want32).abs() / mag).max()) < 1e-5
