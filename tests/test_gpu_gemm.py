@@ -718,6 +718,23 @@ def test_short_a_streaming_kernel_rounding_points(gc, dev, M, N, K):
     assert float(((o32.double() - want32).abs() / mag).max()) < 1e-5
 
 
+def test_short_a_streaming_kernel_strided_operands(gc, dev):
+    """Rows of A, of the weights and of the result further apart than their length (slices of wider tensors, start
+    offsets of 16 bytes): exact on integers, and nothing written between the rows of the result."""
+    M, N, K = 24, 2048, 2048
+    c, _ = gc.tile_config(M, N, K, trans_b=True)
+    assert c.kernel == 4 and c.bn == 64
+    torch.manual_seed(12)
+    wide_a = torch.randint(-3, 4, (M, K + 72), device=dev).to(torch.bfloat16)
+    wide_w = torch.randint(-3, 4, (N, K + 136), device=dev).to(torch.bfloat16)
+    wide_c = torch.full((M, N + 40), 7.0, dtype=torch.float32, device=dev)
+    A, Bt, out = wide_a[:, 8:8 + K], wide_w[:, 16:16 + K], wide_c[:, 4:4 + N]
+    gc.gemm_bf16_nt(A, Bt, out_dtype=gc.F32, out=out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, A.float() @ Bt.float().t())
+    assert bool((wide_c[:, :4] == 7.0).all()) and bool((wide_c[:, 4 + N:] == 7.0).all())
+
+
 def test_bf16_gemm_transposed_b_strided_rows(gc, dev):
     """Rows of Bt further apart than K (a weight that is a slice of a wider one)."""
     torch.manual_seed(6)
