@@ -1,4 +1,4 @@
-// bf16 GEMM for a short A (M <= 32) against wide weights stored [N,K] (k contiguous): C[M,N] = epilogue(A . W^T).
+// bf16 GEMM for a short A (M <= 64) against wide weights stored [N,K] (k contiguous): C[M,N] = epilogue(A . W^T).
 // This is the decode-time shape of the reference's llama2 case (test/benchgc/cases/llama2.mlir: 32 tokens against
 // 4096 x 4096 .. 4096 x 11008 weights), where the reference splits K over threads (KThreads,
 // lib/gc/Analysis/MatmulConfigAnalysis.cpp:149-166).  The arithmetic is negligible; the job is to pull the weights
@@ -8,8 +8,9 @@
 // of 32 rows 3.2-4.4 -- the vector memory pipe pays per cache line it looks up -- and every fragment of A that a
 // wave fetches for itself costs look-ups of its own.  Hence:
 //   * a workgroup is 8 waves on a panel of 64 columns and one slice of K; a stage is 256 bytes of K per row: the A
-//     tile (32 rows, 8 KiB, shared by all waves) and the panel's weights (16 KiB) go to an LDS ring by
-//     global_load_lds_dwordx4, 4 rows x 256 bytes per request, one request for A and two for the weights per wave;
+//     tile (32 rows, 8 KiB, shared by all waves; 64 rows and 16 KiB from 33 rows on) and the panel's weights (16 KiB)
+//     go to an LDS ring by global_load_lds_dwordx4, 4 rows x 256 bytes per request, one request (two) for A and two
+//     for the weights per wave;
 //   * A is re-read once per panel (half the weights' traffic, from L2) instead of once per 16 columns;
 //   * wave w owns column tile w % 4 and k-steps 2 * (w / 4), 2 * (w / 4) + 1 of the stage's four; the two halves are
 //     added through LDS at the end (upper onto lower: a fixed order); one barrier per stage.
@@ -72,10 +73,13 @@ __device__ __forceinline__ void rows32_store4(const GemmParams &p, const f32x4_t
     *reinterpret_cast<f32x4_t *>(reinterpret_cast<float *>(p.C) + m * p.ldc + n) = f32x4_t{o32[0], o32[1], o32[2], o32[3]};
 }
 
-__global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(GemmParams p) {
+// MT: 16-row tiles of A (2: up to 32 rows; 4: up to 64 rows, with an A tile of 16 KiB per stage)
+template <int MT> __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(GemmParams p) {
+  static_assert(MT == 2 || MT == 4, "32 or 64 rows");
   constexpr int KB = R32_KB, BK = KB / 2, NST = R32_NST, BN = R32_BN;
-  constexpr int A_BYTES = R32_BM * KB, B_BYTES = BN * KB, STAGE = A_BYTES + B_BYTES; // 8 + 16 KiB
-  constexpr int PER = 3;
+  constexpr int A_BYTES = 16 * MT * KB, B_BYTES = BN * KB, STAGE = A_BYTES + B_BYTES; // 8 (16) + 16 KiB
+  constexpr int NA_DMA = MT / 2;    // A requests per wave and stage
+  constexpr int PER = NA_DMA + 2;   // requests per wave and stage
   __shared__ __align__(1024) char smem[NST * STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -92,10 +96,14 @@ __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(GemmParams p) {
     const int g0 = (int)((int64_t)slice * KT / p.splits), g1 = (int)((int64_t)(slice + 1) * KT / p.splits);
     k_first = g0, KT = g1 - g0;
   }
-  uint32_t a_src, b_src[2];
+  uint32_t a_src[NA_DMA], b_src[2];
   {
-    const int row = 4 * wave + (lane >> 4), pos = lane & 15;
-    a_src = (uint32_t)(min(row, (int)p.M - 1) * lda_b + ((pos ^ (row & 15)) << 4));
+    const int pos = lane & 15;
+#pragma unroll
+    for (int i = 0; i < NA_DMA; i++) {
+      const int row = 4 * (NA_DMA * wave + i) + (lane >> 4);
+      a_src[i] = (uint32_t)(min(row, (int)p.M - 1) * lda_b + ((pos ^ (row & 15)) << 4));
+    }
 #pragma unroll
     for (int i = 0; i < 2; i++) {
       const int rb = 4 * (2 * wave + i) + (lane >> 4);
@@ -107,24 +115,33 @@ __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(GemmParams p) {
   // (the __restrict__ pointers give the requests and the fragment reads separate alias scopes: without them the
   // compiler makes every fragment read wait for all requests in flight)
   auto issue = [&](char *__restrict__ stage, int kt) {
-    __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(a_ptr + (int64_t)kt * KB + a_src), (GCMI_LDS void *)(stage + wave * 1024), 16,
-                                     0, 0);
+#pragma unroll
+    for (int i = 0; i < NA_DMA; i++)
+      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(a_ptr + (int64_t)kt * KB + a_src[i]),
+                                       (GCMI_LDS void *)(stage + (NA_DMA * wave + i) * 1024), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < 2; i++)
       __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(b_ptr + (int64_t)kt * KB + b_src[i]),
                                        (GCMI_LDS void *)(stage + A_BYTES + (2 * wave + i) * 1024), 16, 0, 0);
   };
-  const uint32_t a_ld0 = (uint32_t)(r16 * KB), a_ld1 = (uint32_t)((16 + r16) * KB), b_ld = (uint32_t)(A_BYTES + (16 * ct + r16) * KB);
-  f32x4_t acc[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
+  const uint32_t a_ld = (uint32_t)(r16 * KB), b_ld = (uint32_t)(A_BYTES + (16 * ct + r16) * KB);
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int it = 0; it < MT; it++)
+    acc[it] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   auto compute = [&](const char *__restrict__ st) {
 #pragma unroll
     for (int u = 0; u < 2; u++) {
       const int sw = ((4 * (2 * half + u) + g16) ^ r16) << 4; // rows 16 * x + r16: row % 16 = r16
-      const uint4 fa0 = *reinterpret_cast<const uint4 *>(st + a_ld0 + sw);
-      const uint4 fa1 = *reinterpret_cast<const uint4 *>(st + a_ld1 + sw);
+      uint4 fa[MT];
+#pragma unroll
+      for (int it = 0; it < MT; it++)
+        fa[it] = *reinterpret_cast<const uint4 *>(st + a_ld + it * 16 * KB + sw);
       const uint4 fb = *reinterpret_cast<const uint4 *>(st + b_ld + sw);
-      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fb), __builtin_bit_cast(bf16x8_t, fa0), acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fb), __builtin_bit_cast(bf16x8_t, fa1), acc[1], 0, 0, 0);
+#pragma unroll
+      for (int it = 0; it < MT; it++)
+        acc[it] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fb), __builtin_bit_cast(bf16x8_t, fa[it]), acc[it],
+                                                          0, 0, 0);
     }
   };
 #pragma unroll
@@ -149,15 +166,15 @@ __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(GemmParams p) {
   float *red = reinterpret_cast<float *>(smem);
   if (half == 1) {
 #pragma unroll
-    for (int it = 0; it < 2; it++)
-      *reinterpret_cast<f32x4_t *>(red + ((ct * 2 + it) * 64 + lane) * 4) = acc[it];
+    for (int it = 0; it < MT; it++)
+      *reinterpret_cast<f32x4_t *>(red + ((ct * MT + it) * 64 + lane) * 4) = acc[it];
   }
   __syncthreads();
   float *part = p.partial + (int64_t)slice * p.M * p.N;
   if (half == 0) {
 #pragma unroll
-    for (int it = 0; it < 2; it++) {
-      const f32x4_t o = *reinterpret_cast<const f32x4_t *>(red + ((ct * 2 + it) * 64 + lane) * 4);
+    for (int it = 0; it < MT; it++) {
+      const f32x4_t o = *reinterpret_cast<const f32x4_t *>(red + ((ct * MT + it) * 64 + lane) * 4);
       const f32x4_t v = {acc[it][0] + o[0], acc[it][1] + o[1], acc[it][2] + o[2], acc[it][3] + o[3]};
       const int64_t m = 16 * it + r16;
       const int col = 16 * ct + 4 * g16;
@@ -181,12 +198,12 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
   const int64_t ws_cap = want ? INT64_MAX : (p.partial ? p.partial_cap : 0);
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const int res_es = p.residual_dt == DT_BF16 ? 2 : 4;
-  if (!p.trans_b || p.batch > 1 || p.M < 1 || p.M > R32_BM || p.N % 4 != 0 || p.K % 128 != 0 || p.K < 512 || !al16(p.A) || !al16(p.B) ||
+  if (!p.trans_b || p.batch > 1 || p.M < 1 || p.M > 2 * R32_BM || p.N % 4 != 0 || p.K % 128 != 0 || p.K < 512 || !al16(p.A) || !al16(p.B) ||
       !al16(p.C) || (p.lda * 2) % 16 != 0 || (p.ldb * 2) % 16 != 0 || p.ldc % 4 != 0 || p.out_dt == DT_S32 ||
       (p.residual && (!al16(p.residual) || (p.ldr * res_es) % 8 != 0)) || p.cfg_tile == 128)
     return -1;
   // rows reachable with 32-bit byte offsets from the tile's first row
-  if (p.lda * 2 * R32_BM >= (int64_t)1 << 31 || p.ldb * 2 * R32_BN >= (int64_t)1 << 31)
+  if (p.lda * 2 * 2 * R32_BM >= (int64_t)1 << 31 || p.ldb * 2 * R32_BN >= (int64_t)1 << 31)
     return -1;
   // the weights must be worth streaming: with few of them the tile kernels' launch is as good
   if (p.N * p.K < (int64_t)1 << 22 || p.N < 512)
@@ -198,6 +215,8 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
   // K slices: one workgroup per compute unit where the panels alone leave a third of them idle, four stages or more
   // each, and a workspace that holds the partial sums.  A caller's slice count (its KThreads) replaces the choice.
   int s = 3 * panels >= 2 * n_cu ? 1 : (n_cu + panels / 2) / panels;
+  if (p.M > R32_BM && panels * s > n_cu) // (the 64-row ring leaves room for one workgroup per compute unit)
+    s = n_cu / panels > 1 ? n_cu / panels : 1;
   if (p.cfg_split_k > 0)
     s = p.cfg_split_k;
   if (s > stages / 4)
@@ -210,8 +229,9 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
     *want = s > 1 ? (int64_t)s * p.M * p.N : 0;
   if (cfg) {
     GemmTileConfig c{};
-    c.kernel = GK_STREAM, c.bm = R32_BM, c.bn = R32_BN, c.kbytes = R32_KB, c.stages = R32_NST;
-    c.waves_m = 1, c.waves_n = 4, c.wave_m = R32_BM, c.wave_n = 16, c.mfma_m = c.mfma_n = 16, c.mfma_k = 32;
+    const int bm = p.M <= R32_BM ? R32_BM : 2 * R32_BM;
+    c.kernel = GK_STREAM, c.bm = bm, c.bn = R32_BN, c.kbytes = R32_KB, c.stages = R32_NST;
+    c.waves_m = 1, c.waves_n = 4, c.wave_m = bm, c.wave_n = 16, c.mfma_m = c.mfma_n = 16, c.mfma_k = 32;
     c.split_k = s, c.group_m = 1, c.workgroups = panels * s;
     c.from_attrs = p.cfg_split_k > 0 ? 1 : 0;
     *cfg = c;
@@ -219,7 +239,10 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
   if (dry)
     return 0;
   p.splits = s;
-  hipLaunchKernelGGL(gemm_rows32_kernel, dim3((unsigned)panels, (unsigned)s), dim3(512), 0, stream, p);
+  if (p.M <= R32_BM)
+    hipLaunchKernelGGL(gemm_rows32_kernel<2>, dim3((unsigned)panels, (unsigned)s), dim3(512), 0, stream, p);
+  else
+    hipLaunchKernelGGL(gemm_rows32_kernel<4>, dim3((unsigned)panels, (unsigned)s), dim3(512), 0, stream, p);
   if (s > 1)
     launch_splitk_reduce(p, stream);
   return hipGetLastError() == hipSuccess ? 0 : 5;

@@ -47,7 +47,8 @@ def _pick(kernels, *parts):
     (("mha_fwd_fast_kernel", "ELi4ELb1"), 2, 80 * 1024),  # pipelined attention: two workgroups per compute unit
     (("gemm_tile256_mi16_kernel",), 2, 160 * 1024),
     (("gemm_skinny_nt_kernel",), 2, 64 * 1024),
-    (("gemm_rows32_kernel",), 2, 72 * 1024),            # 8 waves and a ring of three 24 KiB stages: two per compute unit
+    (("gemm_rows32_kernel", "ILi2E"), 2, 72 * 1024),    # 8 waves and a ring of three 24 KiB stages: two per compute unit
+    (("gemm_rows32_kernel", "ILi4E"), 2, 96 * 1024),    # 64 rows of A: three 32 KiB stages, one workgroup per compute unit
     (("gemm_tile128_kernel",), 2, 80 * 1024),           # small tiles: two workgroups per compute unit share its LDS
 ])
 def test_hot_kernels_have_no_scratch_and_keep_their_occupancy(kernels, parts, occupancy, max_lds):
