@@ -1,4 +1,4 @@
-// bf16 GEMM for a short A (M <= 64) against wide weights stored [N,K] (k contiguous): C[M,N] = epilogue(A . W^T).
+// bf16 GEMM for a short A (M <= 128) against wide weights stored [N,K] (k contiguous): C[M,N] = epilogue(A . W^T).
 // This is the decode-time shape of the reference's llama2 case (test/benchgc/cases/llama2.mlir: 32 tokens against
 // 4096 x 4096 .. 4096 x 11008 weights), where the reference splits K over threads (KThreads,
 // lib/gc/Analysis/MatmulConfigAnalysis.cpp:149-166).  The arithmetic is negligible; the job is to pull the weights
@@ -8,9 +8,9 @@
 // of 32 rows 3.2-4.4 -- the vector memory pipe pays per cache line it looks up -- and every fragment of A that a
 // wave fetches for itself costs look-ups of its own.  Hence:
 //   * a workgroup is 8 waves on a panel of 64 columns and one slice of K; a stage is 256 bytes of K per row: the A
-//     tile (32 rows, 8 KiB, shared by all waves; 64 rows and 16 KiB from 33 rows on) and the panel's weights (16 KiB)
-//     go to an LDS ring by global_load_lds_dwordx4, 4 rows x 256 bytes per request, one request (two) for A and two
-//     for the weights per wave;
+//     tile (32 rows, 8 KiB, shared by all waves; 64 or 128 rows past that) and the panel's weights (16 KiB) go to
+//     an LDS ring by global_load_lds_dwordx4, 4 rows x 256 bytes per request, one request (two, four) for A and
+//     two for the weights per wave;
 //   * A is re-read once per panel (half the weights' traffic, from L2) instead of once per 16 columns;
 //   * wave w owns column tile w % 4 and k-steps 2 * (w / 4), 2 * (w / 4) + 1 of the stage's four; the two halves are
 //     added through LDS at the end (upper onto lower: a fixed order); one barrier per stage.
@@ -73,9 +73,9 @@ __device__ __forceinline__ void rows32_store4(const GemmParams &p, const f32x4_t
     *reinterpret_cast<f32x4_t *>(reinterpret_cast<float *>(p.C) + m * p.ldc + n) = f32x4_t{o32[0], o32[1], o32[2], o32[3]};
 }
 
-// MT: 16-row tiles of A (2: up to 32 rows; 4: up to 64 rows, with an A tile of 16 KiB per stage)
+// MT: 16-row tiles of A (2: up to 32 rows; 4: up to 64; 8: up to 128, with an A tile of 16 / 32 KiB per stage)
 template <int MT> __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(GemmParams p) {
-  static_assert(MT == 2 || MT == 4, "32 or 64 rows");
+  static_assert(MT == 2 || MT == 4 || MT == 8, "32, 64 or 128 rows");
   constexpr int KB = R32_KB, BK = KB / 2, NST = R32_NST, BN = R32_BN;
   constexpr int A_BYTES = 16 * MT * KB, B_BYTES = BN * KB, STAGE = A_BYTES + B_BYTES; // 8 (16) + 16 KiB
   constexpr int NA_DMA = MT / 2;    // A requests per wave and stage
@@ -198,12 +198,12 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
   const int64_t ws_cap = want ? INT64_MAX : (p.partial ? p.partial_cap : 0);
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const int res_es = p.residual_dt == DT_BF16 ? 2 : 4;
-  if (!p.trans_b || p.batch > 1 || p.M < 1 || p.M > 2 * R32_BM || p.N % 4 != 0 || p.K % 128 != 0 || p.K < 512 || !al16(p.A) || !al16(p.B) ||
+  if (!p.trans_b || p.batch > 1 || p.M < 1 || p.M > 4 * R32_BM || p.N % 4 != 0 || p.K % 128 != 0 || p.K < 512 || !al16(p.A) || !al16(p.B) ||
       !al16(p.C) || (p.lda * 2) % 16 != 0 || (p.ldb * 2) % 16 != 0 || p.ldc % 4 != 0 || p.out_dt == DT_S32 ||
       (p.residual && (!al16(p.residual) || (p.ldr * res_es) % 8 != 0)) || p.cfg_tile == 128)
     return -1;
   // rows reachable with 32-bit byte offsets from the tile's first row
-  if (p.lda * 2 * 2 * R32_BM >= (int64_t)1 << 31 || p.ldb * 2 * R32_BN >= (int64_t)1 << 31)
+  if (p.lda * 2 * 4 * R32_BM >= (int64_t)1 << 31 || p.ldb * 2 * R32_BN >= (int64_t)1 << 31)
     return -1;
   // the weights must be worth streaming: with few of them the tile kernels' launch is as good
   if (p.N * p.K < (int64_t)1 << 22 || p.N < 512)
@@ -215,7 +215,7 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
   // K slices: one workgroup per compute unit where the panels alone leave a third of them idle, four stages or more
   // each, and a workspace that holds the partial sums.  A caller's slice count (its KThreads) replaces the choice.
   int s = 3 * panels >= 2 * n_cu ? 1 : (n_cu + panels / 2) / panels;
-  if (p.M > R32_BM && panels * s > n_cu) // (the 64-row ring leaves room for one workgroup per compute unit)
+  if (p.M > R32_BM && panels * s > n_cu) // (the larger rings leave room for one workgroup per compute unit)
     s = n_cu / panels > 1 ? n_cu / panels : 1;
   if (p.cfg_split_k > 0)
     s = p.cfg_split_k;
@@ -229,7 +229,7 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
     *want = s > 1 ? (int64_t)s * p.M * p.N : 0;
   if (cfg) {
     GemmTileConfig c{};
-    const int bm = p.M <= R32_BM ? R32_BM : 2 * R32_BM;
+    const int bm = p.M <= R32_BM ? R32_BM : (p.M <= 2 * R32_BM ? 2 * R32_BM : 4 * R32_BM);
     c.kernel = GK_STREAM, c.bm = bm, c.bn = R32_BN, c.kbytes = R32_KB, c.stages = R32_NST;
     c.waves_m = 1, c.waves_n = 4, c.wave_m = bm, c.wave_n = 16, c.mfma_m = c.mfma_n = 16, c.mfma_k = 32;
     c.split_k = s, c.group_m = 1, c.workgroups = panels * s;
@@ -241,8 +241,10 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
   p.splits = s;
   if (p.M <= R32_BM)
     hipLaunchKernelGGL(gemm_rows32_kernel<2>, dim3((unsigned)panels, (unsigned)s), dim3(512), 0, stream, p);
-  else
+  else if (p.M <= 2 * R32_BM)
     hipLaunchKernelGGL(gemm_rows32_kernel<4>, dim3((unsigned)panels, (unsigned)s), dim3(512), 0, stream, p);
+  else
+    hipLaunchKernelGGL(gemm_rows32_kernel<8>, dim3((unsigned)panels, (unsigned)s), dim3(512), 0, stream, p);
   if (s > 1)
     launch_splitk_reduce(p, stream);
   return hipGetLastError() == hipSuccess ? 0 : 5;

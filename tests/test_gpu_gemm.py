@@ -602,7 +602,7 @@ NT_SHAPES = [(256, 256, 128), (512, 768, 256), (300, 200, 100), (257, 511, 129),
 def _streams_weights(M, N, K):
     """Shapes the [N,K] entry point gives to one of the weight-streaming kernels (short A, enough weights): the
     8-wave kernel with the LDS ring, or the one that loads fragments straight into registers."""
-    ring = M <= 64 and N % 4 == 0 and N >= 512 and K % 128 == 0 and K >= 512 and N * K >= 1 << 22
+    ring = M <= 128 and N % 4 == 0 and N >= 512 and K % 128 == 0 and K >= 512 and N * K >= 1 << 22
     return ring or (M <= 32 and N % 32 == 0 and K % 64 == 0 and K >= 256 and 1 << 20 <= N * K <= 3 << 23)
 
 
@@ -659,15 +659,15 @@ def test_bf16_gemm_streaming_kernel_exact_on_integers(gc, dev):
         assert torch.equal(out2, out)
 
 
-@pytest.mark.parametrize("M", [1, 7, 16, 32, 33, 50, 64])
+@pytest.mark.parametrize("M", [1, 7, 16, 32, 33, 50, 64, 65, 100, 128])
 @pytest.mark.parametrize("N,K", [(4096, 1024), (4100, 4096), (520, 11008), (11008, 4096), (12352, 640)])
 def test_short_a_streaming_kernel_exact_on_integers(gc, dev, M, N, K):
-    """Up to 64 rows against [N,K] weights (from 33 rows on the A tile of the ring holds 64): 8-wave workgroups on panels of 64 columns (the last one 4 or 8 columns
+    """Up to 128 rows against [N,K] weights (the A tile of the ring holds 32, 64 or 128): 8-wave workgroups on panels of 64 columns (the last one 4 or 8 columns
     wide here), K in one piece where the panels fill the GPU and in slices with the second pass where they do not,
     slice lengths that differ (86 and 5 stages), rows past M.  Small integers: every sum is exact in f32, whatever
     the order.  The caller's slice count and a call without workspace (one slice, epilogue in the kernel) agree."""
     c, _ = gc.tile_config(M, N, K, trans_b=True, out_dtype=gc.F32)
-    assert (c.kernel, c.bm, c.bn, c.waves_m * c.waves_n) == (4, 32 if M <= 32 else 64, 64, 4) and c.workgroups == -(-N // 64) * c.split_k
+    assert (c.kernel, c.bm, c.bn, c.waves_m * c.waves_n) == (4, 32 if M <= 32 else (64 if M <= 64 else 128), 64, 4) and c.workgroups == -(-N // 64) * c.split_k
     want_s = (256 + -(-N // 64) // 2) // -(-N // 64)
     if M > 32 and want_s * -(-N // 64) > 256:   # the 64-row ring: one workgroup per compute unit
         want_s = max(1, 256 // -(-N // 64))
@@ -691,7 +691,8 @@ def test_short_a_streaming_kernel_exact_on_integers(gc, dev, M, N, K):
     assert torch.equal(one, want) and torch.equal(three, want)
 
 
-@pytest.mark.parametrize("M,N,K", [(32, 4096, 4096), (9, 11008, 4096), (32, 4096, 11008), (20, 1032, 4096), (64, 4096, 4096), (40, 11008, 4096)])
+@pytest.mark.parametrize("M,N,K", [(32, 4096, 4096), (9, 11008, 4096), (32, 4096, 11008), (20, 1032, 4096), (64, 4096, 4096), (40, 11008, 4096), (128, 4096, 4096),
+                                   (77, 11008, 4096)])
 def test_short_a_streaming_kernel_rounding_points(gc, dev, M, N, K):
     """N(0,1) data through bias, GELU and a residual, bf16 and f32 results: against the same sums in float64 rounded
     at the reference's points (after the matmul and after each op for bf16 results), to one bf16 step of the larger of

@@ -49,6 +49,7 @@ def _pick(kernels, *parts):
     (("gemm_skinny_nt_kernel",), 2, 64 * 1024),
     (("gemm_rows32_kernel", "ILi2E"), 2, 72 * 1024),    # 8 waves and a ring of three 24 KiB stages: two per compute unit
     (("gemm_rows32_kernel", "ILi4E"), 2, 96 * 1024),    # 64 rows of A: three 32 KiB stages, one workgroup per compute unit
+    (("gemm_rows32_kernel", "ILi8E"), 2, 144 * 1024),   # 128 rows of A: three 48 KiB stages
     (("gemm_tile128_kernel",), 2, 80 * 1024),           # small tiles: two workgroups per compute unit share its LDS
 ])
 def test_hot_kernels_have_no_scratch_and_keep_their_occupancy(kernels, parts, occupancy, max_lds):

@@ -48,8 +48,10 @@ def test_defaults_per_shape(gc):
     assert (c.kernel, c.workgroups) == (2, 688)
     c, _ = gc.tile_config(64, 4096, 4096, trans_b=True)                 # [N,K] weights, 64 rows: streamed, A tile of 64 rows
     assert (c.kernel, c.bm, c.bn, c.split_k) == (4, 64, 64, 4)
-    c, _ = gc.tile_config(65, 4096, 4096, trans_b=True)                 # one row more: slices of small tiles
-    assert (c.kernel, c.bm, c.split_k) == (3, 128, 8)
+    c, _ = gc.tile_config(128, 4096, 4096, trans_b=True)                # up to 128 rows likewise
+    assert (c.kernel, c.bm, c.bn, c.split_k) == (4, 128, 64, 4)
+    c, _ = gc.tile_config(129, 4096, 4096, trans_b=True)                # one row more: slices of small tiles
+    assert (c.kernel, c.bm, c.split_k) == (3, 128, 4)
     c, _ = gc.tile_config(32, 4096, 4096, trans_b=True)                 # [N,K] weights, short A: streamed
     assert c.kernel == 4 and c.split_k >= 4
 
