@@ -414,11 +414,9 @@ def main():
             dec["%dx%dx%d" % (Md, Nd, Kdd)] = entry
             del sets
             torch.cuda.empty_cache()
-        others["bf16_decode_gemm"] = {"workload": "A[32 x K] . W bf16 with W stored [K,N] and [N,K]: [K,N] by K slices over 128 x 128 tiles or "
-                                                  "over the 256-wide tile kernel that skips empty row blocks (two launches: partial sums, "
-                                                  "then reduction + epilogue); [N,K] by the 8-wave weight-streaming kernel on panels of 64 "
-                                                  "columns (one launch for N = 11008, K slices + second pass for N = 4096); "
-                                                  "algorithmic bytes = A + W + C once",
+        others["bf16_decode_gemm"] = {"workload": "A[32 x K] . W bf16 with W stored [K,N] and [N,K]: the 8-wave weight-streaming kernel "
+                                                  "on panels of 64 columns (one launch for N = 11008; K slices + reduction and epilogue "
+                                                  "in a second launch for N = 4096); algorithmic bytes = A + W + C once",
                                       "shapes": dec}
 
     # ---------------- the same kernels on shapes off their tile sizes (parity cases elsewhere; here: no cliff)

@@ -669,35 +669,26 @@ void Executable::plan() {
       int64_t N = tB ? bs[Rb - 2] : bs[Rb - 1];
       int sa_slot = slot_for(mm.in[0]), sb_slot = slot_for(mm.in[1]);
       DT out_dt = T(mm.out[0]).dt;
-      // a transposed bf16 copy of an operand (once per executable when the operand is a constant: the analogue of the
-      // reference's weight pre-packing of constant tensors, docs/CPU_pipeline_overview.md:58)
-      auto transposed = [&](int slot, std::vector<int64_t> &shp, bool constant) {
-        std::vector<int64_t> st = dense_strides(shp), d = shp;
-        std::swap(d[d.size() - 1], d[d.size() - 2]);
-        std::swap(st[st.size() - 1], st[st.size() - 2]);
-        int t = new_slot((size_t)prod(shp, 0, shp.size()) * 2);
-        if (d.size() > (size_t)gcmi::ELT_MAX_RANK)
-          throw std::logic_error("tensor rank above 6 is not supported");
-        Step cp;
-        cp.kind = Step::Elt, cp.note = constant ? "transpose copy, once: the operand is constant" : "transpose copy";
-        cp.once = constant, cp.op = gcmi::ELT_COPY, cp.a = slot, cp.out = t;
-        cp.a_dt = cp.out_dt = GCMI_BF16, cp.dims = d, cp.sa = st;
-        v.push_back(cp);
-        shp = d;
-        return t;
-      };
-      if (A.dt == DT::bf16 && tA) // the bf16 kernel reads A row-major [M,K] (B may be stored either way)
+      if (A.dt == DT::bf16 && tA) {
+        // the bf16 kernel reads A row-major [M,K] (B may be stored either way): materialise a transposed A
+        // (once per executable when the operand is a constant: the analogue of the reference's weight
+        // pre-packing of constant tensors, docs/CPU_pipeline_overview.md:58)
+        auto transposed = [&](int slot, std::vector<int64_t> &shp, bool constant) {
+          std::vector<int64_t> st = dense_strides(shp), d = shp;
+          std::swap(d[d.size() - 1], d[d.size() - 2]);
+          std::swap(st[st.size() - 1], st[st.size() - 2]);
+          int t = new_slot((size_t)prod(shp, 0, shp.size()) * 2);
+          if (d.size() > (size_t)gcmi::ELT_MAX_RANK)
+            throw std::logic_error("tensor rank above 6 is not supported");
+          Step cp;
+          cp.kind = Step::Elt, cp.note = constant ? "transpose copy, once: the operand is constant" : "transpose copy";
+          cp.once = constant, cp.op = gcmi::ELT_COPY, cp.a = slot, cp.out = t;
+          cp.a_dt = cp.out_dt = GCMI_BF16, cp.dims = d, cp.sa = st;
+          v.push_back(cp);
+          shp = d;
+          return t;
+        };
         sa_slot = transposed(sa_slot, as, A.constant), tA = false;
-      // Up to 32 rows against a wide constant weight stored [K,N]: the weights have to stream from HBM, and the kernel
-      // that streams them best reads rows of K (gemm_rows32_kernel; 32 x 4096 x 4096 14 against 19 us, 32 x 11008 x
-      // 4096 22 against 27), so the constant is kept as a [N,K] copy as well -- the counterpart of the reference's
-      // VNNI pre-pack of constant weights (lib/gc/Transforms/Microkernel/ConvertLinalgToMicrokernel.cpp:163-176).
-      if (A.dt == DT::bf16 && !tB && !b1 && Rb == 2 && B.constant && !tA) {
-        int64_t rows = M;
-        for (size_t d = 0; d + 2 < Ra; d++)
-          rows *= as[d];
-        if (rows <= 32 && K % 128 == 0 && K >= 512 && N % 4 == 0 && N >= 512 && N * K >= ((int64_t)1 << 22))
-          sb_slot = transposed(sb_slot, bs, true), tB = true;
       }
       std::vector<int64_t> ba(as.begin(), as.end() - 2), bb(bs.begin(), bs.end() - 2), bo;
       broadcast_shape(ba, bb, bo);

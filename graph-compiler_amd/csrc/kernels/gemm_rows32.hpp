@@ -1,4 +1,5 @@
-// bf16 GEMM for a short A (M <= 128) against wide weights stored [N,K] (k contiguous): C[M,N] = epilogue(A . W^T).
+// bf16 GEMM for a short A (M <= 128) against wide weights, stored [N,K] (k contiguous) or [K,N]:
+// C[M,N] = epilogue(A . W).
 // This is the decode-time shape of the reference's llama2 case (test/benchgc/cases/llama2.mlir: 32 tokens against
 // 4096 x 4096 .. 4096 x 11008 weights), where the reference splits K over threads (KThreads,
 // lib/gc/Analysis/MatmulConfigAnalysis.cpp:149-166).  The arithmetic is negligible; the job is to pull the weights
@@ -22,8 +23,9 @@
 // twice and is slower than the second kernel: with device-scope fences every workgroup writes back and invalidates
 // an L2 that the others stream through, 59 against 14 us; with device-scope stores and loads instead of fences the
 // word-sized write-through stores cost more than the launch saves, 12.9 against 11.2 us.)
-// Measured: 32 x 4096 x 4096 11.0 us (13.2 us with 32-byte pieces straight into registers), 32 x 11008 x 4096
-// 22.7 us in one launch (28.9), 32 x 4096 x 11008 23.5 us (28.4).
+// Measured, [N,K] / [K,N]: 32 x 4096 x 4096 11.0 / 11.1 us (13.2 us with 32-byte pieces straight into registers; 16 us
+// on K slices of 128 x 128 tiles), 32 x 11008 x 4096 22.7 / 23.1 us in one launch (28.9; 24), 32 x 4096 x 11008
+// 23.5 / 24.0 us (28.4; 24).
 #pragma once
 #include "gemm_tile256.hpp"
 
@@ -74,7 +76,11 @@ __device__ __forceinline__ void rows32_store4(const GemmParams &p, const f32x4_t
 }
 
 // MT: 16-row tiles of A (2: up to 32 rows; 4: up to 64; 8: up to 128, with an A tile of 16 / 32 KiB per stage)
-template <int MT> __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(GemmParams p) {
+// TB: the weights are stored [N,K]; else [K,N]: a stage's weights are then 128 k-rows of 128 bytes (the panel's 64
+// columns), requested 8 k-rows at a time (whole lines again) and read through the transposing LDS load; a k-row's 8
+// chunks sit at chunk ^ 2 * (k / 2 % 2 + 2 * (k / 8 % 2)), which spreads the 8 k-rows that 32 lanes of a transposing
+// read touch over all banks.
+template <int MT, bool TB> __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(GemmParams p) {
   static_assert(MT == 2 || MT == 4 || MT == 8, "32, 64 or 128 rows");
   constexpr int KB = R32_KB, BK = KB / 2, NST = R32_NST, BN = R32_BN;
   constexpr int A_BYTES = 16 * MT * KB, B_BYTES = BN * KB, STAGE = A_BYTES + B_BYTES; // 8 (16) + 16 KiB
@@ -106,12 +112,19 @@ template <int MT> __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(G
     }
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-      const int rb = 4 * (2 * wave + i) + (lane >> 4);
-      b_src[i] = (uint32_t)(min(rb, cols_in - 1) * ldb_b + ((pos ^ (rb & 15)) << 4));
+      if constexpr (TB) {
+        const int rb = 4 * (2 * wave + i) + (lane >> 4);
+        b_src[i] = (uint32_t)(min(rb, cols_in - 1) * ldb_b + ((pos ^ (rb & 15)) << 4));
+      } else {
+        const int krow = 8 * (2 * wave + i) + (lane >> 3), c8 = lane & 7;
+        const int swz = (((krow >> 1) & 1) | (((krow >> 3) & 1) << 1)) << 1;
+        b_src[i] = (uint32_t)(krow * ldb_b + (min(c8 ^ swz, cols_in / 8 - 1) << 4));
+      }
     }
   }
   const char *a_ptr = reinterpret_cast<const char *>(p.A) + (int64_t)k_first * KB;
-  const char *b_ptr = reinterpret_cast<const char *>(p.B) + n0 * ldb_b + (int64_t)k_first * KB;
+  const int64_t b_step = TB ? (int64_t)KB : (int64_t)BK * ldb_b; // bytes from one stage of the weights to the next
+  const char *b_ptr = reinterpret_cast<const char *>(p.B) + (TB ? n0 * ldb_b : n0 * 2) + (int64_t)k_first * b_step;
   // (the __restrict__ pointers give the requests and the fragment reads separate alias scopes: without them the
   // compiler makes every fragment read wait for all requests in flight)
   auto issue = [&](char *__restrict__ stage, int kt) {
@@ -121,10 +134,16 @@ template <int MT> __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(G
                                        (GCMI_LDS void *)(stage + (NA_DMA * wave + i) * 1024), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < 2; i++)
-      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(b_ptr + (int64_t)kt * KB + b_src[i]),
+      __builtin_amdgcn_global_load_lds((GCMI_GLB const void *)(b_ptr + kt * b_step + b_src[i]),
                                        (GCMI_LDS void *)(stage + A_BYTES + (2 * wave + i) * 1024), 16, 0, 0);
   };
-  const uint32_t a_ld = (uint32_t)(r16 * KB), b_ld = (uint32_t)(A_BYTES + (16 * ct + r16) * KB);
+  const uint32_t a_ld = (uint32_t)(r16 * KB);
+  uint32_t b_ld = (uint32_t)(A_BYTES + (16 * ct + r16) * KB);
+  if constexpr (!TB) { // the 16 lanes of a group hand the transposing read 4 k-rows x 16 columns in 8-byte pieces
+    const int kk = r16 >> 2, cc = r16 & 3;
+    const int swz = (((kk >> 1) & 1) | ((g16 & 1) << 1)) << 1; // of k-row 8 * g16 + kk (+ 4, + 32 per k-step: the same)
+    b_ld = (uint32_t)(A_BYTES + (8 * g16 + kk) * 128 + (((2 * ct + (cc >> 1)) ^ swz) << 4) + (cc & 1) * 8);
+  }
   f32x4_t acc[MT];
 #pragma unroll
   for (int it = 0; it < MT; it++)
@@ -137,7 +156,14 @@ template <int MT> __global__ __launch_bounds__(512, 1) void gemm_rows32_kernel(G
 #pragma unroll
       for (int it = 0; it < MT; it++)
         fa[it] = *reinterpret_cast<const uint4 *>(st + a_ld + it * 16 * KB + sw);
-      const uint4 fb = *reinterpret_cast<const uint4 *>(st + b_ld + sw);
+      uint4 fb;
+      if constexpr (TB) {
+        fb = *reinterpret_cast<const uint4 *>(st + b_ld + sw);
+      } else {
+        const uint2 lo = MfmaOp<2>::tr_read(st + b_ld + (2 * half + u) * 4096);
+        const uint2 hi = MfmaOp<2>::tr_read(st + b_ld + (2 * half + u) * 4096 + 512);
+        fb = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
 #pragma unroll
       for (int it = 0; it < MT; it++)
         acc[it] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fb), __builtin_bit_cast(bf16x8_t, fa[it]), acc[it],
@@ -198,12 +224,16 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
   const int64_t ws_cap = want ? INT64_MAX : (p.partial ? p.partial_cap : 0);
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const int res_es = p.residual_dt == DT_BF16 ? 2 : 4;
-  if (!p.trans_b || p.batch > 1 || p.M < 1 || p.M > 4 * R32_BM || p.N % 4 != 0 || p.K % 128 != 0 || p.K < 512 || !al16(p.A) || !al16(p.B) ||
+  if (p.batch > 1 || p.M < 1 || p.M > 4 * R32_BM || p.N % (p.trans_b ? 4 : 8) != 0 || p.K % 128 != 0 || p.K < 512 || !al16(p.A) || !al16(p.B) ||
       !al16(p.C) || (p.lda * 2) % 16 != 0 || (p.ldb * 2) % 16 != 0 || p.ldc % 4 != 0 || p.out_dt == DT_S32 ||
       (p.residual && (!al16(p.residual) || (p.ldr * res_es) % 8 != 0)) || p.cfg_tile == 128)
     return -1;
+  // [K,N] weights: a caller's MatmulConfig names a workgroup tile, and that tile it gets (with [N,K] weights only the
+  // slice count of such a config is used)
+  if (!p.trans_b && p.cfg_tile != 0)
+    return -1;
   // rows reachable with 32-bit byte offsets from the tile's first row
-  if (p.lda * 2 * 4 * R32_BM >= (int64_t)1 << 31 || p.ldb * 2 * R32_BN >= (int64_t)1 << 31)
+  if (p.lda * 2 * 4 * R32_BM >= (int64_t)1 << 31 || p.ldb * 2 * 128 >= (int64_t)1 << 31)
     return -1;
   // the weights must be worth streaming: with few of them the tile kernels' launch is as good
   if (p.N * p.K < (int64_t)1 << 22 || p.N < 512)
@@ -239,12 +269,23 @@ static int launch_rows32(const GemmParams *pp, hipStream_t stream, int64_t *want
   if (dry)
     return 0;
   p.splits = s;
-  if (p.M <= R32_BM)
-    hipLaunchKernelGGL(gemm_rows32_kernel<2>, dim3((unsigned)panels, (unsigned)s), dim3(512), 0, stream, p);
-  else if (p.M <= 2 * R32_BM)
-    hipLaunchKernelGGL(gemm_rows32_kernel<4>, dim3((unsigned)panels, (unsigned)s), dim3(512), 0, stream, p);
-  else
-    hipLaunchKernelGGL(gemm_rows32_kernel<8>, dim3((unsigned)panels, (unsigned)s), dim3(512), 0, stream, p);
+  const dim3 grid((unsigned)panels, (unsigned)s), block(512);
+  const int mt = p.M <= R32_BM ? 2 : (p.M <= 2 * R32_BM ? 4 : 8);
+  if (p.trans_b) {
+    if (mt == 2)
+      hipLaunchKernelGGL((gemm_rows32_kernel<2, true>), grid, block, 0, stream, p);
+    else if (mt == 4)
+      hipLaunchKernelGGL((gemm_rows32_kernel<4, true>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((gemm_rows32_kernel<8, true>), grid, block, 0, stream, p);
+  } else {
+    if (mt == 2)
+      hipLaunchKernelGGL((gemm_rows32_kernel<2, false>), grid, block, 0, stream, p);
+    else if (mt == 4)
+      hipLaunchKernelGGL((gemm_rows32_kernel<4, false>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((gemm_rows32_kernel<8, false>), grid, block, 0, stream, p);
+  }
   if (s > 1)
     launch_splitk_reduce(p, stream);
   return hipGetLastError() == hipSuccess ? 0 : 5;

@@ -304,38 +304,6 @@ def test_constant_transposed_weight_is_prepared_once(ga, orc, wl, dev):
         comp.close()
 
 
-def test_constant_weight_of_a_short_product_is_kept_row_major_in_k(ga, orc, wl, dev):
-    """x[32,K] . W with a wide W stored [K,N]: as a constant it is copied to [N,K] once, the layout the weight-streaming
-    kernel reads, and the product runs on that kernel; as a variable it is read where it lies.  Both give the oracle's
-    result; the second execute with another buffer under the constant's id still multiplies by the first contents."""
-    M, K, N = 32, 2048, 2048
-    torch.manual_seed(23)
-    x = (torch.randn(M, K) * 0.5).to(torch.bfloat16)
-    W = (torch.randn(K, N) * 0.05).to(torch.bfloat16)
-    W2 = (torch.randn(K, N) * 0.05).to(torch.bfloat16)
-
-    def graph(prop):
-        return ga._graph([{"kind": "MatMul", "inputs": [ga._t(0, "bf16", [M, K]), ga._t(1, "bf16", [K, N], property_type=prop)],
-                           "outputs": [ga._t(2, "bf16", [M, N])]}], [0, 1], [2])
-
-    ref1 = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(x), wl.bf16_bits(W)))
-    ref2 = orc.bf16_to_f32(orc.matmul_bf16(wl.bf16_bits(x), wl.bf16_bits(W2)))
-    for prop, second in (("constant", ref1), ("variable", ref2)):
-        st, plan = ga.explain(graph(prop))
-        assert st == 0, plan
-        assert ("transpose copy, once" in plan) == (prop == "constant"), plan
-        assert ("weight streaming" in plan) == (prop == "constant"), plan
-        comp = ga.Compiler()
-        st, exe = comp.compile(graph(prop))
-        assert st == 0, ga.api().dnnl_graph_compiler_last_error().decode()
-        out = torch.zeros(M, N, dtype=torch.bfloat16)
-        for Wt, ref in ((W, ref1), (W2, second)):
-            assert exe.execute([(0, x.to(dev)), (1, Wt.to(dev))], [(2, out)]) == 0
-            assert_close(ref, out.float().numpy(), 1e-2, "short product, %s weight" % prop)
-        exe.close()
-        comp.close()
-
-
 def test_transposed_b_weight_needs_no_copy(ga, orc, wl, dev):
     """x[32,512] . W^T with W stored [N,K] (transpose_b, as the reference's llama2 case stores its weights):
     one GEMM launch that reads W as it lies."""

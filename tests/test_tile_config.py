@@ -26,16 +26,20 @@ def test_defaults_per_shape(gc):
     assert (c.kernel, c.waves_m * c.waves_n, c.wave_n, c.from_attrs) == (1, 8, 64, 1)
     c, _ = gc.tile_config(300, 200, 100)                                # ragged: bounds-checked tile
     assert c.kernel == 0
-    c, _ = gc.tile_config(32, 4096, 4096)                               # one tile row: K slices fill the GPU
-    assert c.kernel == 3 and (c.bm, c.bn) == (128, 128) and c.split_k == 8 and c.workgroups == 32 * 8
-    c, _ = gc.tile_config(16, 4096, 4096)                               # fewer rows: the kernel that skips empty row blocks
-    assert c.kernel == 3 and (c.bm, c.bn) == (256, 256) and c.split_k == 16 and c.workgroups == 16 * 16
+    c, _ = gc.tile_config(32, 4096, 4096)                               # a short A: the weights are streamed, K slices fill the GPU
+    assert c.kernel == 4 and (c.bm, c.bn) == (32, 64) and c.split_k == 4 and c.workgroups == 64 * 4
+    c, _ = gc.tile_config(16, 11008, 4096)                              # 172 panels: no slices, one launch
+    assert c.kernel == 4 and (c.bm, c.bn) == (32, 64) and c.split_k == 1 and c.workgroups == 172
+    c, _ = gc.tile_config(32, 4096, 4096, matmul_config=_cfg(KThreads=8))   # the 256 x 256 tile by name: K slices of it
+    assert c.kernel == 3 and (c.bm, c.bn) == (256, 256) and c.split_k == 8 and c.workgroups == 16 * 8
     c, _ = gc.tile_config(2048, 2048, 2048)                             # 64 large tiles: small tiles instead
     assert (c.kernel, c.bm, c.wave_m, c.wave_n, c.split_k, c.workgroups) == (5, 128, 64, 64, 1, 256)
     c, _ = gc.tile_config(1024, 1024, 8192)                             # and a deep K: slices of small tiles
     assert (c.kernel, c.bm, c.split_k, c.workgroups) == (3, 128, 4, 256)
-    c, _ = gc.tile_config(128, 4096, 11008)                             # 86 ring groups of K: slices of unequal length
-    assert (c.kernel, c.bm, c.split_k, c.workgroups) == (3, 128, 8, 256)
+    c, _ = gc.tile_config(128, 4096, 11008)                             # up to 128 rows the weights are streamed
+    assert (c.kernel, c.bm, c.bn, c.split_k, c.workgroups) == (4, 128, 64, 4, 256)
+    c, _ = gc.tile_config(192, 4096, 11008)                             # past that: slices of small tiles, of unequal length (86 ring groups)
+    assert (c.kernel, c.bm, c.split_k) == (3, 128, 4)
     c, _ = gc.tile_config(2048, 11008, 4096)                            # 344 large tiles: more than a round, they stay
     assert (c.kernel, c.bm, c.split_k, c.workgroups) == (2, 256, 1, 344)
     c, _ = gc.tile_config(1024, 4096, 4096, a_dtype=gc.U8)              # 8-bit, 64 large tiles: small tiles, never K slices

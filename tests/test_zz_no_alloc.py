@@ -72,7 +72,7 @@ def test_noalloc_allocates_nothing_and_can_be_captured(gc, dev):
     replays to the eager result (several replays with eager work in between: the graph names the static array, whose
     address never changes).  The allocating entry point refuses a capturing stream with a message that names the
     alternatives."""
-    M, N, K = 128, 8192, 4096     # K-sliced, 16 MiB of partial sums: beyond the library workspace's first size
+    M, N, K = 192, 8192, 4096     # K-sliced, 12 MiB of partial sums: beyond the library workspace's first size
     assert gc.lib().gcmi_gemm_bf16_workspace_bytes(M, N, K, 0) > 8 << 20
     torch.manual_seed(3)
     A = (torch.randn(M, K) * 0.5).to(torch.bfloat16).to(dev)
