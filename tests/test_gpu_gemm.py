@@ -682,6 +682,15 @@ def test_short_a_streaming_kernel_exact_on_integers(gc, dev, M, N, K):
     torch.cuda.synchronize()
     assert torch.equal(out, want)
     assert bool((guard[0] == 7.0).all()) and bool((guard[M + 1] == 7.0).all())
+    # the same weights stored [K,N]: the same kernel with transposing fragment reads (N a multiple of 8), else tiles
+    B = Bt.t().contiguous()
+    ckn, _ = gc.tile_config(M, N, K, out_dtype=gc.F32)
+    assert (ckn.kernel == 4) == (N % 8 == 0), (ckn.kernel, N)
+    guard_kn = torch.full((M + 2, N), 7.0, dtype=torch.float32, device=dev)
+    gc.gemm_bf16(A, B, out_dtype=gc.F32, out=guard_kn[1:M + 1])
+    torch.cuda.synchronize()
+    assert torch.equal(guard_kn[1:M + 1], want)
+    assert bool((guard_kn[0] == 7.0).all()) and bool((guard_kn[M + 1] == 7.0).all())
     one = torch.full((M, N), 7.0, dtype=torch.float32, device=dev)
     _gemm_ws(gc, A, Bt, True, one)  # no workspace: K in one piece
     ws = torch.empty(3 * M * N, dtype=torch.float32, device=dev)
@@ -715,6 +724,12 @@ def test_short_a_streaming_kernel_rounding_points(gc, dev, M, N, K):
     _gemm_ws(gc, A, Bt, True, s16, 4, bias=bias, act="gelu_erf", residual=res, ws=ws)
     torch.cuda.synchronize()
     mag = torch.maximum(acc.abs(), torch.maximum(want16.abs(), res.double().abs())) + 1.0
+    # [K,N] weights: the same products in the same order, so the same bits
+    k16 = torch.empty_like(o16)
+    _gemm_ws(gc, A, Bt.t().contiguous(), False, k16, bias=bias, act="gelu_erf", residual=res)
+    torch.cuda.synchronize()
+    if N % 8 == 0:
+        assert torch.equal(k16.view(torch.int16), o16.view(torch.int16))
     # a bias given as f32 holds the same values: the same bits come out
     assert torch.equal(gc.gemm_bf16_nt(A, Bt, bias.float(), "relu", gc.F32), gc.gemm_bf16_nt(A, Bt, bias, "relu", gc.F32))
     assert float(((o16.double() - want16).abs() / mag).max()) < 2.0 ** -7
