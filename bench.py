@@ -388,7 +388,9 @@ def main():
     if want("decode"):
         dec = {}
         for (Md, Nd, Kdd) in [(32, 4096, 4096), (32, 11008, 4096), (32, 4096, 11008)]:
-            nsets = 4  # 4 x 32..90 MB of weights: beyond the Infinity Cache in rotation
+            # weight buffers in rotation: 600 MB or more of them, so that none is left in the 256 MB last-level cache
+            # when its turn comes again (4 x 32 MB would be served from that cache)
+            nsets = max(4, -(-600_000_000 // (2 * Nd * Kdd)))
             sets = []
             for s in range(nsets):
                 torch.manual_seed(100 + s)
