@@ -118,6 +118,8 @@ def time_launches(torch, fn, nsets, steps, warmup):
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script with
 # --copy-calibration: a 1 GiB copy reads FETCH_SIZE = 524304 KiB (scale 2.0)
 # and WRITE_SIZE = 1048580 KiB (scale 1.0).
+# bytes the main kernel of a decode-shaped GEMM fetches per launch (FETCH_SIZE, scaled as above), by (N, K)
+DECODE_TRAFFIC = {(4096, 4096): 35_800_000, (11008, 4096): 92_500_000, (4096, 11008): 95_900_000}
 TRAFFIC = {  # (bytes per launch of the dominant kernel, the committed profile they come from)
     "gemm": (235414490, "profiles/gemm_tile256_w4_bf16_4096cubed.md"),
     "int8": (384693096, "profiles/gemm_tile256_w4_int8_mlp_layer.md"),
@@ -410,7 +412,8 @@ def main():
                 entry["weights_" + layout] = {
                     "ms_per_step": round(t["ms_per_step"], 5), "kernel_ms_mean": round(t["kernel_ms_mean"], 5),
                     "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
+                                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC.get((Nd, Kdd)),
+                                 "traffic_source": "profiles/gemm_rows32_bf16_decode_shapes.md"}}
                 log("bf16 decode gemm %dx%dx%d weights [%s]: %.4f ms  %.0f GB/s of operands" %
                     (Md, Nd, Kdd, layout, t["ms_per_step"], gbs))
             dec["%dx%dx%d" % (Md, Nd, Kdd)] = entry
