@@ -62,7 +62,7 @@ enum GemmKernel : int32_t {
   GK_WAVES8 = 1,  // whole tiles, 8 waves of 128 x 64, 16x16 MFMAs
   GK_WAVES4 = 2,  // whole tiles, 4 waves of 128 x 128 (one per SIMD), 16x16 MFMAs, hand-placed main loop
   GK_SPLITK = 3,  // too few tiles for the GPU: K slices over workgroups + second pass
-  GK_STREAM = 4,  // a short A against [N,K] weights: weight-streaming kernel (+ second pass)
+  GK_STREAM = 4,  // a short A against wide weights: weight-streaming kernel (+ second pass where K is sliced)
   GK_TILE128 = 5, // 128 x 128 tiles, 4 waves of 64 x 64, two workgroups per compute unit: problems of few 256 x 256 tiles
 };
 

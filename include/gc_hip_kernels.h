@@ -145,7 +145,9 @@ int gcmi_gemm_bf16_ws(const void *A, const void *B, void *C, int64_t batch, int6
  * N a multiple of 16 bytes of columns: edge tiles store what lies inside C),
  * 3 K slices over workgroups + second pass (tiles on less than half of the
  * compute units), 4 weight-streaming
- * kernel (a short A against [N,K] weights), 5 tiles of 128 x 128 with 4 waves
+ * kernel (up to 128 rows of A against wide weights in either layout; bn = 64:
+ * the 8-wave kernel with the LDS ring, with split_k > 1 followed by the second
+ * pass), 5 tiles of 128 x 128 with 4 waves
  * of 64 x 64 (problems of few 256 x 256 tiles; with split_k > 1 kind 3 is
  * reported and bm = bn = 128 tells).
  *
